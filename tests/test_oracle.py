@@ -1,0 +1,162 @@
+"""Pins the CPU oracle: four independent restatements against each other, against
+finite differences, and against what the mathematics fixes.  The reference holds no
+golden vectors for this path (its test_fastmax.py only times), so these checks are
+what stands between a plausible mistake and a green parity suite."""
+import itertools
+
+import pytest
+import torch
+
+from oracle import fastmax_oracle as O
+
+torch.set_default_dtype(torch.float32)
+
+CFG = list(itertools.product([False, True], [False, True], [1, 2]))  # mask, normalize, p
+
+
+def _rand(shape, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(shape, generator=g, dtype=torch.float64) for _ in range(4)]
+
+
+@pytest.mark.parametrize("mask,normalize,p", CFG)
+def test_dense_equals_bruteforce_on_reference_demo_shape(mask, normalize, p):
+    # (b,h,n,d) = (2,2,3,2) is the reference's demo shape (example.py:227-230)
+    q, k, v, _ = _rand((2, 2, 3, 2), seed=1)
+    kw = dict(mask=mask, normalize=normalize, a0=0.7, a1=1.3, a2=0.4, lim=1.5, p=p)
+    torch.testing.assert_close(O.fastmax_dense(q, k, v, **kw), O.fastmax_bruteforce(q, k, v, **kw),
+                               rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("mask,normalize,p", CFG)
+def test_reference_form_equals_dense(mask, normalize, p):
+    q, k, v, _ = _rand((2, 3, 17, 8), seed=2)
+    kw = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=p)
+    a = O.fastmax_reference_form(q, k, v, mask=mask, normalize=normalize, **kw)
+    b = O.fastmax_dense(q, k, v, mask=mask, normalize=normalize, **kw)
+    torch.testing.assert_close(a, b, rtol=1e-11, atol=1e-12)
+
+
+def test_reference_form_ignores_temperature():
+    # example.py:102 and :110-111 force temperature to 1 on both branches
+    q, k, v, _ = _rand((1, 2, 9, 4), seed=3)
+    a = O.fastmax_reference_form(q, k, v, mask=1, normalize=0, temperature=7.0)
+    b = O.fastmax_reference_form(q, k, v, mask=1, normalize=0, temperature=1.0)
+    assert torch.equal(a, b)
+
+
+def test_reference_form_rejects_bad_p():
+    q, k, v, _ = _rand((1, 1, 3, 2))
+    with pytest.raises(ValueError):
+        O.fastmax_reference_form(q, k, v, p=3)
+    with pytest.raises(ValueError):
+        O.fastmax_dense(q, k, v, p=3)
+
+
+@pytest.mark.parametrize("mask,normalize,p", CFG)
+def test_three_gradients_agree(mask, normalize, p):
+    q, k, v, go = _rand((2, 2, 13, 6), seed=4)
+    kw = dict(mask=mask, normalize=normalize, a0=0.9, a1=1.1, a2=0.6, lim=1.2, p=p)
+    _, dq1, dk1, dv1 = O.fastmax_grads_autograd(O.fastmax_dense, q, k, v, go, **kw)
+    _, dq2, dk2, dv2 = O.fastmax_grads_autograd(O.fastmax_reference_form, q, k, v, go, **kw)
+    dq3, dk3, dv3 = O.fastmax_grads_closed(q, k, v, go, **kw)
+    for a, b, c in ((dq1, dq2, dq3), (dk1, dk2, dk3), (dv1, dv2, dv3)):
+        torch.testing.assert_close(a, b, rtol=1e-9, atol=1e-11)
+        torch.testing.assert_close(a, c, rtol=1e-9, atol=1e-11)
+
+
+@pytest.mark.parametrize("mask,normalize", [(False, False), (True, True)])
+def test_gradcheck_dense(mask, normalize):
+    q, k, v, _ = _rand((1, 2, 5, 3), seed=5)
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    fn = lambda a, b, c: O.fastmax_dense(a, b, c, mask=mask, normalize=normalize, lim=1.3)
+    assert torch.autograd.gradcheck(fn, (q, k, v), eps=1e-6, atol=1e-6, rtol=1e-5)
+
+
+def test_adjoint_identity_by_finite_difference():
+    q, k, v, go = _rand((1, 2, 11, 4), seed=6)
+    kw = dict(mask=True, normalize=True, lim=0.8, p=2)
+    dq, dk, dv = O.fastmax_grads_closed(q, k, v, go, **kw)
+    g = torch.Generator().manual_seed(7)
+    eq, ek, ev = (torch.randn(q.shape, generator=g, dtype=torch.float64) for _ in range(3))
+    h = 1e-6
+    op = O.fastmax_dense(q + h * eq, k + h * ek, v + h * ev, **kw)
+    om = O.fastmax_dense(q - h * eq, k - h * ek, v - h * ev, **kw)
+    lhs = ((op - om) / (2 * h) * go).sum()
+    rhs = (dq * eq).sum() + (dk * ek).sum() + (dv * ev).sum()
+    assert abs(float(lhs - rhs)) < 1e-7 * max(1.0, abs(float(rhs)))
+
+
+# ---------------------------------------------------------------- invariants
+def test_constant_values_give_constant_output():
+    q, k, _, _ = _rand((2, 2, 9, 4), seed=8)
+    v = torch.full((2, 2, 9, 4), 3.25, dtype=torch.float64)
+    for mask in (False, True):
+        o = O.fastmax_dense(q, k, v, mask=mask, normalize=True)
+        torch.testing.assert_close(o, v, rtol=1e-12, atol=1e-12)
+
+
+def test_a1_a2_zero_is_running_mean():
+    q, k, v, _ = _rand((1, 2, 10, 4), seed=9)
+    o = O.fastmax_dense(q, k, v, mask=True, a0=2.0, a1=0.0, a2=0.0)
+    want = torch.cumsum(v, 2) / torch.arange(1, 11, dtype=torch.float64)[None, None, :, None]
+    torch.testing.assert_close(o, want, rtol=1e-12, atol=1e-12)
+    o = O.fastmax_dense(q, k, v, mask=False, a0=2.0, a1=0.0, a2=0.0)
+    torch.testing.assert_close(o, v.mean(2, keepdim=True).expand_as(v), rtol=1e-12, atol=1e-12)
+
+
+def test_single_token_returns_value():
+    q, k, v, _ = _rand((2, 1, 1, 4), seed=10)
+    for mask in (False, True):
+        torch.testing.assert_close(O.fastmax_dense(q, k, v, mask=mask, normalize=True), v)
+    # causal: the first row only ever sees itself
+    q, k, v, _ = _rand((1, 1, 6, 4), seed=11)
+    torch.testing.assert_close(O.fastmax_dense(q, k, v, mask=True)[..., 0, :], v[..., 0, :])
+
+
+def test_a2_zero_equals_p1():
+    q, k, v, _ = _rand((1, 2, 9, 4), seed=12)
+    for mask in (False, True):
+        a = O.fastmax_dense(q, k, v, mask=mask, normalize=True, a2=0.0, p=2)
+        b = O.fastmax_dense(q, k, v, mask=mask, normalize=True, a2=0.5, p=1)
+        torch.testing.assert_close(a, b, rtol=1e-13, atol=1e-13)
+
+
+def test_normalize_is_scale_invariant_and_bounds_scores():
+    q, k, v, _ = _rand((1, 2, 9, 4), seed=13)
+    a = O.fastmax_dense(q, k, v, mask=True, normalize=True)
+    b = O.fastmax_dense(3.0 * q, 0.25 * k, v, mask=True, normalize=True)
+    torch.testing.assert_close(a, b, rtol=1e-12, atol=1e-12)
+    qh, kh = O.normalize_qk(q, k, 1.0)
+    assert float(torch.linalg.norm(qh, dim=3).max()) == pytest.approx(1.0, abs=1e-12)
+    assert float((qh @ kh.transpose(-1, -2)).abs().max()) <= 1.0 + 1e-12
+
+
+def test_default_coefficients_keep_denominator_positive():
+    q, k, v, _ = _rand((1, 2, 12, 4), seed=14)
+    _, den = O.fastmax_dense(q, k, v, mask=True, normalize=True, return_den=True)
+    counts = torch.arange(1, 13, dtype=torch.float64)
+    assert bool((den >= counts / 2 - 1e-12).all())  # f(s) = ((s+1)^2+1)/2 >= 1/2
+
+
+def test_unmasked_is_permutation_equivariant():
+    q, k, v, _ = _rand((1, 1, 8, 4), seed=15)
+    perm = torch.randperm(8, generator=torch.Generator().manual_seed(1))
+    a = O.fastmax_dense(q, k, v, normalize=True)
+    b = O.fastmax_dense(q[:, :, perm], k[:, :, perm], v[:, :, perm], normalize=True)
+    torch.testing.assert_close(a[:, :, perm], b, rtol=1e-12, atol=1e-12)
+    # keys/values alone may be permuted freely
+    c = O.fastmax_dense(q, k[:, :, perm], v[:, :, perm], normalize=True)
+    torch.testing.assert_close(a, c, rtol=1e-12, atol=1e-12)
+
+
+def test_three_d_layout_matches_four_d():
+    q, k, v, go = _rand((2, 3, 7, 4), seed=16)
+    kw = dict(mask=True, normalize=True)
+    o4 = O.fastmax_dense(q, k, v, **kw)
+    o3 = O.fastmax_dense(q.reshape(6, 7, 4), k.reshape(6, 7, 4), v.reshape(6, 7, 4), **kw)
+    torch.testing.assert_close(o4.reshape(6, 7, 4), o3)
+    d4 = O.fastmax_grads_closed(q, k, v, go, **kw)
+    d3 = O.fastmax_grads_closed(*(t.reshape(6, 7, 4) for t in (q, k, v, go)), **kw)
+    for a, b in zip(d4, d3):
+        torch.testing.assert_close(a.reshape(6, 7, 4), b)
