@@ -1,0 +1,204 @@
+#!/usr/bin/env python3
+"""Headline benchmark: Fastmax attention forward + backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one forward + one backward pass of the attention operator over one batch of
+synthetic q, k, v and upstream gradient already resident in HBM, called through the C ABI
+(include/fastmax_amd.h).  Prints ONE JSON line: whole-job tokens/s (tokens = B*N per step),
+the roofline position of the dominant kernel (algorithmic flops / HIP-event kernel time,
+against the fp32 MFMA peak) and a CPU baseline (the oracle's reference-form restatement of
+the reference's PyTorch path, timed on a bounded sample on this host's cores).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published dense peaks
+PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0}
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # BASELINE.json configs[2]: the shape the metric is quoted on (causal, p=2, fp32)
+    "headline": dict(B=64, H=16, N=10000, D=64, mask=True, p=2, dtype="f32"),
+    "headline-unmasked": dict(B=64, H=16, N=10000, D=64, mask=False, p=2, dtype="f32"),
+    "headline-p1": dict(B=64, H=16, N=10000, D=64, mask=True, p=1, dtype="f32"),
+    "c1": dict(B=8, H=8, N=1024, D=32, mask=False, p=2, dtype="f32"),
+    "c2": dict(B=64, H=8, N=1000, D=32, mask=True, p=2, dtype="f32"),
+    "c4": dict(B=16, H=32, N=16384, D=64, mask=True, p=2, dtype="bf16"),
+}
+COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
+
+
+def algorithmic_flops(d: int, p: int) -> dict:
+    """Per token-head, un-symmetrised reference form (1 MAC = 2 flop)."""
+    feat = 1 + d + (d * d if p == 2 else 0)
+    return {
+        "build": 2 * feat * (d + 1),              # one moment state (prefix or suffix)
+        "fwd_apply": 2 * feat * (d + 1),
+        "bwd_dq": 2 * (feat - 1) * (d + 1),
+        "bwd_dkdv": 2 * (feat - 1) * (d + 1) + 2 * feat * d,
+        "fwd": 4 * feat * (d + 1),
+        "bwd": 2 * (2 * feat * (d + 1) + 2 * (feat - 1) * (d + 1) + feat * d),
+    }
+
+
+def cpu_baseline(cfg: dict, seconds_hint: float) -> dict:
+    """Reference-form fwd+bwd (oracle/fastmax_oracle.py::fastmax_reference_form, the op sequence of
+    the reference's fastmax_function) on one head and a token prefix that fits in memory."""
+    import torch
+    from oracle import fastmax_oracle as O
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    d, p, mask = cfg["D"], cfg["p"], cfg["mask"]
+    # the causal p=2 reference form materialises n*d^2*d floats (and its cumsum)
+    per_tok_bytes = 4 * (d * d * d if p == 2 else d * d) * (6 if mask else 1) + 64 * d * d
+    n_s = int(min(cfg["N"], max(64, (6 << 30) // per_tok_bytes)))
+    q, k, v, go = O.seeded_inputs((1, 1, n_s, d), seed=0)
+    kw = dict(mask=int(mask), normalize=1, a0=COEF["a0"], a1=COEF["a1"], a2=COEF["a2"], lim=COEF["lim"], p=p)
+
+    def step():
+        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = O.fastmax_reference_form(qq, kk, vv, **kw)
+        out.backward(go)
+
+    step()  # warm-up
+    reps, t_tot = 0, 0.0
+    while reps < 3 or (t_tot < seconds_hint and reps < 50):
+        t0 = time.perf_counter()
+        step()
+        t_tot += time.perf_counter() - t0
+        reps += 1
+    t = t_tot / reps
+    token_heads_per_s = n_s / t
+    return {
+        "value": token_heads_per_s / cfg["H"],
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": (f"reference-form fp32 fwd+bwd (autograd) on 1 of {cfg['B'] * cfg['H']} heads, first {n_s} of "
+                   f"{cfg['N']} tokens, {reps} reps of {t:.3f} s; cost is linear in tokens and heads, so "
+                   f"tokens/s = ({n_s}/t)/H"),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures ONE GPU; heads are independent, so N GPUs would each run "
+              "bh/N heads with no communication. Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+    from fastmax_amd import _cabi, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    cfg = WORKLOADS[args.workload]
+    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
+    bh = B * H
+    dtype = torch.float32 if cfg["dtype"] == "f32" else torch.bfloat16
+    dev = torch.device("cuda:0")
+    lib = _cabi.load()
+
+    gen = torch.Generator(device=dev).manual_seed(0)
+    q, k, v, go = (torch.randn((bh, N, D), generator=gen, device=dev, dtype=torch.float32).to(dtype)
+                   for _ in range(4))
+    kw = dict(mask=cfg["mask"], normalize=COEF["normalize"], lim=COEF["lim"], temperature=COEF["temperature"],
+              a0=COEF["a0"], a1=COEF["a1"], a2=COEF["a2"], p=cfg["p"])
+
+    def fwd():
+        return ops.forward(q, k, v, **kw)
+
+    def step():
+        o, den, sc, arg = fwd()
+        return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _cabi.check(lib.fastmax_profile_begin())
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kt = _cabi.KernelTimes()
+    _cabi.check(lib.fastmax_profile_end(C.byref(kt)))
+    ms_step = (t1 - t0) * 1e3 / args.steps
+
+    # forward alone, same inputs
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fwd()
+    torch.cuda.synchronize()
+    ms_fwd = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    fl = algorithmic_flops(D, cfg["p"])
+    token_heads = bh * N
+    kernels = {}
+    for i, name in enumerate(_cabi.KERNEL_NAMES):
+        if kt.launches[i]:
+            kernels[name] = {"ms_per_step": kt.ms[i] / args.steps, "launches_per_step": kt.launches[i] / args.steps}
+    # algorithmic flops each kernel class executes per step (build runs 3x: fwd prefix, bwd prefix, bwd suffix)
+    per_step_flops = {"build": 3 * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
+                      "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dkdv": fl["bwd_dkdv"] * token_heads}
+    dom = max(per_step_flops, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0))
+    dom_ms = kernels[dom]["ms_per_step"]
+    launches = kernels[dom]["launches_per_step"]
+    achieved = per_step_flops[dom] / (dom_ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS["f32"]  # every contraction runs on v_mfma_f32_32x32x2f32, also for bf16 inputs
+    roofline = {
+        "bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
+        "frac": achieved / peak, "traffic": None,
+        "flops_per_launch": per_step_flops[dom] / launches, "avg_launch_ms": dom_ms / launches,
+    }
+    for name, f in per_step_flops.items():
+        if name in kernels:
+            kernels[name]["algorithmic_tflops"] = f / (kernels[name]["ms_per_step"] * 1e-3) / 1e12
+
+    result = {
+        "metric": "fwd+bwd tokens/sec and MFMA % of peak at B64 H16 N10000 D64 p2, 1 GPU",
+        "value": B * N / (ms_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": cfg["dtype"], "data": "synthetic",
+        "config": {"workload": f"{args.workload}: Fastmax {'causal' if cfg['mask'] else 'unmasked'} fwd+bwd, "
+                               f"B={B} H={H} N={N} D={D} p={cfg['p']} {cfg['dtype']}, normalize lim=1, "
+                               "a=(1,1,0.5), q/k/v/grad iid N(0,1) seed 0"},
+        "fwd_ms": ms_fwd, "fwd_tokens_per_s": B * N / (ms_fwd * 1e-3),
+        "fwd_tflops": fl["fwd"] * token_heads / (ms_fwd * 1e-3) / 1e12,
+        "fwd_bwd_tflops": (fl["fwd"] + fl["bwd"]) * token_heads / (ms_step * 1e-3) / 1e12,
+        "mfma_frac_of_peak_fwd_bwd": (fl["fwd"] + fl["bwd"]) * token_heads / (ms_step * 1e-3) / 1e12 / peak,
+        "kernels": kernels,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        del q, k, v, go
+        result["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,12 @@
+"""Fastmax polynomial-kernel linear attention on MI355X (gfx950).
+
+    from fastmax_amd import FASTMultiHeadAttention, fastmax_custom
+
+mirrors the reference's operator API; the C ABI underneath is include/fastmax_amd.h.
+"""
+from .attention import (FASTMultiHeadAttention, FASTMultiHeadAttention_Function, fastmax_custom,
+                        fastmax_function)
+from ._ext import install_as_fastmax_cuda
+
+__all__ = ["FASTMultiHeadAttention", "FASTMultiHeadAttention_Function", "fastmax_custom",
+           "fastmax_function", "install_as_fastmax_cuda"]

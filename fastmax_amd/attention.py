@@ -1,0 +1,157 @@
+"""Operator API of the reference, on the MI355X kernels.
+
+Mirrors example.py:6-223 / model.py:20-218 of the reference: the autograd Function
+`FASTMultiHeadAttention_Function`, the pure-PyTorch `fastmax_function`, the module
+`FASTMultiHeadAttention` and the ready-made instance `fastmax_custom`, with the same
+argument names, order and defaults.
+
+Differences from the reference, all deliberate:
+  * the kernels also serve mask=False (example.py:220 sends that to the PyTorch path);
+  * q and k are never modified; the gradient flows through the normalisation, as autograd
+    does for the reference's PyTorch path (the reference kernels skip that chain rule);
+  * CPU tensors with use_custom_gradient=True raise (the reference returns q unchanged,
+    example.py:10-12);
+  * bfloat16 inputs are accepted (fp32 arithmetic inside).
+"""
+from __future__ import annotations
+
+
+import torch
+
+from . import _ext
+
+
+class FASTMultiHeadAttention_Function(torch.autograd.Function):
+    """Same call signature as example.py:8 / model.py:22."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, drop_noise=None, mask=False, dropout=0.0, normalize=False, temperature=1.0,
+                a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=2):
+        ext = _ext.load()
+        if not q.is_cuda:
+            raise RuntimeError("FASTMultiHeadAttention_Function needs GPU tensors; "
+                               "use FASTMultiHeadAttention(use_custom_gradient=False) on the CPU")
+        if q.dim() not in (3, 4):
+            raise ValueError("q, k, and v should be either 3 or 4 dimensional tensors. "
+                             "If 3D: (b*h,n,d), if 4D: (b,h,n,d).")
+        shape = q.shape
+        q3 = q.reshape(-1, q.shape[-2], q.shape[-1]).contiguous()
+        k3 = k.reshape(-1, k.shape[-2], k.shape[-1]).contiguous()
+        v3 = v.reshape(-1, v.shape[-2], v.shape[-1]).contiguous()
+        o, den, scale, arg = ext.forward_ex(q3, k3, v3, bool(mask), bool(normalize), float(temperature),
+                                            float(a0), float(a1), float(a2), float(lim), int(p))
+        noise = None
+        out = o
+        if dropout and dropout > 0.0:
+            if drop_noise is None:
+                raise ValueError("dropout > 0 needs drop_noise (a standard-normal tensor shaped like q)")
+            # multiplicative Gaussian noise on the output, fastmax_cuda_forward.cu:271-280
+            noise = 1.0 + float(dropout) * drop_noise.reshape(q3.shape).to(o.dtype)
+            out = o * noise
+        ctx.save_for_backward(q3, k3, v3, o, den, scale, arg, noise if noise is not None else o.new_empty(0))
+        ctx.cfg = (bool(mask), bool(normalize), float(temperature), float(a0), float(a1), float(a2), float(lim), int(p))
+        ctx.kshape, ctx.vshape = k.shape, v.shape
+        return out.reshape(shape)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        ext = _ext.load()
+        q3, k3, v3, o, den, scale, arg, noise = ctx.saved_tensors
+        mask, normalize, temperature, a0, a1, a2, lim, p = ctx.cfg
+        go = grad_output.reshape(q3.shape)
+        if noise.numel():
+            go = go * noise
+        go = go.contiguous()
+        dq, dk, dv = ext.backward_ex(q3, k3, v3, o, den, go, scale, arg, mask, normalize, temperature,
+                                     a0, a1, a2, lim, p)
+        return (dq.reshape(grad_output.shape), dk.reshape(ctx.kshape), dv.reshape(ctx.vshape),
+                None, None, None, None, None, None, None, None, None, None)
+
+
+def fastmax_function(q, k, v, mask=0, dropout_rate=0.0, normalize=0, temperature=1, a0=1, a1=1, a2=0.5,
+                     lim=1, p=2, chunk: int = 128):
+    """Pure-PyTorch Fastmax with the semantics of the reference's fastmax_function
+    (example.py:83-197): (b,h,n,d) inputs, normalisation by the per-head max row norm,
+    temperature without effect (example.py:102,110-111), dropout on the k (x) k / q (x) q
+    features for p=2 and on k / q for p=1.  Unlike the reference it never materialises the
+    (b,h,n,d^2,d) cumulative sum: the causal case walks `chunk`-token blocks, carrying the
+    moment state between blocks and using the masked polynomial score inside a block.
+    Differentiable by autograd; runs on any device.
+    """
+    if p not in (1, 2):
+        raise ValueError(f"p must be 1 or 2, got: {p}")
+    if normalize:
+        qn = torch.linalg.norm(q, dim=3)
+        kn = torch.linalg.norm(k, dim=3)
+        q = lim * q / qn.amax(dim=2)[..., None, None]
+        k = lim * k / kn.amax(dim=2)[..., None, None]
+    drop = torch.nn.Dropout(p=dropout_rate)
+
+    def feats(x):
+        if p == 2:
+            return x, drop((x.unsqueeze(-1) * x.unsqueeze(-2)).flatten(-2))
+        return drop(x), None
+
+    b, h, n, d = q.shape
+    if not mask:
+        k1, k2 = feats(k)
+        q1, q2 = feats(q)
+        num = a0 * v.sum(-2, keepdim=True) + a1 * (q1 @ (k1.transpose(-1, -2) @ v))
+        den = a0 * k.shape[2] + a1 * (q1 @ k1.sum(-2).unsqueeze(-1))
+        if p == 2:
+            num = num + a2 * (q2 @ (k2.transpose(-1, -2) @ v))
+            den = den + a2 * (q2 @ k2.sum(-2).unsqueeze(-1))
+        return num / den
+
+    outs = []
+    s0 = v.new_zeros(b, h, 1, d)
+    s1 = v.new_zeros(b, h, d, d)
+    z1 = v.new_zeros(b, h, d, 1)
+    s2 = v.new_zeros(b, h, d * d, d) if p == 2 else None
+    z2 = v.new_zeros(b, h, d * d, 1) if p == 2 else None
+    count = 0
+    for t0 in range(0, n, chunk):
+        qc, kc, vc = q[:, :, t0:t0 + chunk], k[:, :, t0:t0 + chunk], v[:, :, t0:t0 + chunk]
+        c = qc.shape[2]
+        k1, k2 = feats(kc)
+        q1, q2 = feats(qc)
+        s = q1 @ k1.transpose(-1, -2)
+        f = a0 + a1 * s
+        if p == 2:
+            f = f + a2 * (q2 @ k2.transpose(-1, -2))
+        f = torch.tril(f)
+        num = f @ vc + a0 * s0 + a1 * (q1 @ s1)
+        den = f.sum(-1, keepdim=True) + a0 * count + a1 * (q1 @ z1)
+        if p == 2:
+            num = num + a2 * (q2 @ s2)
+            den = den + a2 * (q2 @ z2)
+        outs.append(num / den)
+        s0 = s0 + vc.sum(-2, keepdim=True)
+        s1 = s1 + k1.transpose(-1, -2) @ vc
+        z1 = z1 + k1.sum(-2).unsqueeze(-1)
+        if p == 2:
+            s2 = s2 + k2.transpose(-1, -2) @ vc
+            z2 = z2 + k2.sum(-2).unsqueeze(-1)
+        count += c
+    return torch.cat(outs, dim=2)
+
+
+class FASTMultiHeadAttention(torch.nn.Module):
+    """Same constructor and forward signature as example.py:214-221."""
+
+    def __init__(self, use_custom_gradient=True):
+        super().__init__()
+        self.use_custom_gradient = use_custom_gradient
+
+    def forward(self, q, k, v, drop_noise=None, mask=False, dropout=0.0, normalize=False, temperature=1.0,
+                a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=2):
+        if self.use_custom_gradient:
+            return FASTMultiHeadAttention_Function.apply(q, k, v, drop_noise, mask, dropout, normalize,
+                                                         temperature, a0, a1, a2, lim, p)
+        if q.dim() == 3:
+            return fastmax_function(q[None], k[None], v[None], mask, dropout, normalize, temperature,
+                                    a0, a1, a2, lim, p)[0]
+        return fastmax_function(q, k, v, mask, dropout, normalize, temperature, a0, a1, a2, lim, p)
+
+
+fastmax_custom = FASTMultiHeadAttention()

@@ -1,0 +1,204 @@
+// PyTorch-ROCm binding of the Fastmax C ABI.  The module is named `fastmax_cuda` and exports
+// `forwardpass` / `backwardpass` with the positional signatures of the reference extension
+// (fastmax_cuda.cpp:17-37, minus the rpe_matrix argument the live kernels do not take:
+// fastmax_cuda_forward.cu:297-314), so the reference's autograd Function runs on it unchanged.
+// `forward_ex` / `backward_ex` are the non-mutating entry points the package's own autograd
+// Function uses: they differentiate through the normalisation and accept bf16.
+//
+// Host code only: tensors, the current stream and the device guard come from torch; all device
+// work happens behind include/fastmax_amd.h.
+#include <c10/hip/HIPGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/extension.h>
+
+#include <vector>
+
+#include "fastmax_amd.h"
+
+namespace {
+
+#define CHECK_GPU(x) TORCH_CHECK(x.device().is_cuda(), #x " must be a CUDA tensor")
+#define CHECK_CONTIGUOUS(x) TORCH_CHECK(x.is_contiguous(), #x " must be contiguous")
+#define CHECK_INPUT(x) \
+  CHECK_GPU(x);        \
+  CHECK_CONTIGUOUS(x)
+
+void raise_on(int rc) { TORCH_CHECK(rc == FASTMAX_OK, "fastmax: ", fastmax_last_error(), " (code ", rc, ")"); }
+
+fastmax_desc make_desc(const torch::Tensor& q, const torch::Tensor& k, bool mask, bool normalize,
+                       double temperature, double a0, double a1, double a2, double lim, int64_t p) {
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3, "q, k, v must be (b*h, n, d)");
+  TORCH_CHECK(q.scalar_type() == torch::kFloat32 || q.scalar_type() == torch::kBFloat16,
+              "q must be float32 or bfloat16");
+  fastmax_desc ds;
+  ds.bh = (int32_t)q.size(0);
+  ds.bhkv = (int32_t)k.size(0);
+  ds.nq = (int32_t)q.size(1);
+  ds.nk = (int32_t)k.size(1);
+  ds.d = (int32_t)q.size(2);
+  ds.dtype = q.scalar_type() == torch::kFloat32 ? FASTMAX_F32 : FASTMAX_BF16;
+  ds.mask = mask;
+  ds.normalize = normalize;
+  ds.p = (int32_t)p;
+  ds.lim = (float)lim;
+  ds.temperature = (float)temperature;
+  ds.a0 = (float)a0;
+  ds.a1 = (float)a1;
+  ds.a2 = (float)a2;
+  raise_on(fastmax_check_desc(&ds));
+  return ds;
+}
+
+void check_same(const torch::Tensor& a, const torch::Tensor& b, const char* what) {
+  TORCH_CHECK(a.scalar_type() == b.scalar_type() && a.device() == b.device(), what,
+              " must share dtype and device with q");
+}
+
+torch::Tensor workspace(const fastmax_desc& ds, int pass, const torch::Tensor& like, size_t* bytes) {
+  *bytes = fastmax_workspace_bytes(&ds, pass);
+  TORCH_CHECK(*bytes > 0, "fastmax: ", fastmax_last_error());
+  return torch::empty({(int64_t)*bytes}, like.options().dtype(torch::kUInt8));
+}
+
+fastmax_stream_t current_stream(const torch::Tensor& t) {
+  return reinterpret_cast<fastmax_stream_t>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+// (o, den, qk_scale, qk_argmax); o is (bh, n, d)
+std::vector<torch::Tensor> forward_ex(torch::Tensor q, torch::Tensor k, torch::Tensor v, bool mask,
+                                      bool normalize, double temperature, double a0, double a1,
+                                      double a2, double lim, int64_t p) {
+  CHECK_INPUT(q);
+  CHECK_INPUT(k);
+  CHECK_INPUT(v);
+  check_same(q, k, "k");
+  check_same(q, v, "v");
+  TORCH_CHECK(k.sizes() == v.sizes(), "k and v must have the same shape");
+  const fastmax_desc ds = make_desc(q, k, mask, normalize, temperature, a0, a1, a2, lim, p);
+  const c10::hip::HIPGuard guard(q.device());
+  auto o = torch::empty_like(q);
+  auto den = torch::empty({q.size(0), q.size(1)}, q.options().dtype(torch::kFloat32));
+  auto scale = torch::empty({2 * q.size(0)}, q.options().dtype(torch::kFloat32));
+  auto arg = torch::empty({2 * q.size(0)}, q.options().dtype(torch::kInt32));
+  size_t wsb = 0;
+  auto ws = workspace(ds, FASTMAX_PASS_FORWARD, q, &wsb);
+  raise_on(fastmax_forward(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ds.d,
+                           den.data_ptr<float>(), 1, scale.data_ptr<float>(), arg.data_ptr<int32_t>(),
+                           ws.data_ptr(), wsb, current_stream(q)));
+  return {o, den, scale, arg};
+}
+
+std::vector<torch::Tensor> backward_ex(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                                       torch::Tensor o, torch::Tensor den, torch::Tensor go,
+                                       torch::Tensor scale, torch::Tensor arg, bool mask,
+                                       bool normalize, double temperature, double a0, double a1,
+                                       double a2, double lim, int64_t p) {
+  CHECK_INPUT(q);
+  CHECK_INPUT(k);
+  CHECK_INPUT(v);
+  CHECK_INPUT(o);
+  CHECK_INPUT(den);
+  CHECK_INPUT(go);
+  CHECK_INPUT(scale);
+  CHECK_INPUT(arg);
+  check_same(q, k, "k");
+  check_same(q, v, "v");
+  check_same(q, o, "o");
+  check_same(q, go, "grad_output");
+  TORCH_CHECK(o.sizes() == q.sizes() && go.sizes() == q.sizes(), "o and grad_output must be shaped like q");
+  TORCH_CHECK(den.scalar_type() == torch::kFloat32 && den.numel() == q.size(0) * q.size(1), "den must be float32 (bh, n)");
+  TORCH_CHECK(scale.scalar_type() == torch::kFloat32 && scale.numel() == 2 * q.size(0), "qk_scale must be float32 (2*bh)");
+  TORCH_CHECK(arg.scalar_type() == torch::kInt32 && arg.numel() == 2 * q.size(0), "qk_argmax must be int32 (2*bh)");
+  const fastmax_desc ds = make_desc(q, k, mask, normalize, temperature, a0, a1, a2, lim, p);
+  const c10::hip::HIPGuard guard(q.device());
+  auto dq = torch::empty_like(q);
+  auto dk = torch::empty_like(k);
+  auto dv = torch::empty_like(v);
+  size_t wsb = 0;
+  auto ws = workspace(ds, FASTMAX_PASS_BACKWARD, q, &wsb);
+  raise_on(fastmax_backward(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ds.d,
+                            den.data_ptr<float>(), 1, go.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                            dv.data_ptr(), scale.data_ptr<float>(), arg.data_ptr<int32_t>(),
+                            ws.data_ptr(), wsb, current_stream(q)));
+  return {dq, dk, dv};
+}
+
+// Reference signature and side effects (fastmax_cuda.cpp:17-24, fastmax_cuda_forward.cu:366-399):
+// k is divided by temperature and q, k are normalised IN PLACE, so that the caller's saved
+// q, k are the ones backwardpass expects; the result is (bh, n, d+1) with the row denominators
+// in column d; dropout > 0 multiplies the output by 1 + dropout * drop_noise.
+torch::Tensor forwardpass(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor drop_noise,
+                          bool mask, double dropout, bool normalize, double temperature, double a0,
+                          double a1, double a2, double lim, int64_t p) {
+  CHECK_INPUT(q);
+  CHECK_INPUT(k);
+  CHECK_INPUT(v);
+  check_same(q, k, "k");
+  check_same(q, v, "v");
+  TORCH_CHECK(q.scalar_type() == torch::kFloat32, "forwardpass takes float32 tensors (use forward_ex for bfloat16)");
+  TORCH_CHECK(k.sizes() == v.sizes(), "k and v must have the same shape");
+  fastmax_desc ds = make_desc(q, k, mask, normalize, 1.0, a0, a1, a2, lim, p);
+  const c10::hip::HIPGuard guard(q.device());
+  const fastmax_stream_t stream = current_stream(q);
+  if (temperature != 1.0) k.div_(temperature);
+  if (normalize) {
+    auto nws = torch::empty({16 * (int64_t)ds.bh + 1024}, q.options().dtype(torch::kUInt8));
+    raise_on(fastmax_normalize_inplace(&ds, q.data_ptr(), k.data_ptr(), nws.data_ptr(), (size_t)nws.numel(), stream));
+    ds.normalize = 0;
+  }
+  const int64_t d = q.size(2);
+  auto o = torch::empty({q.size(0), q.size(1), d + 1}, q.options());
+  size_t wsb = 0;
+  auto ws = workspace(ds, FASTMAX_PASS_FORWARD, q, &wsb);
+  raise_on(fastmax_forward(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d + 1,
+                           o.data_ptr<float>() + d, d + 1, nullptr, nullptr, ws.data_ptr(), wsb, stream));
+  if (dropout > 0.0) {
+    TORCH_CHECK(drop_noise.defined() && drop_noise.sizes() == q.sizes(), "drop_noise must be shaped like q");
+    o.narrow(2, 0, d).mul_(drop_noise * dropout + 1.0);
+  }
+  return o;
+}
+
+// Reference signature (fastmax_cuda.cpp:26-32): q, k as left by forwardpass (already scaled),
+// o with the denominator column; no gradient flows through the normalisation here, exactly
+// like the reference kernels (fastmax_cuda_backward.cu:900-1006).  grad_output is not modified.
+std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch::Tensor v,
+                                        torch::Tensor o, torch::Tensor grad_output, bool mask,
+                                        double a0, double a1, double a2, int64_t p) {
+  CHECK_INPUT(q);
+  CHECK_INPUT(k);
+  CHECK_INPUT(v);
+  CHECK_INPUT(o);
+  CHECK_INPUT(grad_output);
+  check_same(q, k, "k");
+  check_same(q, v, "v");
+  check_same(q, o, "o");
+  check_same(q, grad_output, "grad_output");
+  TORCH_CHECK(q.scalar_type() == torch::kFloat32, "backwardpass takes float32 tensors (use backward_ex for bfloat16)");
+  const int64_t d = q.size(2);
+  TORCH_CHECK(o.dim() == 3 && o.size(0) == q.size(0) && o.size(1) == q.size(1) && o.size(2) == d + 1,
+              "o must be the (bh, n, d+1) tensor forwardpass returned");
+  TORCH_CHECK(grad_output.sizes() == q.sizes(), "grad_output must be shaped like q");
+  const fastmax_desc ds = make_desc(q, k, mask, false, 1.0, a0, a1, a2, 1.0, p);
+  const c10::hip::HIPGuard guard(q.device());
+  auto dq = torch::empty_like(q);
+  auto dk = torch::empty_like(k);
+  auto dv = torch::empty_like(v);
+  size_t wsb = 0;
+  auto ws = workspace(ds, FASTMAX_PASS_BACKWARD, q, &wsb);
+  raise_on(fastmax_backward(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d + 1,
+                            o.data_ptr<float>() + d, d + 1, grad_output.data_ptr(), dq.data_ptr(),
+                            dk.data_ptr(), dv.data_ptr(), nullptr, nullptr, ws.data_ptr(), wsb,
+                            current_stream(q)));
+  return {dq, dk, dv};
+}
+
+}  // namespace
+
+PYBIND11_MODULE(fastmax_cuda, m) {
+  m.def("forwardpass", &forwardpass, "forwardpass");
+  m.def("backwardpass", &backwardpass, "backwardpass");
+  m.def("forward_ex", &forward_ex, "forward returning (o, den, qk_scale, qk_argmax)");
+  m.def("backward_ex", &backward_ex, "backward through the normalisation, returns [dq, dk, dv]");
+  m.def("version", []() { return std::string(fastmax_version()); });
+}

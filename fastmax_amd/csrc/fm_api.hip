@@ -1,0 +1,434 @@
+// C ABI of the gfx950 Fastmax library: argument checking, workspace carving, head batching
+// and kernel launches.  No torch, no allocation, no global mutable state.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <vector>
+
+#include "fastmax_amd.h"
+#include "fm_backward.h"
+#include "fm_forward.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// Optional per-thread kernel timing (fastmax_profile_begin/end): every launch is bracketed by
+// two HIP events on the caller's stream; nothing is synchronised until fastmax_profile_end.
+struct Profiler {
+  bool on = false;
+  std::vector<hipEvent_t> ev;   // start/stop pairs
+  std::vector<int> cls;
+  size_t used = 0;
+};
+thread_local Profiler g_prof;
+
+struct ScopedKernel {
+  hipStream_t st;
+  bool on;
+  ScopedKernel(int kclass, hipStream_t stream) : st(stream), on(g_prof.on) {
+    if (!on) return;
+    if (g_prof.used + 2 > g_prof.ev.size()) {
+      hipEvent_t a, b;
+      if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) {
+        on = false;
+        return;
+      }
+      g_prof.ev.push_back(a);
+      g_prof.ev.push_back(b);
+    }
+    g_prof.cls.push_back(kclass);
+    hipEventRecord(g_prof.ev[g_prof.used], st);
+  }
+  ~ScopedKernel() {
+    if (!on) return;
+    hipEventRecord(g_prof.ev[g_prof.used + 1], st);
+    g_prof.used += 2;
+  }
+};
+
+constexpr int kChunk = 256;                       // tokens between causal state snapshots
+constexpr size_t kWorkspaceBudget = 6ull << 30;   // what fastmax_workspace_bytes aims for
+
+struct Plan {
+  int d, p2, masked, n, bh;
+  int rtw, gsplit;     // build kernel: row tiles per wave, feature splits per head
+  int nslots, zlen;    // state slots per head; tokens per slot when unmasked
+  int nblk;            // 128-token blocks per head
+  int64_t state_floats;
+  size_t fixed_bytes;     // scale/argmax/cvec/rpart
+  size_t per_head_bytes;  // states of one head
+};
+
+int64_t state_floats_for(int d, int p2) {
+  return d == 64 ? Geo<64>::state_floats(p2) : Geo<32>::state_floats(p2);
+}
+
+size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+
+Plan make_plan(const fastmax_desc* ds, int pass) {
+  Plan pl;
+  pl.d = ds->d;
+  pl.p2 = ds->p == 2;
+  pl.masked = ds->mask != 0;
+  pl.n = ds->nq;
+  pl.bh = ds->bh;
+  const int rt_total = (pl.p2 ? (pl.d / 2 + 1) * (pl.d / 32) : 0) + pl.d / 32;
+  if (!pl.p2) pl.rtw = 1;
+  else pl.rtw = pl.d == 64 ? 3 : 5;
+  pl.gsplit = (rt_total + 4 * pl.rtw - 1) / (4 * pl.rtw);
+  pl.nblk = (pl.n + 127) / 128;
+  if (pl.masked) {
+    pl.nslots = (pl.n + kChunk - 1) / kChunk;
+    pl.zlen = 0;
+  } else {
+    // enough token splits to put ~1024 blocks in flight, at least 256 tokens each
+    int z = (1024 + pl.gsplit * pl.bh - 1) / (pl.gsplit * pl.bh);
+    const int zmax = (pl.n + 255) / 256;
+    if (z > zmax) z = zmax;
+    if (z < 1) z = 1;
+    int zlen = ((pl.n + z - 1) / z + 31) / 32 * 32;
+    pl.zlen = zlen;
+    pl.nslots = (pl.n + zlen - 1) / zlen;
+  }
+  pl.state_floats = state_floats_for(pl.d, pl.p2);
+  size_t fixed = align256((size_t)2 * pl.bh * sizeof(float)) + align256((size_t)2 * pl.bh * sizeof(int));
+  if (pass == FASTMAX_PASS_BACKWARD) {
+    fixed += align256((size_t)pl.bh * pl.n * sizeof(float));            // c_i
+    fixed += align256((size_t)2 * pl.bh * pl.nblk * sizeof(float));     // norm partials for q, k
+  }
+  pl.fixed_bytes = fixed;
+  pl.per_head_bytes = (size_t)pl.nslots * pl.state_floats * sizeof(float) *
+                      (pass == FASTMAX_PASS_BACKWARD ? 2 : 1);
+  return pl;
+}
+
+int check_desc(const fastmax_desc* ds) {
+  if (!ds) return fail(FASTMAX_E_NULL, "desc is NULL");
+  if (ds->dtype != FASTMAX_F32 && ds->dtype != FASTMAX_BF16)
+    return fail(FASTMAX_E_DTYPE, "dtype %d is neither FASTMAX_F32 nor FASTMAX_BF16", ds->dtype);
+  if (ds->d != 32 && ds->d != 64) return fail(FASTMAX_E_SHAPE, "d = %d; supported head dims are 32 and 64", ds->d);
+  if (ds->bh < 1 || ds->bh > 65535) return fail(FASTMAX_E_SHAPE, "bh = %d outside [1, 65535]", ds->bh);
+  if (ds->bhkv != ds->bh)
+    return fail(FASTMAX_E_SHAPE, "bhkv = %d != bh = %d: grouped key/value heads are not supported", ds->bhkv, ds->bh);
+  if (ds->nq < 1) return fail(FASTMAX_E_SHAPE, "nq = %d < 1", ds->nq);
+  if (ds->nk != ds->nq) return fail(FASTMAX_E_SHAPE, "nk = %d != nq = %d: a key prefix is not supported", ds->nk, ds->nq);
+  if ((int64_t)ds->nq * ds->d * ds->bh >= (int64_t)1 << 40) return fail(FASTMAX_E_SHAPE, "tensor too large");
+  if (ds->p != 1 && ds->p != 2) return fail(FASTMAX_E_PARAM, "p must be 1 or 2, got: %d", ds->p);
+  if (ds->normalize) {
+    if (!(ds->lim > 0.f)) return fail(FASTMAX_E_PARAM, "lim = %g must be positive when normalize is set", (double)ds->lim);
+  } else if (ds->temperature == 0.f || ds->temperature != ds->temperature) {
+    return fail(FASTMAX_E_PARAM, "temperature = %g", (double)ds->temperature);
+  }
+  return FASTMAX_OK;
+}
+
+int check_ws(const Plan& pl, void* ws, size_t ws_bytes) {
+  if (!ws) return fail(FASTMAX_E_WORKSPACE, "workspace is NULL");
+  if (((uintptr_t)ws) & 255) return fail(FASTMAX_E_WORKSPACE, "workspace is not 256-byte aligned");
+  const size_t need = pl.fixed_bytes + pl.per_head_bytes;
+  if (ws_bytes < need)
+    return fail(FASTMAX_E_WORKSPACE, "workspace of %zu bytes is below the minimum of %zu", ws_bytes, need);
+  return FASTMAX_OK;
+}
+
+int launch_status(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(FASTMAX_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return FASTMAX_OK;
+}
+
+#define FM_TRY(expr)            \
+  do {                          \
+    const int rc_ = (expr);     \
+    if (rc_ != FASTMAX_OK) return rc_; \
+  } while (0)
+
+// scale[0..bh) for q, scale[bh..2bh) for k
+template <class T>
+int compute_scales(const fastmax_desc* ds, const T* q, const T* k, float* scale, int* arg,
+                   hipStream_t stream) {
+  const int bh = ds->bh;
+  ScopedKernel sk(FASTMAX_K_ROWSTAT, stream);
+  if (ds->normalize) {
+    rowstat_kernel<T><<<bh, 256, 0, stream>>>(q, ds->nq, ds->d, ds->lim, scale, arg);
+    rowstat_kernel<T><<<bh, 256, 0, stream>>>(k, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
+  } else {
+    fill_scale_kernel<<<(bh + 255) / 256, 256, 0, stream>>>(scale, arg, bh, 1.0f);
+    fill_scale_kernel<<<(bh + 255) / 256, 256, 0, stream>>>(scale + bh, arg + bh, bh, 1.0f / ds->temperature);
+  }
+  return launch_status("scale kernels");
+}
+
+template <int D, class T>
+int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float* xscale,
+                 const float* yden, int64_t yden_stride, const float* ew, float* state, int reverse,
+                 hipStream_t stream) {
+  const dim3 grid(pl.gsplit, heads, pl.masked ? 1 : pl.nslots);
+  if (pl.masked && pl.nslots < 2) return FASTMAX_OK;  // a single chunk never needs a state
+  ScopedKernel sk(FASTMAX_K_BUILD, stream);
+#define FM_BUILD(RTW)                                                                            \
+  build_kernel<D, T, RTW><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, yden_stride, ew, state, \
+                                                    pl.n, kChunk, pl.nslots, pl.masked, reverse, \
+                                                    pl.p2, pl.zlen)
+  if (pl.rtw == 1) {
+    FM_BUILD(1);
+  } else if constexpr (D == 64) {
+    FM_BUILD(3);
+  } else {
+    FM_BUILD(5);
+  }
+#undef FM_BUILD
+  return launch_status("build_kernel");
+}
+
+template <int D, class T>
+int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k, const T* v, T* o,
+                 int64_t ldo, float* den, int64_t den_stride, float* scale_out, int32_t* arg_out,
+                 char* ws, size_t ws_bytes, hipStream_t stream) {
+  const int bh = pl.bh, n = pl.n;
+  float* scale = reinterpret_cast<float*>(ws);
+  int* arg = reinterpret_cast<int*>(ws + align256((size_t)2 * bh * sizeof(float)));
+  float* state = reinterpret_cast<float*>(ws + pl.fixed_bytes);
+  size_t hb_sz = (ws_bytes - pl.fixed_bytes) / pl.per_head_bytes;
+  const int hb = (int)(hb_sz > (size_t)bh ? (size_t)bh : hb_sz);
+
+  FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
+  if (scale_out) hipMemcpyAsync(scale_out, scale, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);
+  if (arg_out) hipMemcpyAsync(arg_out, arg, (size_t)2 * bh * sizeof(int), hipMemcpyDeviceToDevice, stream);
+
+  for (int h0 = 0; h0 < bh; h0 += hb) {
+    const int heads = bh - h0 < hb ? bh - h0 : hb;
+    const int64_t off = (int64_t)h0 * n * D;
+    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, state, 0, stream)));
+    {
+      ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
+      fwd_apply_kernel<D, T><<<dim3(pl.nblk, heads), 256, 0, stream>>>(
+          q + off, k + off, v + off, scale + h0, scale + bh + h0, state, pl.nslots,
+          o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, kChunk,
+          pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
+    }
+    FM_TRY(launch_status("fwd_apply_kernel"));
+  }
+  return FASTMAX_OK;
+}
+
+template <int D, class T>
+int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k, const T* v,
+                  const T* o, int64_t ldo, const float* den, int64_t den_stride, const T* go, T* dq,
+                  T* dk, T* dv, const float* scale_in, const int32_t* arg_in, char* ws,
+                  size_t ws_bytes, hipStream_t stream) {
+  const int bh = pl.bh, n = pl.n;
+  char* p = ws;
+  float* scale = reinterpret_cast<float*>(p);
+  p += align256((size_t)2 * bh * sizeof(float));
+  int* arg = reinterpret_cast<int*>(p);
+  p += align256((size_t)2 * bh * sizeof(int));
+  float* cvec = reinterpret_cast<float*>(p);
+  p += align256((size_t)bh * n * sizeof(float));
+  float* rpart = reinterpret_cast<float*>(p);
+  float* state = reinterpret_cast<float*>(ws + pl.fixed_bytes);
+  size_t hb_sz = (ws_bytes - pl.fixed_bytes) / pl.per_head_bytes;
+  const int hb = (int)(hb_sz > (size_t)bh ? (size_t)bh : hb_sz);
+
+  if (scale_in && arg_in) {
+    hipMemcpyAsync(scale, scale_in, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);
+    hipMemcpyAsync(arg, arg_in, (size_t)2 * bh * sizeof(int), hipMemcpyDeviceToDevice, stream);
+  } else {
+    FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
+  }
+  {
+    const int64_t rows = (int64_t)bh * n;
+    const int rpp = 256 / (D / 4);
+    ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
+    bwd_prep_kernel<T><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
+    FM_TRY(launch_status("bwd_prep_kernel"));
+  }
+  const float a2 = pl.p2 ? ds->a2 : 0.f;
+  for (int h0 = 0; h0 < bh; h0 += hb) {
+    const int heads = bh - h0 < hb ? bh - h0 : hb;
+    const int64_t off = (int64_t)h0 * n * D;
+    float* stS = state;
+    float* stR = state + (int64_t)hb * pl.nslots * pl.state_floats;
+    const float* denh = den + (int64_t)h0 * n * den_stride;
+    const float* ch = cvec + (int64_t)h0 * n;
+    // prefix state of (kh, v, 1) and suffix state of (qh, go/den, c)
+    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, stS, 0, stream)));
+    FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, stream)));
+    const dim3 grid(pl.nblk, heads);
+    {
+      ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
+      bwd_dq_kernel<D, T, false><<<grid, 256, 0, stream>>>(
+          q + off, k + off, v + off, go + off, denh, den_stride, ch, scale + h0, scale + bh + h0, stS,
+          pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, kChunk, pl.masked, pl.p2, ds->a1, a2);
+    }
+    FM_TRY(launch_status("bwd_dq_kernel"));
+    {
+      ScopedKernel sk(FASTMAX_K_BWD_DKDV, stream);
+      bwd_dkdv_kernel<D, T, false><<<grid, 256, 0, stream>>>(
+          q + off, k + off, v + off, go + off, denh, den_stride, ch, scale + h0, scale + bh + h0, stR,
+          pl.nslots, dk + off, dv + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, kChunk, pl.masked,
+          pl.p2, ds->a0, ds->a1, a2);
+    }
+    FM_TRY(launch_status("bwd_dkdv_kernel"));
+  }
+  if (ds->normalize) {
+    ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
+    norm_fix_kernel<T><<<bh, D, 0, stream>>>(dq, q, scale, arg, rpart, pl.nblk, n, D, ds->lim);
+    norm_fix_kernel<T><<<bh, D, 0, stream>>>(dk, k, scale + bh, arg + bh, rpart + (int64_t)bh * pl.nblk, pl.nblk, n, D, ds->lim);
+    FM_TRY(launch_status("norm_fix_kernel"));
+  }
+  return FASTMAX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* fastmax_version(void) { return "0.1"; }
+
+const char* fastmax_last_error(void) { return g_err; }
+
+int fastmax_profile_begin(void) {
+  g_err[0] = 0;
+  g_prof.on = true;
+  g_prof.used = 0;
+  g_prof.cls.clear();
+  return FASTMAX_OK;
+}
+
+int fastmax_profile_end(fastmax_kernel_times* out) {
+  g_err[0] = 0;
+  g_prof.on = false;
+  if (!out) return fail(FASTMAX_E_NULL, "out is NULL");
+  memset(out, 0, sizeof(*out));
+  for (size_t e = 0; e + 1 < g_prof.used; e += 2) {
+    float ms = 0.f;
+    if (hipEventSynchronize(g_prof.ev[e + 1]) != hipSuccess ||
+        hipEventElapsedTime(&ms, g_prof.ev[e], g_prof.ev[e + 1]) != hipSuccess)
+      return fail(FASTMAX_E_LAUNCH, "event timing failed: %s", hipGetErrorString(hipGetLastError()));
+    const int c = g_prof.cls[e / 2];
+    out->ms[c] += ms;
+    out->launches[c] += 1;
+  }
+  g_prof.used = 0;
+  g_prof.cls.clear();
+  return FASTMAX_OK;
+}
+
+int fastmax_check_desc(const fastmax_desc* desc) {
+  g_err[0] = 0;
+  return check_desc(desc);
+}
+
+size_t fastmax_workspace_min_bytes(const fastmax_desc* desc, int pass) {
+  g_err[0] = 0;
+  if (check_desc(desc) != FASTMAX_OK) return 0;
+  if (pass != FASTMAX_PASS_FORWARD && pass != FASTMAX_PASS_BACKWARD) {
+    fail(FASTMAX_E_PARAM, "pass = %d", pass);
+    return 0;
+  }
+  const Plan pl = make_plan(desc, pass);
+  return pl.fixed_bytes + pl.per_head_bytes;
+}
+
+size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass) {
+  const size_t mn = fastmax_workspace_min_bytes(desc, pass);
+  if (!mn) return 0;
+  const Plan pl = make_plan(desc, pass);
+  size_t heads = (kWorkspaceBudget - (pl.fixed_bytes < kWorkspaceBudget ? pl.fixed_bytes : 0)) / pl.per_head_bytes;
+  if (heads < 1) heads = 1;
+  if (heads > (size_t)pl.bh) heads = pl.bh;
+  return pl.fixed_bytes + heads * pl.per_head_bytes;
+}
+
+int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
+                    int64_t ldo, float* den, int64_t den_stride, float* qk_scale,
+                    int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                    fastmax_stream_t stream) {
+  g_err[0] = 0;
+  FM_TRY(check_desc(desc));
+  if (!q || !k || !v || !o || !den) return fail(FASTMAX_E_NULL, "q, k, v, o and den must be non-NULL");
+  if (ldo < desc->d) return fail(FASTMAX_E_PARAM, "ldo = %lld < d = %d", (long long)ldo, desc->d);
+  if (den_stride < 1) return fail(FASTMAX_E_PARAM, "den_stride = %lld < 1", (long long)den_stride);
+  const Plan pl = make_plan(desc, FASTMAX_PASS_FORWARD);
+  FM_TRY(check_ws(pl, workspace, workspace_bytes));
+  char* ws = static_cast<char*>(workspace);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+#define FM_FWD(DD, TT)                                                                             \
+  return forward_impl<DD, TT>(desc, pl, (const TT*)q, (const TT*)k, (const TT*)v, (TT*)o, ldo, den, \
+                              den_stride, qk_scale, qk_argmax, ws, workspace_bytes, st)
+  if (desc->dtype == FASTMAX_F32) {
+    if (desc->d == 64) FM_FWD(64, float);
+    FM_FWD(32, float);
+  }
+  if (desc->d == 64) FM_FWD(64, bf16_t);
+  FM_FWD(32, bf16_t);
+#undef FM_FWD
+}
+
+int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                     const void* o, int64_t ldo, const float* den, int64_t den_stride,
+                     const void* go, void* dq, void* dk, void* dv, const float* qk_scale,
+                     const int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                     fastmax_stream_t stream) {
+  g_err[0] = 0;
+  FM_TRY(check_desc(desc));
+  if (!q || !k || !v || !o || !den || !go || !dq || !dk || !dv)
+    return fail(FASTMAX_E_NULL, "q, k, v, o, den, go, dq, dk and dv must be non-NULL");
+  if (ldo < desc->d) return fail(FASTMAX_E_PARAM, "ldo = %lld < d = %d", (long long)ldo, desc->d);
+  if (den_stride < 1) return fail(FASTMAX_E_PARAM, "den_stride = %lld < 1", (long long)den_stride);
+  const Plan pl = make_plan(desc, FASTMAX_PASS_BACKWARD);
+  FM_TRY(check_ws(pl, workspace, workspace_bytes));
+  char* ws = static_cast<char*>(workspace);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+#define FM_BWD(DD, TT)                                                                              \
+  return backward_impl<DD, TT>(desc, pl, (const TT*)q, (const TT*)k, (const TT*)v, (const TT*)o, ldo, \
+                               den, den_stride, (const TT*)go, (TT*)dq, (TT*)dk, (TT*)dv, qk_scale,  \
+                               qk_argmax, ws, workspace_bytes, st)
+  if (desc->dtype == FASTMAX_F32) {
+    if (desc->d == 64) FM_BWD(64, float);
+    FM_BWD(32, float);
+  }
+  if (desc->d == 64) FM_BWD(64, bf16_t);
+  FM_BWD(32, bf16_t);
+#undef FM_BWD
+}
+
+int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k, void* workspace,
+                              size_t workspace_bytes, fastmax_stream_t stream) {
+  g_err[0] = 0;
+  FM_TRY(check_desc(desc));
+  if (!q || !k) return fail(FASTMAX_E_NULL, "q and k must be non-NULL");
+  if (!workspace || (((uintptr_t)workspace) & 255) || workspace_bytes < (size_t)16 * desc->bh + 512)
+    return fail(FASTMAX_E_WORKSPACE, "workspace must be 256-byte aligned and hold 16*bh+512 bytes");
+  if (!desc->normalize) return FASTMAX_OK;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  const int bh = desc->bh;
+  float* scale = static_cast<float*>(workspace);
+  int* arg = reinterpret_cast<int*>(static_cast<char*>(workspace) + align256((size_t)2 * bh * sizeof(float)));
+  const int64_t per_head = (int64_t)desc->nq * desc->d;
+  const dim3 grid((unsigned)((per_head / 4 + 255) / 256), bh);
+  if (desc->dtype == FASTMAX_F32) {
+    FM_TRY(compute_scales<float>(desc, (const float*)q, (const float*)k, scale, arg, st));
+    scale_rows_kernel<float><<<grid, 256, 0, st>>>((float*)q, scale, per_head);
+    scale_rows_kernel<float><<<grid, 256, 0, st>>>((float*)k, scale + bh, per_head);
+  } else {
+    FM_TRY(compute_scales<bf16_t>(desc, (const bf16_t*)q, (const bf16_t*)k, scale, arg, st));
+    scale_rows_kernel<bf16_t><<<grid, 256, 0, st>>>((bf16_t*)q, scale, per_head);
+    scale_rows_kernel<bf16_t><<<grid, 256, 0, st>>>((bf16_t*)k, scale + bh, per_head);
+  }
+  return launch_status("scale_rows_kernel");
+}
+
+}  // extern "C"

@@ -1,0 +1,194 @@
+// Shared device helpers for the gfx950 Fastmax kernels.
+//
+// Everything here is written for 64-wide wavefronts and the fp32 matrix instruction
+// v_mfma_f32_32x32x2f32.  Operand layouts of that instruction (lane l of the wave):
+//   A (32 x 2):  row  l%32, k = l/32         -> one float per lane
+//   B (2 x 32):  k = l/32,  col l%32         -> one float per lane
+//   D (32 x 32): col  l%32, rows trow(r,l/32) for the 16 accumulator registers r
+// Because the reduction index k of an MFMA can be any permutation as long as A and B agree,
+// an accumulator register can be fed straight back as the A or B operand of the next
+// contraction (k=0/1 then stand for rows trow(r,0)/trow(r,1)); the kernels use that to chain
+// score tiles into value/gradient tiles without going through memory.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+#define FM_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
+
+// row of a 32x32 accumulator tile held by register r in lane half hh
+__device__ __forceinline__ int trow(int r, int hh) { return 8 * (r >> 2) + 4 * hh + (r & 3); }
+
+struct bf16_t {
+  uint16_t x;
+};
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.x) << 16); }
+
+template <class T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) {
+  return v;
+}
+template <>
+__device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) {
+  uint32_t u = __float_as_uint(v);
+  bf16_t o;
+  if ((u & 0x7fffffffu) > 0x7f800000u) {  // NaN stays NaN
+    o.x = (uint16_t)((u >> 16) | 0x40);
+  } else {
+    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+    o.x = (uint16_t)(u >> 16);
+  }
+  return o;
+}
+
+// four consecutive elements <-> four floats
+__device__ __forceinline__ void load4(const float* p, float (&o)[4]) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+}
+__device__ __forceinline__ void load4(const bf16_t* p, float (&o)[4]) {
+  const uint2 t = *reinterpret_cast<const uint2*>(p);
+  o[0] = __uint_as_float(t.x << 16);
+  o[1] = __uint_as_float(t.x & 0xffff0000u);
+  o[2] = __uint_as_float(t.y << 16);
+  o[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4]) {
+  uint2 t;
+  t.x = (uint32_t)from_f32<bf16_t>(v[0]).x | ((uint32_t)from_f32<bf16_t>(v[1]).x << 16);
+  t.y = (uint32_t)from_f32<bf16_t>(v[2]).x | ((uint32_t)from_f32<bf16_t>(v[3]).x << 16);
+  *reinterpret_cast<uint2*>(p) = t;
+}
+
+// Geometry of the symmetric moment state for head dimension D.
+//
+// The order-2 feature of a vector x is stored once per unordered channel pair, indexed by
+// (shift s, channel a) -> x[a] * x[(a+s) mod D], s = 0..D/2.  Shifts 1..D/2-1 carry every
+// pair {a, a+s} exactly once (weight 2 in a full contraction); s = 0 is the diagonal and
+// s = D/2 lists each pair twice (weight 1 each).  Rows of a state, each D+1 floats
+// (D value columns, then the "extra" column that carries the denominator moments):
+//   [0, NS*D)            order 2, row s*D + a        (absent when p == 1)
+//   [.., +D)             order 1, row a
+//   last row             order 0
+template <int D>
+struct Geo {
+  static constexpr int NS = D / 2 + 1;
+  static constexpr int AB = D / 32;  // 32-row blocks per shift
+  static constexpr int CB = D / 32;  // 32-column blocks of the value dimension
+  static constexpr int LD = D + 1;   // row pitch of states and of every LDS tile
+  static constexpr int H2 = D / 2;   // channels handled by each lane half per MFMA sweep
+  __host__ __device__ static constexpr int rows2(int p2) { return p2 ? NS * D : 0; }
+  __host__ __device__ static constexpr int rows(int p2) { return rows2(p2) + D + 1; }
+  __host__ __device__ static constexpr int64_t state_floats(int p2) {
+    return ((int64_t)rows(p2) * LD + 63) / 64 * 64;
+  }
+  // floats of one LDS stage buffer: a state slab of D(+1) rows or a pair of 32-row tiles
+  static constexpr int SLAB = ((D + 1) * LD > 2 * 32 * LD ? (D + 1) * LD : 2 * 32 * LD) + 3;
+  static constexpr int SLABF = (SLAB + 3) / 4 * 4;
+};
+
+// A tile of ROWS token rows x D channels staged global -> registers -> LDS by 256 threads.
+template <int D, class T, int ROWS>
+struct RowTile {
+  static constexpr int VPR = D / 4;
+  static constexpr int TOTAL = ROWS * VPR;
+  static constexpr int NV = (TOTAL + 255) / 256;
+  float v[NV][4];
+
+  // rows tok0.. of one head (base points at the head's first row); rows >= n read as zero.
+  // rowdiv, when given, divides every row by rowdiv[tok * rowdiv_stride].
+  __device__ __forceinline__ void load(const T* base, int tok0, int n, int tid,
+                                       const float* rowdiv = nullptr, int64_t rowdiv_stride = 0) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      const int row = idx / VPR, c4 = idx % VPR;
+      const int tok = tok0 + row;
+      if (idx < TOTAL && tok < n) {
+        load4(base + (int64_t)tok * D + c4 * 4, v[u]);
+        if (rowdiv) {
+          const float s = 1.0f / rowdiv[(int64_t)tok * rowdiv_stride];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[u][e] *= s;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[u][e] = 0.f;
+      }
+    }
+  }
+  // dst is [ROWS][ld] floats in LDS
+  __device__ __forceinline__ void store(float* dst, int ld, float scale, int tid) const {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      const int row = idx / VPR, c4 = idx % VPR;
+      if (idx < TOTAL) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[row * ld + c4 * 4 + e] = v[u][e] * scale;
+      }
+    }
+  }
+};
+
+// A run of `count` floats of a moment state staged global -> registers -> LDS, summed over
+// `nsum` slots (token-split partial states of an unmasked build).
+template <int MAXF>
+struct StateSlab {
+  static constexpr int NV = ((MAXF + 3) / 4 + 255) / 256;
+  float4 v[NV];
+
+  __device__ __forceinline__ void load(const float* src, int64_t slot_stride, int nsum, int count,
+                                       int tid) {
+    const int nvec = (count + 3) >> 2;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (idx < nvec) {
+        a = *reinterpret_cast<const float4*>(src + idx * 4);
+        for (int z = 1; z < nsum; ++z) {
+          const float4 b = *reinterpret_cast<const float4*>(src + z * slot_stride + idx * 4);
+          a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        }
+      }
+      v[u] = a;
+    }
+  }
+  // elements [0, split) are scaled by c_lo, the rest by c_hi
+  __device__ __forceinline__ void store(float* dst, int count, int split, float c_lo, float c_hi,
+                                        int tid) const {
+    const int nvec = (count + 3) >> 2;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      if (idx < nvec) {
+        const int e0 = idx * 4;
+        float4 a = v[u];
+        a.x *= (e0 + 0 < split) ? c_lo : c_hi;
+        a.y *= (e0 + 1 < split) ? c_lo : c_hi;
+        a.z *= (e0 + 2 < split) ? c_lo : c_hi;
+        a.w *= (e0 + 3 < split) ? c_lo : c_hi;
+        *reinterpret_cast<float4*>(dst + e0) = a;
+      }
+    }
+  }
+};
+
+// sum over the 256 threads of a block; red is 4 floats of LDS; result valid in every thread
+__device__ __forceinline__ float block_sum_256(float v, float* red, int tid) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  __syncthreads();
+  if ((tid & 63) == 0) red[tid >> 6] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}

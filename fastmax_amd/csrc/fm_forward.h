@@ -1,0 +1,440 @@
+// Forward-side kernels: per-head row-norm statistics, the moment-state build (used by
+// both passes) and the forward apply.
+#pragma once
+#include "fm_common.h"
+
+// ---------------------------------------------------------------------------------------
+// Per-head normaliser: scale[h] = lim / max_i ||x_i||_2 and the row that attains the max
+// (first one on ties).  Replaces calc_norms / find_max of the reference
+// (fastmax_cuda_forward.cu:223-253) with the PyTorch path's definition (example.py:105-108).
+// One block per head; d/4 threads share a row.
+// ---------------------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(256) void rowstat_kernel(const T* __restrict__ x, int n, int d,
+                                                      float lim, float* __restrict__ scale_out,
+                                                      int* __restrict__ arg_out) {
+  __shared__ float sbest[256];
+  __shared__ int sarg[256];
+  const int tid = threadIdx.x;
+  const int tpr = d >> 2, rpp = 256 / tpr;
+  const int sub = tid % tpr, rowi = tid / tpr;
+  const T* base = x + (int64_t)blockIdx.x * n * d;
+  float best = -1.f;
+  int bi = 0x7fffffff;
+  for (int i0 = 0; i0 < n; i0 += rpp) {
+    const int i = i0 + rowi;
+    float ss = 0.f;
+    if (i < n) {
+      float v[4];
+      load4(base + (int64_t)i * d + sub * 4, v);
+      ss = v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+    for (int off = tpr >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    if (i < n && ss > best) {
+      best = ss;
+      bi = i;
+    }
+  }
+  sbest[tid] = best;
+  sarg[tid] = bi;
+  __syncthreads();
+  for (int off = 128; off > 0; off >>= 1) {
+    if (tid < off) {
+      const float ob = sbest[tid + off];
+      const int oi = sarg[tid + off];
+      if (ob > sbest[tid] || (ob == sbest[tid] && oi < sarg[tid])) {
+        sbest[tid] = ob;
+        sarg[tid] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    scale_out[blockIdx.x] = lim / sqrtf(sbest[0]);
+    arg_out[blockIdx.x] = sarg[0];
+  }
+}
+
+__global__ void fill_scale_kernel(float* scale, int* arg, int count, float value) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) {
+    scale[i] = value;
+    arg[i] = 0;
+  }
+}
+
+// x <- x * scale[head]; the reference's in-place apply_norm (fastmax_cuda_forward.cu:255-269)
+template <class T>
+__global__ void scale_rows_kernel(T* x, const float* __restrict__ scale, int64_t per_head) {
+  const int64_t i4 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i4 < per_head) {
+    T* p = x + (int64_t)blockIdx.y * per_head + i4;
+    float v[4];
+    load4(p, v);
+    const float s = scale[blockIdx.y];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] *= s;
+    store4(p, v);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Moment-state build.
+//
+//   state[row(f)][c] = sum_j feat_f(x_j) * y_j[c]     c < D
+//   state[row(f)][D] = sum_j feat_f(x_j) * e_j        the "extra" column
+//
+// over a token range, with x_j = X_j * xscale[head], y_j = Y_j / yden_j (when given) and
+// e_j = ew_j or 1.  The forward pass uses (X,Y,e) = (k, v, 1); the backward pass also builds
+// the mirror-image suffix state with (q, grad_out/den, c).  A block is four waves; each wave
+// owns RTW row tiles (32 features x D columns) as MFMA accumulators for the whole walk, the
+// features being generated on the fly as products of two LDS reads of the staged X tile.
+// gridDim.x feature splits cover all row tiles of a head, gridDim.y = heads.
+//
+// masked != 0: the walk is a scan over `chunk`-token chunks and a snapshot of the running
+//   state is written before each chunk is added (slot c = everything strictly before chunk
+//   c, or strictly after it when reverse != 0).  The first chunk in scan order needs no
+//   state (it is all zero) and the last one is never added.
+// masked == 0: gridDim.z blocks each sum zlen tokens and write slot blockIdx.z; consumers
+//   add the slots.
+// ---------------------------------------------------------------------------------------
+template <int D, class T, int RTW>
+__global__ __launch_bounds__(256) void build_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const float* __restrict__ xscale,
+    const float* __restrict__ yden, int64_t yden_stride, const float* __restrict__ ew,
+    float* __restrict__ state, int n, int chunk, int nslots, int masked, int reverse, int p2,
+    int zlen) {
+  using G = Geo<D>;
+  constexpr int TS = 32;           // tokens per pipeline step
+  constexpr int LDK = D + 1;       // X tile pitch; column D holds 1 (0 for padding rows)
+  constexpr int CB = G::CB, LD = G::LD;
+  __shared__ float Kl[2][TS * LDK];
+  __shared__ __attribute__((aligned(16))) float Vl[2][TS * D];
+  __shared__ float El[2][TS];
+
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, hh = l >> 5;
+  const int g = blockIdx.x, head = blockIdx.y;
+  const int rows2 = G::rows2(p2);
+  const int rt2 = p2 ? G::NS * G::AB : 0, rt_total = rt2 + G::AB;
+  const int64_t SS = G::state_floats(p2);
+
+  int owncol[RTW], rotcol[RTW], rowbase[RTW];
+  int nx = 0;
+#pragma unroll
+  for (int x = 0; x < RTW; ++x) {
+    const int rt = (g * 4 + w) * RTW + x;
+    owncol[x] = rotcol[x] = rowbase[x] = 0;
+    if (rt < rt_total) {
+      nx = x + 1;
+      if (rt < rt2) {
+        const int s = rt / G::AB, ab = rt % G::AB;
+        owncol[x] = ab * 32 + i;
+        rotcol[x] = (owncol[x] + s) % D;
+        rowbase[x] = s * D + ab * 32;
+      } else {
+        const int ab = rt - rt2;
+        owncol[x] = ab * 32 + i;
+        rotcol[x] = D;  // the column of ones: order-1 feature is x[a] itself
+        rowbase[x] = rows2 + ab * 32;
+      }
+    }
+  }
+
+  f16v acc[RTW][CB];
+  float dacc[RTW];
+#pragma unroll
+  for (int x = 0; x < RTW; ++x) {
+    dacc[x] = 0.f;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[x][cb][r] = 0.f;
+  }
+  float s0 = 0.f;  // order-0 sums: threads 0..D-1 of split 0 own a value column, thread D the extra one
+
+  const T* Xh = X + (int64_t)head * n * D;
+  const T* Yh = Y + (int64_t)head * n * D;
+  const float* ydh = yden ? yden + (int64_t)head * n * yden_stride : nullptr;
+  const float* ewh = ew ? ew + (int64_t)head * n : nullptr;
+  const float xs = xscale[head];
+
+  RowTile<D, T, TS> kx, vy;
+  float ereg = 0.f;
+
+  auto load = [&](int t0, int tend) {
+    kx.load(Xh, t0, tend, tid);
+    vy.load(Yh, t0, tend, tid, ydh, yden_stride);
+    if (tid < TS) {
+      const int tok = t0 + tid;
+      ereg = (tok < tend) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
+    }
+  };
+  auto store = [&](int buf, int t0, int tend) {
+    kx.store(Kl[buf], LDK, xs, tid);
+    vy.store(Vl[buf], D, 1.0f, tid);
+    if (tid < TS) {
+      El[buf][tid] = ereg;
+      Kl[buf][tid * LDK + D] = (t0 + tid < tend) ? 1.0f : 0.f;
+    }
+  };
+  auto compute = [&](int buf) {
+    const float* kb = Kl[buf];
+    const float* vb = Vl[buf];
+#pragma unroll 2
+    for (int t = 0; t < TS / 2; ++t) {
+      const int j = 2 * t + hh;
+      const float* kr = kb + j * LDK;
+      float vv[CB];
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) vv[cb] = vb[j * D + cb * 32 + i];
+      const float e = El[buf][j];
+#pragma unroll
+      for (int x = 0; x < RTW; ++x) {
+        if (x < nx) {
+          const float a = kr[owncol[x]] * kr[rotcol[x]];
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) acc[x][cb] = FM_MFMA(a, vv[cb], acc[x][cb]);
+          dacc[x] += a * e;
+        }
+      }
+    }
+    if (g == 0 && tid <= D) {
+      if (tid < D) {
+#pragma unroll 8
+        for (int j = 0; j < TS; ++j) s0 += vb[j * D + tid];
+      } else {
+#pragma unroll 8
+        for (int j = 0; j < TS; ++j) s0 += El[buf][j];
+      }
+    }
+  };
+  auto run = [&](int tb, int te) {
+    const int nsteps = (te - tb + TS - 1) / TS;
+    if (nsteps <= 0) return;
+    load(tb, te);
+    store(0, tb, te);
+    __syncthreads();
+    for (int st = 0; st < nsteps; ++st) {
+      const bool more = st + 1 < nsteps;
+      if (more) load(tb + (st + 1) * TS, te);
+      compute(st & 1);
+      if (more) store((st + 1) & 1, tb + (st + 1) * TS, te);
+      __syncthreads();
+    }
+  };
+  auto snapshot = [&](int slot) {
+    float* st = state + ((int64_t)head * nslots + slot) * SS;
+#pragma unroll
+    for (int x = 0; x < RTW; ++x) {
+      if (x < nx) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            st[(int64_t)(rowbase[x] + trow(r, hh)) * LD + cb * 32 + i] = acc[x][cb][r];
+        const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
+        if (hh == 0) st[(int64_t)(rowbase[x] + i) * LD + D] = ds;
+      }
+    }
+    if (g == 0 && tid <= D) st[(int64_t)(rows2 + D) * LD + tid] = s0;
+  };
+
+  if (masked) {
+    const int nc = (n + chunk - 1) / chunk;
+    for (int cc = 0; cc + 1 < nc; ++cc) {
+      const int c = reverse ? nc - 1 - cc : cc;
+      const int te = (c + 1) * chunk < n ? (c + 1) * chunk : n;
+      run(c * chunk, te);
+      snapshot(reverse ? c - 1 : c + 1);
+    }
+  } else {
+    const int z = blockIdx.z;
+    const int te = (z + 1) * zlen < n ? (z + 1) * zlen : n;
+    run(z * zlen, te);
+    snapshot(z);
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Forward apply:  [num_i, den_i] = phi(q_i) . S  (+ the causal intra-chunk tile), o = num/den.
+//
+// One block = 128 query tokens of one head, one wave = 32 of them.  Lane (i = l%32, hh = l/32)
+// keeps q_i[t + hh*D/2] in registers (A-operand side of the order-2 feature) and reads the
+// rotated partner q_i[(a+s)%D] from the LDS copy of the tile, so a feature costs one LDS
+// read and one multiply per MFMA pair.  The state streams through a double-buffered LDS slab
+// (one shift = D rows at a time), coefficients a2*w_s / a1 / a0 applied while staging.
+// For causal attention the same stream then carries the 32-key tiles of the block's own
+// chunk: scores are formed transposed (keys x queries) so that the polynomial of the score
+// tile is directly the A operand of the P.V product.
+// ---------------------------------------------------------------------------------------
+template <int D, class T>
+__global__ __launch_bounds__(256) void fwd_apply_kernel(
+    const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+    const float* __restrict__ qscale, const float* __restrict__ kscale,
+    const float* __restrict__ state, int nslots, T* __restrict__ O, int64_t ldo,
+    float* __restrict__ den, int64_t den_stride, int n, int chunk, int masked, int p2, float a0,
+    float a1, float a2) {
+  using G = Geo<D>;
+  constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
+  __shared__ float Ql[128 * LD];
+  __shared__ __attribute__((aligned(16))) float Sl[2][SLABF];
+  __shared__ float denl[128];
+
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, hh = l >> 5;
+  const int head = blockIdx.y, tok0 = blockIdx.x * 128;
+  const int c = tok0 / chunk;
+  const int rows2 = G::rows2(p2);
+  const int64_t SS = G::state_floats(p2);
+  const T* Qh = Q + (int64_t)head * n * D;
+  const T* Kh = K + (int64_t)head * n * D;
+  const T* Vh = V + (int64_t)head * n * D;
+  const float qs = qscale[head], ks = kscale[head];
+
+  {  // stage the query tile; column D is the constant 1 used by the order-1 sweep
+    RowTile<D, T, 128> qt;
+    qt.load(Qh, tok0, n, tid);
+    qt.store(Ql, LD, qs, tid);
+    if (tid < 128) Ql[tid * LD + D] = 1.0f;
+  }
+
+  const int n_state = (masked && c == 0) ? 0 : (p2 ? NS : 0) + 1;
+  int n_key = 0, kt0 = 0;
+  if (masked) {
+    kt0 = (c * chunk) >> 5;
+    int last = tok0 + 127 < n ? tok0 + 127 : n - 1;
+    n_key = (last >> 5) - kt0 + 1;
+  }
+  const int n_stage = n_state + n_key;
+  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
+  const int nsum = masked ? 1 : nslots;
+
+  StateSlab<(D + 1) * LD> slab;
+  RowTile<D, T, 32> kt_k, kt_v;
+
+  // stage st is a state slab (st < n_state) or a key tile
+  auto stage_load = [&](int st) {
+    if (st < n_state) {
+      const bool ord2 = p2 && st < NS;
+      const int off = ord2 ? st * D * LD : rows2 * LD;
+      const int cnt = ord2 ? D * LD : (D + 1) * LD;
+      slab.load(sbase + off, SS, nsum, cnt, tid);
+    } else {
+      const int kt = kt0 + (st - n_state);
+      kt_k.load(Kh, kt * 32, n, tid);
+      kt_v.load(Vh, kt * 32, n, tid);
+    }
+  };
+  auto stage_store = [&](int st) {
+    float* dst = Sl[st & 1];
+    if (st < n_state) {
+      const bool ord2 = p2 && st < NS;
+      if (ord2) {
+        const float cf = (st == 0 || st == H2) ? a2 : 2.0f * a2;
+        slab.store(dst, D * LD, D * LD, cf, cf, tid);
+      } else {
+        slab.store(dst, (D + 1) * LD, D * LD, a1, a0, tid);
+      }
+    } else {
+      kt_k.store(dst, LD, ks, tid);
+      kt_v.store(dst + 32 * LD, LD, 1.0f, tid);
+    }
+  };
+
+  __syncthreads();
+  const int qrow = w * 32 + i;
+  float Qr[H2];
+#pragma unroll
+  for (int t = 0; t < H2; ++t) Qr[t] = Ql[qrow * LD + t + hh * H2];
+
+  f16v acc[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[cb][r] = 0.f;
+  float dn = 0.f;
+
+  if (n_stage > 0) {
+    stage_load(0);
+    stage_store(0);
+  }
+  __syncthreads();
+  const int qt_mine = (tok0 >> 5) + w;
+  for (int st = 0; st < n_stage; ++st) {
+    const bool more = st + 1 < n_stage;
+    if (more) stage_load(st + 1);
+    const float* sl = Sl[st & 1];
+    if (st < n_state) {
+      const bool ord2 = p2 && st < NS;
+      const int rbase = hh * H2 + st;  // (a + s) for t = 0; order-1 reads the ones column
+      const float* qr = Ql + qrow * LD;
+#pragma unroll
+      for (int t = 0; t < H2; ++t) {
+        int rc = rbase + t;
+        rc -= (rc >= D) ? D : 0;
+        rc = ord2 ? rc : D;
+        const float a = Qr[t] * qr[rc];
+        const float* srow = sl + (t + hh * H2) * LD;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA(a, srow[cb * 32 + i], acc[cb]);
+        dn += a * srow[D];
+      }
+      if (!ord2) {  // order 0 rides at the end of the order-1 slab
+        const float* s0 = sl + D * LD;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+          const float z = s0[cb * 32 + i];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[cb][r] += z;
+        }
+        if (hh == 0) dn += s0[D];
+      }
+    } else {
+      const int kt = kt0 + (st - n_state);
+      if (kt <= qt_mine) {
+        const float* kl = sl;
+        const float* vl = sl + 32 * LD;
+        f16v sc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < H2; ++t) sc = FM_MFMA(kl[i * LD + t + hh * H2], Qr[t], sc);
+        const bool diag = kt == qt_mine;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float s = sc[r];
+          float f = a0 + s * (a1 + a2 * s);
+          if (diag && trow(r, hh) > i) f = 0.f;
+          sc[r] = f;
+          dn += f;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float* vrow = vl + trow(r, hh) * LD;
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA(sc[r], vrow[cb * 32 + i], acc[cb]);
+        }
+      }
+    }
+    if (more) stage_store(st + 1);
+    __syncthreads();
+  }
+
+  const float dtot = dn + __shfl_xor(dn, 32, 64);
+  const int tok = tok0 + qrow;
+  if (hh == 0) {
+    denl[qrow] = dtot;
+    if (tok < n) den[((int64_t)head * n + tok) * den_stride] = dtot;
+  }
+  __syncthreads();
+  T* Oh = O + (int64_t)head * n * ldo;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = w * 32 + trow(r, hh);
+    const int tk = tok0 + row;
+    if (tk < n) {
+      const float inv = 1.0f / denl[row];
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) Oh[(int64_t)tk * ldo + cb * 32 + i] = from_f32<T>(acc[cb][r] * inv);
+    }
+  }
+}

@@ -1,0 +1,127 @@
+"""Tensor-level calls into the C ABI: torch supplies device memory and the current stream,
+the library does the work.  Layout (bh, n, d) contiguous, fp32 or bf16."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _cabi
+
+_WS: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return _cabi.FASTMAX_F32
+    if t.dtype == torch.bfloat16:
+        return _cabi.FASTMAX_BF16
+    raise TypeError(f"fastmax: dtype {t.dtype} is not supported (float32 or bfloat16)")
+
+
+def _check_inputs(*ts: torch.Tensor) -> None:
+    first = ts[0]
+    for t in ts:
+        if not t.is_cuda:
+            raise RuntimeError("fastmax: tensors must live on a GPU (the HIP kernels have no CPU path)")
+        if not t.is_contiguous():
+            raise RuntimeError("fastmax: tensors must be contiguous")
+        if t.dtype != first.dtype or t.device != first.device:
+            raise RuntimeError("fastmax: tensors must share dtype and device")
+        if t.dim() != 3:
+            raise RuntimeError("fastmax: expected (b*h, n, d) tensors at this level")
+
+
+def _workspace(dev: torch.device, nbytes: int, slot: int) -> torch.Tensor:
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), slot)
+    ws = _WS.get(key)
+    if ws is None or ws.numel() < nbytes:
+        _WS[key] = ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    return ws
+
+
+def release_workspaces() -> None:
+    _WS.clear()
+
+
+def _desc(q, k, mask, normalize, p, lim, temperature, a0, a1, a2):
+    return _cabi.make_desc(q.shape[0], q.shape[1], q.shape[2], _dtype_code(q), mask, normalize, p, lim,
+                           temperature, a0, a1, a2, bhkv=k.shape[0], nk=k.shape[1])
+
+
+def forward(q, k, v, *, mask=False, normalize=False, lim=1.0, temperature=1.0, a0=1.0, a1=1.0, a2=0.5,
+            p=2, denominator_column: bool = False, workspace_bytes: Optional[int] = None):
+    """Returns (o, den, qk_scale, qk_argmax).
+
+    denominator_column=True gives the reference extension's layout: o is (bh, n, d+1) with the
+    row denominators in column d (fastmax_cuda_forward.cu:353); den is then a view of it.
+    """
+    _check_inputs(q, k, v)
+    lib = _cabi.load()
+    bh, n, d = q.shape
+    ds = _desc(q, k, mask, normalize, p, lim, temperature, a0, a1, a2)
+    _cabi.check(lib.fastmax_check_desc(C.byref(ds)))
+    if v.shape != k.shape:
+        raise RuntimeError("fastmax: k and v must have the same shape")
+    with torch.cuda.device(q.device):
+        nbytes = workspace_bytes or lib.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD)
+        ws = _workspace(q.device, nbytes, 0)
+        if denominator_column:
+            if q.dtype != torch.float32:
+                raise RuntimeError("fastmax: the (d+1)-column output exists for float32 only")
+            o = torch.empty((bh, n, d + 1), dtype=q.dtype, device=q.device)
+            den = o[:, :, d]
+            ldo, den_ptr, den_stride = d + 1, o.data_ptr() + 4 * d, d + 1
+        else:
+            o = torch.empty((bh, n, d), dtype=q.dtype, device=q.device)
+            den = torch.empty((bh, n), dtype=torch.float32, device=q.device)
+            ldo, den_ptr, den_stride = d, den.data_ptr(), 1
+        scale = torch.empty(2 * bh, dtype=torch.float32, device=q.device)
+        arg = torch.empty(2 * bh, dtype=torch.int32, device=q.device)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        _cabi.check(lib.fastmax_forward(C.byref(ds), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                        ldo, den_ptr, den_stride, scale.data_ptr(), arg.data_ptr(),
+                                        ws.data_ptr(), nbytes, stream))
+    return o, den, scale, arg
+
+
+def backward(q, k, v, o, den, go, *, mask=False, normalize=False, lim=1.0, temperature=1.0, a0=1.0,
+             a1=1.0, a2=0.5, p=2, qk_scale: Optional[torch.Tensor] = None,
+             qk_argmax: Optional[torch.Tensor] = None, workspace_bytes: Optional[int] = None):
+    """Returns (dq, dk, dv).  o may be (bh,n,d) or (bh,n,d+1); den any strided (bh,n) fp32 view."""
+    _check_inputs(q, k, v, go)
+    lib = _cabi.load()
+    bh, n, d = q.shape
+    ds = _desc(q, k, mask, normalize, p, lim, temperature, a0, a1, a2)
+    _cabi.check(lib.fastmax_check_desc(C.byref(ds)))
+    if o.dtype != q.dtype or o.stride(2) != 1 or o.stride(0) != n * o.stride(1):
+        raise RuntimeError("fastmax: o must be (bh, n, ldo) with unit column stride")
+    if den.dtype != torch.float32 or den.shape != (bh, n) or den.stride(0) != n * den.stride(1):
+        raise RuntimeError("fastmax: den must be a float32 (bh, n) view with a uniform stride")
+    with torch.cuda.device(q.device):
+        nbytes = workspace_bytes or lib.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_BACKWARD)
+        ws = _workspace(q.device, nbytes, 1)
+        dq = torch.empty_like(q)
+        dk = torch.empty_like(k)
+        dv = torch.empty_like(v)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        _cabi.check(lib.fastmax_backward(
+            C.byref(ds), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), o.stride(1), den.data_ptr(),
+            den.stride(1), go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+            qk_scale.data_ptr() if qk_scale is not None else None,
+            qk_argmax.data_ptr() if qk_argmax is not None else None, ws.data_ptr(), nbytes, stream))
+    return dq, dk, dv
+
+
+def normalize_inplace(q, k, *, lim=1.0):
+    """q <- lim*q/max||q_n||, k likewise, in place (the reference forward's side effect)."""
+    _check_inputs(q, k)
+    lib = _cabi.load()
+    ds = _desc(q, k, False, True, 2, lim, 1.0, 1.0, 1.0, 0.5)
+    with torch.cuda.device(q.device):
+        nbytes = 16 * q.shape[0] + 1024
+        ws = _workspace(q.device, nbytes, 2)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        _cabi.check(lib.fastmax_normalize_inplace(C.byref(ds), q.data_ptr(), k.data_ptr(), ws.data_ptr(),
+                                                  nbytes, stream))

@@ -1,0 +1,142 @@
+/*
+ * fastmax_amd.h -- C ABI of the MI355X (gfx950) Fastmax attention library.
+ *
+ * Fastmax attention replaces the softmax by a row-normalised polynomial score
+ *     o_i = sum_j f(q_i.k_j) v_j / sum_j f(q_i.k_j),   f(s) = a0 + a1 s + a2 s^2  (p=2)
+ * (j <= i when mask != 0).  This header is the whole drop-in boundary for that path:
+ * plain pointers and sizes, no torch types.  Every entry point is asynchronous on the
+ * given stream, allocates nothing on the device, keeps no state between calls (the opt-in
+ * kernel timer at the end of this header aside) and returns 0 or a negative FASTMAX_E_* code (text via fastmax_last_error()).
+ *
+ * Layout contract (reference: fastmax_cuda_forward.cu:331-336): q, k, v, grad_output and
+ * the gradients are (bh, n, d) row-major with d contiguous; a (b,h,n,d) tensor is the
+ * same memory.  The output may carry a row pitch ldo >= d so that the reference's
+ * (bh, n, d+1) "o with the denominator in column d" (fastmax_cuda_forward.cu:353,
+ * example.py:47) is written in place: pass ldo = d+1, den = o + d, den_stride = d+1.
+ */
+#ifndef FASTMAX_AMD_H
+#define FASTMAX_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* fastmax_stream_t; /* == hipStream_t */
+
+enum {
+  FASTMAX_OK = 0,
+  FASTMAX_E_NULL = -1,        /* a required pointer is NULL                         */
+  FASTMAX_E_SHAPE = -2,       /* unsupported bh / n / d / bhkv / nq != nk           */
+  FASTMAX_E_DTYPE = -3,       /* dtype not FASTMAX_F32 / FASTMAX_BF16               */
+  FASTMAX_E_PARAM = -4,       /* p not in {1,2}, bad lim / temperature / pitch      */
+  FASTMAX_E_WORKSPACE = -5,   /* workspace NULL, misaligned or too small            */
+  FASTMAX_E_LAUNCH = -6,      /* the HIP runtime refused a launch                   */
+  FASTMAX_E_NO_DEVICE = -7    /* no gfx950 device is current                        */
+};
+
+enum { FASTMAX_F32 = 0, FASTMAX_BF16 = 1 };
+enum { FASTMAX_PASS_FORWARD = 0, FASTMAX_PASS_BACKWARD = 1 };
+
+/* Problem descriptor.  Mirrors the scalar arguments of the reference's
+ * forwardpass(q,k,v,drop_noise,mask,dropout,normalize,temperature,a0,a1,a2,lim,p)
+ * (fastmax_cuda.cpp:17, fastmax_cuda_forward.cu:297-314) plus the sizes its launcher reads
+ * from the tensors (fastmax_cuda_forward.cu:331-336). */
+typedef struct fastmax_desc {
+  int32_t bh;          /* query heads  (b*h)                                             */
+  int32_t bhkv;        /* key/value heads; must equal bh                                 */
+  int32_t nq;          /* query tokens                                                   */
+  int32_t nk;          /* key tokens; must equal nq                                      */
+  int32_t d;           /* head dimension: 32 or 64                                        */
+  int32_t dtype;       /* FASTMAX_F32 or FASTMAX_BF16 (bf16 in/out, fp32 arithmetic)     */
+  int32_t mask;        /* 0: every key visible, 1: causal (j <= i)                       */
+  int32_t normalize;   /* 1: x <- lim * x / max_n ||x_n||_2 per head for q and k,
+                          differentiated through (example.py:101-108)                    */
+  int32_t p;           /* polynomial order, 1 or 2                                       */
+  float lim;           /* see normalize                                                  */
+  float temperature;   /* used only when normalize == 0: k <- k / temperature
+                          (fastmax_cuda_forward.cu:212-221,366; gradk / temperature at
+                          example.py:80)                                                 */
+  float a0, a1, a2;    /* score coefficients                                             */
+} fastmax_desc;
+
+/* Library version, "major.minor". */
+const char* fastmax_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char* fastmax_last_error(void);
+
+/* Checks a descriptor without touching the device.  Replaces the shape reads and the
+ * implicit assumptions of fastmax_cuda_forward.cu:331-345 (d == 64, bh == bhkv). */
+int fastmax_check_desc(const fastmax_desc* desc);
+
+/* Bytes of device workspace that let a pass run all heads in as few batches as a 6 GiB
+ * budget allows (the passes accept anything >= fastmax_workspace_min_bytes and then loop
+ * over smaller head batches).  Replaces the torch::zeros scratch tensors of
+ * fastmax_cuda_forward.cu:353-357 and fastmax_cuda_backward.cu:957-959.  0 on error. */
+size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass);
+size_t fastmax_workspace_min_bytes(const fastmax_desc* desc, int pass);
+
+/* Forward pass.  Replaces forward_cuda (fastmax_cuda_forward.cu:297-411).
+ *   q, k, v     (bh, n, d)             inputs, never modified
+ *   o           (bh, n, ldo >= d)      out: attention output, columns [0,d)
+ *   den         den[(h*n+i)*den_stride] out: row denominators sum_j f(s_ij); may alias
+ *                                      column d of o (see layout contract)
+ *   qk_scale    2*bh floats or NULL    out: per-head factors applied to q then k
+ *                                      (lim / max row norm, 1/temperature, or 1)
+ *   qk_argmax   2*bh int32 or NULL     out: row index of the max-norm row per head
+ *   workspace   256-byte aligned device memory of workspace_bytes bytes               */
+int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                    void* o, int64_t ldo, float* den, int64_t den_stride,
+                    float* qk_scale, int32_t* qk_argmax,
+                    void* workspace, size_t workspace_bytes, fastmax_stream_t stream);
+
+/* Backward pass.  Replaces backward_cuda (fastmax_cuda_backward.cu:900-1006) and adds the
+ * chain rule through the normalisation that autograd applies to the reference's PyTorch
+ * path (example.py:101-108).
+ *   q, k, v, o, den  as given to / produced by fastmax_forward (q, k un-normalised)
+ *   go               (bh, n, d) upstream gradient, never modified (the reference divides it
+ *                    in place, fastmax_cuda_backward.cu:874-882,970)
+ *   dq, dk, dv       (bh, n, d) out
+ *   qk_scale, qk_argmax  values written by fastmax_forward, or NULL to recompute them   */
+int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                     const void* o, int64_t ldo, const float* den, int64_t den_stride,
+                     const void* go, void* dq, void* dk, void* dv,
+                     const float* qk_scale, const int32_t* qk_argmax,
+                     void* workspace, size_t workspace_bytes, fastmax_stream_t stream);
+
+/* In-place q <- lim*q/max||q_n||, k likewise: the side effect the reference's forward has
+ * on its inputs (calc_norms/find_max/apply_norm, fastmax_cuda_forward.cu:223-269,368-382,
+ * with the PyTorch path's definition of the norm, example.py:105-108).  Only the legacy
+ * forwardpass binding uses it.  workspace: >= 16*bh bytes. */
+int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k,
+                              void* workspace, size_t workspace_bytes, fastmax_stream_t stream);
+
+/* Kernel timing aid (no counterpart in the reference, which only wall-clocks whole calls,
+ * test_fastmax.py:351-356).  Between begin and end every kernel the calling thread launches
+ * through this library is bracketed by two HIP events on the caller's stream; end waits for
+ * them and adds up milliseconds and launch counts per kernel class.  Events are created on
+ * first use and kept by the thread. */
+enum {
+  FASTMAX_K_ROWSTAT = 0,   /* per-head max row norm (or the constant fill)               */
+  FASTMAX_K_BUILD = 1,     /* moment-state build (prefix and suffix states)              */
+  FASTMAX_K_FWD_APPLY = 2, /* forward apply + divide                                     */
+  FASTMAX_K_BWD_PREP = 3,  /* c_i = go_i.o_i/den_i                                       */
+  FASTMAX_K_BWD_DQ = 4,    /* dq                                                         */
+  FASTMAX_K_BWD_DKDV = 5,  /* dk and dv                                                  */
+  FASTMAX_K_NORM_FIX = 6,  /* normalisation chain rule on the max-norm rows              */
+  FASTMAX_NUM_KERNELS = 7
+};
+typedef struct fastmax_kernel_times {
+  float ms[FASTMAX_NUM_KERNELS];
+  int32_t launches[FASTMAX_NUM_KERNELS];
+} fastmax_kernel_times;
+int fastmax_profile_begin(void);
+int fastmax_profile_end(fastmax_kernel_times* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FASTMAX_AMD_H */
