@@ -7,8 +7,8 @@
 //
 // Host code only: tensors, the current stream and the device guard come from torch; all device
 // work happens behind include/fastmax_amd.h.
-#include <c10/hip/HIPGuard.h>
-#include <c10/hip/HIPStream.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
 #include <vector>
@@ -61,7 +61,7 @@ torch::Tensor workspace(const fastmax_desc& ds, int pass, const torch::Tensor& l
 }
 
 fastmax_stream_t current_stream(const torch::Tensor& t) {
-  return reinterpret_cast<fastmax_stream_t>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+  return reinterpret_cast<fastmax_stream_t>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream());
 }
 
 // (o, den, qk_scale, qk_argmax); o is (bh, n, d)
@@ -75,7 +75,7 @@ std::vector<torch::Tensor> forward_ex(torch::Tensor q, torch::Tensor k, torch::T
   check_same(q, v, "v");
   TORCH_CHECK(k.sizes() == v.sizes(), "k and v must have the same shape");
   const fastmax_desc ds = make_desc(q, k, mask, normalize, temperature, a0, a1, a2, lim, p);
-  const c10::hip::HIPGuard guard(q.device());
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
   auto o = torch::empty_like(q);
   auto den = torch::empty({q.size(0), q.size(1)}, q.options().dtype(torch::kFloat32));
   auto scale = torch::empty({2 * q.size(0)}, q.options().dtype(torch::kFloat32));
@@ -110,7 +110,7 @@ std::vector<torch::Tensor> backward_ex(torch::Tensor q, torch::Tensor k, torch::
   TORCH_CHECK(scale.scalar_type() == torch::kFloat32 && scale.numel() == 2 * q.size(0), "qk_scale must be float32 (2*bh)");
   TORCH_CHECK(arg.scalar_type() == torch::kInt32 && arg.numel() == 2 * q.size(0), "qk_argmax must be int32 (2*bh)");
   const fastmax_desc ds = make_desc(q, k, mask, normalize, temperature, a0, a1, a2, lim, p);
-  const c10::hip::HIPGuard guard(q.device());
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
   auto dq = torch::empty_like(q);
   auto dk = torch::empty_like(k);
   auto dv = torch::empty_like(v);
@@ -138,7 +138,7 @@ torch::Tensor forwardpass(torch::Tensor q, torch::Tensor k, torch::Tensor v, tor
   TORCH_CHECK(q.scalar_type() == torch::kFloat32, "forwardpass takes float32 tensors (use forward_ex for bfloat16)");
   TORCH_CHECK(k.sizes() == v.sizes(), "k and v must have the same shape");
   fastmax_desc ds = make_desc(q, k, mask, normalize, 1.0, a0, a1, a2, lim, p);
-  const c10::hip::HIPGuard guard(q.device());
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
   const fastmax_stream_t stream = current_stream(q);
   if (temperature != 1.0) k.div_(temperature);
   if (normalize) {
@@ -180,7 +180,7 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
               "o must be the (bh, n, d+1) tensor forwardpass returned");
   TORCH_CHECK(grad_output.sizes() == q.sizes(), "grad_output must be shaped like q");
   const fastmax_desc ds = make_desc(q, k, mask, false, 1.0, a0, a1, a2, 1.0, p);
-  const c10::hip::HIPGuard guard(q.device());
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
   auto dq = torch::empty_like(q);
   auto dk = torch::empty_like(k);
   auto dv = torch::empty_like(v);

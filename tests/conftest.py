@@ -21,3 +21,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(scope="session")
+def built():
+    """The in-tree native libraries; compiled only if nothing is there yet."""
+    from fastmax_amd import _cabi, _ext
+
+    if not (os.path.exists(_cabi.LIB_PATH) and os.path.exists(_ext.EXT_PATH)):
+        from fastmax_amd import build
+
+        build.build_all()
+    return _cabi.load()

@@ -1,0 +1,99 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares,
+and rejects bad descriptors / pointers / workspaces before anything reaches a device."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from fastmax_amd import _cabi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FAKE = 0x10000  # a non-NULL pointer that is never dereferenced: validation fails first
+
+
+def desc(**over):
+    base = dict(bh=4, n=100, d=64, dtype=_cabi.FASTMAX_F32, mask=True, normalize=True, p=2)
+    base.update(over)
+    return _cabi.make_desc(**base)
+
+
+def test_exports_match_header(built):
+    text = open(os.path.join(ROOT, "include", "fastmax_amd.h")).read()
+    declared = set(re.findall(r"\b(fastmax_[a-z_]+)\s*\(", text))
+    assert declared == set(_cabi.EXPORTS)
+    for name in declared:
+        assert getattr(built, name) is not None
+
+
+def test_version_and_clean_error(built):
+    assert built.fastmax_version().decode() == "0.1"
+    assert built.fastmax_check_desc(C.byref(desc())) == 0
+    assert _cabi.last_error() == ""
+
+
+@pytest.mark.parametrize("over,code", [
+    (dict(d=48), -2), (dict(d=128), -2), (dict(bh=0), -2), (dict(bhkv=2), -2), (dict(nk=50), -2), (dict(n=0), -2),
+    (dict(dtype=7), -3), (dict(p=3), -4), (dict(p=0), -4), (dict(lim=0.0), -4),
+    (dict(normalize=False, temperature=0.0), -4),
+])
+def test_bad_descriptors(built, over, code):
+    assert built.fastmax_check_desc(C.byref(desc(**over))) == code
+    assert _cabi.last_error() != ""
+    assert built.fastmax_workspace_bytes(C.byref(desc(**over)), _cabi.PASS_FORWARD) == 0
+
+
+def test_bad_p_message_matches_reference_wording(built):
+    # the reference raises ValueError(f"p must be 1 or 2, got: {p}") (example.py:195-196)
+    built.fastmax_check_desc(C.byref(desc(p=5)))
+    assert _cabi.last_error() == "p must be 1 or 2, got: 5"
+
+
+def test_null_desc(built):
+    assert built.fastmax_check_desc(None) == -1
+
+
+def test_workspace_sizes(built):
+    for mask in (False, True):
+        for pas in (_cabi.PASS_FORWARD, _cabi.PASS_BACKWARD):
+            ds = desc(bh=1024, n=10000, mask=mask)
+            lo = built.fastmax_workspace_min_bytes(C.byref(ds), pas)
+            hi = built.fastmax_workspace_bytes(C.byref(ds), pas)
+            assert 0 < lo <= hi
+            assert hi <= (6 << 30) + lo
+    # causal d=64 p=2: one state is (33*64 + 64 + 1) rows of 65 floats, one per 256-token chunk
+    ds = desc(bh=1, n=1000, mask=True)
+    state = ((33 * 64 + 65) * 65 + 63) // 64 * 64 * 4
+    assert built.fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_FORWARD) == 512 + 4 * state
+    assert built.fastmax_workspace_bytes(C.byref(ds), 9) == 0  # unknown pass
+
+
+def test_forward_rejects_before_touching_device(built):
+    ds = desc()
+    f = built.fastmax_forward
+    assert f(C.byref(ds), None, FAKE, FAKE, FAKE, 64, FAKE, 1, None, None, FAKE, 1 << 30, None) == -1
+    assert f(C.byref(ds), FAKE, FAKE, FAKE, FAKE, 63, FAKE, 1, None, None, FAKE, 1 << 30, None) == -4  # ldo < d
+    assert f(C.byref(ds), FAKE, FAKE, FAKE, FAKE, 64, FAKE, 0, None, None, FAKE, 1 << 30, None) == -4  # den stride
+    assert f(C.byref(ds), FAKE, FAKE, FAKE, FAKE, 64, FAKE, 1, None, None, None, 1 << 30, None) == -5
+    assert f(C.byref(ds), FAKE, FAKE, FAKE, FAKE, 64, FAKE, 1, None, None, FAKE + 4, 1 << 30, None) == -5  # alignment
+    assert f(C.byref(ds), FAKE, FAKE, FAKE, FAKE, 64, FAKE, 1, None, None, FAKE, 16, None) == -5  # too small
+    assert "minimum" in _cabi.last_error()
+
+
+def test_backward_rejects_before_touching_device(built):
+    ds = desc()
+    b = built.fastmax_backward
+    args = [FAKE] * 3 + [FAKE, 64, FAKE, 1, FAKE, FAKE, FAKE, FAKE, None, None]
+    assert b(C.byref(ds), *args, FAKE, 16, None) == -5
+    args[0] = None
+    assert b(C.byref(ds), *args, FAKE, 1 << 30, None) == -1
+    assert built.fastmax_normalize_inplace(C.byref(ds), None, FAKE, FAKE, 1 << 20, None) == -1
+    assert built.fastmax_normalize_inplace(C.byref(ds), FAKE, FAKE, FAKE, 8, None) == -5
+
+
+def test_profile_end_without_launches(built):
+    kt = _cabi.KernelTimes()
+    assert built.fastmax_profile_begin() == 0
+    assert built.fastmax_profile_end(C.byref(kt)) == 0
+    assert sum(kt.launches) == 0
+    assert built.fastmax_profile_end(None) == -1

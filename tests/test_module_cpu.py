@@ -1,0 +1,112 @@
+"""Host-side mirror of the reference's operator API: signatures, the PyTorch path
+(use_custom_gradient=False) against the oracle, the golden vectors, and the loud failures."""
+import inspect
+
+import pytest
+import torch
+
+import fastmax_amd
+from fastmax_amd import FASTMultiHeadAttention, FASTMultiHeadAttention_Function, fastmax_function
+from oracle import fastmax_oracle as O
+
+from helpers import assert_close, load_golden
+
+GOLD = load_golden()
+
+
+def test_forward_signature_matches_reference():
+    # example.py:219: forward(self, q,k,v,drop_noise=None, mask=False, dropout=0.0, normalize=False,
+    #                         temperature=1.0, a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=2)
+    sig = inspect.signature(FASTMultiHeadAttention.forward)
+    names = list(sig.parameters)
+    assert names == ["self", "q", "k", "v", "drop_noise", "mask", "dropout", "normalize", "temperature",
+                     "a0", "a1", "a2", "lim", "p"]
+    defaults = {k: v.default for k, v in sig.parameters.items() if v.default is not inspect.Parameter.empty}
+    assert defaults == dict(drop_noise=None, mask=False, dropout=0.0, normalize=False, temperature=1.0,
+                            a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=2)
+    assert isinstance(fastmax_amd.fastmax_custom, FASTMultiHeadAttention)
+    assert fastmax_amd.fastmax_custom.use_custom_gradient is True
+    # example.py:83
+    fsig = inspect.signature(fastmax_function)
+    assert list(fsig.parameters)[:12] == ["q", "k", "v", "mask", "dropout_rate", "normalize", "temperature",
+                                          "a0", "a1", "a2", "lim", "p"]
+
+
+@pytest.mark.parametrize("name", sorted(GOLD))
+def test_oracle_reproduces_golden_vectors(name):
+    c = GOLD[name]
+    o, dq, dk, dv = O.dense_truth(c["q"], c["k"], c["v"], c["go"], **c["kw"])
+    _, den = O.dense_truth(c["q"], c["k"], c["v"], None, **c["kw"])
+    for key, got in (("o", o), ("den", den), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert_close(f"{name}/{key}", got, c[key], 2e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("name", sorted(GOLD))
+def test_pytorch_path_matches_golden_vectors(name):
+    c = GOLD[name]
+    kw = c["kw"]
+    q, k, v = (c[t].double().requires_grad_(True) for t in ("q", "k", "v"))
+    mod = FASTMultiHeadAttention(use_custom_gradient=False)
+    o = mod(q, k, v, None, kw["mask"], 0.0, kw["normalize"], 1.0, kw["a0"], kw["a1"], kw["a2"], kw["lim"], kw["p"])
+    o.backward(c["go"].double())
+    for key, got in (("o", o), ("dq", q.grad), ("dk", k.grad), ("dv", v.grad)):
+        assert_close(f"{name}/{key}", got, c[key], 2e-6, atol=1e-9)
+
+
+def test_pytorch_path_chunking_is_exact_across_block_sizes():
+    q, k, v, _ = (t.double() for t in O.seeded_inputs((1, 2, 150, 8), seed=5))
+    ref = O.fastmax_dense(q, k, v, mask=True, normalize=True)
+    for chunk in (1, 7, 64, 150, 1000):
+        got = fastmax_function(q, k, v, 1, 0.0, 1, 1.0, 1.0, 1.0, 0.5, 1.0, 2, chunk=chunk)
+        torch.testing.assert_close(got, ref, rtol=1e-11, atol=1e-12)
+
+
+def test_pytorch_path_ignores_temperature_and_rejects_bad_p():
+    q, k, v, _ = O.seeded_inputs((1, 2, 9, 4), seed=6)
+    a = fastmax_function(q, k, v, 1, 0.0, 0, 5.0)
+    b = fastmax_function(q, k, v, 1, 0.0, 0, 1.0)
+    assert torch.equal(a, b)  # example.py:110-111
+    with pytest.raises(ValueError, match="p must be 1 or 2"):
+        fastmax_function(q, k, v, p=3)
+
+
+def test_pytorch_path_dropout_zeroes_features_only_in_training_semantics():
+    q, k, v, _ = O.seeded_inputs((1, 1, 12, 4), seed=7)
+    torch.manual_seed(0)
+    a = fastmax_function(q, k, v, 0, 0.5, 1)
+    b = fastmax_function(q, k, v, 0, 0.0, 1)
+    assert a.shape == b.shape and not torch.allclose(a, b)
+
+
+def test_custom_path_fails_loudly_on_cpu(built):
+    q, k, v, _ = O.seeded_inputs((1, 2, 9, 4), seed=8)
+    with pytest.raises(RuntimeError, match="GPU"):
+        FASTMultiHeadAttention()(q, k, v)
+    with pytest.raises(RuntimeError, match="GPU"):
+        FASTMultiHeadAttention_Function.apply(q, k, v, None, True)
+
+
+def test_extension_entry_points_and_checks(built):
+    from fastmax_amd import _ext
+
+    ext = _ext.load()
+    for name in ("forwardpass", "backwardpass", "forward_ex", "backward_ex"):
+        assert callable(getattr(ext, name))
+    t = torch.zeros(2, 3, 32)
+    # fastmax_cuda.cpp:13-15: CHECK_CUDA on q, k, v
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        ext.forwardpass(t, t, t, t, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        ext.backwardpass(t, t, t, torch.zeros(2, 3, 33), t, True, 1.0, 1.0, 0.5, 2)
+    mod = fastmax_amd.install_as_fastmax_cuda()
+    import fastmax_cuda  # the name the reference's files import (example.py:4)
+
+    assert fastmax_cuda is mod
+
+
+def test_ops_reject_cpu_and_bad_dtype(built):
+    from fastmax_amd import ops
+
+    t = torch.zeros(2, 3, 32)
+    with pytest.raises(RuntimeError, match="GPU"):
+        ops.forward(t, t, t)

@@ -1,0 +1,282 @@
+"""Parity of the HIP path with the CPU oracle, called through the C ABI (fastmax_amd.ops is a
+ctypes shim over include/fastmax_amd.h) and through the torch extension / module.
+
+Tolerances are the ones the path is specified to: normwise and max-abs relative error
+<= 1e-4 for fp32, <= 2e-2 for bf16 inputs with fp32 accumulation, against the fp64 closed
+form evaluated on the same (bf16-rounded, where applicable) inputs."""
+import pytest
+import torch
+
+from oracle import fastmax_oracle as O
+
+from helpers import TOL, assert_close, load_golden
+
+pytestmark = pytest.mark.gpu
+GOLD = load_golden()
+
+
+@pytest.fixture(scope="module")
+def ops(built):
+    from fastmax_amd import ops as _ops
+
+    return _ops
+
+
+def run_case(ops, shape, dtype=torch.float32, seed=0, check_bwd=True, **kw):
+    q, k, v, go = O.seeded_inputs(shape, seed=seed, dtype=dtype)
+    print("case", shape, dtype, kw, flush=True)
+    qd, kd, vd, god = (t.cuda() for t in (q, k, v, go))
+    o, den, sc, arg = ops.forward(qd, kd, vd, **kw)
+    tol = TOL[dtype]
+    if check_bwd:
+        dq, dk, dv = ops.backward(qd, kd, vd, o, den, god, qk_scale=sc, qk_argmax=arg, **kw)
+        ro, rdq, rdk, rdv = O.dense_truth(q.float(), k.float(), v.float(), go.float(), **kw)
+        for name, got, ref in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+            assert_close(name, got.float(), ref, tol, atol=1e-6)
+    _, rden = O.dense_truth(q.float(), k.float(), v.float(), None, **kw)
+    ro = O.dense_truth(q.float(), k.float(), v.float(), None, **kw)[0]
+    assert_close("o", o.float(), ro, tol)
+    assert_close("den", den, rden, tol if dtype == torch.float32 else 3e-2)
+    return o, den
+
+
+@pytest.mark.parametrize("name", sorted(GOLD))
+def test_golden_vectors(ops, name):
+    c = GOLD[name]
+    q, k, v, go = (c[t].cuda() for t in ("q", "k", "v", "go"))
+    if q.shape[-1] not in (32, 64):
+        from fastmax_amd import _cabi
+
+        with pytest.raises(_cabi.FastmaxError, match="supported head dims"):
+            ops.forward(q, k, v, **c["kw"])
+        return
+    o, den, sc, arg = ops.forward(q, k, v, **c["kw"])
+    dq, dk, dv = ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **c["kw"])
+    for key, got in (("o", o), ("den", den), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert_close(f"{name}/{key}", got, c[key], 1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("d", [32, 64])
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("p", [1, 2])
+@pytest.mark.parametrize("n", [1, 31, 128, 257, 700])
+def test_shapes_fp32(ops, d, mask, p, n):
+    run_case(ops, (3, n, d), seed=n + d, mask=mask, normalize=True, p=p)
+
+
+@pytest.mark.parametrize("mask", [False, True])
+def test_coefficients_lim_and_single_head(ops, mask):
+    run_case(ops, (1, 333, 64), seed=3, mask=mask, normalize=True, p=2, a0=0.7, a1=1.3, a2=0.4, lim=1.5)
+    run_case(ops, (1, 333, 32), seed=4, mask=mask, normalize=True, p=2, a0=2.0, a1=0.5, a2=0.25, lim=0.5)
+
+
+@pytest.mark.parametrize("mask", [False, True])
+def test_unnormalised_small_scores(ops, mask):
+    # without normalisation keep |q.k| small so that the denominator stays well away from zero
+    q, k, v, go = O.seeded_inputs((2, 300, 64), seed=9)
+    q, k = 0.1 * q, 0.1 * k
+    kw = dict(mask=mask, normalize=False, p=2)
+    o, den, sc, arg = ops.forward(q.cuda(), k.cuda(), v.cuda(), **kw)
+    dq, dk, dv = ops.backward(q.cuda(), k.cuda(), v.cuda(), o, den, go.cuda(), **kw)  # scales recomputed
+    ro, rdq, rdk, rdv = O.dense_truth(q, k, v, go, **kw)
+    for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert_close(name, got, ref, 1e-4)
+
+
+def test_temperature_divides_keys_when_not_normalising(ops):
+    # kernel semantics of the reference: k /= temperature (fastmax_cuda_forward.cu:212-221,366)
+    q, k, v, go = O.seeded_inputs((2, 200, 32), seed=10)
+    q, k = 0.2 * q, 0.2 * k
+    T = 2.5
+    o, den, sc, arg = ops.forward(q.cuda(), k.cuda(), v.cuda(), mask=True, normalize=False, temperature=T)
+    dq, dk, dv = ops.backward(q.cuda(), k.cuda(), v.cuda(), o, den, go.cuda(), mask=True, normalize=False,
+                              temperature=T, qk_scale=sc, qk_argmax=arg)
+    ro, rdq, rdk, rdv = O.dense_truth(q, k / T, v, go, mask=True, normalize=False)
+    assert_close("o", o, ro, 1e-4)
+    assert_close("dq", dq, rdq, 1e-4)
+    assert_close("dk", dk, rdk / T, 1e-4)
+    assert_close("dv", dv, rdv, 1e-4)
+
+
+@pytest.mark.parametrize("mask", [False, True])
+def test_bf16_inputs(ops, mask):
+    run_case(ops, (2, 600, 64), dtype=torch.bfloat16, seed=11, mask=mask, normalize=True, p=2)
+    run_case(ops, (2, 300, 32), dtype=torch.bfloat16, seed=12, mask=mask, normalize=True, p=1)
+
+
+def test_deterministic_and_independent_of_head_batching(ops, built):
+    import ctypes as C
+
+    from fastmax_amd import _cabi
+
+    q, k, v, go = (t.cuda() for t in O.seeded_inputs((5, 600, 64), seed=13))
+    kw = dict(mask=True, normalize=True, p=2)
+    a = ops.forward(q, k, v, **kw)
+    b = ops.forward(q, k, v, **kw)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    ga = ops.backward(q, k, v, a[0], a[1], go, qk_scale=a[2], qk_argmax=a[3], **kw)
+    # smallest workspace: one head per batch
+    ds = _cabi.make_desc(5, 600, 64, _cabi.FASTMAX_F32, True, True, 2)
+    wf = built.fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_FORWARD)
+    wb = built.fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_BACKWARD)
+    c = ops.forward(q, k, v, workspace_bytes=wf, **kw)
+    gc = ops.backward(q, k, v, c[0], c[1], go, qk_scale=c[2], qk_argmax=c[3], workspace_bytes=wb, **kw)
+    assert torch.equal(a[0], c[0])
+    for x, y in zip(ga, gc):
+        assert torch.equal(x, y)
+    ops.release_workspaces()
+
+
+def test_denominator_column_layout(ops):
+    q, k, v, _ = (t.cuda() for t in O.seeded_inputs((2, 130, 32), seed=14))
+    o1, den1, _, _ = ops.forward(q, k, v, mask=True, normalize=True)
+    o2, den2, _, _ = ops.forward(q, k, v, mask=True, normalize=True, denominator_column=True)
+    assert o2.shape == (2, 130, 33)
+    assert torch.equal(o2[:, :, :32], o1) and torch.equal(o2[:, :, 32], den1)
+
+
+# ------------------------------------------------------------------ invariants at size
+def test_constant_values_and_running_mean_at_length(ops):
+    bh, n, d = 4, 5000, 64
+    q, k, _, _ = (t.cuda() for t in O.seeded_inputs((bh, n, d), seed=15))
+    v = torch.full((bh, n, d), -1.75, device="cuda")
+    for mask in (False, True):
+        o, den, _, _ = ops.forward(q, k, v, mask=mask, normalize=True)
+        assert float((o - v).abs().max()) < 1e-5
+        assert bool((den > 0).all())
+    v = torch.randn((bh, n, d), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
+    o, den, _, _ = ops.forward(q, k, v, mask=True, normalize=True, a0=2.0, a1=0.0, a2=0.0)
+    want = torch.cumsum(v.double(), 1) / torch.arange(1, n + 1, device="cuda", dtype=torch.float64)[None, :, None]
+    assert_close("running mean", o, want, 1e-4)
+    assert_close("count", den, 2.0 * torch.arange(1, n + 1, dtype=torch.float64).expand(bh, n), 1e-6)
+
+
+def test_linearity_in_values_and_adjoint_identity(ops):
+    bh, n, d = 3, 2000, 64
+    g = torch.Generator(device="cuda").manual_seed(2)
+    q, k, v1, v2, go = (torch.randn((bh, n, d), device="cuda", generator=g) for _ in range(5))
+    kw = dict(mask=True, normalize=True, p=2)
+    o1, den, sc, arg = ops.forward(q, k, v1, **kw)
+    o2 = ops.forward(q, k, v2, **kw)[0]
+    o12 = ops.forward(q, k, 2.0 * v1 - 3.0 * v2, **kw)[0]
+    assert_close("linearity", o12, 2.0 * o1.double() - 3.0 * o2.double(), 1e-4)
+    # <go, o(v2)> == <dv(go), v2> because o is linear in v
+    dv = ops.backward(q, k, v1, o1, den, go, qk_scale=sc, qk_argmax=arg, **kw)[2]
+    lhs = float((go.double() * o2.double()).sum())
+    rhs = float((dv.double() * v2.double()).sum())
+    assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), 1.0)
+
+
+# ------------------------------------------------------------------ configurations of record
+def test_config1_unmasked_b8_h8_n1024_d32(ops):
+    run_case(ops, (64, 1024, 32), seed=0, mask=False, normalize=True, p=2)
+
+
+def test_config2_causal_b64_h8_n1000_d32(ops):
+    run_case(ops, (512, 1000, 32), seed=0, mask=True, normalize=True, p=2)
+
+
+@pytest.mark.parametrize("mask,p", [(True, 2), (False, 2), (True, 1)])
+def test_config3_headline_sampled_heads(ops, mask, p):
+    """B=64 H=16 N=10000 D=64 through the kernels at full size; heads are independent (the
+    normaliser is per head), so fp64 truth on a sample of heads is exact for those heads."""
+    bh, n, d = 1024, 10000, 64
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v, go = (torch.randn((bh, n, d), device="cuda", generator=g) for _ in range(4))
+    kw = dict(mask=mask, normalize=True, p=p)
+    o, den, sc, arg = ops.forward(q, k, v, **kw)
+    dq, dk, dv = ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+    torch.cuda.synchronize()
+    for h in (0, 517, 1023) if (mask and p == 2) else (700,):
+        print("head", h, flush=True)
+        sl = slice(h, h + 1)
+        ro, rdq, rdk, rdv = O.dense_truth(q[sl].cpu(), k[sl].cpu(), v[sl].cpu(), go[sl].cpu(), **kw)
+        for name, got, ref in (("o", o[sl], ro), ("dq", dq[sl], rdq), ("dk", dk[sl], rdk), ("dv", dv[sl], rdv)):
+            assert_close(f"head{h}/{name}", got, ref, 1e-4)
+    del q, k, v, go, o, den, dq, dk, dv
+    ops.release_workspaces()
+    torch.cuda.empty_cache()
+
+
+def test_config4_bf16_long_context_sampled_head(ops):
+    bh, n, d = 512, 16384, 64
+    g = torch.Generator(device="cuda").manual_seed(0)
+    q, k, v, go = (torch.randn((bh, n, d), device="cuda", generator=g).bfloat16() for _ in range(4))
+    kw = dict(mask=True, normalize=True, p=2)
+    o, den, sc, arg = ops.forward(q, k, v, **kw)
+    dq, dk, dv = ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+    torch.cuda.synchronize()
+    sl = slice(311, 312)
+    q1, k1, v1, go1 = (t[sl].float().cpu().double() for t in (q, k, v, go))
+    ro = O.fastmax_dense(q1, k1, v1, **kw)
+    rdq, rdk, rdv = O.fastmax_grads_closed(q1, k1, v1, go1, **kw)
+    for name, got, ref in (("o", o[sl], ro), ("dq", dq[sl], rdq), ("dk", dk[sl], rdk), ("dv", dv[sl], rdv)):
+        assert_close(name, got.float(), ref, 2e-2)
+    del q, k, v, go, o, den, dq, dk, dv
+    ops.release_workspaces()
+    torch.cuda.empty_cache()
+
+
+# ------------------------------------------------------------------ extension and module
+def test_module_autograd_4d(built):
+    from fastmax_amd import FASTMultiHeadAttention
+
+    shape = (2, 3, 300, 64)
+    q, k, v, go = O.seeded_inputs(shape, seed=20)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    mod = FASTMultiHeadAttention()
+    o = mod(qd, kd, vd, None, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
+    assert o.shape == shape
+    o.backward(go.cuda())
+    ro, rdq, rdk, rdv = O.dense_truth(q, k, v, go, mask=True, normalize=True)
+    for name, got, ref in (("o", o, ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+        assert_close(name, got, ref, 1e-4)
+    # unmasked goes through the kernels too, 3-D input keeps its shape
+    o3 = mod(qd.detach().reshape(6, 300, 64), kd.detach().reshape(6, 300, 64), vd.detach().reshape(6, 300, 64),
+             None, False, 0.0, True)
+    assert o3.shape == (6, 300, 64)
+    assert_close("unmasked", o3.reshape(shape), O.dense_truth(q, k, v, None, mask=False, normalize=True)[0], 1e-4)
+
+
+def test_module_output_noise_dropout(built):
+    from fastmax_amd import FASTMultiHeadAttention
+
+    shape = (1, 2, 130, 32)
+    q, k, v, go = O.seeded_inputs(shape, seed=21)
+    noise = O.seeded_inputs(shape, seed=22)[0]
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = FASTMultiHeadAttention()(qd, kd, vd, noise.cuda(), True, 0.3, True)
+    o.backward(go.cuda())
+    fac = 1.0 + 0.3 * noise.double()
+    ro, rdq, rdk, rdv = O.dense_truth(q, k, v, go.double() * fac, mask=True, normalize=True)
+    assert_close("o", o, ro * fac, 1e-4)  # fastmax_cuda_forward.cu:271-280
+    for name, got, ref in (("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+        assert_close(name, got, ref, 1e-4)
+
+
+def test_legacy_extension_entry_points(built):
+    """forwardpass / backwardpass with the reference's positional signatures and side effects."""
+    from fastmax_amd import _ext
+
+    ext = _ext.load()
+    q, k, v, go = O.seeded_inputs((4, 300, 64), seed=23)
+    qd, kd, vd, god = (t.cuda() for t in (q, k, v, go))
+    go_copy = god.clone()
+    o = ext.forwardpass(qd, kd, vd, torch.zeros_like(qd), True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
+    assert o.shape == (4, 300, 65)
+    qh, kh = O.normalize_qk(q[None].double(), k[None].double(), 1.0)
+    assert_close("q normalised in place", qd, qh[0], 1e-6)
+    assert_close("k normalised in place", kd, kh[0], 1e-6)
+    ro, rden = O.dense_truth(q, k, v, None, mask=True, normalize=True)
+    assert_close("o", o[:, :, :64], ro, 1e-4)
+    assert_close("den column", o[:, :, 64], rden, 1e-4)
+    dq, dk, dv = ext.backwardpass(qd, kd, vd, o, god, True, 1.0, 1.0, 0.5, 2)
+    assert torch.equal(god, go_copy)  # not divided in place
+    # gradients w.r.t. the normalised q, k (no chain rule through the normaliser at this boundary)
+    _, rdq, rdk, rdv = O.dense_truth(qh[0], kh[0], v, go, mask=True, normalize=False)
+    for name, got, ref in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert_close(name, got, ref, 1e-4)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ext.forwardpass(qd.transpose(0, 1), kd, vd, qd, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
+    with pytest.raises(RuntimeError, match="p must be 1 or 2"):
+        ext.forwardpass(qd, kd, vd, qd, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 3)
