@@ -98,6 +98,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch", type=int, default=0, help="override B of the workload (profiling aid; "
+                    "the metric is only quoted at the workload's own B)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -112,7 +114,9 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3
-    cfg = WORKLOADS[args.workload]
+    cfg = dict(WORKLOADS[args.workload])
+    if args.batch:
+        cfg["B"] = args.batch
     B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
     bh = B * H
     dtype = torch.float32 if cfg["dtype"] == "f32" else torch.bfloat16

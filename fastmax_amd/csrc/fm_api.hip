@@ -58,7 +58,7 @@ struct ScopedKernel {
 };
 
 constexpr int kChunk = 256;                       // tokens between causal state snapshots
-constexpr size_t kWorkspaceBudget = 6ull << 30;   // what fastmax_workspace_bytes aims for
+constexpr size_t kWorkspaceBudget = 16ull << 30;   // what fastmax_workspace_bytes aims for
 
 struct Plan {
   int d, p2, masked, n, bh;
@@ -111,6 +111,21 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   pl.per_head_bytes = (size_t)pl.nslots * pl.state_floats * sizeof(float) *
                       (pass == FASTMAX_PASS_BACKWARD ? 2 : 1);
   return pl;
+}
+
+// Heads per launch that fit the workspace.  When several batches are needed the batch is
+// rounded down so that the build grid (gsplit blocks per head, two resident blocks per CU)
+// is a whole number of rounds over the 256 CUs; a ragged last round would idle most of the chip.
+int heads_per_batch(const Plan& pl, size_t ws_bytes) {
+  size_t hb = (ws_bytes - pl.fixed_bytes) / pl.per_head_bytes;
+  if (hb >= (size_t)pl.bh) return pl.bh;
+  int g = pl.gsplit, m = 512;
+  while (g % 2 == 0 && m > 1) {
+    g /= 2;
+    m /= 2;
+  }
+  if (hb >= (size_t)m) hb = hb / m * m;
+  return (int)hb;
 }
 
 int check_desc(const fastmax_desc* ds) {
@@ -200,8 +215,7 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   float* scale = reinterpret_cast<float*>(ws);
   int* arg = reinterpret_cast<int*>(ws + align256((size_t)2 * bh * sizeof(float)));
   float* state = reinterpret_cast<float*>(ws + pl.fixed_bytes);
-  size_t hb_sz = (ws_bytes - pl.fixed_bytes) / pl.per_head_bytes;
-  const int hb = (int)(hb_sz > (size_t)bh ? (size_t)bh : hb_sz);
+  const int hb = heads_per_batch(pl, ws_bytes);
 
   FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
   if (scale_out) hipMemcpyAsync(scale_out, scale, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);
@@ -238,8 +252,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
   p += align256((size_t)bh * n * sizeof(float));
   float* rpart = reinterpret_cast<float*>(p);
   float* state = reinterpret_cast<float*>(ws + pl.fixed_bytes);
-  size_t hb_sz = (ws_bytes - pl.fixed_bytes) / pl.per_head_bytes;
-  const int hb = (int)(hb_sz > (size_t)bh ? (size_t)bh : hb_sz);
+  const int hb = heads_per_batch(pl, ws_bytes);
 
   if (scale_in && arg_in) {
     hipMemcpyAsync(scale, scale_in, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);

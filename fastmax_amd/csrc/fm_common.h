@@ -137,6 +137,18 @@ struct RowTile {
       }
     }
   }
+  // transposed: dst is [D][ld] floats in LDS, token rows become columns
+  __device__ __forceinline__ void store_t(float* dst, int ld, float scale, int tid) const {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      const int row = idx / VPR, c4 = idx % VPR;
+      if (idx < TOTAL) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[(c4 * 4 + e) * ld + row] = v[u][e] * scale;
+      }
+    }
+  }
 };
 
 // A run of `count` floats of a moment state staged global -> registers -> LDS, summed over

@@ -99,18 +99,22 @@ __global__ void scale_rows_kernel(T* x, const float* __restrict__ scale, int64_t
 //   add the slots.
 // ---------------------------------------------------------------------------------------
 template <int D, class T, int RTW>
-__global__ __launch_bounds__(256) void build_kernel(
+__global__ __launch_bounds__(256, 2) void build_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const float* __restrict__ xscale,
     const float* __restrict__ yden, int64_t yden_stride, const float* __restrict__ ew,
     float* __restrict__ state, int n, int chunk, int nslots, int masked, int reverse, int p2,
     int zlen) {
   using G = Geo<D>;
-  constexpr int TS = 32;           // tokens per pipeline step
-  constexpr int LDK = D + 1;       // X tile pitch; column D holds 1 (0 for padding rows)
+  constexpr int TS = 32;        // tokens per pipeline step
+  constexpr int TP = TS + 4;    // pitch of the transposed tiles: 16-byte aligned rows, and the
+                                // 8 lanes of a 128-bit LDS access phase fall in distinct banks
   constexpr int CB = G::CB, LD = G::LD;
-  __shared__ float Kl[2][TS * LDK];
-  __shared__ __attribute__((aligned(16))) float Vl[2][TS * D];
-  __shared__ float El[2][TS];
+  // X and Y tiles are staged TRANSPOSED ([channel][token]) so that the four tokens a lane feeds
+  // into four consecutive MFMAs come from one 128-bit LDS read.  Row D of the X tile is 1 for
+  // real tokens and 0 for padding: order-1 features are x[a] * 1.
+  __shared__ __attribute__((aligned(16))) float Kt[2][(D + 1) * TP];
+  __shared__ __attribute__((aligned(16))) float Vt[2][D * TP];
+  __shared__ __attribute__((aligned(16))) float El[2][TS];
 
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, hh = l >> 5;
   const int g = blockIdx.x, head = blockIdx.y;
@@ -118,27 +122,32 @@ __global__ __launch_bounds__(256) void build_kernel(
   const int rt2 = p2 ? G::NS * G::AB : 0, rt_total = rt2 + G::AB;
   const int64_t SS = G::state_floats(p2);
 
-  int owncol[RTW], rotcol[RTW], rowbase[RTW];
+  // per owned row tile: LDS offsets of the lane's own channel row and of its rotated partner
+  int ownoff[RTW], rotoff[RTW], rowbase[RTW];
   int nx = 0;
 #pragma unroll
   for (int x = 0; x < RTW; ++x) {
     const int rt = (g * 4 + w) * RTW + x;
-    owncol[x] = rotcol[x] = rowbase[x] = 0;
+    ownoff[x] = rotoff[x] = 4 * hh;
+    rowbase[x] = 0;
     if (rt < rt_total) {
       nx = x + 1;
       if (rt < rt2) {
         const int s = rt / G::AB, ab = rt % G::AB;
-        owncol[x] = ab * 32 + i;
-        rotcol[x] = (owncol[x] + s) % D;
+        ownoff[x] = (ab * 32 + i) * TP + 4 * hh;
+        rotoff[x] = ((ab * 32 + i + s) % D) * TP + 4 * hh;
         rowbase[x] = s * D + ab * 32;
       } else {
         const int ab = rt - rt2;
-        owncol[x] = ab * 32 + i;
-        rotcol[x] = D;  // the column of ones: order-1 feature is x[a] itself
+        ownoff[x] = (ab * 32 + i) * TP + 4 * hh;
+        rotoff[x] = D * TP + 4 * hh;
         rowbase[x] = rows2 + ab * 32;
       }
     }
   }
+  int voff[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) voff[cb] = (cb * 32 + i) * TP + 4 * hh;
 
   f16v acc[RTW][CB];
   float dacc[RTW];
@@ -170,41 +179,48 @@ __global__ __launch_bounds__(256) void build_kernel(
     }
   };
   auto store = [&](int buf, int t0, int tend) {
-    kx.store(Kl[buf], LDK, xs, tid);
-    vy.store(Vl[buf], D, 1.0f, tid);
+    kx.store_t(Kt[buf], TP, xs, tid);
+    vy.store_t(Vt[buf], TP, 1.0f, tid);
     if (tid < TS) {
       El[buf][tid] = ereg;
-      Kl[buf][tid * LDK + D] = (t0 + tid < tend) ? 1.0f : 0.f;
+      Kt[buf][D * TP + tid] = (t0 + tid < tend) ? 1.0f : 0.f;
     }
   };
   auto compute = [&](int buf) {
-    const float* kb = Kl[buf];
-    const float* vb = Vl[buf];
+    const float* kb = Kt[buf];
+    const float* vb = Vt[buf];
+    const float* eb = El[buf];
 #pragma unroll 2
-    for (int t = 0; t < TS / 2; ++t) {
-      const int j = 2 * t + hh;
-      const float* kr = kb + j * LDK;
-      float vv[CB];
+    for (int grp = 0; grp < TS / 8; ++grp) {
+      // lane half hh takes tokens 8*grp + 4*hh + u, u = 0..3, as the k index of MFMA u
+      const int go8 = 8 * grp;
+      float4 vv[CB];
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) vv[cb] = vb[j * D + cb * 32 + i];
-      const float e = El[buf][j];
+      for (int cb = 0; cb < CB; ++cb) vv[cb] = *reinterpret_cast<const float4*>(vb + voff[cb] + go8);
+      const float4 e4 = *reinterpret_cast<const float4*>(eb + go8 + 4 * hh);
 #pragma unroll
       for (int x = 0; x < RTW; ++x) {
         if (x < nx) {
-          const float a = kr[owncol[x]] * kr[rotcol[x]];
+          const float4 o4 = *reinterpret_cast<const float4*>(kb + ownoff[x] + go8);
+          const float4 r4 = *reinterpret_cast<const float4*>(kb + rotoff[x] + go8);
+          const float a0 = o4.x * r4.x, a1 = o4.y * r4.y, a2 = o4.z * r4.z, a3 = o4.w * r4.w;
 #pragma unroll
-          for (int cb = 0; cb < CB; ++cb) acc[x][cb] = FM_MFMA(a, vv[cb], acc[x][cb]);
-          dacc[x] += a * e;
+          for (int cb = 0; cb < CB; ++cb) {
+            acc[x][cb] = FM_MFMA(a0, vv[cb].x, acc[x][cb]);
+            acc[x][cb] = FM_MFMA(a1, vv[cb].y, acc[x][cb]);
+            acc[x][cb] = FM_MFMA(a2, vv[cb].z, acc[x][cb]);
+            acc[x][cb] = FM_MFMA(a3, vv[cb].w, acc[x][cb]);
+          }
+          dacc[x] += a0 * e4.x + a1 * e4.y + a2 * e4.z + a3 * e4.w;
         }
       }
     }
     if (g == 0 && tid <= D) {
-      if (tid < D) {
-#pragma unroll 8
-        for (int j = 0; j < TS; ++j) s0 += vb[j * D + tid];
-      } else {
-#pragma unroll 8
-        for (int j = 0; j < TS; ++j) s0 += El[buf][j];
+      const float* src = tid < D ? vb + tid * TP : eb;
+#pragma unroll
+      for (int j = 0; j < TS; j += 4) {
+        const float4 t4 = *reinterpret_cast<const float4*>(src + j);
+        s0 += (t4.x + t4.y) + (t4.z + t4.w);
       }
     }
   };

@@ -72,7 +72,7 @@ const char* fastmax_last_error(void);
  * implicit assumptions of fastmax_cuda_forward.cu:331-345 (d == 64, bh == bhkv). */
 int fastmax_check_desc(const fastmax_desc* desc);
 
-/* Bytes of device workspace that let a pass run all heads in as few batches as a 6 GiB
+/* Bytes of device workspace that let a pass run all heads in as few batches as a 16 GiB
  * budget allows (the passes accept anything >= fastmax_workspace_min_bytes and then loop
  * over smaller head batches).  Replaces the torch::zeros scratch tensors of
  * fastmax_cuda_forward.cu:353-357 and fastmax_cuda_backward.cu:957-959.  0 on error. */
