@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const T* __restrict__ go,
 template <int D>
 __device__ __forceinline__ f16v contract_cols(const float* sl, int arow, int hh,
                                               const float (&Gr)[D / 2], float gx) {
-  constexpr int LD = D + 1, H2 = D / 2;
+  constexpr int LD = D + 4, H2 = D / 2;
   f16v t;
 #pragma unroll
   for (int r = 0; r < 16; ++r) t[r] = 0.f;
@@ -114,7 +114,7 @@ __device__ __forceinline__ float write_grad_tile(const f16v (&g)[D / 32], float*
                                                  const float* xl,   // nullable LDS [128][LD]
                                                  T* out_head, int tok0, int n, float scale, int w,
                                                  int i, int hh, int tid) {
-  constexpr int LD = D + 1, AB = D / 32, VPR = D / 4;
+  constexpr int LD = D + 4, AB = D / 32, VPR = D / 4;
   const int qrow = w * 32 + i;
 #pragma unroll
   for (int ab = 0; ab < AB; ++ab)
@@ -152,12 +152,12 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(
     float a2) {
   using G = Geo<D>;
   constexpr int LD = G::LD, AB = G::AB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
-  __shared__ float Ql[128 * LD];
+  __shared__ __attribute__((aligned(16))) float Ql[128 * LD];
   __shared__ __attribute__((aligned(16))) float Sl[2 * SLABF];
   __shared__ float Ml[SYM ? 128 * LD : 1];
   __shared__ float red[4];
 
-  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, hh = l >> 5;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int head = blockIdx.y, tok0 = blockIdx.x * 128;
   const int c = tok0 / chunk;
   const int rows2 = G::rows2(p2);
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(
 // block's own chunk from its own position to the chunk end.
 // ---------------------------------------------------------------------------------------
 template <int D, class T, bool SYM>
-__global__ __launch_bounds__(256) void bwd_dkdv_kernel(
+__global__ __launch_bounds__(256, 2) void bwd_dkdv_kernel(
     const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
     const T* __restrict__ GO, const float* __restrict__ den, int64_t den_stride,
     const float* __restrict__ cvec, const float* __restrict__ qscale,
@@ -296,13 +296,13 @@ __global__ __launch_bounds__(256) void bwd_dkdv_kernel(
     int masked, int p2, float a0, float a1, float a2) {
   using G = Geo<D>;
   constexpr int LD = G::LD, AB = G::AB, CB = G::CB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
-  __shared__ float Kl[128 * LD];
+  __shared__ __attribute__((aligned(16))) float Kl[128 * LD];
   __shared__ __attribute__((aligned(16))) float Sl[2 * SLABF];
   __shared__ float Cl[2][32];
   __shared__ float Ml[SYM ? 128 * LD : 1];
   __shared__ float red[4];
 
-  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, hh = l >> 5;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int head = blockIdx.y, tok0 = blockIdx.x * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;

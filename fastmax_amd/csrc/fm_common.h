@@ -73,8 +73,8 @@ __device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4]) {
 // The order-2 feature of a vector x is stored once per unordered channel pair, indexed by
 // (shift s, channel a) -> x[a] * x[(a+s) mod D], s = 0..D/2.  Shifts 1..D/2-1 carry every
 // pair {a, a+s} exactly once (weight 2 in a full contraction); s = 0 is the diagonal and
-// s = D/2 lists each pair twice (weight 1 each).  Rows of a state, each D+1 floats
-// (D value columns, then the "extra" column that carries the denominator moments):
+// s = D/2 lists each pair twice (weight 1 each).  Rows of a state, each LD = D+4 floats
+// (D value columns, the "extra" column that carries the denominator moments, 3 of padding):
 //   [0, NS*D)            order 2, row s*D + a        (absent when p == 1)
 //   [.., +D)             order 1, row a
 //   last row             order 0
@@ -83,7 +83,9 @@ struct Geo {
   static constexpr int NS = D / 2 + 1;
   static constexpr int AB = D / 32;  // 32-row blocks per shift
   static constexpr int CB = D / 32;  // 32-column blocks of the value dimension
-  static constexpr int LD = D + 1;   // row pitch of states and of every LDS tile
+  static constexpr int LD = D + 4;   // row pitch of states and of every LDS tile: column D is the
+                                     // extra column, D+1..D+3 pad the row to 16 bytes so that
+                                     // row-strided accesses can be 128-bit and bank-conflict-free
   static constexpr int H2 = D / 2;   // channels handled by each lane half per MFMA sweep
   __host__ __device__ static constexpr int rows2(int p2) { return p2 ? NS * D : 0; }
   __host__ __device__ static constexpr int rows(int p2) { return rows2(p2) + D + 1; }
@@ -125,16 +127,15 @@ struct RowTile {
       }
     }
   }
-  // dst is [ROWS][ld] floats in LDS
+  // dst is [ROWS][ld] floats in LDS, 16-byte aligned, ld a multiple of 4
   __device__ __forceinline__ void store(float* dst, int ld, float scale, int tid) const {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
       const int row = idx / VPR, c4 = idx % VPR;
-      if (idx < TOTAL) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) dst[row * ld + c4 * 4 + e] = v[u][e] * scale;
-      }
+      if (idx < TOTAL)
+        *reinterpret_cast<float4*>(dst + row * ld + c4 * 4) =
+            make_float4(v[u][0] * scale, v[u][1] * scale, v[u][2] * scale, v[u][3] * scale);
     }
   }
   // transposed: dst is [D][ld] floats in LDS, token rows become columns

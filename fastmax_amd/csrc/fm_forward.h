@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   __shared__ __attribute__((aligned(16))) float Vt[2][D * TP];
   __shared__ __attribute__((aligned(16))) float El[2][TS];
 
-  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, hh = l >> 5;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int g = blockIdx.x, head = blockIdx.y;
   const int rows2 = G::rows2(p2);
   const int rt2 = p2 ? G::NS * G::AB : 0, rt_total = rt2 + G::AB;
@@ -186,34 +186,46 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       Kt[buf][D * TP + tid] = (t0 + tid < tend) ? 1.0f : 0.f;
     }
   };
+  // operands of one group of 8 tokens (lane half hh takes tokens 8*grp + 4*hh + u, u = 0..3,
+  // as the k index of MFMA u)
+  struct GroupOps {
+    float4 own[RTW], rot[RTW], vv[CB], e4;
+  };
+  auto fetch = [&](const float* kb, const float* vb, const float* eb, int grp, GroupOps& g4) {
+    const int go8 = 8 * grp;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) g4.vv[cb] = *reinterpret_cast<const float4*>(vb + voff[cb] + go8);
+    g4.e4 = *reinterpret_cast<const float4*>(eb + go8 + 4 * hh);
+#pragma unroll
+    for (int x = 0; x < RTW; ++x) {
+      g4.own[x] = *reinterpret_cast<const float4*>(kb + ownoff[x] + go8);
+      g4.rot[x] = *reinterpret_cast<const float4*>(kb + rotoff[x] + go8);
+    }
+  };
   auto compute = [&](int buf) {
     const float* kb = Kt[buf];
     const float* vb = Vt[buf];
     const float* eb = El[buf];
-#pragma unroll 2
-    for (int grp = 0; grp < TS / 8; ++grp) {
-      // lane half hh takes tokens 8*grp + 4*hh + u, u = 0..3, as the k index of MFMA u
-      const int go8 = 8 * grp;
-      float4 vv[CB];
+    GroupOps cur, nxt;
+    fetch(kb, vb, eb, 0, cur);
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) vv[cb] = *reinterpret_cast<const float4*>(vb + voff[cb] + go8);
-      const float4 e4 = *reinterpret_cast<const float4*>(eb + go8 + 4 * hh);
+    for (int grp = 0; grp < TS / 8; ++grp) {
+      if (grp + 1 < TS / 8) fetch(kb, vb, eb, grp + 1, nxt);
+      // tiles past the end of the feature list (x >= nx) run on dummy operands and are never stored
 #pragma unroll
       for (int x = 0; x < RTW; ++x) {
-        if (x < nx) {
-          const float4 o4 = *reinterpret_cast<const float4*>(kb + ownoff[x] + go8);
-          const float4 r4 = *reinterpret_cast<const float4*>(kb + rotoff[x] + go8);
-          const float a0 = o4.x * r4.x, a1 = o4.y * r4.y, a2 = o4.z * r4.z, a3 = o4.w * r4.w;
+        const float a0 = cur.own[x].x * cur.rot[x].x, a1 = cur.own[x].y * cur.rot[x].y;
+        const float a2 = cur.own[x].z * cur.rot[x].z, a3 = cur.own[x].w * cur.rot[x].w;
 #pragma unroll
-          for (int cb = 0; cb < CB; ++cb) {
-            acc[x][cb] = FM_MFMA(a0, vv[cb].x, acc[x][cb]);
-            acc[x][cb] = FM_MFMA(a1, vv[cb].y, acc[x][cb]);
-            acc[x][cb] = FM_MFMA(a2, vv[cb].z, acc[x][cb]);
-            acc[x][cb] = FM_MFMA(a3, vv[cb].w, acc[x][cb]);
-          }
-          dacc[x] += a0 * e4.x + a1 * e4.y + a2 * e4.z + a3 * e4.w;
+        for (int cb = 0; cb < CB; ++cb) {
+          acc[x][cb] = FM_MFMA(a0, cur.vv[cb].x, acc[x][cb]);
+          acc[x][cb] = FM_MFMA(a1, cur.vv[cb].y, acc[x][cb]);
+          acc[x][cb] = FM_MFMA(a2, cur.vv[cb].z, acc[x][cb]);
+          acc[x][cb] = FM_MFMA(a3, cur.vv[cb].w, acc[x][cb]);
         }
+        dacc[x] += a0 * cur.e4.x + a1 * cur.e4.y + a2 * cur.e4.z + a3 * cur.e4.w;
       }
+      if (grp + 1 < TS / 8) cur = nxt;
     }
     if (g == 0 && tid <= D) {
       const float* src = tid < D ? vb + tid * TP : eb;
@@ -292,11 +304,11 @@ __global__ __launch_bounds__(256) void fwd_apply_kernel(
     float a1, float a2) {
   using G = Geo<D>;
   constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
-  __shared__ float Ql[128 * LD];
+  __shared__ __attribute__((aligned(16))) float Ql[128 * LD];
   __shared__ __attribute__((aligned(16))) float Sl[2][SLABF];
   __shared__ float denl[128];
 
-  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, i = l & 31, hh = l >> 5;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int head = blockIdx.y, tok0 = blockIdx.x * 128;
   const int c = tok0 / chunk;
   const int rows2 = G::rows2(p2);
