@@ -46,7 +46,8 @@ def algorithmic_flops(d: int, p: int) -> dict:
         "build": 2 * feat * (d + 1),              # one moment state (prefix or suffix)
         "fwd_apply": 2 * feat * (d + 1),
         "bwd_dq": 2 * (feat - 1) * (d + 1),
-        "bwd_dkdv": 2 * (feat - 1) * (d + 1) + 2 * feat * d,
+        "bwd_dk": 2 * (feat - 1) * (d + 1),
+        "bwd_dv": 2 * feat * d,
         "fwd": 4 * feat * (d + 1),
         "bwd": 2 * (2 * feat * (d + 1) + 2 * (feat - 1) * (d + 1) + feat * d),
     }
@@ -165,7 +166,8 @@ def main() -> int:
             kernels[name] = {"ms_per_step": kt.ms[i] / args.steps, "launches_per_step": kt.launches[i] / args.steps}
     # algorithmic flops each kernel class executes per step (build runs 3x: fwd prefix, bwd prefix, bwd suffix)
     per_step_flops = {"build": 3 * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
-                      "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dkdv": fl["bwd_dkdv"] * token_heads}
+                      "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dk": fl["bwd_dk"] * token_heads,
+                      "bwd_dv": fl["bwd_dv"] * token_heads}
     dom = max(per_step_flops, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0))
     dom_ms = kernels[dom]["ms_per_step"]
     launches = kernels[dom]["launches_per_step"]

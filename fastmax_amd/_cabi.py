@@ -27,11 +27,11 @@ EXPORTS = (
     "fastmax_profile_begin", "fastmax_profile_end",
 )
 
-KERNEL_NAMES = ("rowstat", "build", "fwd_apply", "bwd_prep", "bwd_dq", "bwd_dkdv", "norm_fix")
+KERNEL_NAMES = ("rowstat", "build", "fwd_apply", "bwd_prep", "bwd_dq", "bwd_dk", "bwd_dv", "norm_fix")
 
 
 class KernelTimes(C.Structure):
-    _fields_ = [("ms", C.c_float * 7), ("launches", C.c_int32 * 7)]
+    _fields_ = [("ms", C.c_float * 8), ("launches", C.c_int32 * 8)]
 
 
 class FastmaxDesc(C.Structure):

@@ -8,8 +8,10 @@
 #include <vector>
 
 #include "fastmax_amd.h"
+#include "fm_apply.h"
 #include "fm_backward.h"
 #include "fm_forward.h"
+#include "fm_grad.h"
 
 namespace {
 
@@ -227,8 +229,8 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
     FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, state, 0, stream)));
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
-      fwd_apply_kernel<D, T><<<dim3(pl.nblk, heads), 256, 0, stream>>>(
-          q + off, k + off, v + off, scale + h0, scale + bh + h0, state, pl.nslots,
+      apply_kernel<D, T, 0><<<dim3(pl.nblk, heads), 256, 0, stream>>>(
+          q + off, k + off, v + off, scale + h0, scale + bh + h0, nullptr, 0, state, pl.nslots,
           o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, kChunk,
           pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
     }
@@ -281,19 +283,27 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     const dim3 grid(pl.nblk, heads);
     {
       ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
-      bwd_dq_kernel<D, T, false><<<grid, 256, 0, stream>>>(
-          q + off, k + off, v + off, go + off, denh, den_stride, ch, scale + h0, scale + bh + h0, stS,
-          pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, kChunk, pl.masked, pl.p2, ds->a1, a2);
+      grad_kernel<D, T, 0><<<grid, 256, 0, stream>>>(
+          q + off, go + off, denh, den_stride, ch, k + off, v + off, nullptr, 0, scale + h0,
+          scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, kChunk, pl.masked,
+          pl.p2, ds->a1, a2);
     }
-    FM_TRY(launch_status("bwd_dq_kernel"));
+    FM_TRY(launch_status("grad_kernel (dq)"));
     {
-      ScopedKernel sk(FASTMAX_K_BWD_DKDV, stream);
-      bwd_dkdv_kernel<D, T, false><<<grid, 256, 0, stream>>>(
-          q + off, k + off, v + off, go + off, denh, den_stride, ch, scale + h0, scale + bh + h0, stR,
-          pl.nslots, dk + off, dv + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, kChunk, pl.masked,
-          pl.p2, ds->a0, ds->a1, a2);
+      ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
+      grad_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
+          k + off, v + off, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + h0,
+          scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, kChunk,
+          pl.masked, pl.p2, ds->a1, a2);
     }
-    FM_TRY(launch_status("bwd_dkdv_kernel"));
+    FM_TRY(launch_status("grad_kernel (dk)"));
+    {
+      ScopedKernel sk(FASTMAX_K_BWD_DV, stream);
+      apply_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
+          k + off, q + off, go + off, scale + bh + h0, scale + h0, denh, den_stride, stR, pl.nslots,
+          dv + off, D, nullptr, 0, n, kChunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
+    }
+    FM_TRY(launch_status("apply_kernel (dv)"));
   }
   if (ds->normalize) {
     ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);

@@ -1,0 +1,274 @@
+// Row-apply kernel: contracts generated features of the block's own tokens with a moment state.
+//   MODE 0  forward:  [num_i, den_i] = phi(qh_i) . S (+ causal intra-chunk tile), o = num/den
+//   MODE 1  dv:       dv_j = phi(kh_j) . R (+ causal intra-chunk tile  sum_{i>=j} f(s_ij) g_i)
+#pragma once
+#include <type_traits>
+
+#include "fm_common.h"
+
+// interleave hint for the instruction scheduler: n x (1 MFMA, 1 LDS read, 1 VALU)
+#define FM_SCHED_MFMA_DS_VALU(n)                            \
+  _Pragma("unroll") for (int q_ = 0; q_ < (n); ++q_) {      \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      \
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      \
+    __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);      \
+  }
+
+// ---------------------------------------------------------------------------------------
+// One block = 128 tokens of one head, one wave = 32 of them.  Lane (i = l%32, hh = l/32) keeps
+// its own half of x_i in registers (channels t + hh*D/2) and a sliding window of the rotated
+// partners x_i[(a+s)%D] (reloaded from LDS every fourth shift, slid by one register in
+// between), so an order-2 feature costs one multiply of two registers.  The state streams
+// through a double-buffered LDS slab (one shift = D rows at a time), coefficients a2*w_s / a1 /
+// a0 applied while staging; its rows are the B operands (two column tiles per feature) and, in
+// the forward pass, its extra column gives the denominator.
+// For causal attention 32-token tiles of the block's own chunk follow through the same
+// buffers: scores are formed transposed (streamed tokens x own tokens) so that the polynomial
+// of the score tile, still in accumulator registers, is directly the A operand of the product
+// with the streamed value rows.
+//
+// A wave cannot overlap its own VALU/LDS work with its own MFMAs, so the kernel is built for
+// two resident blocks per CU and keeps the non-MFMA instruction count low: operands of eight
+// MFMA k-steps are fetched one batch ahead of their use.
+//
+//   X   own rows (q forward, k for dv), scaled by xscale[head]
+//   A1  streamed rows the scores are taken with (k forward, q for dv), scaled by a1scale[head]
+//   A2  streamed value rows (v forward; grad_out for dv, divided by a2den per row)
+// ---------------------------------------------------------------------------------------
+template <int D, class T, int MODE>
+__global__ __launch_bounds__(256, 2) void apply_kernel(
+    const T* __restrict__ X, const T* __restrict__ A1, const T* __restrict__ A2,
+    const float* __restrict__ xscale, const float* __restrict__ a1scale,
+    const float* __restrict__ a2den, int64_t a2den_stride, const float* __restrict__ state,
+    int nslots, T* __restrict__ OUT, int64_t ldo, float* __restrict__ den, int64_t den_stride, int n,
+    int chunk, int masked, int p2, float a0, float a1, float a2) {
+  using G = Geo<D>;
+  constexpr bool FWD = MODE == 0;
+  constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
+  constexpr int KB = 8;  // k-steps per operand batch
+  __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
+  __shared__ __attribute__((aligned(16))) float Sl[2][SLABF];
+  __shared__ float denl[128];
+
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
+  const int head = blockIdx.y, tok0 = blockIdx.x * 128;
+  const int c = tok0 / chunk;
+  const int nc = (n + chunk - 1) / chunk;
+  const int rows2 = G::rows2(p2);
+  const int64_t SS = G::state_floats(p2);
+  const T* Xh = X + (int64_t)head * n * D;
+  const T* A1h = A1 + (int64_t)head * n * D;
+  const T* A2h = A2 + (int64_t)head * n * D;
+  const float* a2dh = a2den ? a2den + (int64_t)head * n * a2den_stride : nullptr;
+  const float xs = xscale[head], a1s = a1scale[head];
+
+  {
+    RowTile<D, T, 128> xt;
+    xt.load(Xh, tok0, n, tid);
+    xt.store(Xl, LD, xs, tid);
+  }
+
+  // the state is all zero for the first chunk in scan order
+  const bool no_state = masked && (FWD ? c == 0 : c == nc - 1);
+  const int n_state = no_state ? 0 : (p2 ? NS : 0) + 1;
+  // streamed tiles: forward = key tiles from the chunk start to this block's last tile;
+  // dv = query tiles from this block's first tile to the chunk end
+  int n_tile = 0, tile0 = 0;
+  if (masked) {
+    if (FWD) {
+      tile0 = (c * chunk) >> 5;
+      const int last = tok0 + 127 < n ? tok0 + 127 : n - 1;
+      n_tile = (last >> 5) - tile0 + 1;
+    } else {
+      tile0 = tok0 >> 5;
+      const int cend = (c + 1) * chunk < n ? (c + 1) * chunk : n;
+      n_tile = ((cend - 1) >> 5) - tile0 + 1;
+    }
+  }
+  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
+  const int nsum = masked ? 1 : nslots;
+
+  StateSlab<(D + 1) * LD> slab;
+  RowTile<D, T, 32> t1, t2;
+  auto slab_load = [&](int st) {
+    const bool ord2 = p2 && st < NS;
+    slab.load(sbase + (ord2 ? st * D * LD : rows2 * LD), SS, nsum, ord2 ? D * LD : (D + 1) * LD, tid);
+  };
+  auto slab_store = [&](int st) {
+    if (p2 && st < NS) {
+      const float cf = (st == 0 || st == H2) ? a2 : 2.0f * a2;
+      slab.store(Sl[st & 1], D * LD, D * LD, cf, cf, tid);
+    } else {
+      slab.store(Sl[st & 1], (D + 1) * LD, D * LD, a1, a0, tid);
+    }
+  };
+  auto tiles_load = [&](int kk) {
+    t1.load(A1h, (tile0 + kk) * 32, n, tid);
+    t2.load(A2h, (tile0 + kk) * 32, n, tid, a2dh, a2den_stride);
+  };
+  auto tiles_store = [&](int buf) {
+    t1.store(Sl[buf], LD, a1s, tid);
+    t2.store(Sl[buf] + 32 * LD, LD, 1.0f, tid);
+  };
+
+  if (n_tile > 0) tiles_load(0);
+  if (n_state > 0) {
+    slab_load(0);
+    slab_store(0);
+  } else if (n_tile > 0) {
+    tiles_store(0);
+  }
+  __syncthreads();
+
+  const int xrow = w * 32 + i;
+  float Xr[H2];
+#pragma unroll
+  for (int t = 0; t < H2; t += 4) {
+    const float4 q4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + hh * H2 + t);
+    Xr[t] = q4.x; Xr[t + 1] = q4.y; Xr[t + 2] = q4.z; Xr[t + 3] = q4.w;
+  }
+
+  f16v acc[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[cb][r] = 0.f;
+  float dn = 0.f;
+
+  // rotated partners: after window_load(s0) (s0 % 4 == 0), Wn[x] = x_i[(hh*H2 + s0 + x) % D]
+  float Wn[H2 + 4];
+  auto window_load = [&](int s0) {
+#pragma unroll
+    for (int j = 0; j < H2 / 4 + 1; ++j) {
+      const int c0 = (hh * H2 + s0 + 4 * j) & (D - 1);
+      const float4 q4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + c0);
+      Wn[4 * j] = q4.x; Wn[4 * j + 1] = q4.y; Wn[4 * j + 2] = q4.z; Wn[4 * j + 3] = q4.w;
+    }
+  };
+
+  // operands of KB k-steps of a slab: rows a = t + hh*H2, value columns i and 32+i, extra column
+  struct Batch {
+    float b[KB][CB], dd[KB];
+  };
+  auto batch_fetch = [&](const float* sl, int t0, Batch& bt) {
+    const float* base = sl + (hh * H2 + t0) * LD;
+#pragma unroll
+    for (int e = 0; e < KB; ++e) {
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) bt.b[e][cb] = base[e * LD + cb * 32 + i];
+      if (FWD) bt.dd[e] = base[e * LD + D];
+    }
+  };
+  // one slab; ORD2 = false is the order-1 sweep (feature = x[a] itself)
+  auto slab_compute = [&](const float* sl, auto tag) {
+    constexpr bool ORD2 = decltype(tag)::value;
+    Batch cur, nxt;
+    batch_fetch(sl, 0, cur);
+#pragma unroll
+    for (int t0 = 0; t0 < H2; t0 += KB) {
+      if (t0 + KB < H2) batch_fetch(sl, t0 + KB, nxt);
+#pragma unroll
+      for (int e = 0; e < KB; ++e) {
+        const float a = ORD2 ? Xr[t0 + e] * Wn[t0 + e] : Xr[t0 + e];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA(a, cur.b[e][cb], acc[cb]);
+        if (FWD) dn += a * cur.dd[e];
+      }
+      FM_SCHED_MFMA_DS_VALU(KB * CB)
+      if (t0 + KB < H2) cur = nxt;
+    }
+  };
+
+  for (int st = 0; st < n_state; ++st) {
+    slab_load(st + 1 < n_state ? st + 1 : st);
+    const float* sl = Sl[st & 1];
+    if (p2 && st < NS) {
+      // window of rotated partners for shift st: reloaded every fourth shift, slid by one otherwise
+      if ((st & 3) == 0) {
+        window_load(st);
+      } else {
+#pragma unroll
+        for (int x = 0; x < H2 + 3; ++x) Wn[x] = Wn[x + 1];
+      }
+      slab_compute(sl, std::true_type{});
+    } else {
+      slab_compute(sl, std::false_type{});
+      const float* s0 = sl + D * LD;  // order 0 rides at the end of the order-1 slab
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const float z = s0[cb * 32 + i];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[cb][r] += z;
+      }
+      if (FWD && hh == 0) dn += s0[D];
+    }
+    if (st + 1 < n_state) slab_store(st + 1);
+    else if (n_tile > 0) tiles_store((st + 1) & 1);
+    __syncthreads();
+  }
+
+  const int mine = (tok0 >> 5) + w;
+  for (int kk = 0; kk < n_tile; ++kk) {
+    const int buf = (n_state + kk) & 1;
+    tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
+    const int tl = tile0 + kk;
+    if (FWD ? tl <= mine : tl >= mine) {
+      const float* l1 = Sl[buf];
+      const float* l2 = Sl[buf] + 32 * LD;
+      // scores, transposed: rows = streamed tokens trow(r,hh), lanes = own tokens
+      f16v sc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+      for (int t = 0; t < H2; t += 4) {
+        const float4 k4 = *reinterpret_cast<const float4*>(l1 + i * LD + hh * H2 + t);
+        sc = FM_MFMA(k4.x, Xr[t], sc);
+        sc = FM_MFMA(k4.y, Xr[t + 1], sc);
+        sc = FM_MFMA(k4.z, Xr[t + 2], sc);
+        sc = FM_MFMA(k4.w, Xr[t + 3], sc);
+      }
+      float vv[16][CB];
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) vv[r][cb] = l2[trow(r, hh) * LD + cb * 32 + i];
+      const bool diag = tl == mine;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float s = sc[r];
+        float f = a0 + s * (a1 + a2 * s);
+        // causal: a key may not lie after the query
+        if (diag && (FWD ? trow(r, hh) > i : trow(r, hh) < i)) f = 0.f;
+        sc[r] = f;
+        if (FWD) dn += f;
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA(sc[r], vv[r][cb], acc[cb]);
+    }
+    if (kk + 1 < n_tile) tiles_store(buf ^ 1);
+    __syncthreads();
+  }
+
+  if (FWD) {
+    const float dtot = dn + __shfl_xor(dn, 32, 64);
+    const int tok = tok0 + xrow;
+    if (hh == 0) {
+      denl[xrow] = dtot;
+      if (tok < n) den[((int64_t)head * n + tok) * den_stride] = dtot;
+    }
+    __syncthreads();
+  }
+  T* Oh = OUT + (int64_t)head * n * ldo;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = w * 32 + trow(r, hh);
+    const int tk = tok0 + row;
+    if (tk < n) {
+      const float inv = FWD ? 1.0f / denl[row] : 1.0f;
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) Oh[(int64_t)tk * ldo + cb * 32 + i] = from_f32<T>(acc[cb][r] * inv);
+    }
+  }
+}

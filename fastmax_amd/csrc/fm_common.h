@@ -138,6 +138,18 @@ struct RowTile {
             make_float4(v[u][0] * scale, v[u][1] * scale, v[u][2] * scale, v[u][3] * scale);
     }
   }
+  // same with scalar stores, for an odd pitch
+  __device__ __forceinline__ void store_s(float* dst, int ld, float scale, int tid) const {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      const int row = idx / VPR, c4 = idx % VPR;
+      if (idx < TOTAL) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[row * ld + c4 * 4 + e] = v[u][e] * scale;
+      }
+    }
+  }
   // transposed: dst is [D][ld] floats in LDS, token rows become columns
   __device__ __forceinline__ void store_t(float* dst, int ld, float scale, int tid) const {
 #pragma unroll

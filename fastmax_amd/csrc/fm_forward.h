@@ -1,6 +1,8 @@
 // Forward-side kernels: per-head row-norm statistics, the moment-state build (used by
 // both passes) and the forward apply.
 #pragma once
+#include <type_traits>
+
 #include "fm_common.h"
 
 // ---------------------------------------------------------------------------------------
@@ -280,189 +282,5 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     const int te = (z + 1) * zlen < n ? (z + 1) * zlen : n;
     run(z * zlen, te);
     snapshot(z);
-  }
-}
-
-// ---------------------------------------------------------------------------------------
-// Forward apply:  [num_i, den_i] = phi(q_i) . S  (+ the causal intra-chunk tile), o = num/den.
-//
-// One block = 128 query tokens of one head, one wave = 32 of them.  Lane (i = l%32, hh = l/32)
-// keeps q_i[t + hh*D/2] in registers (A-operand side of the order-2 feature) and reads the
-// rotated partner q_i[(a+s)%D] from the LDS copy of the tile, so a feature costs one LDS
-// read and one multiply per MFMA pair.  The state streams through a double-buffered LDS slab
-// (one shift = D rows at a time), coefficients a2*w_s / a1 / a0 applied while staging.
-// For causal attention the same stream then carries the 32-key tiles of the block's own
-// chunk: scores are formed transposed (keys x queries) so that the polynomial of the score
-// tile is directly the A operand of the P.V product.
-// ---------------------------------------------------------------------------------------
-template <int D, class T>
-__global__ __launch_bounds__(256) void fwd_apply_kernel(
-    const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
-    const float* __restrict__ qscale, const float* __restrict__ kscale,
-    const float* __restrict__ state, int nslots, T* __restrict__ O, int64_t ldo,
-    float* __restrict__ den, int64_t den_stride, int n, int chunk, int masked, int p2, float a0,
-    float a1, float a2) {
-  using G = Geo<D>;
-  constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
-  __shared__ __attribute__((aligned(16))) float Ql[128 * LD];
-  __shared__ __attribute__((aligned(16))) float Sl[2][SLABF];
-  __shared__ float denl[128];
-
-  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
-  const int head = blockIdx.y, tok0 = blockIdx.x * 128;
-  const int c = tok0 / chunk;
-  const int rows2 = G::rows2(p2);
-  const int64_t SS = G::state_floats(p2);
-  const T* Qh = Q + (int64_t)head * n * D;
-  const T* Kh = K + (int64_t)head * n * D;
-  const T* Vh = V + (int64_t)head * n * D;
-  const float qs = qscale[head], ks = kscale[head];
-
-  {  // stage the query tile; column D is the constant 1 used by the order-1 sweep
-    RowTile<D, T, 128> qt;
-    qt.load(Qh, tok0, n, tid);
-    qt.store(Ql, LD, qs, tid);
-    if (tid < 128) Ql[tid * LD + D] = 1.0f;
-  }
-
-  const int n_state = (masked && c == 0) ? 0 : (p2 ? NS : 0) + 1;
-  int n_key = 0, kt0 = 0;
-  if (masked) {
-    kt0 = (c * chunk) >> 5;
-    int last = tok0 + 127 < n ? tok0 + 127 : n - 1;
-    n_key = (last >> 5) - kt0 + 1;
-  }
-  const int n_stage = n_state + n_key;
-  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
-  const int nsum = masked ? 1 : nslots;
-
-  StateSlab<(D + 1) * LD> slab;
-  RowTile<D, T, 32> kt_k, kt_v;
-
-  // stage st is a state slab (st < n_state) or a key tile
-  auto stage_load = [&](int st) {
-    if (st < n_state) {
-      const bool ord2 = p2 && st < NS;
-      const int off = ord2 ? st * D * LD : rows2 * LD;
-      const int cnt = ord2 ? D * LD : (D + 1) * LD;
-      slab.load(sbase + off, SS, nsum, cnt, tid);
-    } else {
-      const int kt = kt0 + (st - n_state);
-      kt_k.load(Kh, kt * 32, n, tid);
-      kt_v.load(Vh, kt * 32, n, tid);
-    }
-  };
-  auto stage_store = [&](int st) {
-    float* dst = Sl[st & 1];
-    if (st < n_state) {
-      const bool ord2 = p2 && st < NS;
-      if (ord2) {
-        const float cf = (st == 0 || st == H2) ? a2 : 2.0f * a2;
-        slab.store(dst, D * LD, D * LD, cf, cf, tid);
-      } else {
-        slab.store(dst, (D + 1) * LD, D * LD, a1, a0, tid);
-      }
-    } else {
-      kt_k.store(dst, LD, ks, tid);
-      kt_v.store(dst + 32 * LD, LD, 1.0f, tid);
-    }
-  };
-
-  __syncthreads();
-  const int qrow = w * 32 + i;
-  float Qr[H2];
-#pragma unroll
-  for (int t = 0; t < H2; ++t) Qr[t] = Ql[qrow * LD + t + hh * H2];
-
-  f16v acc[CB];
-#pragma unroll
-  for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[cb][r] = 0.f;
-  float dn = 0.f;
-
-  if (n_stage > 0) {
-    stage_load(0);
-    stage_store(0);
-  }
-  __syncthreads();
-  const int qt_mine = (tok0 >> 5) + w;
-  for (int st = 0; st < n_stage; ++st) {
-    const bool more = st + 1 < n_stage;
-    if (more) stage_load(st + 1);
-    const float* sl = Sl[st & 1];
-    if (st < n_state) {
-      const bool ord2 = p2 && st < NS;
-      const int rbase = hh * H2 + st;  // (a + s) for t = 0; order-1 reads the ones column
-      const float* qr = Ql + qrow * LD;
-#pragma unroll
-      for (int t = 0; t < H2; ++t) {
-        int rc = rbase + t;
-        rc -= (rc >= D) ? D : 0;
-        rc = ord2 ? rc : D;
-        const float a = Qr[t] * qr[rc];
-        const float* srow = sl + (t + hh * H2) * LD;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA(a, srow[cb * 32 + i], acc[cb]);
-        dn += a * srow[D];
-      }
-      if (!ord2) {  // order 0 rides at the end of the order-1 slab
-        const float* s0 = sl + D * LD;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-          const float z = s0[cb * 32 + i];
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[cb][r] += z;
-        }
-        if (hh == 0) dn += s0[D];
-      }
-    } else {
-      const int kt = kt0 + (st - n_state);
-      if (kt <= qt_mine) {
-        const float* kl = sl;
-        const float* vl = sl + 32 * LD;
-        f16v sc;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-#pragma unroll
-        for (int t = 0; t < H2; ++t) sc = FM_MFMA(kl[i * LD + t + hh * H2], Qr[t], sc);
-        const bool diag = kt == qt_mine;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float s = sc[r];
-          float f = a0 + s * (a1 + a2 * s);
-          if (diag && trow(r, hh) > i) f = 0.f;
-          sc[r] = f;
-          dn += f;
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float* vrow = vl + trow(r, hh) * LD;
-#pragma unroll
-          for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA(sc[r], vrow[cb * 32 + i], acc[cb]);
-        }
-      }
-    }
-    if (more) stage_store(st + 1);
-    __syncthreads();
-  }
-
-  const float dtot = dn + __shfl_xor(dn, 32, 64);
-  const int tok = tok0 + qrow;
-  if (hh == 0) {
-    denl[qrow] = dtot;
-    if (tok < n) den[((int64_t)head * n + tok) * den_stride] = dtot;
-  }
-  __syncthreads();
-  T* Oh = O + (int64_t)head * n * ldo;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = w * 32 + trow(r, hh);
-    const int tk = tok0 + row;
-    if (tk < n) {
-      const float inv = 1.0f / denl[row];
-#pragma unroll
-      for (int cb = 0; cb < CB; ++cb) Oh[(int64_t)tk * ldo + cb * 32 + i] = from_f32<T>(acc[cb][r] * inv);
-    }
   }
 }

@@ -1,0 +1,283 @@
+// Column-contraction kernel: gradients with respect to the normalised q (MODE 0) or k (MODE 1).
+//
+// With g_i = go_i/den_i, c_i = g_i.o_i and W_ij = f'(s_ij)(g_i.v_j - c_i):
+//   dqh_i = sum_j W_ij kh_j = a1 S1 [g_i,-c_i] + 2 a2 sum_b qh_i[b] (S2[.,b,:] [g_i,-c_i])   (+ intra-chunk)
+//   dkh_j = sum_i W_ij qh_i = a1 R1 [v_j,-1]  + 2 a2 sum_b kh_j[b] (R2[.,b,:] [v_j,-1])     (+ intra-chunk)
+// where S = sum phi(kh) (x) [v,1] over the keys before the chunk and R = sum phi(qh) (x) [g,c] over
+// the queries after it.  Both are the same computation with the roles of the operands swapped.
+#pragma once
+#include "fm_apply.h"
+#include "fm_common.h"
+
+// ---------------------------------------------------------------------------------------
+// One block = 128 own tokens of one head, one wave = 32 of them, tokens in lanes.  Per shift
+// slab of the state the kernel contracts 32 state rows at a time over the D+1 columns with the
+// token's extended value vector y_ext = [y, yx] (B operand straight from registers, one extra
+// MFMA for the extra column); the result T[r] is the entry (a, a+s) of the token's symmetric
+// matrix for channel a = ab*32 + trow(r,hh), and out[a] += T * x[(a+s)%D] is a register FMA
+// with one LDS read.  The state stores each unordered pair {a, a+s} once, so for 0 < s < D/2
+// the same slab is contracted a second time over rows rotated by -s to credit the pair's
+// other member (twice the minimal MFMA work).
+// Causal intra-chunk part: for every streamed 32-token tile the transposed score and g.v tiles
+// are formed, W is built in registers and fed back as the B operand of  out^T += A1^T W.
+//
+//   MODE 0 (dq): X = q, Y = grad_out/den, yx = -c_i, state S, streamed A1 = k, A2 = v over tiles
+//                at or before the own tile, W = f'(s)(g.v - c_own)
+//   MODE 1 (dk): X = k, Y = v, yx = -1, state R, streamed A1 = q, A2 = grad_out/den over tiles
+//                at or after the own tile, W = f'(s)(g.v - c_streamed)
+// rpart[head*gridDim.x + block] = sum over the block of out . x_hat (normalisation backward).
+// ---------------------------------------------------------------------------------------
+template <int D, class T, int MODE>
+__global__ __launch_bounds__(256, 2) void grad_kernel(
+    const T* __restrict__ X, const T* __restrict__ Y, const float* __restrict__ yden,
+    int64_t yden_stride, const float* __restrict__ cvec, const T* __restrict__ A1,
+    const T* __restrict__ A2, const float* __restrict__ a2den, int64_t a2den_stride,
+    const float* __restrict__ xscale, const float* __restrict__ a1scale,
+    const float* __restrict__ state, int nslots, T* __restrict__ OUT, float* __restrict__ rpart,
+    int n, int chunk, int masked, int p2, float a1, float a2) {
+  using G = Geo<D>;
+  constexpr bool DQ = MODE == 0;
+  constexpr int LD = G::LD, AB = G::AB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
+  constexpr int LX = D + 1;  // odd pitch: the scalar rotated reads of x are bank-conflict-free
+  __shared__ float Xl[128 * LX];
+  __shared__ __attribute__((aligned(16))) float Sl[2 * SLABF];
+  __shared__ float Cl[2][32];
+  __shared__ float red[4];
+
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
+  const int head = blockIdx.y, tok0 = blockIdx.x * 128;
+  const int c = tok0 / chunk;
+  const int nc = (n + chunk - 1) / chunk;
+  const int rows2 = G::rows2(p2);
+  const int64_t SS = G::state_floats(p2);
+  const T* Xh = X + (int64_t)head * n * D;
+  const T* Yh = Y + (int64_t)head * n * D;
+  const T* A1h = A1 + (int64_t)head * n * D;
+  const T* A2h = A2 + (int64_t)head * n * D;
+  const float* ydh = yden ? yden + (int64_t)head * n * yden_stride : nullptr;
+  const float* a2dh = a2den ? a2den + (int64_t)head * n * a2den_stride : nullptr;
+  const float* ch = cvec + (int64_t)head * n;
+  const float xs = xscale[head], a1s = a1scale[head];
+  const int xrow = w * 32 + i, tok = tok0 + xrow;
+
+  {
+    RowTile<D, T, 128> t;
+    t.load(Xh, tok0, n, tid);
+    t.store_s(Xl, LX, xs, tid);
+    t.load(Yh, tok0, n, tid, ydh, yden_stride);
+    t.store(Sl, LD, 1.0f, tid);
+  }
+  __syncthreads();
+  float Yr[H2];
+#pragma unroll
+  for (int t = 0; t < H2; t += 4) {
+    const float4 y4 = *reinterpret_cast<const float4*>(Sl + xrow * LD + hh * H2 + t);
+    Yr[t] = y4.x; Yr[t + 1] = y4.y; Yr[t + 2] = y4.z; Yr[t + 3] = y4.w;
+  }
+  const float c_own = (DQ && tok < n) ? ch[tok] : 0.f;
+  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f;
+  __syncthreads();
+
+  const bool no_state = masked && (DQ ? c == 0 : c == nc - 1);
+  const int n_state = no_state ? 0 : (p2 ? NS : 0) + 1;
+  int n_tile = 0, tile0 = 0;
+  if (masked) {
+    if (DQ) {
+      tile0 = (c * chunk) >> 5;
+      const int last = tok0 + 127 < n ? tok0 + 127 : n - 1;
+      n_tile = (last >> 5) - tile0 + 1;
+    } else {
+      tile0 = tok0 >> 5;
+      const int cend = (c + 1) * chunk < n ? (c + 1) * chunk : n;
+      n_tile = ((cend - 1) >> 5) - tile0 + 1;
+    }
+  }
+  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
+  const int nsum = masked ? 1 : nslots;
+
+  StateSlab<D * LD> slab;
+  RowTile<D, T, 32> t1, t2;
+  float creg = 0.f;
+  auto slab_load = [&](int st) {
+    slab.load(sbase + ((p2 && st < NS) ? st * D * LD : rows2 * LD), SS, nsum, D * LD, tid);
+  };
+  auto slab_store = [&](int st) {
+    const float cf = (p2 && st < NS) ? 2.0f * a2 : a1;
+    slab.store(Sl + (st & 1) * SLABF, D * LD, D * LD, cf, cf, tid);
+  };
+  auto tiles_load = [&](int kk) {
+    const int r0 = (tile0 + kk) * 32;
+    t1.load(A1h, r0, n, tid);
+    t2.load(A2h, r0, n, tid, a2dh, a2den_stride);
+    if (!DQ && tid < 32) creg = (r0 + tid < n) ? ch[r0 + tid] : 0.f;
+  };
+  auto tiles_store = [&](int buf) {
+    t1.store(Sl + buf * SLABF, LD, a1s, tid);
+    t2.store(Sl + buf * SLABF + 32 * LD, LD, 1.0f, tid);
+    if (!DQ && tid < 32) Cl[buf][tid] = creg;
+  };
+
+  f16v out[AB];
+#pragma unroll
+  for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) out[ab][r] = 0.f;
+
+  if (n_tile > 0) tiles_load(0);
+  if (n_state > 0) {
+    slab_load(0);
+    slab_store(0);
+  } else if (n_tile > 0) {
+    tiles_store(0);
+  }
+  __syncthreads();
+
+  // A operands of one 32-row tile of a slab: the row's D value columns and its extra column
+  struct AOps {
+    float4 a4[H2 / 4];
+    float ax;
+  };
+  auto fetch = [&](const float* sl, int arow, AOps& o) {
+    const float* ar = sl + arow * LD;
+#pragma unroll
+    for (int k = 0; k < H2 / 4; ++k) o.a4[k] = *reinterpret_cast<const float4*>(ar + hh * H2 + 4 * k);
+    o.ax = ar[D];
+  };
+  auto chain = [&](const AOps& o) {
+    f16v t;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t[r] = 0.f;
+#pragma unroll
+    for (int k = 0; k < H2 / 4; ++k) {
+      t = FM_MFMA(o.a4[k].x, Yr[4 * k], t);
+      t = FM_MFMA(o.a4[k].y, Yr[4 * k + 1], t);
+      t = FM_MFMA(o.a4[k].z, Yr[4 * k + 2], t);
+      t = FM_MFMA(o.a4[k].w, Yr[4 * k + 3], t);
+    }
+    return FM_MFMA(o.ax, yx, t);
+  };
+  const float* xl_row = Xl + xrow * LX;
+  // out[a] += T[a] * x[(a + qo) % D]
+  auto credit = [&](const f16v& t, int ab, int qo) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int rc = (ab * 32 + trow(r, hh) + qo) & (D - 1);
+      out[ab][r] += t[r] * xl_row[rc];
+    }
+  };
+
+  for (int st = 0; st < n_state; ++st) {
+    slab_load(st + 1 < n_state ? st + 1 : st);
+    const float* sl = Sl + (st & 1) * SLABF;
+    if (p2 && st < NS) {
+      const int s = st;
+      // tile n: ab = n % AB, pass = n / AB; the second pass (rows rotated by -s) exists for 0 < s < D/2
+      const int ntile = (s > 0 && s < H2) ? 2 * AB : AB;
+      AOps ops[2];
+      f16v tprev;
+      fetch(sl, i, ops[0]);
+#pragma unroll
+      for (int nn = 0; nn < 2 * AB; ++nn) {
+        if (nn < ntile) {
+          if (nn + 1 < ntile) {
+            const int ab1 = (nn + 1) % AB, ro1 = (nn + 1) / AB ? D - s : 0;
+            fetch(sl, (ab1 * 32 + i + ro1) & (D - 1), ops[(nn + 1) & 1]);
+          }
+          const f16v tcur = chain(ops[nn & 1]);
+          if (nn > 0) credit(tprev, (nn - 1) % AB, (nn - 1) / AB ? D - s : s);
+          FM_SCHED_MFMA_DS_VALU(H2 + 1)
+          tprev = tcur;
+        }
+      }
+      credit(tprev, (ntile - 1) % AB, (ntile - 1) / AB ? D - s : s);
+    } else {
+      AOps ops[2];
+      fetch(sl, i, ops[0]);
+#pragma unroll
+      for (int ab = 0; ab < AB; ++ab) {
+        if (ab + 1 < AB) fetch(sl, (ab + 1) * 32 + i, ops[(ab + 1) & 1]);
+        const f16v t = chain(ops[ab & 1]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out[ab][r] += t[r];
+      }
+    }
+    if (st + 1 < n_state) slab_store(st + 1);
+    else if (n_tile > 0) tiles_store((st + 1) & 1);
+    __syncthreads();
+  }
+
+  if (n_tile > 0) {
+    float Xr[H2];
+#pragma unroll
+    for (int t = 0; t < H2; ++t) Xr[t] = xl_row[hh * H2 + t];
+    const int mine = (tok0 >> 5) + w;
+    const float twoa2 = 2.0f * a2;
+    for (int kk = 0; kk < n_tile; ++kk) {
+      const int buf = (n_state + kk) & 1;
+      tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
+      const int tl = tile0 + kk;
+      if (DQ ? tl <= mine : tl >= mine) {
+        const float* l1 = Sl + buf * SLABF;
+        const float* l2 = l1 + 32 * LD;
+        // rows = streamed tokens trow(r,hh), lanes = own tokens
+        f16v sc, gv;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = gv[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < H2; t += 4) {
+          const float4 p4 = *reinterpret_cast<const float4*>(l1 + i * LD + hh * H2 + t);
+          const float4 v4 = *reinterpret_cast<const float4*>(l2 + i * LD + hh * H2 + t);
+          sc = FM_MFMA(p4.x, Xr[t], sc);
+          gv = FM_MFMA(v4.x, Yr[t], gv);
+          sc = FM_MFMA(p4.y, Xr[t + 1], sc);
+          gv = FM_MFMA(v4.y, Yr[t + 1], gv);
+          sc = FM_MFMA(p4.z, Xr[t + 2], sc);
+          gv = FM_MFMA(v4.z, Yr[t + 2], gv);
+          sc = FM_MFMA(p4.w, Xr[t + 3], sc);
+          gv = FM_MFMA(v4.w, Yr[t + 3], gv);
+        }
+        float pa[16][AB];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+          for (int ab = 0; ab < AB; ++ab) pa[r][ab] = l1[trow(r, hh) * LD + ab * 32 + i];
+        const bool diag = tl == mine;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float cc = DQ ? c_own : Cl[buf][trow(r, hh)];
+          float wv = (a1 + twoa2 * sc[r]) * (gv[r] - cc);
+          if (diag && (DQ ? trow(r, hh) > i : trow(r, hh) < i)) wv = 0.f;
+          sc[r] = wv;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+          for (int ab = 0; ab < AB; ++ab) out[ab] = FM_MFMA(pa[r][ab], sc[r], out[ab]);
+      }
+      if (kk + 1 < n_tile) tiles_store(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // transposed accumulators -> LDS -> coalesced global rows, scaled by the normaliser; sum out.x_hat
+  constexpr int VPR = D / 4;
+#pragma unroll
+  for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      *reinterpret_cast<float4*>(Sl + xrow * LD + ab * 32 + 8 * j + 4 * hh) =
+          make_float4(out[ab][4 * j], out[ab][4 * j + 1], out[ab][4 * j + 2], out[ab][4 * j + 3]);
+  __syncthreads();
+  float rs = 0.f;
+  T* Oh = OUT + (int64_t)head * n * D;
+  for (int idx = tid; idx < 128 * VPR; idx += 256) {
+    const int row = idx / VPR, c4 = idx % VPR;
+    const float4 g4 = *reinterpret_cast<const float4*>(Sl + row * LD + c4 * 4);
+    const float* xr = Xl + row * LX + c4 * 4;
+    rs += g4.x * xr[0] + g4.y * xr[1] + g4.z * xr[2] + g4.w * xr[3];
+    const float v[4] = {g4.x * xs, g4.y * xs, g4.z * xs, g4.w * xs};
+    if (tok0 + row < n) store4(Oh + (int64_t)(tok0 + row) * D + c4 * 4, v);
+  }
+  rs = block_sum_256(rs, red, tid);
+  if (tid == 0) rpart[(int64_t)head * gridDim.x + blockIdx.x] = rs;
+}

@@ -125,9 +125,10 @@ enum {
   FASTMAX_K_FWD_APPLY = 2, /* forward apply + divide                                     */
   FASTMAX_K_BWD_PREP = 3,  /* c_i = go_i.o_i/den_i                                       */
   FASTMAX_K_BWD_DQ = 4,    /* dq                                                         */
-  FASTMAX_K_BWD_DKDV = 5,  /* dk and dv                                                  */
-  FASTMAX_K_NORM_FIX = 6,  /* normalisation chain rule on the max-norm rows              */
-  FASTMAX_NUM_KERNELS = 7
+  FASTMAX_K_BWD_DK = 5,    /* dk                                                         */
+  FASTMAX_K_BWD_DV = 6,    /* dv                                                         */
+  FASTMAX_K_NORM_FIX = 7,  /* normalisation chain rule on the max-norm rows              */
+  FASTMAX_NUM_KERNELS = 8
 };
 typedef struct fastmax_kernel_times {
   float ms[FASTMAX_NUM_KERNELS];
