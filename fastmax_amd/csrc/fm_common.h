@@ -98,29 +98,34 @@ struct Geo {
 };
 
 // A tile of ROWS token rows x D channels staged global -> registers -> LDS by 256 threads.
-template <int D, class T, int ROWS>
+// ROWFAST = false: consecutive threads take consecutive 16-byte pieces of a row (coalesced
+// global reads, conflict-free row-major LDS writes).  ROWFAST = true: consecutive threads
+// take consecutive rows, which makes the TRANSPOSED LDS write (store_t) conflict-free.
+template <int D, class T, int ROWS, bool ROWFAST = false>
 struct RowTile {
   static constexpr int VPR = D / 4;
   static constexpr int TOTAL = ROWS * VPR;
   static constexpr int NV = (TOTAL + 255) / 256;
   float v[NV][4];
+  __device__ __forceinline__ static int row_of(int idx) { return ROWFAST ? idx % ROWS : idx / VPR; }
+  __device__ __forceinline__ static int c4_of(int idx) { return ROWFAST ? idx / ROWS : idx % VPR; }
+
+  float rdiv[NV];  // per-row divisors fetched by load(), applied by the stores
 
   // rows tok0.. of one head (base points at the head's first row); rows >= n read as zero.
-  // rowdiv, when given, divides every row by rowdiv[tok * rowdiv_stride].
+  // rowdiv, when given, makes the stores divide every row by rowdiv[tok * rowdiv_stride]; the
+  // division is deferred to the store so that no load has to be waited for here.
   __device__ __forceinline__ void load(const T* base, int tok0, int n, int tid,
                                        const float* rowdiv = nullptr, int64_t rowdiv_stride = 0) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
-      const int row = idx / VPR, c4 = idx % VPR;
+      const int row = row_of(idx), c4 = c4_of(idx);
       const int tok = tok0 + row;
+      rdiv[u] = 1.0f;
       if (idx < TOTAL && tok < n) {
         load4(base + (int64_t)tok * D + c4 * 4, v[u]);
-        if (rowdiv) {
-          const float s = 1.0f / rowdiv[(int64_t)tok * rowdiv_stride];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[u][e] *= s;
-        }
+        if (rowdiv) rdiv[u] = rowdiv[(int64_t)tok * rowdiv_stride];
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[u][e] = 0.f;
@@ -132,10 +137,12 @@ struct RowTile {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
-      const int row = idx / VPR, c4 = idx % VPR;
-      if (idx < TOTAL)
+      const int row = row_of(idx), c4 = c4_of(idx);
+      if (idx < TOTAL) {
+        const float sc = scale / rdiv[u];
         *reinterpret_cast<float4*>(dst + row * ld + c4 * 4) =
-            make_float4(v[u][0] * scale, v[u][1] * scale, v[u][2] * scale, v[u][3] * scale);
+            make_float4(v[u][0] * sc, v[u][1] * sc, v[u][2] * sc, v[u][3] * sc);
+      }
     }
   }
   // same with scalar stores, for an odd pitch
@@ -143,10 +150,11 @@ struct RowTile {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
-      const int row = idx / VPR, c4 = idx % VPR;
+      const int row = row_of(idx), c4 = c4_of(idx);
       if (idx < TOTAL) {
+        const float sc = scale / rdiv[u];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dst[row * ld + c4 * 4 + e] = v[u][e] * scale;
+        for (int e = 0; e < 4; ++e) dst[row * ld + c4 * 4 + e] = v[u][e] * sc;
       }
     }
   }
@@ -155,10 +163,11 @@ struct RowTile {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
-      const int row = idx / VPR, c4 = idx % VPR;
+      const int row = row_of(idx), c4 = c4_of(idx);
       if (idx < TOTAL) {
+        const float sc = scale / rdiv[u];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dst[(c4 * 4 + e) * ld + row] = v[u][e] * scale;
+        for (int e = 0; e < 4; ++e) dst[(c4 * 4 + e) * ld + row] = v[u][e] * sc;
       }
     }
   }

@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   const float* ewh = ew ? ew + (int64_t)head * n : nullptr;
   const float xs = xscale[head];
 
-  RowTile<D, T, TS> kx, vy;
+  RowTile<D, T, TS, true> kx, vy;
   float ereg = 0.f;
 
   auto load = [&](int t0, int tend) {
