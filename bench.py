@@ -101,6 +101,9 @@ def main() -> int:
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
     ap.add_argument("--batch", type=int, default=0, help="override B of the workload (profiling aid; "
                     "the metric is only quoted at the workload's own B)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy, so that a counter profile of this command "
+                         "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
@@ -157,6 +160,14 @@ def main() -> int:
         fwd()
     torch.cuda.synchronize()
     ms_fwd = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     fl = algorithmic_flops(D, cfg["p"])
     token_heads = bh * N
