@@ -51,7 +51,9 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
   __shared__ float denl[128];
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
-  const int head = blockIdx.y, tok0 = blockIdx.x * 128;
+  // logical block = (128-token block fastest, then head): neighbours in a chunk share their state
+  const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
+  const int head = lid / gridDim.x, tblk = lid % gridDim.x, tok0 = tblk * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);

@@ -20,6 +20,17 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 // row of a 32x32 accumulator tile held by register r in lane half hh
 __device__ __forceinline__ int trow(int r, int hh) { return 8 * (r >> 2) + 4 * hh + (r & 3); }
 
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2) in linear block-id
+// order.  This permutation makes a run of consecutive LOGICAL ids land on one XCD, in order,
+// so that blocks that read the same data (feature splits of a head, the two halves of a chunk)
+// share an L2.  The ragged tail (total not a multiple of 8) keeps its place.
+__device__ __forceinline__ int xcd_logical_id(int linear, int total) {
+  constexpr int NX = 8;
+  const int per = total / NX;
+  if (linear >= per * NX) return linear;
+  return (linear % NX) * per + linear / NX;
+}
+
 struct bf16_t {
   uint16_t x;
 };

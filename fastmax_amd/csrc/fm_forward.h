@@ -119,7 +119,10 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   __shared__ __attribute__((aligned(16))) float El[2][TS];
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
-  const int g = blockIdx.x, head = blockIdx.y;
+  // logical block = (feature split g fastest, then head, then token split z)
+  const int lid = xcd_logical_id(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z),
+                                 gridDim.x * gridDim.y * gridDim.z);
+  const int g = lid % gridDim.x, head = (lid / gridDim.x) % gridDim.y, zsplit = lid / (gridDim.x * gridDim.y);
   const int rows2 = G::rows2(p2);
   const int rt2 = p2 ? G::NS * G::AB : 0, rt_total = rt2 + G::AB;
   const int64_t SS = G::state_floats(p2);
@@ -278,7 +281,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       snapshot(reverse ? c - 1 : c + 1);
     }
   } else {
-    const int z = blockIdx.z;
+    const int z = zsplit;
     const int te = (z + 1) * zlen < n ? (z + 1) * zlen : n;
     run(z * zlen, te);
     snapshot(z);

@@ -10,16 +10,19 @@
 #include "fm_common.h"
 
 // ---------------------------------------------------------------------------------------
-// One block = 128 own tokens of one head, one wave = 32 of them, tokens in lanes.  Per shift
-// slab of the state the kernel contracts 32 state rows at a time over the D+1 columns with the
-// token's extended value vector y_ext = [y, yx] (B operand straight from registers, one extra
-// MFMA for the extra column); the result T[r] is the entry (a, a+s) of the token's symmetric
-// matrix for channel a = ab*32 + trow(r,hh), and out[a] += T * x[(a+s)%D] is a register FMA
-// with one LDS read.  The state stores each unordered pair {a, a+s} once, so for 0 < s < D/2
-// the same slab is contracted a second time over rows rotated by -s to credit the pair's
-// other member (twice the minimal MFMA work).
+// One block = 128 own tokens of one head, one wave = 32 of them.  Per shift slab s of the state
+// the kernel contracts the token's extended value vector y_ext = [y, yx] (A operand straight
+// from registers, one extra MFMA for the extra column) with 32 state rows at a time (B operand,
+// 128-bit LDS reads along the columns).  The result tile T (tokens x channels a) holds entry
+// (a, a+s) of every token's symmetric matrix; the state stores each unordered pair once, so
+// both members are credited from the same T:
+//     out[tok][a]         += T[tok][a] * x[tok][(a+s)%D]        (one LDS read, lanes = channels)
+//     out[tok][(a+s)%D]   += T[tok][a] * x[tok][a]              (0 < s < D/2 only)
+// The second credit moves along the channel ring, which is the lane dimension here: the two
+// 32-channel blocks are merged by a lane select and rotated by s with one ds_bpermute.
 // Causal intra-chunk part: for every streamed 32-token tile the transposed score and g.v tiles
-// are formed, W is built in registers and fed back as the B operand of  out^T += A1^T W.
+// are formed (streamed x own), W is built in registers and fed back as the A operand of
+// out += W^T-as-rows . A1.
 //
 //   MODE 0 (dq): X = q, Y = grad_out/den, yx = -c_i, state S, streamed A1 = k, A2 = v over tiles
 //                at or before the own tile, W = f'(s)(g.v - c_own)
@@ -38,14 +41,15 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   using G = Geo<D>;
   constexpr bool DQ = MODE == 0;
   constexpr int LD = G::LD, AB = G::AB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
-  constexpr int LX = D + 1;  // odd pitch: the scalar rotated reads of x are bank-conflict-free
-  __shared__ float Xl[128 * LX];
+  __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
   __shared__ __attribute__((aligned(16))) float Sl[2 * SLABF];
   __shared__ float Cl[2][32];
   __shared__ float red[4];
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
-  const int head = blockIdx.y, tok0 = blockIdx.x * 128;
+  // logical block = (128-token block fastest, then head): neighbours in a chunk share their state
+  const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
+  const int head = lid / gridDim.x, tblk = lid % gridDim.x, tok0 = tblk * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
@@ -63,11 +67,12 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   {
     RowTile<D, T, 128> t;
     t.load(Xh, tok0, n, tid);
-    t.store_s(Xl, LX, xs, tid);
+    t.store(Xl, LD, xs, tid);
     t.load(Yh, tok0, n, tid, ydh, yden_stride);
     t.store(Sl, LD, 1.0f, tid);
   }
   __syncthreads();
+  // own token of this lane = row xrow: its half of y (A operand of the state contraction, B of g.v)
   float Yr[H2];
 #pragma unroll
   for (int t = 0; t < H2; t += 4) {
@@ -117,6 +122,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
     if (!DQ && tid < 32) Cl[buf][tid] = creg;
   };
 
+  // out[ab][r]: token w*32 + trow(r,hh), channel ab*32 + i
   f16v out[AB];
 #pragma unroll
   for (int ab = 0; ab < AB; ++ab)
@@ -132,74 +138,73 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   }
   __syncthreads();
 
-  // A operands of one 32-row tile of a slab: the row's D value columns and its extra column
-  struct AOps {
-    float4 a4[H2 / 4];
-    float ax;
+  // B operands of one 32-row tile of a slab: the row's D value columns and its extra column
+  struct BOps {
+    float4 b4[H2 / 4];
+    float bx;
   };
-  auto fetch = [&](const float* sl, int arow, AOps& o) {
-    const float* ar = sl + arow * LD;
+  auto fetch = [&](const float* sl, int ab, BOps& o) {
+    const float* ar = sl + (ab * 32 + i) * LD;
 #pragma unroll
-    for (int k = 0; k < H2 / 4; ++k) o.a4[k] = *reinterpret_cast<const float4*>(ar + hh * H2 + 4 * k);
-    o.ax = ar[D];
+    for (int k = 0; k < H2 / 4; ++k) o.b4[k] = *reinterpret_cast<const float4*>(ar + hh * H2 + 4 * k);
+    o.bx = ar[D];
   };
-  auto chain = [&](const AOps& o) {
+  auto chain = [&](const BOps& o) {
     f16v t;
 #pragma unroll
     for (int r = 0; r < 16; ++r) t[r] = 0.f;
 #pragma unroll
     for (int k = 0; k < H2 / 4; ++k) {
-      t = FM_MFMA(o.a4[k].x, Yr[4 * k], t);
-      t = FM_MFMA(o.a4[k].y, Yr[4 * k + 1], t);
-      t = FM_MFMA(o.a4[k].z, Yr[4 * k + 2], t);
-      t = FM_MFMA(o.a4[k].w, Yr[4 * k + 3], t);
+      t = FM_MFMA(Yr[4 * k], o.b4[k].x, t);
+      t = FM_MFMA(Yr[4 * k + 1], o.b4[k].y, t);
+      t = FM_MFMA(Yr[4 * k + 2], o.b4[k].z, t);
+      t = FM_MFMA(Yr[4 * k + 3], o.b4[k].w, t);
     }
-    return FM_MFMA(o.ax, yx, t);
+    return FM_MFMA(yx, o.bx, t);
   };
-  const float* xl_row = Xl + xrow * LX;
-  // out[a] += T[a] * x[(a + qo) % D]
-  auto credit = [&](const f16v& t, int ab, int qo) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int rc = (ab * 32 + trow(r, hh) + qo) & (D - 1);
-      out[ab][r] += t[r] * xl_row[rc];
-    }
-  };
+  // x rows of the 16 tokens this lane holds results for: row w*32 + trow(r,hh), r = 4j+e
+  const float* xtok = Xl + (w * 32 + 4 * hh) * LD;
+  auto xat = [&](int r, int col) { return xtok[((r >> 2) * 8 + (r & 3)) * LD + col]; };
 
   for (int st = 0; st < n_state; ++st) {
     slab_load(st + 1 < n_state ? st + 1 : st);
     const float* sl = Sl + (st & 1) * SLABF;
+    BOps ops[AB];
+#pragma unroll
+    for (int ab = 0; ab < AB; ++ab) fetch(sl, ab, ops[ab]);
+    f16v tt[AB];
+#pragma unroll
+    for (int ab = 0; ab < AB; ++ab) tt[ab] = chain(ops[ab]);
     if (p2 && st < NS) {
       const int s = st;
-      // tile n: ab = n % AB, pass = n / AB; the second pass (rows rotated by -s) exists for 0 < s < D/2
-      const int ntile = (s > 0 && s < H2) ? 2 * AB : AB;
-      AOps ops[2];
-      f16v tprev;
-      fetch(sl, i, ops[0]);
-#pragma unroll
-      for (int nn = 0; nn < 2 * AB; ++nn) {
-        if (nn < ntile) {
-          if (nn + 1 < ntile) {
-            const int ab1 = (nn + 1) % AB, ro1 = (nn + 1) / AB ? D - s : 0;
-            fetch(sl, (ab1 * 32 + i + ro1) & (D - 1), ops[(nn + 1) & 1]);
-          }
-          const f16v tcur = chain(ops[nn & 1]);
-          if (nn > 0) credit(tprev, (nn - 1) % AB, (nn - 1) / AB ? D - s : s);
-          FM_SCHED_MFMA_DS_VALU(H2 + 1)
-          tprev = tcur;
-        }
-      }
-      credit(tprev, (ntile - 1) % AB, (ntile - 1) / AB ? D - s : s);
-    } else {
-      AOps ops[2];
-      fetch(sl, i, ops[0]);
 #pragma unroll
       for (int ab = 0; ab < AB; ++ab) {
-        if (ab + 1 < AB) fetch(sl, (ab + 1) * 32 + i, ops[(ab + 1) & 1]);
-        const f16v t = chain(ops[ab & 1]);
+        const int rc = (ab * 32 + i + s) & (D - 1);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) out[ab][r] += t[r];
+        for (int r = 0; r < 16; ++r) out[ab][r] += tt[ab][r] * xat(r, rc);
       }
+      if (s > 0 && s < H2) {
+        // credit the other member of each pair: channel (a+s)%D gets T[a]*x[a]
+#pragma unroll
+        for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tt[ab][r] *= xat(r, ab * 32 + i);
+        const bool keep = i < 32 - s;                    // source lanes that stay in their block
+        const int src = (((i - s) & 31) + 32 * hh) << 2;  // byte index of the source lane
+#pragma unroll
+        for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            // lanes i >= s of block ab take U[ab][i-s]; lanes i < s take U[ab-1][i-s+32]
+            const float v = keep ? tt[ab][r] : tt[(ab + 1) % AB][r];
+            out[ab][r] += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, v)));
+          }
+      }
+    } else {
+#pragma unroll
+      for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out[ab][r] += tt[ab][r];
     }
     if (st + 1 < n_state) slab_store(st + 1);
     else if (n_tile > 0) tiles_store((st + 1) & 1);
@@ -209,7 +214,10 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   if (n_tile > 0) {
     float Xr[H2];
 #pragma unroll
-    for (int t = 0; t < H2; ++t) Xr[t] = xl_row[hh * H2 + t];
+    for (int t = 0; t < H2; t += 4) {
+      const float4 x4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + hh * H2 + t);
+      Xr[t] = x4.x; Xr[t + 1] = x4.y; Xr[t + 2] = x4.z; Xr[t + 3] = x4.w;
+    }
     const int mine = (tok0 >> 5) + w;
     const float twoa2 = 2.0f * a2;
     for (int kk = 0; kk < n_tile; ++kk) {
@@ -249,35 +257,30 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
           if (diag && (DQ ? trow(r, hh) > i : trow(r, hh) < i)) wv = 0.f;
           sc[r] = wv;
         }
+        // out (own x channels) += W (own x streamed) . A1 (streamed x channels)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
 #pragma unroll
-          for (int ab = 0; ab < AB; ++ab) out[ab] = FM_MFMA(pa[r][ab], sc[r], out[ab]);
+          for (int ab = 0; ab < AB; ++ab) out[ab] = FM_MFMA(sc[r], pa[r][ab], out[ab]);
       }
       if (kk + 1 < n_tile) tiles_store(buf ^ 1);
       __syncthreads();
     }
   }
 
-  // transposed accumulators -> LDS -> coalesced global rows, scaled by the normaliser; sum out.x_hat
-  constexpr int VPR = D / 4;
-#pragma unroll
-  for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      *reinterpret_cast<float4*>(Sl + xrow * LD + ab * 32 + 8 * j + 4 * hh) =
-          make_float4(out[ab][4 * j], out[ab][4 * j + 1], out[ab][4 * j + 2], out[ab][4 * j + 3]);
-  __syncthreads();
+  // rows of out are tokens, lanes are channels: store directly, scaled by the normaliser
   float rs = 0.f;
   T* Oh = OUT + (int64_t)head * n * D;
-  for (int idx = tid; idx < 128 * VPR; idx += 256) {
-    const int row = idx / VPR, c4 = idx % VPR;
-    const float4 g4 = *reinterpret_cast<const float4*>(Sl + row * LD + c4 * 4);
-    const float* xr = Xl + row * LX + c4 * 4;
-    rs += g4.x * xr[0] + g4.y * xr[1] + g4.z * xr[2] + g4.w * xr[3];
-    const float v[4] = {g4.x * xs, g4.y * xs, g4.z * xs, g4.w * xs};
-    if (tok0 + row < n) store4(Oh + (int64_t)(tok0 + row) * D + c4 * 4, v);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int tk = tok0 + w * 32 + trow(r, hh);
+#pragma unroll
+    for (int ab = 0; ab < AB; ++ab) {
+      const float g = out[ab][r];
+      rs += g * xat(r, ab * 32 + i);
+      if (tk < n) Oh[(int64_t)tk * D + ab * 32 + i] = from_f32<T>(g * xs);
+    }
   }
   rs = block_sum_256(rs, red, tid);
-  if (tid == 0) rpart[(int64_t)head * gridDim.x + blockIdx.x] = rs;
+  if (tid == 0) rpart[(int64_t)head * gridDim.x + tblk] = rs;
 }
