@@ -241,49 +241,82 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       }
     }
   };
-  auto run = [&](int tb, int te) {
-    const int nsteps = (te - tb + TS - 1) / TS;
-    if (nsteps <= 0) return;
-    load(tb, te);
-    store(0, tb, te);
-    __syncthreads();
-    for (int st = 0; st < nsteps; ++st) {
-      const bool more = st + 1 < nsteps;
-      if (more) load(tb + (st + 1) * TS, te);
-      compute(st & 1);
-      if (more) store((st + 1) & 1, tb + (st + 1) * TS, te);
-      __syncthreads();
-    }
-  };
+  // lane part of a snapshot address: row 4*hh (+ 8j + e per register), column i (+ 32*cb)
+  const unsigned lane_off = (unsigned)(4 * hh * LD + i);
   auto snapshot = [&](int slot) {
-    float* st = state + ((int64_t)head * nslots + slot) * SS;
+    float* st = state + ((int64_t)head * nslots + slot) * SS;  // uniform: scalar base + 32-bit lane offsets
 #pragma unroll
     for (int x = 0; x < RTW; ++x) {
       if (x < nx) {
+        float* sx = st + (unsigned)(rowbase[x] * LD);
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
+        for (int j = 0; j < 4; ++j) {
+          const unsigned oj = lane_off + (unsigned)(8 * j * LD);
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
-            st[(int64_t)(rowbase[x] + trow(r, hh)) * LD + cb * 32 + i] = acc[x][cb][r];
+          for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) sx[oj + (unsigned)(e * LD + cb * 32)] = acc[x][cb][4 * j + e];
+        }
         const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
-        if (hh == 0) st[(int64_t)(rowbase[x] + i) * LD + D] = ds;
+        if (hh == 0) sx[(unsigned)(i * LD + D)] = ds;
       }
     }
-    if (g == 0 && tid <= D) st[(int64_t)(rows2 + D) * LD + tid] = s0;
+    if (g == 0 && tid <= D) st[(unsigned)((rows2 + D) * LD + tid)] = s0;
   };
 
+  // The walk is one software pipeline over all 32-token steps: the loads of step p+1 are issued
+  // before the MFMAs of step p, and a snapshot is written between the two, so neither the tile
+  // loads nor the snapshot stores are ever waited for on their own.
+  //   masked, forward : chunks 0 .. nc-2 in order; after chunk c the state goes to slot c+1
+  //   masked, reverse : chunks nc-1 .. 1;          after chunk c the state goes to slot c-1
+  //   unmasked        : tokens [z*zlen, (z+1)*zlen) ; at the end the state goes to slot z
+  const int spc = chunk / TS;  // steps per full chunk
+  int nsteps, first_len = 0, tbase = 0, tend = n;
   if (masked) {
     const int nc = (n + chunk - 1) / chunk;
-    for (int cc = 0; cc + 1 < nc; ++cc) {
-      const int c = reverse ? nc - 1 - cc : cc;
-      const int te = (c + 1) * chunk < n ? (c + 1) * chunk : n;
-      run(c * chunk, te);
-      snapshot(reverse ? c - 1 : c + 1);
+    if (reverse) {
+      first_len = (n - (nc - 1) * chunk + TS - 1) / TS;  // the last chunk may be short
+      nsteps = nc > 1 ? first_len + (nc - 2) * spc : 0;
+    } else {
+      nsteps = (nc - 1) * spc;
     }
   } else {
-    const int z = zsplit;
-    const int te = (z + 1) * zlen < n ? (z + 1) * zlen : n;
-    run(z * zlen, te);
-    snapshot(z);
+    tbase = zsplit * zlen;
+    tend = tbase + zlen < n ? tbase + zlen : n;
+    nsteps = (tend - tbase + TS - 1) / TS;
   }
+  // token base of step p and the slot to write after it (-1: none)
+  auto step_tok = [&](int p) {
+    if (!masked) return tbase + p * TS;
+    if (!reverse) return p * TS;
+    const int nc = (n + chunk - 1) / chunk;
+    if (p < first_len) return (nc - 1) * chunk + p * TS;
+    const int q = p - first_len;
+    return (nc - 2 - q / spc) * chunk + (q % spc) * TS;
+  };
+  auto step_slot = [&](int p) {
+    if (!masked) return p + 1 == nsteps ? zsplit : -1;
+    if (!reverse) return (p + 1) % spc == 0 ? (p + 1) / spc : -1;
+    const int nc = (n + chunk - 1) / chunk;
+    if (p < first_len) return p + 1 == first_len ? nc - 2 : -1;
+    const int q = p - first_len;
+    return (q + 1) % spc == 0 ? nc - 3 - q / spc : -1;
+  };
+
+  if (nsteps > 0) {
+    load(step_tok(0), tend);
+    store(0, step_tok(0), tend);
+  }
+  __syncthreads();
+  for (int p = 0; p < nsteps; ++p) {
+    const bool more = p + 1 < nsteps;
+    const int tnext = step_tok(more ? p + 1 : p);
+    if (more) load(tnext, tend);
+    compute(p & 1);
+    const int slot = step_slot(p);
+    if (slot >= 0) snapshot(slot);
+    if (more) store((p + 1) & 1, tnext, tend);
+    __syncthreads();
+  }
+  if (!masked && nsteps == 0) snapshot(zsplit);  // an empty token split still owns its slot
 }
