@@ -38,6 +38,13 @@ WORKLOADS = {
 }
 COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 
+# HBM bytes per token-head moved by each kernel class at the headline workload, from the
+# FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/headline_causal_fp32_all_kernels.txt
+# (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch x2.0, write x1.0).
+MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD = {
+    "headline": {"build": 3785.0, "fwd_apply": 3502.0, "bwd_dq": 3754.0, "bwd_dk": 3939.0, "bwd_dv": 3582.0},
+}
+
 
 def algorithmic_flops(d: int, p: int) -> dict:
     """Per token-head, un-symmetrised reference form (1 MAC = 2 flop)."""
@@ -189,6 +196,11 @@ def main() -> int:
         "frac": achieved / peak, "traffic": None,
         "flops_per_launch": per_step_flops[dom] / launches, "avg_launch_ms": dom_ms / launches,
     }
+    per_th = MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD.get(args.workload if not args.batch else "", {}).get(dom)
+    if per_th is not None:
+        n_states = 3 if dom == "build" else 1
+        roofline["traffic"] = per_th * token_heads * n_states / launches  # bytes per launch (profiled, not live)
+        roofline["traffic_source"] = "profiles/headline_causal_fp32_all_kernels.txt"
     for name, f in per_step_flops.items():
         if name in kernels:
             kernels[name]["algorithmic_tflops"] = f / (kernels[name]["ms_per_step"] * 1e-3) / 1e12

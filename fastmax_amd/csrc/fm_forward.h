@@ -265,8 +265,8 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   };
 
   // The walk is one software pipeline over all 32-token steps: the loads of step p+1 are issued
-  // before the MFMAs of step p, and a snapshot is written between the two, so neither the tile
-  // loads nor the snapshot stores are ever waited for on their own.
+  // before the MFMAs of step p and consumed after them; a snapshot is stored right after that,
+  // so its stores drain under the next step's MFMAs.
   //   masked, forward : chunks 0 .. nc-2 in order; after chunk c the state goes to slot c+1
   //   masked, reverse : chunks nc-1 .. 1;          after chunk c the state goes to slot c-1
   //   unmasked        : tokens [z*zlen, (z+1)*zlen) ; at the end the state goes to slot z
@@ -313,9 +313,11 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     const int tnext = step_tok(more ? p + 1 : p);
     if (more) load(tnext, tend);
     compute(p & 1);
+    if (more) store((p + 1) & 1, tnext, tend);
+    // after the staged tile has been consumed: waiting for loads while stores are pending
+    // would wait for the stores too (one in-order counter covers both)
     const int slot = step_slot(p);
     if (slot >= 0) snapshot(slot);
-    if (more) store((p + 1) & 1, tnext, tend);
     __syncthreads();
   }
   if (!masked && nsteps == 0) snapshot(zsplit);  // an empty token split still owns its slot
