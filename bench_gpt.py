@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""End-to-end GPT training step with Fastmax causal attention in every layer (the caller side of
+the attention path: reference model.py:464-603 calls fastmax_custom on contiguous (B,H,T,hs)
+q, k, v with RoPE applied and transposes the result back).
+
+    python bench_gpt.py [--steps K] [--warmup W] [--p 2] [--layers 12] [--batch 8] [--seq 2048]
+
+A step = forward + loss + backward + AdamW update, bf16 autocast, random-init weights (std 0.02,
+as reference model.py:267-274), token ids uniform over the vocabulary from a seed.  Prints one JSON
+line with tokens/s and the share of the step spent in attention forward + backward (HIP events
+around the attention module and around its backward, summed over layers).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+import torch.nn as nn  # noqa: E402
+import torch.nn.functional as F  # noqa: E402
+
+
+def rope_cache(seq: int, hs: int, device, base: float = 10000.0):
+    theta = 1.0 / (base ** (torch.arange(0, hs, 2, device=device).float() / hs))
+    idx = torch.outer(torch.arange(seq, device=device).float(), theta).repeat(1, 2)
+    return torch.cos(idx), torch.sin(idx)
+
+
+def apply_rope(x, cos, sin):
+    hs = x.size(-1)
+    x1, x2 = x[..., : hs // 2], x[..., hs // 2:]
+    rotated = torch.cat((-x2, x1), dim=-1)
+    return (x * cos + rotated * sin).to(x.dtype)
+
+
+class Block(nn.Module):
+    def __init__(self, d_model, n_head, d_mlp, attn, p):
+        super().__init__()
+        self.n_head, self.hs, self.p = n_head, d_model // n_head, p
+        self.ln1 = nn.LayerNorm(d_model)
+        self.qkv = nn.Linear(d_model, 3 * d_model)
+        self.proj = nn.Linear(d_model, d_model)
+        self.ln2 = nn.LayerNorm(d_model)
+        self.fc = nn.Linear(d_model, d_mlp)
+        self.out = nn.Linear(d_mlp, d_model)
+        self.attn = attn
+
+    def forward(self, x, cos, sin):
+        B, T, C = x.shape
+        q, k, v = self.qkv(self.ln1(x)).view(B, T, 3, self.n_head, self.hs).permute(2, 0, 3, 1, 4)
+        q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+        # same call as reference model.py:575: mask, no dropout, normalize, lim 1, a = (1, 1, 0.5)
+        y = self.attn(q.contiguous(), k.contiguous(), v.contiguous(), None, True, 0.0, True, 1.0, 1.0, 1.0, 0.5,
+                      1.0, self.p)
+        x = x + self.proj(y.transpose(1, 2).reshape(B, T, C))
+        return x + self.out(F.gelu(self.fc(self.ln2(x))))
+
+
+class MiniGPT(nn.Module):
+    def __init__(self, vocab, d_model, n_layer, n_head, d_mlp, seq, attn, p):
+        super().__init__()
+        self.wte = nn.Embedding(vocab, d_model)
+        self.blocks = nn.ModuleList(Block(d_model, n_head, d_mlp, attn, p) for _ in range(n_layer))
+        self.ln_f = nn.LayerNorm(d_model)
+        self.lm_head = nn.Linear(d_model, vocab, bias=False)
+        self.seq, self.hs = seq, d_model // n_head
+        self.apply(self._init)
+
+    @staticmethod
+    def _init(m):
+        if isinstance(m, (nn.Linear, nn.Embedding)):
+            nn.init.normal_(m.weight, mean=0.0, std=0.02)
+            if isinstance(m, nn.Linear) and m.bias is not None:
+                nn.init.zeros_(m.bias)
+
+    def forward(self, idx):
+        cos, sin = rope_cache(idx.size(1), self.hs, idx.device)
+        x = self.wte(idx)
+        for b in self.blocks:
+            x = b(x, cos, sin)
+        return self.lm_head(self.ln_f(x))
+
+
+class TimedAttention(nn.Module):
+    """Wraps the attention module with HIP events around its forward and its backward."""
+
+    def __init__(self, inner):
+        super().__init__()
+        self.inner = inner
+        self.events = []
+        self.register_full_backward_pre_hook(self._bwd_start)
+        self.register_full_backward_hook(self._bwd_end)
+
+    def _mark(self):
+        e = torch.cuda.Event(enable_timing=True)
+        e.record()
+        return e
+
+    def _bwd_start(self, module, grad_output):
+        self._b0 = self._mark()
+
+    def _bwd_end(self, module, grad_input, grad_output):
+        self.events.append((self._b0, self._mark()))
+
+    def forward(self, *args):
+        e0 = self._mark()
+        y = self.inner(*args)
+        self.events.append((e0, self._mark()))
+        return y
+
+    def total_ms(self):
+        torch.cuda.synchronize()
+        t = sum(a.elapsed_time(b) for a, b in self.events)
+        self.events.clear()
+        return t
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--p", type=int, default=2, help="polynomial order (the reference model hard-codes 1)")
+    ap.add_argument("--layers", type=int, default=12)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--seq", type=int, default=2048)
+    ap.add_argument("--pytorch-attention", action="store_true", help="use_custom_gradient=False path")
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        print("bench_gpt.py: no GPU visible", file=sys.stderr)
+        return 3
+    from fastmax_amd import FASTMultiHeadAttention
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    attn = TimedAttention(FASTMultiHeadAttention(use_custom_gradient=not args.pytorch_attention))
+    model = MiniGPT(50304, 768, args.layers, 12, 3072, args.seq, attn, args.p).to(dev)
+    opt = torch.optim.AdamW(model.parameters(), lr=3e-4, weight_decay=0.1)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    idx = torch.randint(0, 50304, (args.batch, args.seq + 1), device=dev, generator=gen)
+    x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
+
+    def step():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits = model(x)
+        loss = F.cross_entropy(logits.float().view(-1, logits.size(-1)), y.view(-1))
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        opt.step()
+        return loss.detach()
+
+    losses = []
+    for _ in range(args.warmup):
+        losses.append(float(step()))
+    attn.total_ms()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        losses.append(float(step()))
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    attn_ms = attn.total_ms() / args.steps
+    print(json.dumps({
+        "metric": "GPT training step with Fastmax causal attention in every layer",
+        "value": args.batch * args.seq / (ms * 1e-3), "unit": "tokens/s", "ms_per_step": ms,
+        "attention_fwd_bwd_ms_per_step": attn_ms, "attention_share_of_step": attn_ms / ms,
+        "dtype": "bf16 autocast (attention: bf16 in/out, fp32 arithmetic)", "data": "synthetic",
+        "config": {"workload": f"{args.layers} layers, d_model 768, 12 heads x 64, MLP 3072 GELU, RoPE, vocab 50304, "
+                               f"seq {args.seq}, batch {args.batch}, p={args.p}, AdamW",
+                   "attention": "pytorch function" if args.pytorch_attention else "hip kernels"},
+        "loss_first_last": [losses[0], losses[-1]], "steps": args.steps, "warmup": args.warmup,
+    }))
+    return 0 if all(math.isfinite(v) for v in losses) else 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

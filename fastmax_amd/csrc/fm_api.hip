@@ -86,9 +86,18 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   pl.n = ds->nq;
   pl.bh = ds->bh;
   const int rt_total = (pl.p2 ? (pl.d / 2 + 1) * (pl.d / 32) : 0) + pl.d / 32;
-  if (!pl.p2) pl.rtw = 1;
-  else pl.rtw = pl.d == 64 ? 3 : 5;
-  pl.gsplit = (rt_total + 4 * pl.rtw - 1) / (4 * pl.rtw);
+  auto splits = [&](int rtw) { return (rt_total + 4 * rtw - 1) / (4 * rtw); };
+  if (!pl.p2) {
+    pl.rtw = 1;
+  } else if (pl.d == 64) {
+    // 3 or 4 row tiles per wave (6 or 5 blocks per head): a block's run time grows with its tile
+    // count and 512 blocks are resident at once, so pick the one with fewer tile-rounds
+    auto cost = [&](int rtw) { return (int64_t)((splits(rtw) * pl.bh + 511) / 512) * rtw; };
+    pl.rtw = cost(4) < cost(3) ? 4 : 3;
+  } else {
+    pl.rtw = 5;
+  }
+  pl.gsplit = splits(pl.rtw);
   pl.nblk = (pl.n + 127) / 128;
   if (pl.masked) {
     pl.nslots = (pl.n + kChunk - 1) / kChunk;
@@ -201,7 +210,11 @@ int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float*
   if (pl.rtw == 1) {
     FM_BUILD(1);
   } else if constexpr (D == 64) {
-    FM_BUILD(3);
+    if (pl.rtw == 4) {
+      FM_BUILD(4);
+    } else {
+      FM_BUILD(3);
+    }
   } else {
     FM_BUILD(5);
   }
