@@ -196,6 +196,12 @@ int compute_scales(const fastmax_desc* ds, const T* q, const T* k, float* scale,
   return launch_status("scale kernels");
 }
 
+// bf16 inputs run the contractions on the bf16 matrix instruction (fp32 accumulate)
+template <class T>
+constexpr bool kBf16Mfma = false;
+template <>
+constexpr bool kBf16Mfma<bf16_t> = true;
+
 template <int D, class T>
 int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float* xscale,
                  const float* yden, int64_t yden_stride, const float* ew, float* state, int reverse,
@@ -204,7 +210,7 @@ int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float*
   if (pl.masked && pl.nslots < 2) return FASTMAX_OK;  // a single chunk never needs a state
   ScopedKernel sk(FASTMAX_K_BUILD, stream);
 #define FM_BUILD(RTW)                                                                            \
-  build_kernel<D, T, RTW><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, yden_stride, ew, state, \
+  build_kernel<D, T, RTW, kBf16Mfma<T>><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, yden_stride, ew, state, \
                                                     pl.n, kChunk, pl.nslots, pl.masked, reverse, \
                                                     pl.p2, pl.zlen)
   if (pl.rtw == 1) {

@@ -17,6 +17,27 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 
 #define FM_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
 
+// bf16 matrix instruction used when the inputs are bf16: v_mfma_f32_32x32x8_bf16, fp32 accumulate.
+//   A (32 x 8): row l%32, k = 4*(l/32) + {0,1,2,3}  -> four bf16 per lane (s4v)
+//   B (8 x 32): col l%32, k = 4*(l/32) + {0,1,2,3}
+//   D (32 x 32): as for the fp32 instruction
+// One of these replaces four fp32 MFMAs whose k indices were 2*u + l/32, u = 0..3.
+typedef short s4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
+#define FM_MFMA_BF(a, b, c) __builtin_amdgcn_mfma_f32_32x32x8bf16_1k((a), (b), (c), 0, 0, 0)
+
+__device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
+  const bf2v p = {(__bf16)lo, (__bf16)hi};  // round to nearest even (v_cvt_pk_bf16_f32)
+  return __builtin_bit_cast(uint32_t, p);
+}
+__device__ __forceinline__ s4v pack_bf4(float a, float b, float c, float d) {
+  const uint2 u = make_uint2(pack_bf2(a, b), pack_bf2(c, d));
+  return __builtin_bit_cast(s4v, u);
+}
+__device__ __forceinline__ s4v as_s4v(uint2 u) { return __builtin_bit_cast(s4v, u); }
+__device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+
 // row of a 32x32 accumulator tile held by register r in lane half hh
 __device__ __forceinline__ int trow(int r, int hh) { return 8 * (r >> 2) + 4 * hh + (r & 3); }
 
@@ -166,6 +187,35 @@ struct RowTile {
         const float sc = scale / rdiv[u];
 #pragma unroll
         for (int e = 0; e < 4; ++e) dst[row * ld + c4 * 4 + e] = v[u][e] * sc;
+      }
+    }
+  }
+  // transposed and rounded to bf16: dst is [D][ld] 16-bit elements in LDS
+  __device__ __forceinline__ void store_t_bf(uint16_t* dst, int ld, float scale, int tid) const {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      const int row = row_of(idx), c4 = c4_of(idx);
+      if (idx < TOTAL) {
+        const float sc = scale / rdiv[u];
+        const uint32_t p01 = pack_bf2(v[u][0] * sc, v[u][1] * sc), p23 = pack_bf2(v[u][2] * sc, v[u][3] * sc);
+        dst[(c4 * 4 + 0) * ld + row] = (uint16_t)p01;
+        dst[(c4 * 4 + 1) * ld + row] = (uint16_t)(p01 >> 16);
+        dst[(c4 * 4 + 2) * ld + row] = (uint16_t)p23;
+        dst[(c4 * 4 + 3) * ld + row] = (uint16_t)(p23 >> 16);
+      }
+    }
+  }
+  // row-major, rounded to bf16: dst is [ROWS][ld] 16-bit elements in LDS, 8-byte aligned rows
+  __device__ __forceinline__ void store_bf(uint16_t* dst, int ld, float scale, int tid) const {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      const int row = row_of(idx), c4 = c4_of(idx);
+      if (idx < TOTAL) {
+        const float sc = scale / rdiv[u];
+        *reinterpret_cast<uint2*>(dst + row * ld + c4 * 4) =
+            make_uint2(pack_bf2(v[u][0] * sc, v[u][1] * sc), pack_bf2(v[u][2] * sc, v[u][3] * sc));
       }
     }
   }

@@ -100,7 +100,7 @@ __global__ void scale_rows_kernel(T* x, const float* __restrict__ scale, int64_t
 // masked == 0: gridDim.z blocks each sum zlen tokens and write slot blockIdx.z; consumers
 //   add the slots.
 // ---------------------------------------------------------------------------------------
-template <int D, class T, int RTW>
+template <int D, class T, int RTW, bool BF>
 __global__ __launch_bounds__(256, 2) void build_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const float* __restrict__ xscale,
     const float* __restrict__ yden, int64_t yden_stride, const float* __restrict__ ew,
@@ -115,7 +115,12 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   // into four consecutive MFMAs come from one 128-bit LDS read.  Row D of the X tile is 1 for
   // real tokens and 0 for padding: order-1 features are x[a] * 1.
   __shared__ __attribute__((aligned(16))) float Kt[2][(D + 1) * TP];
-  __shared__ __attribute__((aligned(16))) float Vt[2][D * TP];
+  // BF: the value tile is kept as bf16 (pitch TPB 16-bit elements: 8-byte aligned rows, the 16
+  // lanes of a 64-bit access phase in distinct banks) and every four fp32 MFMAs become one
+  // bf16 MFMA on features rounded after the fp32 product
+  constexpr int TPB = TS + 4;
+  __shared__ __attribute__((aligned(16))) float Vt[BF ? 1 : 2][BF ? 4 : D * TP];
+  __shared__ __attribute__((aligned(16))) uint16_t Vtb[BF ? 2 : 1][BF ? D * TPB : 4];
   __shared__ __attribute__((aligned(16))) float El[2][TS];
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   }
   int voff[CB];
 #pragma unroll
-  for (int cb = 0; cb < CB; ++cb) voff[cb] = (cb * 32 + i) * TP + 4 * hh;
+  for (int cb = 0; cb < CB; ++cb) voff[cb] = (cb * 32 + i) * (BF ? TPB : TP) + 4 * hh;
 
   f16v acc[RTW][CB];
   float dacc[RTW];
@@ -185,7 +190,8 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   };
   auto store = [&](int buf, int t0, int tend) {
     kx.store_t(Kt[buf], TP, xs, tid);
-    vy.store_t(Vt[buf], TP, 1.0f, tid);
+    if constexpr (BF) vy.store_t_bf(Vtb[buf], TPB, 1.0f, tid);
+    else vy.store_t(Vt[buf], TP, 1.0f, tid);
     if (tid < TS) {
       El[buf][tid] = ereg;
       Kt[buf][D * TP + tid] = (t0 + tid < tend) ? 1.0f : 0.f;
@@ -194,12 +200,16 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   // operands of one group of 8 tokens (lane half hh takes tokens 8*grp + 4*hh + u, u = 0..3,
   // as the k index of MFMA u)
   struct GroupOps {
-    float4 own[RTW], rot[RTW], vv[CB], e4;
+    float4 own[RTW], rot[RTW], vv[BF ? 1 : CB], e4;
+    uint2 vb[BF ? CB : 1];
   };
-  auto fetch = [&](const float* kb, const float* vb, const float* eb, int grp, GroupOps& g4) {
+  auto fetch = [&](const float* kb, int buf, const float* eb, int grp, GroupOps& g4) {
     const int go8 = 8 * grp;
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb) g4.vv[cb] = *reinterpret_cast<const float4*>(vb + voff[cb] + go8);
+    for (int cb = 0; cb < CB; ++cb) {
+      if constexpr (BF) g4.vb[cb] = *reinterpret_cast<const uint2*>(Vtb[buf] + voff[cb] + go8);
+      else g4.vv[cb] = *reinterpret_cast<const float4*>(Vt[buf] + voff[cb] + go8);
+    }
     g4.e4 = *reinterpret_cast<const float4*>(eb + go8 + 4 * hh);
 #pragma unroll
     for (int x = 0; x < RTW; ++x) {
@@ -209,35 +219,49 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   };
   auto compute = [&](int buf) {
     const float* kb = Kt[buf];
-    const float* vb = Vt[buf];
     const float* eb = El[buf];
     GroupOps cur, nxt;
-    fetch(kb, vb, eb, 0, cur);
+    fetch(kb, buf, eb, 0, cur);
 #pragma unroll
     for (int grp = 0; grp < TS / 8; ++grp) {
-      if (grp + 1 < TS / 8) fetch(kb, vb, eb, grp + 1, nxt);
+      if (grp + 1 < TS / 8) fetch(kb, buf, eb, grp + 1, nxt);
       // tiles past the end of the feature list (x >= nx) run on dummy operands and are never stored
 #pragma unroll
       for (int x = 0; x < RTW; ++x) {
         const float a0 = cur.own[x].x * cur.rot[x].x, a1 = cur.own[x].y * cur.rot[x].y;
         const float a2 = cur.own[x].z * cur.rot[x].z, a3 = cur.own[x].w * cur.rot[x].w;
+        if constexpr (BF) {
+          const s4v ap = pack_bf4(a0, a1, a2, a3);
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-          acc[x][cb] = FM_MFMA(a0, cur.vv[cb].x, acc[x][cb]);
-          acc[x][cb] = FM_MFMA(a1, cur.vv[cb].y, acc[x][cb]);
-          acc[x][cb] = FM_MFMA(a2, cur.vv[cb].z, acc[x][cb]);
-          acc[x][cb] = FM_MFMA(a3, cur.vv[cb].w, acc[x][cb]);
+          for (int cb = 0; cb < CB; ++cb) acc[x][cb] = FM_MFMA_BF(ap, as_s4v(cur.vb[cb]), acc[x][cb]);
+        } else {
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) {
+            acc[x][cb] = FM_MFMA(a0, cur.vv[cb].x, acc[x][cb]);
+            acc[x][cb] = FM_MFMA(a1, cur.vv[cb].y, acc[x][cb]);
+            acc[x][cb] = FM_MFMA(a2, cur.vv[cb].z, acc[x][cb]);
+            acc[x][cb] = FM_MFMA(a3, cur.vv[cb].w, acc[x][cb]);
+          }
         }
         dacc[x] += a0 * cur.e4.x + a1 * cur.e4.y + a2 * cur.e4.z + a3 * cur.e4.w;
       }
       if (grp + 1 < TS / 8) cur = nxt;
     }
     if (g == 0 && tid <= D) {
-      const float* src = tid < D ? vb + tid * TP : eb;
+      if (BF && tid < D) {
+        const uint16_t* src = Vtb[buf] + tid * TPB;
 #pragma unroll
-      for (int j = 0; j < TS; j += 4) {
-        const float4 t4 = *reinterpret_cast<const float4*>(src + j);
-        s0 += (t4.x + t4.y) + (t4.z + t4.w);
+        for (int j = 0; j < TS; j += 2) {
+          const uint32_t u = *reinterpret_cast<const uint32_t*>(src + j);
+          s0 += bf_lo(u) + bf_hi(u);
+        }
+      } else {
+        const float* src = tid < D ? Vt[buf] + tid * TP : eb;
+#pragma unroll
+        for (int j = 0; j < TS; j += 4) {
+          const float4 t4 = *reinterpret_cast<const float4*>(src + j);
+          s0 += (t4.x + t4.y) + (t4.z + t4.w);
+        }
       }
     }
   };
