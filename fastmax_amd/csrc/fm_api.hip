@@ -248,10 +248,18 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
     FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, state, 0, stream)));
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
-      apply_kernel<D, T, 0><<<dim3(pl.nblk, heads), 256, 0, stream>>>(
-          q + off, k + off, v + off, scale + h0, scale + bh + h0, nullptr, 0, state, pl.nslots,
-          o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, kChunk,
-          pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
+      const dim3 agrid(pl.nblk, heads);
+      if constexpr (kBf16Mfma<T>) {
+        apply_kernel_bf<D, 0><<<agrid, 256, 0, stream>>>(
+            q + off, k + off, v + off, scale + h0, scale + bh + h0, nullptr, 0, state, pl.nslots,
+            o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, kChunk,
+            pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
+      } else {
+        apply_kernel<D, T, 0><<<agrid, 256, 0, stream>>>(
+            q + off, k + off, v + off, scale + h0, scale + bh + h0, nullptr, 0, state, pl.nslots,
+            o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, kChunk,
+            pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
+      }
     }
     FM_TRY(launch_status("fwd_apply_kernel"));
   }
@@ -318,9 +326,15 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     FM_TRY(launch_status("grad_kernel (dk)"));
     {
       ScopedKernel sk(FASTMAX_K_BWD_DV, stream);
-      apply_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
-          k + off, q + off, go + off, scale + bh + h0, scale + h0, denh, den_stride, stR, pl.nslots,
-          dv + off, D, nullptr, 0, n, kChunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
+      if constexpr (kBf16Mfma<T>) {
+        apply_kernel_bf<D, 1><<<grid, 256, 0, stream>>>(
+            k + off, q + off, go + off, scale + bh + h0, scale + h0, denh, den_stride, stR, pl.nslots,
+            dv + off, D, nullptr, 0, n, kChunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
+      } else {
+        apply_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
+            k + off, q + off, go + off, scale + bh + h0, scale + h0, denh, den_stride, stR, pl.nslots,
+            dv + off, D, nullptr, 0, n, kChunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
+      }
     }
     FM_TRY(launch_status("apply_kernel (dv)"));
   }

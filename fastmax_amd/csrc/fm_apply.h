@@ -274,3 +274,246 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
     }
   }
 }
+
+// ---------------------------------------------------------------------------------------
+// bf16 variant of apply_kernel (bf16 inputs and outputs): same decomposition, but every
+// contraction runs on v_mfma_f32_32x32x8_bf16 with fp32 accumulation.  Features are formed in
+// fp32 from the fp32-scaled inputs and rounded when packed; the state slab is transposed and
+// rounded to bf16 while it is staged ([column][feature], so that the four features of a lane's
+// k-slots are one 64-bit LDS read); the order-0 row stays fp32.  The forward denominator comes
+// from a third accumulator tile whose B operand is the state's extra column broadcast to every
+// lane, which leaves den[row] in every lane that holds that row of the output.
+// Lane half hh owns features/channels 32*hh + t as in the fp32 kernel; MFMA g of a sweep takes
+// t = 4g..4g+3 from both halves.
+// ---------------------------------------------------------------------------------------
+template <int D, int MODE>
+__global__ __launch_bounds__(256, 2) void apply_kernel_bf(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ A1, const bf16_t* __restrict__ A2,
+    const float* __restrict__ xscale, const float* __restrict__ a1scale,
+    const float* __restrict__ a2den, int64_t a2den_stride, const float* __restrict__ state,
+    int nslots, bf16_t* __restrict__ OUT, int64_t ldo, float* __restrict__ den, int64_t den_stride,
+    int n, int chunk, int masked, int p2, float a0, float a1, float a2) {
+  using G = Geo<D>;
+  using T = bf16_t;
+  constexpr bool FWD = MODE == 0;
+  constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS;
+  constexpr int LB = D + 4;            // pitch of bf16 rows (16-bit elements): 8-byte aligned, and the
+                                       // 16 lanes of a 64-bit access phase fall in distinct banks
+  constexpr int TPB = 36;              // pitch of the transposed 32-token value tile
+  constexpr int SLB0 = (D + 2) * LB, SLB1 = 32 * LB + D * TPB;  // D+1 state columns, or both tiles
+  constexpr int SLB = (SLB0 > SLB1 ? SLB0 : SLB1 + 7) / 8 * 8;
+  __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb[2][SLB];
+  __shared__ float S0l[2][D + 4];      // order-0 row (fp32), one per stage buffer
+
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
+  const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
+  const int head = lid / gridDim.x, tblk = lid % gridDim.x, tok0 = tblk * 128;
+  const int c = tok0 / chunk;
+  const int nc = (n + chunk - 1) / chunk;
+  const int rows2 = G::rows2(p2);
+  const int64_t SS = G::state_floats(p2);
+  const T* Xh = X + (int64_t)head * n * D;
+  const T* A1h = A1 + (int64_t)head * n * D;
+  const T* A2h = A2 + (int64_t)head * n * D;
+  const float* a2dh = a2den ? a2den + (int64_t)head * n * a2den_stride : nullptr;
+  const float xs = xscale[head], a1s = a1scale[head];
+
+  {
+    RowTile<D, T, 128> xt;
+    xt.load(Xh, tok0, n, tid);
+    xt.store(Xl, LD, xs, tid);
+  }
+
+  const bool no_state = masked && (FWD ? c == 0 : c == nc - 1);
+  const int n_state = no_state ? 0 : (p2 ? NS : 0) + 1;
+  int n_tile = 0, tile0 = 0;
+  if (masked) {
+    if (FWD) {
+      tile0 = (c * chunk) >> 5;
+      const int last = tok0 + 127 < n ? tok0 + 127 : n - 1;
+      n_tile = (last >> 5) - tile0 + 1;
+    } else {
+      tile0 = tok0 >> 5;
+      const int cend = (c + 1) * chunk < n ? (c + 1) * chunk : n;
+      n_tile = ((cend - 1) >> 5) - tile0 + 1;
+    }
+  }
+  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
+  const int nsum = masked ? 1 : nslots;
+
+  StateSlab<(D + 1) * LD> slab;
+  RowTile<D, T, 32> t1, t2;
+  auto slab_load = [&](int st) {
+    const bool ord2 = p2 && st < NS;
+    slab.load(sbase + (ord2 ? st * D * LD : rows2 * LD), SS, nsum, ord2 ? D * LD : (D + 1) * LD, tid);
+  };
+  // fp32 [feature][LD] rows in registers -> bf16 [column][LB] in LDS, coefficient applied on the way
+  auto slab_store = [&](int st) {
+    const bool ord2 = p2 && st < NS;
+    const float cf = ord2 ? ((st == 0 || st == H2) ? a2 : 2.0f * a2) : a1;
+    uint16_t* dst = Sb[st & 1];
+    constexpr int VPR = LD / 4;  // float4 pieces per state row
+    const int nvec = ((ord2 ? D * LD : (D + 1) * LD) + 3) >> 2;
+#pragma unroll
+    for (int u = 0; u < decltype(slab)::NV; ++u) {
+      const int idx = tid + u * 256;
+      if (idx < nvec) {
+        const int f = idx / VPR, c0 = (idx % VPR) * 4;
+        const float4 v4 = slab.v[u];
+        const float e4[4] = {v4.x, v4.y, v4.z, v4.w};
+        if (f < D) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (c0 + e <= D) dst[(c0 + e) * LB + f] = (uint16_t)pack_bf2(e4[e] * cf, 0.f);
+        } else {  // the order-0 row that follows the order-1 rows
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (c0 + e <= D) S0l[st & 1][c0 + e] = e4[e] * a0;
+        }
+      }
+    }
+  };
+  auto tiles_load = [&](int kk) {
+    t1.load(A1h, (tile0 + kk) * 32, n, tid);
+    t2.load(A2h, (tile0 + kk) * 32, n, tid, a2dh, a2den_stride);
+  };
+  auto tiles_store = [&](int buf) {
+    t1.store_bf(Sb[buf], LB, a1s, tid);
+    t2.store_t_bf(Sb[buf] + 32 * LB, TPB, 1.0f, tid);
+  };
+
+  if (n_tile > 0) tiles_load(0);
+  if (n_state > 0) {
+    slab_load(0);
+    slab_store(0);
+  } else if (n_tile > 0) {
+    tiles_store(0);
+  }
+  __syncthreads();
+
+  const int xrow = w * 32 + i;
+  float Xr[H2];
+#pragma unroll
+  for (int t = 0; t < H2; t += 4) {
+    const float4 q4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + hh * H2 + t);
+    Xr[t] = q4.x; Xr[t + 1] = q4.y; Xr[t + 2] = q4.z; Xr[t + 3] = q4.w;
+  }
+
+  f16v acc[CB], accd;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    accd[r] = 0.f;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) acc[cb][r] = 0.f;
+  }
+
+  float Wn[H2 + 4];
+  auto window_load = [&](int s0) {
+#pragma unroll
+    for (int j = 0; j < H2 / 4 + 1; ++j) {
+      const int c0 = (hh * H2 + s0 + 4 * j) & (D - 1);
+      const float4 q4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + c0);
+      Wn[4 * j] = q4.x; Wn[4 * j + 1] = q4.y; Wn[4 * j + 2] = q4.z; Wn[4 * j + 3] = q4.w;
+    }
+  };
+
+  auto slab_compute = [&](const uint16_t* sl, auto tag) {
+    constexpr bool ORD2 = decltype(tag)::value;
+    const uint16_t* brow = sl + hh * H2;
+#pragma unroll
+    for (int g4 = 0; g4 < H2 / 4; ++g4) {
+      const int t = 4 * g4;
+      const s4v ap = ORD2 ? pack_bf4(Xr[t] * Wn[t], Xr[t + 1] * Wn[t + 1], Xr[t + 2] * Wn[t + 2], Xr[t + 3] * Wn[t + 3])
+                          : pack_bf4(Xr[t], Xr[t + 1], Xr[t + 2], Xr[t + 3]);
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+        acc[cb] = FM_MFMA_BF(ap, as_s4v(*reinterpret_cast<const uint2*>(brow + (cb * 32 + i) * LB + t)), acc[cb]);
+      if (FWD) accd = FM_MFMA_BF(ap, as_s4v(*reinterpret_cast<const uint2*>(brow + D * LB + t)), accd);
+    }
+  };
+
+  for (int st = 0; st < n_state; ++st) {
+    slab_load(st + 1 < n_state ? st + 1 : st);
+    const uint16_t* sl = Sb[st & 1];
+    if (p2 && st < NS) {
+      if ((st & 3) == 0) {
+        window_load(st);
+      } else {
+#pragma unroll
+        for (int x = 0; x < H2 + 3; ++x) Wn[x] = Wn[x + 1];
+      }
+      slab_compute(sl, std::true_type{});
+    } else {
+      slab_compute(sl, std::false_type{});
+      const float* s0 = S0l[st & 1];
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const float z = s0[cb * 32 + i];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[cb][r] += z;
+      }
+      if (FWD) {
+        const float z = s0[D];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) accd[r] += z;
+      }
+    }
+    if (st + 1 < n_state) slab_store(st + 1);
+    else if (n_tile > 0) tiles_store((st + 1) & 1);
+    __syncthreads();
+  }
+
+  if (n_tile > 0) {
+    s4v Xp[H2 / 4];
+#pragma unroll
+    for (int g4 = 0; g4 < H2 / 4; ++g4) Xp[g4] = pack_bf4(Xr[4 * g4], Xr[4 * g4 + 1], Xr[4 * g4 + 2], Xr[4 * g4 + 3]);
+    const s4v ones = as_s4v(make_uint2(0x3f803f80u, 0x3f803f80u));
+    const int mine = (tok0 >> 5) + w;
+    for (int kk = 0; kk < n_tile; ++kk) {
+      const int buf = (n_state + kk) & 1;
+      tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
+      const int tl = tile0 + kk;
+      if (FWD ? tl <= mine : tl >= mine) {
+        const uint16_t* l1 = Sb[buf];
+        const uint16_t* l2 = Sb[buf] + 32 * LB;
+        f16v sc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+        for (int g4 = 0; g4 < H2 / 4; ++g4)
+          sc = FM_MFMA_BF(as_s4v(*reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 4 * g4)), Xp[g4], sc);
+        const bool diag = tl == mine;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float s = sc[r];
+          float f = a0 + s * (a1 + a2 * s);
+          if (diag && (FWD ? trow(r, hh) > i : trow(r, hh) < i)) f = 0.f;
+          sc[r] = f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const s4v pp = pack_bf4(sc[4 * j], sc[4 * j + 1], sc[4 * j + 2], sc[4 * j + 3]);
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb)
+            acc[cb] = FM_MFMA_BF(pp, as_s4v(*reinterpret_cast<const uint2*>(l2 + (cb * 32 + i) * TPB + 8 * j + 4 * hh)), acc[cb]);
+          if (FWD) accd = FM_MFMA_BF(pp, ones, accd);
+        }
+      }
+      if (kk + 1 < n_tile) tiles_store(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  T* Oh = OUT + (int64_t)head * n * ldo;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int tk = tok0 + w * 32 + trow(r, hh);
+    if (tk < n) {
+      const float inv = FWD ? 1.0f / accd[r] : 1.0f;
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) Oh[(int64_t)tk * ldo + cb * 32 + i] = from_f32<T>(acc[cb][r] * inv);
+      if (FWD && i == 0) den[((int64_t)head * n + tk) * den_stride] = accd[r];
+    }
+  }
+}
