@@ -310,18 +310,32 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     const dim3 grid(pl.nblk, heads);
     {
       ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
-      grad_kernel<D, T, 0><<<grid, 256, 0, stream>>>(
-          q + off, go + off, denh, den_stride, ch, k + off, v + off, nullptr, 0, scale + h0,
-          scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, kChunk, pl.masked,
-          pl.p2, ds->a1, a2);
+      if constexpr (kBf16Mfma<T>) {
+        grad_kernel_bf<D, 0><<<grid, 256, 0, stream>>>(
+            q + off, go + off, denh, den_stride, ch, k + off, v + off, nullptr, 0, scale + h0,
+            scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, kChunk, pl.masked,
+            pl.p2, ds->a1, a2);
+      } else {
+        grad_kernel<D, T, 0><<<grid, 256, 0, stream>>>(
+            q + off, go + off, denh, den_stride, ch, k + off, v + off, nullptr, 0, scale + h0,
+            scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, kChunk, pl.masked,
+            pl.p2, ds->a1, a2);
+      }
     }
     FM_TRY(launch_status("grad_kernel (dq)"));
     {
       ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
-      grad_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
-          k + off, v + off, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + h0,
-          scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, kChunk,
-          pl.masked, pl.p2, ds->a1, a2);
+      if constexpr (kBf16Mfma<T>) {
+        grad_kernel_bf<D, 1><<<grid, 256, 0, stream>>>(
+            k + off, v + off, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + h0,
+            scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, kChunk,
+            pl.masked, pl.p2, ds->a1, a2);
+      } else {
+        grad_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
+            k + off, v + off, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + h0,
+            scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, kChunk,
+            pl.masked, pl.p2, ds->a1, a2);
+      }
     }
     FM_TRY(launch_status("grad_kernel (dk)"));
     {

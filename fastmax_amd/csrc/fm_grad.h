@@ -284,3 +284,262 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   rs = block_sum_256(rs, red, tid);
   if (tid == 0) rpart[(int64_t)head * gridDim.x + tblk] = rs;
 }
+
+// ---------------------------------------------------------------------------------------
+// bf16 variant of grad_kernel (bf16 inputs and outputs): every contraction runs on
+// v_mfma_f32_32x32x8_bf16 with fp32 accumulation.  The state slab keeps its [row][column]
+// layout and is rounded to bf16 while staged (coefficient applied in fp32 first), the token's
+// extended value vector is packed once, so a 32-row tile costs D/8 + 1 MFMAs; the credits are
+// the fp32 register/LDS work of the fp32 kernel.  Streamed tiles are staged as bf16, the first
+// one in both orientations (rows for the scores, transposed for the product with W).
+// ---------------------------------------------------------------------------------------
+template <int D, int MODE>
+__global__ __launch_bounds__(256, 2) void grad_kernel_bf(
+    const bf16_t* __restrict__ X, const bf16_t* __restrict__ Y, const float* __restrict__ yden,
+    int64_t yden_stride, const float* __restrict__ cvec, const bf16_t* __restrict__ A1,
+    const bf16_t* __restrict__ A2, const float* __restrict__ a2den, int64_t a2den_stride,
+    const float* __restrict__ xscale, const float* __restrict__ a1scale,
+    const float* __restrict__ state, int nslots, bf16_t* __restrict__ OUT, float* __restrict__ rpart,
+    int n, int chunk, int masked, int p2, float a1, float a2) {
+  using G = Geo<D>;
+  using T = bf16_t;
+  constexpr bool DQ = MODE == 0;
+  constexpr int LD = G::LD, AB = G::AB, H2 = G::H2, NS = G::NS;
+  constexpr int LB = D + 4;   // bf16 row pitch (elements)
+  constexpr int TPB = 36;     // pitch of the transposed 32-token tile
+  constexpr int SLB0 = D * LB, SLB1 = 2 * 32 * LB + D * TPB;
+  constexpr int SLB = ((SLB0 > SLB1 ? SLB0 : SLB1) + 7) / 8 * 8;
+  __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb[2][SLB];
+  __shared__ float Cl[2][32];
+  __shared__ float red[4];
+
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
+  const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
+  const int head = lid / gridDim.x, tblk = lid % gridDim.x, tok0 = tblk * 128;
+  const int c = tok0 / chunk;
+  const int nc = (n + chunk - 1) / chunk;
+  const int rows2 = G::rows2(p2);
+  const int64_t SS = G::state_floats(p2);
+  const T* Xh = X + (int64_t)head * n * D;
+  const T* Yh = Y + (int64_t)head * n * D;
+  const T* A1h = A1 + (int64_t)head * n * D;
+  const T* A2h = A2 + (int64_t)head * n * D;
+  const float* ydh = yden ? yden + (int64_t)head * n * yden_stride : nullptr;
+  const float* a2dh = a2den ? a2den + (int64_t)head * n * a2den_stride : nullptr;
+  const float* ch = cvec + (int64_t)head * n;
+  const float xs = xscale[head], a1s = a1scale[head];
+  const int xrow = w * 32 + i, tok = tok0 + xrow;
+
+  {
+    RowTile<D, T, 128> t;
+    t.load(Xh, tok0, n, tid);
+    t.store(Xl, LD, xs, tid);
+    t.load(Yh, tok0, n, tid, ydh, yden_stride);
+    // the own y rows only pass through LDS to reach their lanes: [128][LB] bf16 fits one stage pair
+    static_assert(128 * LB <= 2 * SLB, "own-row staging must fit the stage buffers");
+    t.store_bf(&Sb[0][0], LB, 1.0f, tid);
+  }
+  __syncthreads();
+  // own token of this lane = row xrow: its half of y, packed (A operand of the state
+  // contraction, B operand of g.v)
+  s4v Yp[H2 / 4];
+#pragma unroll
+  for (int g4 = 0; g4 < H2 / 4; ++g4)
+    Yp[g4] = as_s4v(*reinterpret_cast<const uint2*>(&Sb[0][0] + xrow * LB + hh * H2 + 4 * g4));
+  const float c_own = (DQ && tok < n) ? ch[tok] : 0.f;
+  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
+  const s4v yxp = pack_bf4(yxhi, yx - yxhi, yxhi, yx - yxhi);  // pairs with (e_hi, e_hi, e_lo, e_lo)
+  __syncthreads();
+
+  const bool no_state = masked && (DQ ? c == 0 : c == nc - 1);
+  const int n_state = no_state ? 0 : (p2 ? NS : 0) + 1;
+  int n_tile = 0, tile0 = 0;
+  if (masked) {
+    if (DQ) {
+      tile0 = (c * chunk) >> 5;
+      const int last = tok0 + 127 < n ? tok0 + 127 : n - 1;
+      n_tile = (last >> 5) - tile0 + 1;
+    } else {
+      tile0 = tok0 >> 5;
+      const int cend = (c + 1) * chunk < n ? (c + 1) * chunk : n;
+      n_tile = ((cend - 1) >> 5) - tile0 + 1;
+    }
+  }
+  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
+  const int nsum = masked ? 1 : nslots;
+
+  StateSlab<D * LD> slab;
+  RowTile<D, T, 32> t1, t2;
+  float creg = 0.f;
+  auto slab_load = [&](int st) {
+    slab.load(sbase + ((p2 && st < NS) ? st * D * LD : rows2 * LD), SS, nsum, D * LD, tid);
+  };
+  // fp32 [row][LD] -> bf16 [row][LB] (same pitch in elements), coefficient applied first
+  auto slab_store = [&](int st) {
+    const float cf = (p2 && st < NS) ? 2.0f * a2 : a1;
+    uint16_t* dst = Sb[st & 1];
+#pragma unroll
+    for (int u = 0; u < decltype(slab)::NV; ++u) {
+      const int idx = tid + u * 256;
+      if (idx < D * LD / 4) {
+        float4 v4 = slab.v[u];
+        if (idx % (LD / 4) == D / 4) {
+          // extra column e and three floats of padding the build never writes: store
+          // (e_hi, e_hi, e_lo, e_lo); with yx as (hi, lo, hi, lo) the extra-column MFMA then forms
+          // yx * e to 16 bits of mantissa -- this term nearly cancels the value columns' sum
+          const float e = v4.x * cf, ehi = bf_lo(pack_bf2(e, 0.f));
+          v4 = make_float4(ehi, ehi, e - ehi, e - ehi);
+          *reinterpret_cast<uint2*>(dst + idx * 4) = make_uint2(pack_bf2(v4.x, v4.y), pack_bf2(v4.z, v4.w));
+        } else {
+          *reinterpret_cast<uint2*>(dst + idx * 4) =
+              make_uint2(pack_bf2(v4.x * cf, v4.y * cf), pack_bf2(v4.z * cf, v4.w * cf));
+        }
+      }
+    }
+  };
+  auto tiles_load = [&](int kk) {
+    const int r0 = (tile0 + kk) * 32;
+    t1.load(A1h, r0, n, tid);
+    t2.load(A2h, r0, n, tid, a2dh, a2den_stride);
+    if (!DQ && tid < 32) creg = (r0 + tid < n) ? ch[r0 + tid] : 0.f;
+  };
+  auto tiles_store = [&](int buf) {
+    t1.store_bf(Sb[buf], LB, a1s, tid);
+    t2.store_bf(Sb[buf] + 32 * LB, LB, 1.0f, tid);
+    t1.store_t_bf(Sb[buf] + 2 * 32 * LB, TPB, a1s, tid);
+    if (!DQ && tid < 32) Cl[buf][tid] = creg;
+  };
+
+  f16v out[AB];
+#pragma unroll
+  for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) out[ab][r] = 0.f;
+
+  if (n_tile > 0) tiles_load(0);
+  if (n_state > 0) {
+    slab_load(0);
+    slab_store(0);
+  } else if (n_tile > 0) {
+    tiles_store(0);
+  }
+  __syncthreads();
+
+  auto chain = [&](const uint16_t* sl, int ab) {
+    const uint16_t* ar = sl + (ab * 32 + i) * LB;
+    uint2 b[H2 / 4 + 1];
+#pragma unroll
+    for (int g4 = 0; g4 < H2 / 4; ++g4) b[g4] = *reinterpret_cast<const uint2*>(ar + hh * H2 + 4 * g4);
+    b[H2 / 4] = *reinterpret_cast<const uint2*>(ar + D);  // extra column and its zero padding
+    f16v t;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) t[r] = 0.f;
+#pragma unroll
+    for (int g4 = 0; g4 < H2 / 4; ++g4) t = FM_MFMA_BF(Yp[g4], as_s4v(b[g4]), t);
+    return FM_MFMA_BF(yxp, as_s4v(b[H2 / 4]), t);
+  };
+  const float* xtok = Xl + (w * 32 + 4 * hh) * LD;
+  auto xat = [&](int r, int col) { return xtok[((r >> 2) * 8 + (r & 3)) * LD + col]; };
+
+  for (int st = 0; st < n_state; ++st) {
+    slab_load(st + 1 < n_state ? st + 1 : st);
+    const uint16_t* sl = Sb[st & 1];
+    f16v tt[AB];
+#pragma unroll
+    for (int ab = 0; ab < AB; ++ab) tt[ab] = chain(sl, ab);
+    if (p2 && st < NS) {
+      const int s = st;
+#pragma unroll
+      for (int ab = 0; ab < AB; ++ab) {
+        const int rc = (ab * 32 + i + s) & (D - 1);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out[ab][r] += tt[ab][r] * xat(r, rc);
+      }
+      if (s > 0 && s < H2) {
+#pragma unroll
+        for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tt[ab][r] *= xat(r, ab * 32 + i);
+        const bool keep = i < 32 - s;
+        const int src = (((i - s) & 31) + 32 * hh) << 2;
+#pragma unroll
+        for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float v = keep ? tt[ab][r] : tt[(ab + 1) % AB][r];
+            out[ab][r] += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, v)));
+          }
+      }
+    } else {
+#pragma unroll
+      for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out[ab][r] += tt[ab][r];
+    }
+    if (st + 1 < n_state) slab_store(st + 1);
+    else if (n_tile > 0) tiles_store((st + 1) & 1);
+    __syncthreads();
+  }
+
+  if (n_tile > 0) {
+    s4v Xp[H2 / 4];
+#pragma unroll
+    for (int g4 = 0; g4 < H2 / 4; ++g4) {
+      const float4 x4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + hh * H2 + 4 * g4);
+      Xp[g4] = pack_bf4(x4.x, x4.y, x4.z, x4.w);
+    }
+    const int mine = (tok0 >> 5) + w;
+    const float twoa2 = 2.0f * a2;
+    for (int kk = 0; kk < n_tile; ++kk) {
+      const int buf = (n_state + kk) & 1;
+      tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
+      const int tl = tile0 + kk;
+      if (DQ ? tl <= mine : tl >= mine) {
+        const uint16_t* l1 = Sb[buf];
+        const uint16_t* l2 = l1 + 32 * LB;
+        const uint16_t* l1t = l1 + 2 * 32 * LB;
+        f16v sc, gv;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = gv[r] = 0.f;
+#pragma unroll
+        for (int g4 = 0; g4 < H2 / 4; ++g4) {
+          sc = FM_MFMA_BF(as_s4v(*reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 4 * g4)), Xp[g4], sc);
+          gv = FM_MFMA_BF(as_s4v(*reinterpret_cast<const uint2*>(l2 + i * LB + hh * H2 + 4 * g4)), Yp[g4], gv);
+        }
+        const bool diag = tl == mine;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float cc = DQ ? c_own : Cl[buf][trow(r, hh)];
+          float wv = (a1 + twoa2 * sc[r]) * (gv[r] - cc);
+          if (diag && (DQ ? trow(r, hh) > i : trow(r, hh) < i)) wv = 0.f;
+          sc[r] = wv;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const s4v wp = pack_bf4(sc[4 * j], sc[4 * j + 1], sc[4 * j + 2], sc[4 * j + 3]);
+#pragma unroll
+          for (int ab = 0; ab < AB; ++ab)
+            out[ab] = FM_MFMA_BF(wp, as_s4v(*reinterpret_cast<const uint2*>(l1t + (ab * 32 + i) * TPB + 8 * j + 4 * hh)), out[ab]);
+        }
+      }
+      if (kk + 1 < n_tile) tiles_store(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  float rs = 0.f;
+  T* Oh = OUT + (int64_t)head * n * D;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int tk = tok0 + w * 32 + trow(r, hh);
+#pragma unroll
+    for (int ab = 0; ab < AB; ++ab) {
+      const float g = out[ab][r];
+      rs += g * xat(r, ab * 32 + i);
+      if (tk < n) Oh[(int64_t)tk * D + ab * 32 + i] = from_f32<T>(g * xs);
+    }
+  }
+  rs = block_sum_256(rs, red, tid);
+  if (tid == 0) rpart[(int64_t)head * gridDim.x + tblk] = rs;
+}
