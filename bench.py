@@ -7,7 +7,7 @@ A step is one forward + one backward pass of the attention operator over one bat
 synthetic q, k, v and upstream gradient already resident in HBM, called through the C ABI
 (include/fastmax_amd.h).  Prints ONE JSON line: whole-job tokens/s (tokens = B*N per step),
 the roofline position of the dominant kernel (algorithmic flops / HIP-event kernel time,
-against the fp32 MFMA peak) and a CPU baseline (the oracle's reference-form restatement of
+against the MFMA peak of the input type) and a CPU baseline (the oracle's reference-form restatement of
 the reference's PyTorch path, timed on a bounded sample on this host's cores).
 """
 from __future__ import annotations
@@ -190,7 +190,8 @@ def main() -> int:
     dom_ms = kernels[dom]["ms_per_step"]
     launches = kernels[dom]["launches_per_step"]
     achieved = per_step_flops[dom] / (dom_ms * 1e-3) / 1e12
-    peak = PEAK_TFLOPS["f32"]  # every contraction runs on v_mfma_f32_32x32x2f32, also for bf16 inputs
+    # fp32 inputs run every contraction on v_mfma_f32_32x32x2f32; bf16 inputs on v_mfma_f32_32x32x8_bf16
+    peak = PEAK_TFLOPS[cfg["dtype"]]
     roofline = {
         "bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
         "frac": achieved / peak, "traffic": None,
@@ -211,7 +212,7 @@ def main() -> int:
         "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": cfg["dtype"], "data": "synthetic",
+        "dtype": cfg["dtype"] if cfg["dtype"] == "f32" else "bf16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": f"{args.workload}: Fastmax {'causal' if cfg['mask'] else 'unmasked'} fwd+bwd, "
                                f"B={B} H={H} N={N} D={D} p={cfg['p']} {cfg['dtype']}, normalize lim=1, "
                                "a=(1,1,0.5), q/k/v/grad iid N(0,1) seed 0"},

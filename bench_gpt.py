@@ -171,7 +171,7 @@ def main() -> int:
         "metric": "GPT training step with Fastmax causal attention in every layer",
         "value": args.batch * args.seq / (ms * 1e-3), "unit": "tokens/s", "ms_per_step": ms,
         "attention_fwd_bwd_ms_per_step": attn_ms, "attention_share_of_step": attn_ms / ms,
-        "dtype": "bf16 autocast (attention: bf16 in/out, fp32 arithmetic)", "data": "synthetic",
+        "dtype": "bf16 autocast (attention: bf16 in/out, bf16 matrix instructions, fp32 accumulate)", "data": "synthetic",
         "config": {"workload": f"{args.layers} layers, d_model 768, 12 heads x 64, MLP 3072 GELU, RoPE, vocab 50304, "
                                f"seq {args.seq}, batch {args.batch}, p={args.p}, AdamW",
                    "attention": "pytorch function" if args.pytorch_attention else "hip kernels"},

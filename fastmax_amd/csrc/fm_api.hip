@@ -59,13 +59,17 @@ struct ScopedKernel {
   }
 };
 
-constexpr int kChunk = 256;                       // tokens between causal state snapshots
+constexpr int kChunk = 256;      // tokens between causal state snapshots (fp32 arithmetic)
+constexpr int kChunkBf16 = 512;  // ... when the contractions run on the bf16 matrix instruction: the
+                                 // moment work is ~8x cheaper there, so snapshot traffic is worth
+                                 // halving at the price of more intra-chunk tiles
 constexpr size_t kWorkspaceBudget = 16ull << 30;   // what fastmax_workspace_bytes aims for
 
 struct Plan {
   int d, p2, masked, n, bh;
   int rtw, gsplit;     // build kernel: row tiles per wave, feature splits per head
   int nslots, zlen;    // state slots per head; tokens per slot when unmasked
+  int chunk;           // tokens between causal state snapshots
   int nblk;            // 128-token blocks per head
   int64_t state_floats;
   size_t fixed_bytes;     // scale/argmax/cvec/rpart
@@ -99,8 +103,9 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   }
   pl.gsplit = splits(pl.rtw);
   pl.nblk = (pl.n + 127) / 128;
+  pl.chunk = ds->dtype == FASTMAX_BF16 ? kChunkBf16 : kChunk;
   if (pl.masked) {
-    pl.nslots = (pl.n + kChunk - 1) / kChunk;
+    pl.nslots = (pl.n + pl.chunk - 1) / pl.chunk;
     pl.zlen = 0;
   } else {
     // enough token splits to put ~1024 blocks in flight, at least 256 tokens each
@@ -211,7 +216,7 @@ int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float*
   ScopedKernel sk(FASTMAX_K_BUILD, stream);
 #define FM_BUILD(RTW)                                                                            \
   build_kernel<D, T, RTW, kBf16Mfma<T>><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, yden_stride, ew, state, \
-                                                    pl.n, kChunk, pl.nslots, pl.masked, reverse, \
+                                                    pl.n, pl.chunk, pl.nslots, pl.masked, reverse, \
                                                     pl.p2, pl.zlen)
   if (pl.rtw == 1) {
     FM_BUILD(1);
@@ -252,12 +257,12 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
       if constexpr (kBf16Mfma<T>) {
         apply_kernel_bf<D, 0><<<agrid, 256, 0, stream>>>(
             q + off, k + off, v + off, scale + h0, scale + bh + h0, nullptr, 0, state, pl.nslots,
-            o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, kChunk,
+            o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, pl.chunk,
             pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
       } else {
         apply_kernel<D, T, 0><<<agrid, 256, 0, stream>>>(
             q + off, k + off, v + off, scale + h0, scale + bh + h0, nullptr, 0, state, pl.nslots,
-            o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, kChunk,
+            o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, pl.chunk,
             pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
       }
     }
@@ -313,12 +318,12 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       if constexpr (kBf16Mfma<T>) {
         grad_kernel_bf<D, 0><<<grid, 256, 0, stream>>>(
             q + off, go + off, denh, den_stride, ch, k + off, v + off, nullptr, 0, scale + h0,
-            scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, kChunk, pl.masked,
+            scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, pl.chunk, pl.masked,
             pl.p2, ds->a1, a2);
       } else {
         grad_kernel<D, T, 0><<<grid, 256, 0, stream>>>(
             q + off, go + off, denh, den_stride, ch, k + off, v + off, nullptr, 0, scale + h0,
-            scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, kChunk, pl.masked,
+            scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, pl.chunk, pl.masked,
             pl.p2, ds->a1, a2);
       }
     }
@@ -328,12 +333,12 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       if constexpr (kBf16Mfma<T>) {
         grad_kernel_bf<D, 1><<<grid, 256, 0, stream>>>(
             k + off, v + off, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + h0,
-            scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, kChunk,
+            scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, pl.chunk,
             pl.masked, pl.p2, ds->a1, a2);
       } else {
         grad_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
             k + off, v + off, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + h0,
-            scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, kChunk,
+            scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, pl.chunk,
             pl.masked, pl.p2, ds->a1, a2);
       }
     }
@@ -343,11 +348,11 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       if constexpr (kBf16Mfma<T>) {
         apply_kernel_bf<D, 1><<<grid, 256, 0, stream>>>(
             k + off, q + off, go + off, scale + bh + h0, scale + h0, denh, den_stride, stR, pl.nslots,
-            dv + off, D, nullptr, 0, n, kChunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
+            dv + off, D, nullptr, 0, n, pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
       } else {
         apply_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
             k + off, q + off, go + off, scale + bh + h0, scale + h0, denh, den_stride, stR, pl.nslots,
-            dv + off, D, nullptr, 0, n, kChunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
+            dv + off, D, nullptr, 0, n, pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
       }
     }
     FM_TRY(launch_status("apply_kernel (dv)"));

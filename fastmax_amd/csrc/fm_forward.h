@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
 
   // per owned row tile: LDS offsets of the lane's own channel row and of its rotated partner
   int ownoff[RTW], rotoff[RTW], rowbase[RTW];
-  int nx = 0;
+  int nx = 0;  // row tiles this wave really owns (wave-uniform)
 #pragma unroll
   for (int x = 0; x < RTW; ++x) {
     const int rt = (g * 4 + w) * RTW + x;
