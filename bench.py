@@ -35,6 +35,7 @@ WORKLOADS = {
     "c1": dict(B=8, H=8, N=1024, D=32, mask=False, p=2, dtype="f32"),
     "c2": dict(B=64, H=8, N=1000, D=32, mask=True, p=2, dtype="f32"),
     "c4": dict(B=16, H=32, N=16384, D=64, mask=True, p=2, dtype="bf16"),
+    "c5-layer": dict(B=8, H=12, N=2048, D=64, mask=True, p=2, dtype="bf16"),  # one layer of the GPT step
 }
 COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 

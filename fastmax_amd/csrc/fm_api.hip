@@ -69,6 +69,8 @@ struct Plan {
   int d, p2, masked, n, bh;
   int rtw, gsplit;     // build kernel: row tiles per wave, feature splits per head
   int nslots, zlen;    // state slots per head; tokens per slot when unmasked
+  int nparts;          // token splits the unmasked build sums separately (1 when masked); bf16
+                       // inputs add one slot that receives their sum in packed form
   int chunk;           // tokens between causal state snapshots
   int nblk;            // 128-token blocks per head
   int64_t state_floats;
@@ -106,6 +108,7 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   pl.chunk = ds->dtype == FASTMAX_BF16 ? kChunkBf16 : kChunk;
   if (pl.masked) {
     pl.nslots = (pl.n + pl.chunk - 1) / pl.chunk;
+    pl.nparts = 1;
     pl.zlen = 0;
   } else {
     // enough token splits to put ~1024 blocks in flight, at least 256 tokens each
@@ -115,7 +118,9 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
     if (z < 1) z = 1;
     int zlen = ((pl.n + z - 1) / z + 31) / 32 * 32;
     pl.zlen = zlen;
-    pl.nslots = (pl.n + zlen - 1) / zlen;
+    pl.nparts = (pl.n + zlen - 1) / zlen;
+    // bf16: one more slot for the summed state in the packed form the consumers read
+    pl.nslots = pl.nparts + (ds->dtype == FASTMAX_BF16 ? 1 : 0);
   }
   pl.state_floats = state_floats_for(pl.d, pl.p2);
   size_t fixed = align256((size_t)2 * pl.bh * sizeof(float)) + align256((size_t)2 * pl.bh * sizeof(int));
@@ -207,17 +212,19 @@ constexpr bool kBf16Mfma = false;
 template <>
 constexpr bool kBf16Mfma<bf16_t> = true;
 
+// sections (bf16 inputs, masked): which packed layouts the consumers of this state read --
+// 1 = feature-packed (apply kernels), 2 = column-packed (grad kernels)
 template <int D, class T>
 int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float* xscale,
                  const float* yden, int64_t yden_stride, const float* ew, float* state, int reverse,
-                 hipStream_t stream) {
-  const dim3 grid(pl.gsplit, heads, pl.masked ? 1 : pl.nslots);
+                 int sections, hipStream_t stream) {
+  const dim3 grid(pl.gsplit, heads, pl.nparts);
   if (pl.masked && pl.nslots < 2) return FASTMAX_OK;  // a single chunk never needs a state
   ScopedKernel sk(FASTMAX_K_BUILD, stream);
 #define FM_BUILD(RTW)                                                                            \
   build_kernel<D, T, RTW, kBf16Mfma<T>><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, yden_stride, ew, state, \
                                                     pl.n, pl.chunk, pl.nslots, pl.masked, reverse, \
-                                                    pl.p2, pl.zlen)
+                                                    pl.p2, pl.zlen, sections)
   if (pl.rtw == 1) {
     FM_BUILD(1);
   } else if constexpr (D == 64) {
@@ -230,6 +237,10 @@ int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float*
     FM_BUILD(5);
   }
 #undef FM_BUILD
+  if constexpr (kBf16Mfma<T>) {
+    if (!pl.masked)
+      state_pack_kernel<D><<<dim3(PackedGeo<D>::nslab(pl.p2), heads), 256, 0, stream>>>(state, pl.nslots, pl.nparts, pl.p2);
+  }
   return launch_status("build_kernel");
 }
 
@@ -250,7 +261,7 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
     const int64_t off = (int64_t)h0 * n * D;
-    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, state, 0, stream)));
+    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, state, 0, 1, stream)));
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       const dim3 agrid(pl.nblk, heads);
@@ -310,8 +321,8 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     const float* denh = den + (int64_t)h0 * n * den_stride;
     const float* ch = cvec + (int64_t)h0 * n;
     // prefix state of (kh, v, 1) and suffix state of (qh, go/den, c)
-    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, stS, 0, stream)));
-    FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, stream)));
+    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, stS, 0, 2, stream)));
+    FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, 3, stream)));
     const dim3 grid(pl.nblk, heads);
     {
       ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);

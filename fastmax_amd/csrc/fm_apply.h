@@ -278,10 +278,12 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
 // ---------------------------------------------------------------------------------------
 // bf16 variant of apply_kernel (bf16 inputs and outputs): same decomposition, but every
 // contraction runs on v_mfma_f32_32x32x8_bf16 with fp32 accumulation.  Features are formed in
-// fp32 from the fp32-scaled inputs and rounded when packed; the state slab is transposed and
-// rounded to bf16 while it is staged ([column][feature], so that the four features of a lane's
-// k-slots are one 64-bit LDS read); the order-0 row stays fp32.  The forward denominator comes
-// from a third accumulator tile whose B operand is the state's extra column broadcast to every
+// fp32 from the fp32-scaled inputs and rounded when packed.  The state arrives in the packed
+// bf16 form (PackedGeo): a feature-packed slab is copied to LDS as it is and the four features
+// of a lane's k-slots are one 64-bit LDS read; the order-2 slabs carry their pair weights, a2
+// multiplies their accumulated sum, a1 the order-1 features and a0 the fp32 order-0 row.  The
+// forward denominator comes from a third accumulator tile whose B operand is the state's extra
+// column broadcast to every
 // lane, which leaves den[row] in every lane that holds that row of the output.
 // Lane half hh owns features/channels 32*hh + t as in the fp32 kernel; MFMA g of a sweep takes
 // t = 4g..4g+3 from both halves.
@@ -290,21 +292,22 @@ template <int D, int MODE>
 __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     const bf16_t* __restrict__ X, const bf16_t* __restrict__ A1, const bf16_t* __restrict__ A2,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
-    const float* __restrict__ a2den, int64_t a2den_stride, const float* __restrict__ state,
+    const float* __restrict__ a2den, int64_t a2den_stride, const float* state,
     int nslots, bf16_t* __restrict__ OUT, int64_t ldo, float* __restrict__ den, int64_t den_stride,
     int n, int chunk, int masked, int p2, float a0, float a1, float a2) {
   using G = Geo<D>;
   using T = bf16_t;
   constexpr bool FWD = MODE == 0;
   constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS;
+  using PG = PackedGeo<D>;
   constexpr int LB = D + 4;            // pitch of bf16 rows (16-bit elements): 8-byte aligned, and the
                                        // 16 lanes of a 64-bit access phase fall in distinct banks
   constexpr int TPB = 36;              // pitch of the transposed 32-token value tile
-  constexpr int SLB0 = (D + 2) * LB, SLB1 = 32 * LB + D * TPB;  // D+1 state columns, or both tiles
-  constexpr int SLB = (SLB0 > SLB1 ? SLB0 : SLB1 + 7) / 8 * 8;
+  constexpr int NCF = PG::NCF, FSL = PG::FSL;
+  constexpr int SLB1 = 32 * LB + D * TPB;  // both 32-token tiles
+  constexpr int SLB = ((FSL > SLB1 ? FSL : SLB1) + 7) / 8 * 8;
   __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
   __shared__ __attribute__((aligned(16))) uint16_t Sb[2][SLB];
-  __shared__ float S0l[2][D + 4];      // order-0 row (fp32), one per stage buffer
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
@@ -339,40 +342,29 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
       n_tile = ((cend - 1) >> 5) - tile0 + 1;
     }
   }
-  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
-  const int nsum = masked ? 1 : nslots;
+  // packed state of this block's chunk (masked) or the head's summed state (last slot)
+  const char* sbase = reinterpret_cast<const char*>(state + ((int64_t)head * nslots + (masked ? c : nslots - 1)) * SS);
+  const uint16_t* fsec = reinterpret_cast<const uint16_t*>(sbase);
+  const float* zsec = reinterpret_cast<const float*>(sbase + PG::z_off(p2));
 
-  StateSlab<(D + 1) * LD> slab;
+  // an F slab is copied as it is: 16-byte pieces global -> registers -> LDS
+  // (no branches: threads past the end wrap round and copy an early piece a second time, so that
+  // every load is issued up front and stays in flight under the MFMAs)
+  constexpr int NPC = FSL / 8, NVS = (NPC + 255) / 256;
+  static_assert(NVS <= 3, "three named pieces per thread (an indexed array would live in scratch)");
+  uint4 sv0, sv1, sv2;
   RowTile<D, T, 32> t1, t2;
   auto slab_load = [&](int st) {
-    const bool ord2 = p2 && st < NS;
-    slab.load(sbase + (ord2 ? st * D * LD : rows2 * LD), SS, nsum, ord2 ? D * LD : (D + 1) * LD, tid);
+    const uint4* src = reinterpret_cast<const uint4*>(fsec + st * FSL);
+    sv0 = src[tid % NPC];
+    if constexpr (NVS > 1) sv1 = src[(tid + 256) % NPC];
+    if constexpr (NVS > 2) sv2 = src[(tid + 512) % NPC];
   };
-  // fp32 [feature][LD] rows in registers -> bf16 [column][LB] in LDS, coefficient applied on the way
   auto slab_store = [&](int st) {
-    const bool ord2 = p2 && st < NS;
-    const float cf = ord2 ? ((st == 0 || st == H2) ? a2 : 2.0f * a2) : a1;
-    uint16_t* dst = Sb[st & 1];
-    constexpr int VPR = LD / 4;  // float4 pieces per state row
-    const int nvec = ((ord2 ? D * LD : (D + 1) * LD) + 3) >> 2;
-#pragma unroll
-    for (int u = 0; u < decltype(slab)::NV; ++u) {
-      const int idx = tid + u * 256;
-      if (idx < nvec) {
-        const int f = idx / VPR, c0 = (idx % VPR) * 4;
-        const float4 v4 = slab.v[u];
-        const float e4[4] = {v4.x, v4.y, v4.z, v4.w};
-        if (f < D) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (c0 + e <= D) dst[(c0 + e) * LB + f] = (uint16_t)pack_bf2(e4[e] * cf, 0.f);
-        } else {  // the order-0 row that follows the order-1 rows
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (c0 + e <= D) S0l[st & 1][c0 + e] = e4[e] * a0;
-        }
-      }
-    }
+    uint4* dst = reinterpret_cast<uint4*>(Sb[st & 1]);
+    dst[tid % NPC] = sv0;
+    if constexpr (NVS > 1) dst[(tid + 256) % NPC] = sv1;
+    if constexpr (NVS > 2) dst[(tid + 512) % NPC] = sv2;
   };
   auto tiles_load = [&](int kk) {
     t1.load(A1h, (tile0 + kk) * 32, n, tid);
@@ -418,23 +410,30 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     }
   };
 
+  // one slab: B operands are 64-bit reads of [feature group][column][4 features]
   auto slab_compute = [&](const uint16_t* sl, auto tag) {
     constexpr bool ORD2 = decltype(tag)::value;
-    const uint16_t* brow = sl + hh * H2;
+    const uint16_t* brow = sl + (hh * (H2 / 4) * NCF + i) * 4;
 #pragma unroll
     for (int g4 = 0; g4 < H2 / 4; ++g4) {
       const int t = 4 * g4;
       const s4v ap = ORD2 ? pack_bf4(Xr[t] * Wn[t], Xr[t + 1] * Wn[t + 1], Xr[t + 2] * Wn[t + 2], Xr[t + 3] * Wn[t + 3])
-                          : pack_bf4(Xr[t], Xr[t + 1], Xr[t + 2], Xr[t + 3]);
+                          : pack_bf4(Xr[t] * a1, Xr[t + 1] * a1, Xr[t + 2] * a1, Xr[t + 3] * a1);
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb)
-        acc[cb] = FM_MFMA_BF(ap, as_s4v(*reinterpret_cast<const uint2*>(brow + (cb * 32 + i) * LB + t)), acc[cb]);
-      if (FWD) accd = FM_MFMA_BF(ap, as_s4v(*reinterpret_cast<const uint2*>(brow + D * LB + t)), accd);
+        acc[cb] = FM_MFMA_BF(ap, as_s4v(*reinterpret_cast<const uint2*>(brow + (g4 * NCF + cb * 32) * 4)), acc[cb]);
+      if (FWD) accd = FM_MFMA_BF(ap, as_s4v(*reinterpret_cast<const uint2*>(sl + ((hh * (H2 / 4) + g4) * NCF + D) * 4)), accd);
     }
   };
 
-  for (int st = 0; st < n_state; ++st) {
-    slab_load(st + 1 < n_state ? st + 1 : st);
+  // the order-2 slabs carry their pair weights; a2 is applied to their sum, a1 to the order-1
+  // features and a0 to the order-0 row
+  float zc[CB], zd = 0.f;
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) zc[cb] = n_state > 0 ? a0 * zsec[cb * 32 + i] : 0.f;
+  if (FWD && n_state > 0) zd = a0 * zsec[D];
+
+  auto slab_step = [&](int st) {
     const uint16_t* sl = Sb[st & 1];
     if (p2 && st < NS) {
       if ((st & 3) == 0) {
@@ -444,23 +443,35 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
         for (int x = 0; x < H2 + 3; ++x) Wn[x] = Wn[x + 1];
       }
       slab_compute(sl, std::true_type{});
+      if (st == NS - 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) acc[cb][r] *= a2;
+          accd[r] *= a2;
+        }
+      }
     } else {
       slab_compute(sl, std::false_type{});
-      const float* s0 = S0l[st & 1];
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) {
-        const float z = s0[cb * 32 + i];
+      for (int r = 0; r < 16; ++r) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[cb][r] += z;
-      }
-      if (FWD) {
-        const float z = s0[D];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) accd[r] += z;
+        for (int cb = 0; cb < CB; ++cb) acc[cb][r] += zc[cb];
+        if (FWD) accd[r] += zd;
       }
     }
-    if (st + 1 < n_state) slab_store(st + 1);
-    else if (n_tile > 0) tiles_store((st + 1) & 1);
+  };
+  // the last slab is peeled off so that load and store of the next slab are unconditional in
+  // the loop (a load whose only use sits in a branch is moved there and waited for at once)
+  for (int st = 0; st + 1 < n_state; ++st) {
+    slab_load(st + 1);
+    slab_step(st);
+    slab_store(st + 1);
+    __syncthreads();
+  }
+  if (n_state > 0) {
+    slab_step(n_state - 1);
+    if (n_tile > 0) tiles_store(n_state & 1);
     __syncthreads();
   }
 

@@ -129,6 +129,32 @@ struct Geo {
   static constexpr int SLABF = (SLAB + 3) / 4 * 4;
 };
 
+// Packed bf16 form of a state, used when the inputs are bf16 (it occupies the same
+// state_floats slot as the fp32 form).  A "slab" is the D feature rows of one shift s
+// (order 2; rows carry their pair weight: x2 for 0 < s < D/2) or the D order-1 rows (slab
+// NS, or slab 0 when p == 1).  Each slab is stored twice, in the two operand layouts of
+// v_mfma_f32_32x32x8_bf16, so that consumers stage it with plain 16-byte copies:
+//   F, feature-packed  [a/4][column 0..D (+1 pad)][a%4]   contraction over features (apply)
+//   C, column-packed   [a][LB = D+4]                        contraction over columns (grad);
+//      columns D..D+3 hold the extra column as (hi, hi, lo, lo) bf16 pairs
+// followed by the order-0 row as D+1 floats.  Column D is the extra (denominator) column.
+template <int D>
+struct PackedGeo {
+  using G = Geo<D>;
+  static constexpr int NCF = D + 2;
+  static constexpr int FSL = (D / 4) * NCF * 4;  // bf16 elements of an F slab (a multiple of 128)
+  static constexpr int LB = D + 4;
+  static constexpr int CSL = D * LB;             // bf16 elements of a C slab (a multiple of 128)
+  __host__ __device__ static constexpr int nslab(int p2) { return (p2 ? G::NS : 0) + 1; }
+  __host__ __device__ static constexpr int64_t c_off(int p2) { return ((int64_t)nslab(p2) * FSL * 2 + 255) / 256 * 256; }
+  __host__ __device__ static constexpr int64_t z_off(int p2) {
+    return c_off(p2) + ((int64_t)nslab(p2) * CSL * 2 + 255) / 256 * 256;
+  }
+  __host__ __device__ static constexpr int64_t bytes(int p2) { return z_off(p2) + (D + 1) * 4; }
+  static_assert(bytes(1) <= G::state_floats(1) * 4 && bytes(0) <= G::state_floats(0) * 4,
+                "the packed form must fit the fp32 state slot");
+};
+
 // A tile of ROWS token rows x D channels staged global -> registers -> LDS by 256 threads.
 // ROWFAST = false: consecutive threads take consecutive 16-byte pieces of a row (coalesced
 // global reads, conflict-free row-major LDS writes).  ROWFAST = true: consecutive threads

@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const float* __restrict__ xscale,
     const float* __restrict__ yden, int64_t yden_stride, const float* __restrict__ ew,
     float* __restrict__ state, int n, int chunk, int nslots, int masked, int reverse, int p2,
-    int zlen) {
+    int zlen, int sections) {
   using G = Geo<D>;
   constexpr int TS = 32;        // tokens per pipeline step
   constexpr int TP = TS + 4;    // pitch of the transposed tiles: 16-byte aligned rows, and the
@@ -288,6 +288,66 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     if (g == 0 && tid <= D) st[(unsigned)((rows2 + D) * LD + tid)] = s0;
   };
 
+  // BF, masked: the snapshot goes out in the packed bf16 form (PackedGeo): section F when
+  // sections & 1, section C when sections & 2, and the fp32 order-0 row.
+  auto snapshot_packed = [&](int slot) {
+    using PG = PackedGeo<D>;
+    char* sb = reinterpret_cast<char*>(state + ((int64_t)head * nslots + slot) * SS);  // uniform
+    uint16_t* fsec = reinterpret_cast<uint16_t*>(sb);
+    uint16_t* csec = reinterpret_cast<uint16_t*>(sb + PG::c_off(p2));
+#pragma unroll
+    for (int x = 0; x < RTW; ++x) {
+      if (x < nx) {
+        const int slab = rowbase[x] / D, arow = rowbase[x] % D;
+        const bool dbl = rowbase[x] < rows2 && slab != 0 && slab != G::H2;  // pair weight 2
+        const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
+        if (sections & 1) {
+          const float wgt = dbl ? 2.0f : 1.0f;
+          uint16_t* fx = fsec + (unsigned)(slab * PG::FSL + (arow >> 2) * PG::NCF * 4);
+          const unsigned lo = (unsigned)((hh * PG::NCF + i) * 4);
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+              const f16v& a = acc[x][cb];
+              *reinterpret_cast<uint2*>(fx + lo + (unsigned)((2 * j * PG::NCF + cb * 32) * 4)) =
+                  make_uint2(pack_bf2(a[4 * j] * wgt, a[4 * j + 1] * wgt), pack_bf2(a[4 * j + 2] * wgt, a[4 * j + 3] * wgt));
+            }
+          if (hh == 0) fx[(unsigned)(((i >> 2) * PG::NCF + D) * 4 + (i & 3))] = (uint16_t)pack_bf2(ds * wgt, 0.f);
+        }
+        if (sections & 2) {
+          uint16_t* cx = csec + (unsigned)(slab * PG::CSL + arow * PG::LB);
+          const unsigned lo = (unsigned)(4 * hh * PG::LB + i);
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; e += 2)
+#pragma unroll
+              for (int cb = 0; cb < CB; ++cb) {
+                const uint32_t u = pack_bf2(acc[x][cb][4 * j + e], acc[x][cb][4 * j + e + 1]);
+                cx[lo + (unsigned)((8 * j + e) * PG::LB + cb * 32)] = (uint16_t)u;
+                cx[lo + (unsigned)((8 * j + e + 1) * PG::LB + cb * 32)] = (uint16_t)(u >> 16);
+              }
+          if (hh == 0) {
+            const float ehi = bf_lo(pack_bf2(ds, 0.f));
+            *reinterpret_cast<uint2*>(cx + (unsigned)(i * PG::LB + D)) =
+                make_uint2(pack_bf2(ehi, ehi), pack_bf2(ds - ehi, ds - ehi));
+          }
+        }
+      }
+    }
+    if (g == 0 && tid <= D) reinterpret_cast<float*>(sb + PG::z_off(p2))[tid] = s0;
+  };
+  auto emit = [&](int slot) {
+    if constexpr (BF) {
+      if (masked) {
+        snapshot_packed(slot);
+        return;
+      }
+    }
+    snapshot(slot);
+  };
+
   // The walk is one software pipeline over all 32-token steps: the loads of step p+1 are issued
   // before the MFMAs of step p and consumed after them; a snapshot is stored right after that,
   // so its stores drain under the next step's MFMAs.
@@ -341,8 +401,55 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     // after the staged tile has been consumed: waiting for loads while stores are pending
     // would wait for the stores too (one in-order counter covers both)
     const int slot = step_slot(p);
-    if (slot >= 0) snapshot(slot);
+    if (slot >= 0) emit(slot);
     __syncthreads();
   }
-  if (!masked && nsteps == 0) snapshot(zsplit);  // an empty token split still owns its slot
+  if (!masked && nsteps == 0) emit(zsplit);  // an empty token split still owns its slot
+}
+
+// ---------------------------------------------------------------------------------------
+// bf16 inputs, unmasked: sums the nparts fp32 partial states of a head (slots 0..nparts-1)
+// and writes the packed bf16 form (PackedGeo) into the head's last slot, nslots-1.
+// grid = (slabs, heads), 256 threads.
+// ---------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void state_pack_kernel(float* __restrict__ state, int nslots, int nparts, int p2) {
+  using G = Geo<D>;
+  using PG = PackedGeo<D>;
+  constexpr int LD = G::LD;
+  __shared__ __attribute__((aligned(16))) float Sl[(D + 1) * LD];
+  const int slab = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+  const int64_t SS = G::state_floats(p2);
+  const bool ord1 = slab == PG::nslab(p2) - 1;  // the order-1 rows, followed by the order-0 row
+  const float* src = state + (int64_t)head * nslots * SS + (int64_t)slab * D * LD;
+  const int nf = (ord1 ? D + 1 : D) * LD;
+  for (int idx = tid * 4; idx < nf; idx += 1024) {
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int part = 0; part < nparts; ++part) {
+      const float4 t = *reinterpret_cast<const float4*>(src + part * SS + idx);
+      a.x += t.x; a.y += t.y; a.z += t.z; a.w += t.w;
+    }
+    *reinterpret_cast<float4*>(Sl + idx) = a;
+  }
+  __syncthreads();
+  char* sb = reinterpret_cast<char*>(state + ((int64_t)head * nslots + nslots - 1) * SS);
+  uint16_t* fsec = reinterpret_cast<uint16_t*>(sb) + slab * PG::FSL;
+  uint16_t* csec = reinterpret_cast<uint16_t*>(sb + PG::c_off(p2)) + slab * PG::CSL;
+  const float wgt = (!ord1 && slab != 0 && slab != G::H2) ? 2.0f : 1.0f;
+  for (int idx = tid; idx < (D / 4) * (D + 1); idx += 256) {
+    const int tg = idx / (D + 1), col = idx % (D + 1);
+    const float* f = Sl + 4 * tg * LD + col;
+    *reinterpret_cast<uint2*>(fsec + (tg * PG::NCF + col) * 4) =
+        make_uint2(pack_bf2(f[0] * wgt, f[LD] * wgt), pack_bf2(f[2 * LD] * wgt, f[3 * LD] * wgt));
+  }
+  for (int idx = tid; idx < D * (D / 4); idx += 256) {
+    const int a = idx / (D / 4), c4 = (idx % (D / 4)) * 4;
+    const float4 t = *reinterpret_cast<const float4*>(Sl + a * LD + c4);
+    *reinterpret_cast<uint2*>(csec + a * PG::LB + c4) = make_uint2(pack_bf2(t.x, t.y), pack_bf2(t.z, t.w));
+  }
+  if (tid < D) {
+    const float e = Sl[tid * LD + D], ehi = bf_lo(pack_bf2(e, 0.f));
+    *reinterpret_cast<uint2*>(csec + tid * PG::LB + D) = make_uint2(pack_bf2(ehi, ehi), pack_bf2(e - ehi, e - ehi));
+  }
+  if (ord1 && tid <= D) reinterpret_cast<float*>(sb + PG::z_off(p2))[tid] = Sl[D * LD + tid];
 }

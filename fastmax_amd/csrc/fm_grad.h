@@ -287,10 +287,11 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 
 // ---------------------------------------------------------------------------------------
 // bf16 variant of grad_kernel (bf16 inputs and outputs): every contraction runs on
-// v_mfma_f32_32x32x8_bf16 with fp32 accumulation.  The state slab keeps its [row][column]
-// layout and is rounded to bf16 while staged (coefficient applied in fp32 first), the token's
-// extended value vector is packed once, so a 32-row tile costs D/8 + 1 MFMAs; the credits are
-// the fp32 register/LDS work of the fp32 kernel.  Streamed tiles are staged as bf16, the first
+// v_mfma_f32_32x32x8_bf16 with fp32 accumulation.  The state arrives in the packed bf16 form
+// (PackedGeo): a column-packed slab ([row][column], unweighted, extra column split into hi + lo
+// parts) is copied to LDS as it is; 2*a2 multiplies the accumulated order-2 credits and a1 the
+// order-1 tile.  The token's extended value vector is packed once, so a 32-row tile costs
+// D/8 + 1 MFMAs; the credits are the fp32 register/LDS work of the fp32 kernel.  Streamed tiles are staged as bf16, the first
 // one in both orientations (rows for the scores, transposed for the product with W).
 // ---------------------------------------------------------------------------------------
 template <int D, int MODE>
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     int64_t yden_stride, const float* __restrict__ cvec, const bf16_t* __restrict__ A1,
     const bf16_t* __restrict__ A2, const float* __restrict__ a2den, int64_t a2den_stride,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
-    const float* __restrict__ state, int nslots, bf16_t* __restrict__ OUT, float* __restrict__ rpart,
+    const float* state, int nslots, bf16_t* __restrict__ OUT, float* __restrict__ rpart,
     int n, int chunk, int masked, int p2, float a1, float a2) {
   using G = Geo<D>;
   using T = bf16_t;
@@ -366,37 +367,31 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
       n_tile = ((cend - 1) >> 5) - tile0 + 1;
     }
   }
-  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
-  const int nsum = masked ? 1 : nslots;
+  // packed state of this block's chunk (masked) or the head's summed state (last slot)
+  using PG = PackedGeo<D>;
+  static_assert(PG::LB == LB && PG::CSL == D * LB, "stage layout = column-packed slab layout");
+  const char* sbase = reinterpret_cast<const char*>(state + ((int64_t)head * nslots + (masked ? c : nslots - 1)) * SS);
+  const uint16_t* csec = reinterpret_cast<const uint16_t*>(sbase + PG::c_off(p2));
 
-  StateSlab<D * LD> slab;
+  // a C slab is copied as it is: 16-byte pieces global -> registers -> LDS
+  // (no branches: threads past the end wrap round and copy an early piece a second time, so that
+  // every load is issued up front and stays in flight under the MFMAs)
+  constexpr int NPC = PG::CSL / 8, NVS = (NPC + 255) / 256;
+  static_assert(NVS <= 3, "three named pieces per thread (an indexed array would live in scratch)");
+  uint4 sv0, sv1, sv2;
   RowTile<D, T, 32> t1, t2;
   float creg = 0.f;
   auto slab_load = [&](int st) {
-    slab.load(sbase + ((p2 && st < NS) ? st * D * LD : rows2 * LD), SS, nsum, D * LD, tid);
+    const uint4* src = reinterpret_cast<const uint4*>(csec + st * PG::CSL);
+    sv0 = src[tid % NPC];
+    if constexpr (NVS > 1) sv1 = src[(tid + 256) % NPC];
+    if constexpr (NVS > 2) sv2 = src[(tid + 512) % NPC];
   };
-  // fp32 [row][LD] -> bf16 [row][LB] (same pitch in elements), coefficient applied first
   auto slab_store = [&](int st) {
-    const float cf = (p2 && st < NS) ? 2.0f * a2 : a1;
-    uint16_t* dst = Sb[st & 1];
-#pragma unroll
-    for (int u = 0; u < decltype(slab)::NV; ++u) {
-      const int idx = tid + u * 256;
-      if (idx < D * LD / 4) {
-        float4 v4 = slab.v[u];
-        if (idx % (LD / 4) == D / 4) {
-          // extra column e and three floats of padding the build never writes: store
-          // (e_hi, e_hi, e_lo, e_lo); with yx as (hi, lo, hi, lo) the extra-column MFMA then forms
-          // yx * e to 16 bits of mantissa -- this term nearly cancels the value columns' sum
-          const float e = v4.x * cf, ehi = bf_lo(pack_bf2(e, 0.f));
-          v4 = make_float4(ehi, ehi, e - ehi, e - ehi);
-          *reinterpret_cast<uint2*>(dst + idx * 4) = make_uint2(pack_bf2(v4.x, v4.y), pack_bf2(v4.z, v4.w));
-        } else {
-          *reinterpret_cast<uint2*>(dst + idx * 4) =
-              make_uint2(pack_bf2(v4.x * cf, v4.y * cf), pack_bf2(v4.z * cf, v4.w * cf));
-        }
-      }
-    }
+    uint4* dst = reinterpret_cast<uint4*>(Sb[st & 1]);
+    dst[tid % NPC] = sv0;
+    if constexpr (NVS > 1) dst[(tid + 256) % NPC] = sv1;
+    if constexpr (NVS > 2) dst[(tid + 512) % NPC] = sv2;
   };
   auto tiles_load = [&](int kk) {
     const int r0 = (tile0 + kk) * 32;
@@ -442,8 +437,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   const float* xtok = Xl + (w * 32 + 4 * hh) * LD;
   auto xat = [&](int r, int col) { return xtok[((r >> 2) * 8 + (r & 3)) * LD + col]; };
 
-  for (int st = 0; st < n_state; ++st) {
-    slab_load(st + 1 < n_state ? st + 1 : st);
+  auto slab_step = [&](int st) {
     const uint16_t* sl = Sb[st & 1];
     f16v tt[AB];
 #pragma unroll
@@ -471,14 +465,30 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
             out[ab][r] += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, v)));
           }
       }
+      if (st == NS - 1) {  // the order-2 slabs are stored raw: f'(s) contributes 2*a2 to their sum
+#pragma unroll
+        for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) out[ab][r] *= 2.0f * a2;
+      }
     } else {
 #pragma unroll
       for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) out[ab][r] += tt[ab][r];
+        for (int r = 0; r < 16; ++r) out[ab][r] += a1 * tt[ab][r];
     }
-    if (st + 1 < n_state) slab_store(st + 1);
-    else if (n_tile > 0) tiles_store((st + 1) & 1);
+  };
+  // the last slab is peeled off so that load and store of the next slab are unconditional in
+  // the loop (a load whose only use sits in a branch is moved there and waited for at once)
+  for (int st = 0; st + 1 < n_state; ++st) {
+    slab_load(st + 1);
+    slab_step(st);
+    slab_store(st + 1);
+    __syncthreads();
+  }
+  if (n_state > 0) {
+    slab_step(n_state - 1);
+    if (n_tile > 0) tiles_store(n_state & 1);
     __syncthreads();
   }
 
