@@ -410,19 +410,45 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     }
   };
 
-  // one slab: B operands are 64-bit reads of [feature group][column][4 features]
+  // one slab: B operands are 64-bit reads of [feature group][column][4 features], fetched one
+  // group ahead of the MFMAs that use them
   auto slab_compute = [&](const uint16_t* sl, auto tag) {
     constexpr bool ORD2 = decltype(tag)::value;
+    constexpr int NB = FWD ? CB + 1 : CB;
     const uint16_t* brow = sl + (hh * (H2 / 4) * NCF + i) * 4;
+    const uint16_t* erow = sl + (hh * (H2 / 4) * NCF + D) * 4;
+    auto fetch = [&](int g4, uint2 (&b)[NB]) {
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) b[cb] = *reinterpret_cast<const uint2*>(brow + (g4 * NCF + cb * 32) * 4);
+      if (FWD) b[NB - 1] = *reinterpret_cast<const uint2*>(erow + g4 * NCF * 4);
+    };
+    auto feat = [&](int g4) {
+      const int t = 4 * g4;
+      return ORD2 ? pack_bf4(Xr[t] * Wn[t], Xr[t + 1] * Wn[t + 1], Xr[t + 2] * Wn[t + 2], Xr[t + 3] * Wn[t + 3])
+                  : pack_bf4(Xr[t] * a1, Xr[t + 1] * a1, Xr[t + 2] * a1, Xr[t + 3] * a1);
+    };
+    uint2 bc[NB], bn[NB];
+    fetch(0, bc);
+    s4v apc = feat(0), apn = apc;
 #pragma unroll
     for (int g4 = 0; g4 < H2 / 4; ++g4) {
-      const int t = 4 * g4;
-      const s4v ap = ORD2 ? pack_bf4(Xr[t] * Wn[t], Xr[t + 1] * Wn[t + 1], Xr[t + 2] * Wn[t + 2], Xr[t + 3] * Wn[t + 3])
-                          : pack_bf4(Xr[t] * a1, Xr[t + 1] * a1, Xr[t + 2] * a1, Xr[t + 3] * a1);
+      if (g4 + 1 < H2 / 4) {
+        fetch(g4 + 1, bn);
+        apn = feat(g4 + 1);
+      }
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb)
-        acc[cb] = FM_MFMA_BF(ap, as_s4v(*reinterpret_cast<const uint2*>(brow + (g4 * NCF + cb * 32) * 4)), acc[cb]);
-      if (FWD) accd = FM_MFMA_BF(ap, as_s4v(*reinterpret_cast<const uint2*>(sl + ((hh * (H2 / 4) + g4) * NCF + D) * 4)), accd);
+      for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA_BF(apc, as_s4v(bc[cb]), acc[cb]);
+      if (FWD) accd = FM_MFMA_BF(apc, as_s4v(bc[NB - 1]), accd);
+      // interleave: each MFMA is followed by one of the next group's LDS reads and two of its VALU ops
+#pragma unroll
+      for (int x = 0; x < NB; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      }
+#pragma unroll
+      for (int x = 0; x < NB; ++x) bc[x] = bn[x];
+      apc = apn;
     }
   };
 

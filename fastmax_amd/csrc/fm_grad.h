@@ -165,6 +165,13 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   // x rows of the 16 tokens this lane holds results for: row w*32 + trow(r,hh), r = 4j+e
   const float* xtok = Xl + (w * 32 + 4 * hh) * LD;
   auto xat = [&](int r, int col) { return xtok[((r >> 2) * 8 + (r & 3)) * LD + col]; };
+  // x of the lane's own channels for the 16 token rows of its accumulator registers (the factor
+  // of the mirrored credit and of the normalisation partial), read once
+  float xown[AB][16];
+#pragma unroll
+  for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) xown[ab][r] = xat(r, ab * 32 + i);
 
   for (int st = 0; st < n_state; ++st) {
     slab_load(st + 1 < n_state ? st + 1 : st);
@@ -188,7 +195,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 #pragma unroll
         for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) tt[ab][r] *= xat(r, ab * 32 + i);
+          for (int r = 0; r < 16; ++r) tt[ab][r] *= xown[ab][r];
         const bool keep = i < 32 - s;                    // source lanes that stay in their block
         const int src = (((i - s) & 31) + 32 * hh) << 2;  // byte index of the source lane
 #pragma unroll
@@ -277,7 +284,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 #pragma unroll
     for (int ab = 0; ab < AB; ++ab) {
       const float g = out[ab][r];
-      rs += g * xat(r, ab * 32 + i);
+      rs += g * xown[ab][r];
       if (tk < n) Oh[(int64_t)tk * D + ab * 32 + i] = from_f32<T>(g * xs);
     }
   }
@@ -436,6 +443,13 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   };
   const float* xtok = Xl + (w * 32 + 4 * hh) * LD;
   auto xat = [&](int r, int col) { return xtok[((r >> 2) * 8 + (r & 3)) * LD + col]; };
+  // x of the lane's own channels for the 16 token rows of its accumulator registers (the factor
+  // of the mirrored credit and of the normalisation partial), read once
+  float xown[AB][16];
+#pragma unroll
+  for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) xown[ab][r] = xat(r, ab * 32 + i);
 
   auto slab_step = [&](int st) {
     const uint16_t* sl = Sb[st & 1];
@@ -454,7 +468,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
 #pragma unroll
         for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) tt[ab][r] *= xat(r, ab * 32 + i);
+          for (int r = 0; r < 16; ++r) tt[ab][r] *= xown[ab][r];
         const bool keep = i < 32 - s;
         const int src = (((i - s) & 31) + 32 * hh) << 2;
 #pragma unroll
@@ -546,7 +560,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
 #pragma unroll
     for (int ab = 0; ab < AB; ++ab) {
       const float g = out[ab][r];
-      rs += g * xat(r, ab * 32 + i);
+      rs += g * xown[ab][r];
       if (tk < n) Oh[(int64_t)tk * D + ab * 32 + i] = from_f32<T>(g * xs);
     }
   }
