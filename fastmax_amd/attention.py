@@ -11,7 +11,8 @@ Differences from the reference, all deliberate:
     does for the reference's PyTorch path (the reference kernels skip that chain rule);
   * CPU tensors with use_custom_gradient=True raise (the reference returns q unchanged,
     example.py:10-12);
-  * bfloat16 inputs are accepted (fp32 arithmetic inside).
+  * bfloat16 inputs are accepted (bf16 matrix instructions, fp32 accumulation);
+  * head dimensions other than 32 and 64 (up to 64) run zero-padded to the next kernel size.
 """
 from __future__ import annotations
 
@@ -35,9 +36,17 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             raise ValueError("q, k, and v should be either 3 or 4 dimensional tensors. "
                              "If 3D: (b*h,n,d), if 4D: (b,h,n,d).")
         shape = q.shape
-        q3 = q.reshape(-1, q.shape[-2], q.shape[-1]).contiguous()
-        k3 = k.reshape(-1, k.shape[-2], k.shape[-1]).contiguous()
-        v3 = v.reshape(-1, v.shape[-2], v.shape[-1]).contiguous()
+        d = q.shape[-1]
+        if d > 64:
+            raise ValueError(f"head dimension {d} is not supported (kernels exist for d <= 64)")
+        pad = (32 if d <= 32 else 64) - d
+        q3 = q.reshape(-1, q.shape[-2], d)
+        k3 = k.reshape(-1, k.shape[-2], d)
+        v3 = v.reshape(-1, v.shape[-2], d)
+        if pad:
+            # zero channels change neither q.k nor the row norms, and give zero output columns
+            q3, k3, v3 = (torch.nn.functional.pad(t, (0, pad)) for t in (q3, k3, v3))
+        q3, k3, v3 = q3.contiguous(), k3.contiguous(), v3.contiguous()
         o, den, scale, arg = ext.forward_ex(q3, k3, v3, bool(mask), bool(normalize), float(temperature),
                                             float(a0), float(a1), float(a2), float(lim), int(p))
         noise = None
@@ -46,11 +55,15 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             if drop_noise is None:
                 raise ValueError("dropout > 0 needs drop_noise (a standard-normal tensor shaped like q)")
             # multiplicative Gaussian noise on the output, fastmax_cuda_forward.cu:271-280
-            noise = 1.0 + float(dropout) * drop_noise.reshape(q3.shape).to(o.dtype)
+            noise = 1.0 + float(dropout) * drop_noise.reshape(q3.shape[0], q3.shape[1], -1).to(o.dtype)
+            if pad:
+                noise = torch.nn.functional.pad(noise, (0, pad), value=1.0)
             out = o * noise
         ctx.save_for_backward(q3, k3, v3, o, den, scale, arg, noise if noise is not None else o.new_empty(0))
         ctx.cfg = (bool(mask), bool(normalize), float(temperature), float(a0), float(a1), float(a2), float(lim), int(p))
-        ctx.kshape, ctx.vshape = k.shape, v.shape
+        ctx.kshape, ctx.vshape, ctx.pad = k.shape, v.shape, pad
+        if pad:
+            out = out[..., :d]
         return out.reshape(shape)
 
     @staticmethod
@@ -58,12 +71,17 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
         ext = _ext.load()
         q3, k3, v3, o, den, scale, arg, noise = ctx.saved_tensors
         mask, normalize, temperature, a0, a1, a2, lim, p = ctx.cfg
-        go = grad_output.reshape(q3.shape)
+        go = grad_output.reshape(q3.shape[0], q3.shape[1], -1)
+        if ctx.pad:
+            go = torch.nn.functional.pad(go, (0, ctx.pad))
         if noise.numel():
             go = go * noise
         go = go.contiguous()
         dq, dk, dv = ext.backward_ex(q3, k3, v3, o, den, go, scale, arg, mask, normalize, temperature,
                                      a0, a1, a2, lim, p)
+        if ctx.pad:
+            d = grad_output.shape[-1]
+            dq, dk, dv = dq[..., :d], dk[..., :d], dv[..., :d]
         return (dq.reshape(grad_output.shape), dk.reshape(ctx.kshape), dv.reshape(ctx.vshape),
                 None, None, None, None, None, None, None, None, None, None)
 

@@ -59,6 +59,7 @@ struct ScopedKernel {
   }
 };
 
+constexpr int kChunkP1 = 128;    // p = 1
 constexpr int kChunk = 256;      // tokens between causal state snapshots (fp32 arithmetic)
 constexpr int kChunkBf16 = 512;  // ... when the contractions run on the bf16 matrix instruction: the
                                  // moment work is ~8x cheaper there, so snapshot traffic is worth
@@ -105,7 +106,9 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   }
   pl.gsplit = splits(pl.rtw);
   pl.nblk = (pl.n + 127) / 128;
-  pl.chunk = ds->dtype == FASTMAX_BF16 ? kChunkBf16 : kChunk;
+  // p = 1: a state is only (d+1) rows, so a snapshot per 128-token block is cheaper than a longer
+  // intra-chunk part
+  pl.chunk = !pl.p2 ? kChunkP1 : ds->dtype == FASTMAX_BF16 ? kChunkBf16 : kChunk;
   if (pl.masked) {
     pl.nslots = (pl.n + pl.chunk - 1) / pl.chunk;
     pl.nparts = 1;

@@ -238,6 +238,27 @@ def test_module_autograd_4d(built):
     assert_close("unmasked", o3.reshape(shape), O.dense_truth(q, k, v, None, mask=False, normalize=True)[0], 1e-4)
 
 
+@pytest.mark.parametrize("shape,mask", [((2, 2, 3, 2), True), ((2, 2, 3, 2), False), ((1, 3, 200, 16), True),
+                                         ((2, 2, 150, 48), True), ((1, 2, 90, 20), False)])
+def test_module_other_head_dims(built, shape, mask):
+    """Head dims below 64 other than 32 run zero-padded; (2,2,3,2) is the reference's demo shape
+    (example.py:227-230)."""
+    from fastmax_amd import FASTMultiHeadAttention
+
+    q, k, v, go = O.seeded_inputs(shape, seed=24)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = FASTMultiHeadAttention()(qd, kd, vd, None, mask, 0.0, True)
+    assert o.shape == shape
+    o.backward(go.cuda())
+    ro, rdq, rdk, rdv = O.dense_truth(q, k, v, go, mask=mask, normalize=True)
+    for name, got, ref in (("o", o, ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+        assert got.shape == ref.shape
+        assert_close(name, got, ref, 1e-4, atol=1e-6)
+    with pytest.raises(ValueError, match="head dimension"):
+        FASTMultiHeadAttention()(torch.zeros(1, 1, 4, 128, device="cuda"), torch.zeros(1, 1, 4, 128, device="cuda"),
+                                 torch.zeros(1, 1, 4, 128, device="cuda"))
+
+
 def test_module_output_noise_dropout(built):
     from fastmax_amd import FASTMultiHeadAttention
 
