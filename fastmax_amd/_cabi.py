@@ -25,6 +25,7 @@ EXPORTS = (
     "fastmax_version", "fastmax_last_error", "fastmax_check_desc", "fastmax_workspace_bytes",
     "fastmax_workspace_min_bytes", "fastmax_forward", "fastmax_backward", "fastmax_normalize_inplace",
     "fastmax_profile_begin", "fastmax_profile_end",
+    "fastmax_state_bytes", "fastmax_decode_workspace_bytes", "fastmax_state_update", "fastmax_decode_step",
 )
 
 KERNEL_NAMES = ("rowstat", "build", "fwd_apply", "bwd_prep", "bwd_dq", "bwd_dk", "bwd_dv", "norm_fix")
@@ -79,6 +80,14 @@ def load() -> C.CDLL:
     lib.fastmax_backward.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, sz, vp]
     lib.fastmax_normalize_inplace.restype = C.c_int
     lib.fastmax_normalize_inplace.argtypes = [dp, vp, vp, vp, sz, vp]
+    lib.fastmax_state_bytes.restype = sz
+    lib.fastmax_state_bytes.argtypes = [dp]
+    lib.fastmax_decode_workspace_bytes.restype = sz
+    lib.fastmax_decode_workspace_bytes.argtypes = [dp]
+    lib.fastmax_state_update.restype = C.c_int
+    lib.fastmax_state_update.argtypes = [dp, vp, vp, vp, vp, C.c_int, vp, sz, vp]
+    lib.fastmax_decode_step.restype = C.c_int
+    lib.fastmax_decode_step.argtypes = [dp, vp, vp, vp, vp, vp, vp, vp, i64, vp, i64, vp, sz, vp]
     lib.fastmax_profile_begin.restype = C.c_int
     lib.fastmax_profile_begin.argtypes = []
     lib.fastmax_profile_end.restype = C.c_int

@@ -10,6 +10,7 @@
 #include "fastmax_amd.h"
 #include "fm_apply.h"
 #include "fm_backward.h"
+#include "fm_decode.h"
 #include "fm_forward.h"
 #include "fm_grad.h"
 
@@ -93,7 +94,8 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   pl.n = ds->nq;
   pl.bh = ds->bh;
   const int rt_total = (pl.p2 ? (pl.d / 2 + 1) * (pl.d / 32) : 0) + pl.d / 32;
-  auto splits = [&](int rtw) { return (rt_total + 4 * rtw - 1) / (4 * rtw); };
+  // (p = 1, d = 64: the four waves of a block share its two row tiles, one column tile each)
+  auto splits = [&](int rtw) { return !pl.p2 && pl.d == 64 ? 1 : (rt_total + 4 * rtw - 1) / (4 * rtw); };
   if (!pl.p2) {
     pl.rtw = 1;
   } else if (pl.d == 64) {
@@ -380,6 +382,46 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
   return FASTMAX_OK;
 }
 
+constexpr int kDecodeSplits = 8;  // blocks per head in a decode step (row slices of the state)
+
+size_t decode_ws_bytes(const fastmax_desc* ds) {
+  return align256((size_t)ds->bh * kDecodeSplits * (ds->d + 4) * sizeof(float));
+}
+
+template <int D, class T>
+int state_update_impl(const fastmax_desc* ds, const Plan& pl, const T* k, const T* v, const float* kscale,
+                      float* state, int accumulate, char* ws, size_t ws_bytes, hipStream_t stream) {
+  const int bh = pl.bh, n = pl.n;
+  float* scale = reinterpret_cast<float*>(ws);
+  int* arg = reinterpret_cast<int*>(ws + align256((size_t)2 * bh * sizeof(float)));
+  float* slots = reinterpret_cast<float*>(ws + pl.fixed_bytes);
+  const int hb = heads_per_batch(pl, ws_bytes);
+  if (!kscale) {
+    fill_scale_kernel<<<(bh + 255) / 256, 256, 0, stream>>>(scale + bh, arg + bh, bh, 1.0f / ds->temperature);
+    kscale = scale + bh;
+  }
+  const int64_t ss = pl.state_floats;
+  for (int h0 = 0; h0 < bh; h0 += hb) {
+    const int heads = bh - h0 < hb ? bh - h0 : hb;
+    const int64_t off = (int64_t)h0 * n * D;
+    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, kscale + h0, nullptr, 0, nullptr, slots, 0, 0, stream)));
+    state_accumulate_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads), 256, 0, stream>>>(
+        state + (int64_t)h0 * ss, slots, pl.nslots, pl.nparts, ss, accumulate);
+  }
+  return launch_status("state_accumulate_kernel");
+}
+
+template <int D, class T>
+int decode_impl(const fastmax_desc* ds, const T* q, const T* k, const T* v, const float* qscale,
+                const float* kscale, float* state, T* o, int64_t ldo, float* den, int64_t den_stride,
+                float* part, hipStream_t stream) {
+  const int p2 = ds->p == 2;
+  decode_update_kernel<D, T><<<dim3(kDecodeSplits, ds->bh), 256, 0, stream>>>(
+      q, k, v, qscale, kscale, 1.0f / ds->temperature, state, part, p2, ds->a0, ds->a1, p2 ? ds->a2 : 0.f);
+  decode_finish_kernel<D, T><<<ds->bh, D + 4, 0, stream>>>(part, kDecodeSplits, o, ldo, den, den_stride);
+  return launch_status("decode kernels");
+}
+
 }  // namespace
 
 extern "C" {
@@ -518,6 +560,71 @@ int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k, void* 
     scale_rows_kernel<bf16_t><<<grid, 256, 0, st>>>((bf16_t*)k, scale + bh, per_head);
   }
   return launch_status("scale_rows_kernel");
+}
+
+size_t fastmax_state_bytes(const fastmax_desc* desc) {
+  g_err[0] = 0;
+  if (check_desc(desc) != FASTMAX_OK) return 0;
+  return (size_t)state_floats_for(desc->d, desc->p == 2) * sizeof(float);
+}
+
+size_t fastmax_decode_workspace_bytes(const fastmax_desc* desc) {
+  g_err[0] = 0;
+  if (check_desc(desc) != FASTMAX_OK) return 0;
+  return decode_ws_bytes(desc);
+}
+
+int fastmax_state_update(const fastmax_desc* desc, const void* k, const void* v, const float* k_scale,
+                         void* state, int accumulate, void* workspace, size_t workspace_bytes,
+                         fastmax_stream_t stream) {
+  g_err[0] = 0;
+  FM_TRY(check_desc(desc));
+  if (!k || !v || !state) return fail(FASTMAX_E_NULL, "k, v and state must be non-NULL");
+  if (desc->normalize && !k_scale)
+    return fail(FASTMAX_E_NULL, "normalize is set: k_scale (the factor a forward pass reported) is required");
+  fastmax_desc d2 = *desc;
+  d2.mask = 0;
+  const Plan pl = make_plan(&d2, FASTMAX_PASS_FORWARD);
+  FM_TRY(check_ws(pl, workspace, workspace_bytes));
+  char* ws = static_cast<char*>(workspace);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+#define FM_UPD(DD, TT)                                                                            \
+  return state_update_impl<DD, TT>(&d2, pl, (const TT*)k, (const TT*)v, k_scale, (float*)state, \
+                                   accumulate, ws, workspace_bytes, st)
+  if (desc->dtype == FASTMAX_F32) {
+    if (desc->d == 64) FM_UPD(64, float);
+    FM_UPD(32, float);
+  }
+  if (desc->d == 64) FM_UPD(64, bf16_t);
+  FM_UPD(32, bf16_t);
+#undef FM_UPD
+}
+
+int fastmax_decode_step(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                        const float* q_scale, const float* k_scale, void* state, void* o, int64_t ldo,
+                        float* den, int64_t den_stride, void* workspace, size_t workspace_bytes,
+                        fastmax_stream_t stream) {
+  g_err[0] = 0;
+  FM_TRY(check_desc(desc));
+  if (!q || !k || !v || !state || !o) return fail(FASTMAX_E_NULL, "q, k, v, state and o must be non-NULL");
+  if (desc->nq != 1) return fail(FASTMAX_E_SHAPE, "a decode step takes one token per head (nq = nk = 1), got nq = %d", desc->nq);
+  if (desc->normalize && (!q_scale || !k_scale))
+    return fail(FASTMAX_E_NULL, "normalize is set: q_scale and k_scale (the factors a forward pass reported) are required");
+  if (ldo < desc->d) return fail(FASTMAX_E_PARAM, "ldo = %lld < d = %d", (long long)ldo, desc->d);
+  if (den && den_stride < 1) return fail(FASTMAX_E_PARAM, "den_stride = %lld < 1", (long long)den_stride);
+  if (!workspace || (((uintptr_t)workspace) & 255) || workspace_bytes < decode_ws_bytes(desc))
+    return fail(FASTMAX_E_WORKSPACE, "workspace must be 256-byte aligned and hold %zu bytes", decode_ws_bytes(desc));
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+#define FM_DEC(DD, TT)                                                                              \
+  return decode_impl<DD, TT>(desc, (const TT*)q, (const TT*)k, (const TT*)v, q_scale, k_scale,     \
+                             (float*)state, (TT*)o, ldo, den, den_stride, (float*)workspace, st)
+  if (desc->dtype == FASTMAX_F32) {
+    if (desc->d == 64) FM_DEC(64, float);
+    FM_DEC(32, float);
+  }
+  if (desc->d == 64) FM_DEC(64, bf16_t);
+  FM_DEC(32, bf16_t);
+#undef FM_DEC
 }
 
 }  // extern "C"

@@ -110,7 +110,11 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   constexpr int TS = 32;        // tokens per pipeline step
   constexpr int TP = TS + 4;    // pitch of the transposed tiles: 16-byte aligned rows, and the
                                 // 8 lanes of a 128-bit LDS access phase fall in distinct banks
-  constexpr int CB = G::CB, LD = G::LD;
+  constexpr int LD = G::LD;
+  // RTW == 1 is the p = 1 configuration: a head has only D/32 row tiles, so for D = 64 the four
+  // waves split the 2 x 2 (row tile, column tile) grid instead of leaving two waves without work
+  constexpr bool CSPLIT = RTW == 1 && G::CB == 2;
+  constexpr int CB = CSPLIT ? 1 : G::CB;  // column tiles per wave
   // X and Y tiles are staged TRANSPOSED ([channel][token]) so that the four tokens a lane feeds
   // into four consecutive MFMAs come from one 128-bit LDS read.  Row D of the X tile is 1 for
   // real tokens and 0 for padding: order-1 features are x[a] * 1.
@@ -137,7 +141,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   int nx = 0;  // row tiles this wave really owns (wave-uniform)
 #pragma unroll
   for (int x = 0; x < RTW; ++x) {
-    const int rt = (g * 4 + w) * RTW + x;
+    const int rt = CSPLIT ? g * 2 + (w & 1) : (g * 4 + w) * RTW + x;
     ownoff[x] = rotoff[x] = 4 * hh;
     rowbase[x] = 0;
     if (rt < rt_total) {
@@ -155,9 +159,10 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       }
     }
   }
+  const int cbase = CSPLIT ? w >> 1 : 0;  // first column tile of this wave
   int voff[CB];
 #pragma unroll
-  for (int cb = 0; cb < CB; ++cb) voff[cb] = (cb * 32 + i) * (BF ? TPB : TP) + 4 * hh;
+  for (int cb = 0; cb < CB; ++cb) voff[cb] = ((cbase + cb) * 32 + i) * (BF ? TPB : TP) + 4 * hh;
 
   f16v acc[RTW][CB];
   float dacc[RTW];
@@ -266,7 +271,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     }
   };
   // lane part of a snapshot address: row 4*hh (+ 8j + e per register), column i (+ 32*cb)
-  const unsigned lane_off = (unsigned)(4 * hh * LD + i);
+  const unsigned lane_off = (unsigned)(4 * hh * LD + cbase * 32 + i);
   auto snapshot = [&](int slot) {
     float* st = state + ((int64_t)head * nslots + slot) * SS;  // uniform: scalar base + 32-bit lane offsets
 #pragma unroll
@@ -282,7 +287,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
             for (int cb = 0; cb < CB; ++cb) sx[oj + (unsigned)(e * LD + cb * 32)] = acc[x][cb][4 * j + e];
         }
         const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
-        if (hh == 0) sx[(unsigned)(i * LD + D)] = ds;
+        if (hh == 0 && cbase == 0) sx[(unsigned)(i * LD + D)] = ds;
       }
     }
     if (g == 0 && tid <= D) st[(unsigned)((rows2 + D) * LD + tid)] = s0;
@@ -304,7 +309,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
         if (sections & 1) {
           const float wgt = dbl ? 2.0f : 1.0f;
           uint16_t* fx = fsec + (unsigned)(slab * PG::FSL + (arow >> 2) * PG::NCF * 4);
-          const unsigned lo = (unsigned)((hh * PG::NCF + i) * 4);
+          const unsigned lo = (unsigned)((hh * PG::NCF + cbase * 32 + i) * 4);
 #pragma unroll
           for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -313,11 +318,11 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
               *reinterpret_cast<uint2*>(fx + lo + (unsigned)((2 * j * PG::NCF + cb * 32) * 4)) =
                   make_uint2(pack_bf2(a[4 * j] * wgt, a[4 * j + 1] * wgt), pack_bf2(a[4 * j + 2] * wgt, a[4 * j + 3] * wgt));
             }
-          if (hh == 0) fx[(unsigned)(((i >> 2) * PG::NCF + D) * 4 + (i & 3))] = (uint16_t)pack_bf2(ds * wgt, 0.f);
+          if (hh == 0 && cbase == 0) fx[(unsigned)(((i >> 2) * PG::NCF + D) * 4 + (i & 3))] = (uint16_t)pack_bf2(ds * wgt, 0.f);
         }
         if (sections & 2) {
           uint16_t* cx = csec + (unsigned)(slab * PG::CSL + arow * PG::LB);
-          const unsigned lo = (unsigned)(4 * hh * PG::LB + i);
+          const unsigned lo = (unsigned)(4 * hh * PG::LB + cbase * 32 + i);
 #pragma unroll
           for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -328,7 +333,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
                 cx[lo + (unsigned)((8 * j + e) * PG::LB + cb * 32)] = (uint16_t)u;
                 cx[lo + (unsigned)((8 * j + e + 1) * PG::LB + cb * 32)] = (uint16_t)(u >> 16);
               }
-          if (hh == 0) {
+          if (hh == 0 && cbase == 0) {
             const float ehi = bf_lo(pack_bf2(ds, 0.f));
             *reinterpret_cast<uint2*>(cx + (unsigned)(i * PG::LB + D)) =
                 make_uint2(pack_bf2(ehi, ehi), pack_bf2(ds - ehi, ds - ehi));

@@ -125,3 +125,58 @@ def normalize_inplace(q, k, *, lim=1.0):
         stream = torch.cuda.current_stream(q.device).cuda_stream
         _cabi.check(lib.fastmax_normalize_inplace(C.byref(ds), q.data_ptr(), k.data_ptr(), ws.data_ptr(),
                                                   nbytes, stream))
+
+
+def new_state(bh: int, d: int, *, p=2, dtype=torch.float32, device="cuda") -> torch.Tensor:
+    """A zeroed recurrent state for bh heads (fp32 whatever the input dtype): the moment state
+    that stands in for a key/value cache.  Its layout is private to the library."""
+    lib = _cabi.load()
+    ds = _cabi.make_desc(bh, 1, d, _cabi.FASTMAX_BF16 if dtype == torch.bfloat16 else _cabi.FASTMAX_F32,
+                         False, False, p)
+    nbytes = lib.fastmax_state_bytes(C.byref(ds))
+    if nbytes == 0:
+        raise _cabi.FastmaxError(-2, _cabi.last_error())
+    return torch.zeros((bh, nbytes // 4), dtype=torch.float32, device=device)
+
+
+def state_update(state, k, v, *, k_scale: Optional[torch.Tensor] = None, accumulate=True, normalize=False,
+                 lim=1.0, temperature=1.0, a0=1.0, a1=1.0, a2=0.5, p=2) -> None:
+    """state (+)= sum over the tokens of k, v (bh, n, d).  With normalize, k_scale is the k half
+    of the qk_scale a forward pass over the prompt returned."""
+    _check_inputs(k, v)
+    lib = _cabi.load()
+    ds = _desc(k, k, False, normalize, p, lim, temperature, a0, a1, a2)
+    with torch.cuda.device(k.device):
+        nbytes = lib.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD)
+        if nbytes == 0:
+            raise _cabi.FastmaxError(-2, _cabi.last_error())
+        ws = _workspace(k.device, nbytes, 0)
+        stream = torch.cuda.current_stream(k.device).cuda_stream
+        _cabi.check(lib.fastmax_state_update(
+            C.byref(ds), k.data_ptr(), v.data_ptr(), k_scale.data_ptr() if k_scale is not None else None,
+            state.data_ptr(), int(bool(accumulate)), ws.data_ptr(), nbytes, stream))
+
+
+def decode_step(state, q, k, v, *, q_scale: Optional[torch.Tensor] = None,
+                k_scale: Optional[torch.Tensor] = None, normalize=False, lim=1.0, temperature=1.0,
+                a0=1.0, a1=1.0, a2=0.5, p=2):
+    """One new token per head, q, k, v (bh, 1, d): the state takes in (k, v) and the token's causal
+    output row comes back as (o, den)."""
+    _check_inputs(q, k, v)
+    lib = _cabi.load()
+    bh, n, d = q.shape
+    ds = _desc(q, k, True, normalize, p, lim, temperature, a0, a1, a2)
+    with torch.cuda.device(q.device):
+        nbytes = lib.fastmax_decode_workspace_bytes(C.byref(ds))
+        if nbytes == 0:
+            raise _cabi.FastmaxError(-2, _cabi.last_error())
+        ws = _workspace(q.device, nbytes, 3)
+        o = torch.empty_like(q)
+        den = torch.empty((bh, 1), dtype=torch.float32, device=q.device)
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        _cabi.check(lib.fastmax_decode_step(
+            C.byref(ds), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            q_scale.data_ptr() if q_scale is not None else None,
+            k_scale.data_ptr() if k_scale is not None else None, state.data_ptr(), o.data_ptr(), d,
+            den.data_ptr(), 1, ws.data_ptr(), nbytes, stream))
+    return o, den

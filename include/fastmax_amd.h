@@ -50,7 +50,7 @@ typedef struct fastmax_desc {
   int32_t nq;          /* query tokens                                                   */
   int32_t nk;          /* key tokens; must equal nq                                      */
   int32_t d;           /* head dimension: 32 or 64                                        */
-  int32_t dtype;       /* FASTMAX_F32 or FASTMAX_BF16 (bf16 in/out, fp32 arithmetic)     */
+  int32_t dtype;       /* FASTMAX_F32 or FASTMAX_BF16 (bf16 in/out, fp32 accumulation)    */
   int32_t mask;        /* 0: every key visible, 1: causal (j <= i)                       */
   int32_t normalize;   /* 1: x <- lim * x / max_n ||x_n||_2 per head for q and k,
                           differentiated through (example.py:101-108)                    */
@@ -113,6 +113,33 @@ int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, con
  * forwardpass binding uses it.  workspace: >= 16*bh bytes. */
 int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k,
                               void* workspace, size_t workspace_bytes, fastmax_stream_t stream);
+
+/* Recurrent form: the moment state S = sum_j phi(k_j) (x) [v_j, 1] of a head is kept by the
+ * caller between calls and plays the part of the key/value cache (reference model.py:828-852,
+ * which caches k and v because its attention is recomputed from them).  The reference has
+ * no such kernel; the arithmetic is the running state of its causal loop
+ * (fastmax_cuda_forward.cu:102-197).  A state is fastmax_state_bytes(desc) bytes of fp32 per
+ * head, heads contiguous; its layout is private to the library.  The normalisation by the
+ * maximum row norm is not causal, so with normalize != 0 the caller passes the per-head
+ * factors (bh floats each, device memory) that a forward pass over the prompt reported in
+ * qk_scale (q factors first, then k factors); with normalize == 0 they may be NULL (q: 1,
+ * k: 1/temperature).  mask is ignored by these calls.
+ *
+ * fastmax_state_update: state (+)= the sum over desc->nk tokens of k, v (bh, nk, d); with
+ *   accumulate == 0 the state is overwritten.  workspace: as fastmax_forward for the same
+ *   descriptor with mask = 0.
+ * fastmax_decode_step: one new token per head (desc->nq = desc->nk = 1; q, k, v are (bh, 1, d)):
+ *   the state takes in (k, v), then o = phi(q).S / den -- the causal output row of that token.
+ *   den may be NULL.  workspace: fastmax_decode_workspace_bytes(desc), 256-byte aligned. */
+size_t fastmax_state_bytes(const fastmax_desc* desc);
+size_t fastmax_decode_workspace_bytes(const fastmax_desc* desc);
+int fastmax_state_update(const fastmax_desc* desc, const void* k, const void* v, const float* k_scale,
+                         void* state, int accumulate, void* workspace, size_t workspace_bytes,
+                         fastmax_stream_t stream);
+int fastmax_decode_step(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                        const float* q_scale, const float* k_scale, void* state, void* o, int64_t ldo,
+                        float* den, int64_t den_stride, void* workspace, size_t workspace_bytes,
+                        fastmax_stream_t stream);
 
 /* Kernel timing aid (no counterpart in the reference, which only wall-clocks whole calls,
  * test_fastmax.py:351-356).  Between begin and end every kernel the calling thread launches
