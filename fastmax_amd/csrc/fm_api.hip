@@ -69,6 +69,7 @@ constexpr size_t kWorkspaceBudget = 16ull << 30;   // what fastmax_workspace_byt
 
 struct Plan {
   int d, p2, masked, n, bh;
+  int bhkv, ratio;     // key/value heads; query heads per key/value head
   int rtw, gsplit;     // build kernel: row tiles per wave, feature splits per head
   int nslots, zlen;    // state slots per head; tokens per slot when unmasked
   int nparts;          // token splits the unmasked build sums separately (1 when masked); bf16
@@ -93,6 +94,8 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   pl.masked = ds->mask != 0;
   pl.n = ds->nq;
   pl.bh = ds->bh;
+  pl.bhkv = ds->bhkv;
+  pl.ratio = ds->bh / ds->bhkv;
   const int rt_total = (pl.p2 ? (pl.d / 2 + 1) * (pl.d / 32) : 0) + pl.d / 32;
   // (p = 1, d = 64: the four waves of a block share its two row tiles, one column tile each)
   auto splits = [&](int rtw) { return !pl.p2 && pl.d == 64 ? 1 : (rt_total + 4 * rtw - 1) / (4 * rtw); };
@@ -136,6 +139,9 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   pl.fixed_bytes = fixed;
   pl.per_head_bytes = (size_t)pl.nslots * pl.state_floats * sizeof(float) *
                       (pass == FASTMAX_PASS_BACKWARD ? 2 : 1);
+  // grouped key/value heads, backward: dk and dv are formed per query head and then added up
+  if (pass == FASTMAX_PASS_BACKWARD && pl.ratio > 1)
+    pl.per_head_bytes += 2 * (size_t)pl.n * pl.d * (ds->dtype == FASTMAX_BF16 ? 2 : 4);
   return pl;
 }
 
@@ -151,6 +157,7 @@ int heads_per_batch(const Plan& pl, size_t ws_bytes) {
     m /= 2;
   }
   if (hb >= (size_t)m) hb = hb / m * m;
+  hb = hb / pl.ratio * pl.ratio;  // whole key/value groups
   return (int)hb;
 }
 
@@ -160,8 +167,8 @@ int check_desc(const fastmax_desc* ds) {
     return fail(FASTMAX_E_DTYPE, "dtype %d is neither FASTMAX_F32 nor FASTMAX_BF16", ds->dtype);
   if (ds->d != 32 && ds->d != 64) return fail(FASTMAX_E_SHAPE, "d = %d; supported head dims are 32 and 64", ds->d);
   if (ds->bh < 1 || ds->bh > 65535) return fail(FASTMAX_E_SHAPE, "bh = %d outside [1, 65535]", ds->bh);
-  if (ds->bhkv != ds->bh)
-    return fail(FASTMAX_E_SHAPE, "bhkv = %d != bh = %d: grouped key/value heads are not supported", ds->bhkv, ds->bh);
+  if (ds->bhkv < 1 || ds->bh % ds->bhkv != 0)
+    return fail(FASTMAX_E_SHAPE, "bhkv = %d does not divide bh = %d", ds->bhkv, ds->bh);
   if (ds->nq < 1) return fail(FASTMAX_E_SHAPE, "nq = %d < 1", ds->nq);
   if (ds->nk != ds->nq) return fail(FASTMAX_E_SHAPE, "nk = %d != nq = %d: a key prefix is not supported", ds->nk, ds->nq);
   if ((int64_t)ds->nq * ds->d * ds->bh >= (int64_t)1 << 40) return fail(FASTMAX_E_SHAPE, "tensor too large");
@@ -177,7 +184,7 @@ int check_desc(const fastmax_desc* ds) {
 int check_ws(const Plan& pl, void* ws, size_t ws_bytes) {
   if (!ws) return fail(FASTMAX_E_WORKSPACE, "workspace is NULL");
   if (((uintptr_t)ws) & 255) return fail(FASTMAX_E_WORKSPACE, "workspace is not 256-byte aligned");
-  const size_t need = pl.fixed_bytes + pl.per_head_bytes;
+  const size_t need = pl.fixed_bytes + pl.ratio * pl.per_head_bytes;
   if (ws_bytes < need)
     return fail(FASTMAX_E_WORKSPACE, "workspace of %zu bytes is below the minimum of %zu", ws_bytes, need);
   return FASTMAX_OK;
@@ -199,14 +206,14 @@ int launch_status(const char* what) {
 template <class T>
 int compute_scales(const fastmax_desc* ds, const T* q, const T* k, float* scale, int* arg,
                    hipStream_t stream) {
-  const int bh = ds->bh;
+  const int bh = ds->bh, bhkv = ds->bhkv;
   ScopedKernel sk(FASTMAX_K_ROWSTAT, stream);
   if (ds->normalize) {
     rowstat_kernel<T><<<bh, 256, 0, stream>>>(q, ds->nq, ds->d, ds->lim, scale, arg);
-    rowstat_kernel<T><<<bh, 256, 0, stream>>>(k, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
+    rowstat_kernel<T><<<bhkv, 256, 0, stream>>>(k, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
   } else {
     fill_scale_kernel<<<(bh + 255) / 256, 256, 0, stream>>>(scale, arg, bh, 1.0f);
-    fill_scale_kernel<<<(bh + 255) / 256, 256, 0, stream>>>(scale + bh, arg + bh, bh, 1.0f / ds->temperature);
+    fill_scale_kernel<<<(bhkv + 255) / 256, 256, 0, stream>>>(scale + bh, arg + bh, bhkv, 1.0f / ds->temperature);
   }
   return launch_status("scale kernels");
 }
@@ -263,23 +270,27 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   if (scale_out) hipMemcpyAsync(scale_out, scale, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);
   if (arg_out) hipMemcpyAsync(arg_out, arg, (size_t)2 * bh * sizeof(int), hipMemcpyDeviceToDevice, stream);
 
+  const int ratio = pl.ratio;
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
-    const int64_t off = (int64_t)h0 * n * D;
-    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, state, 0, 1, stream)));
+    const int64_t off = (int64_t)h0 * n * D;             // query-head tensors
+    const int kv0 = h0 / ratio;                          // first key/value head of the batch
+    const int64_t koff = (int64_t)kv0 * n * D;
+    FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr,
+                               state, 0, 1, stream)));
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       const dim3 agrid(pl.nblk, heads);
       if constexpr (kBf16Mfma<T>) {
         apply_kernel_bf<D, 0><<<agrid, 256, 0, stream>>>(
-            q + off, k + off, v + off, scale + h0, scale + bh + h0, nullptr, 0, state, pl.nslots,
+            q + off, k + koff, v + koff, scale + h0, scale + bh + kv0, nullptr, 0, state, pl.nslots,
             o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, pl.chunk,
-            pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
+            pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f, 1, ratio);
       } else {
         apply_kernel<D, T, 0><<<agrid, 256, 0, stream>>>(
-            q + off, k + off, v + off, scale + h0, scale + bh + h0, nullptr, 0, state, pl.nslots,
+            q + off, k + koff, v + koff, scale + h0, scale + bh + kv0, nullptr, 0, state, pl.nslots,
             o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, pl.chunk,
-            pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f);
+            pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f, 1, ratio);
       }
     }
     FM_TRY(launch_status("fwd_apply_kernel"));
@@ -318,29 +329,42 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     FM_TRY(launch_status("bwd_prep_kernel"));
   }
   const float a2 = pl.p2 ? ds->a2 : 0.f;
+  const int ratio = pl.ratio, bhkv = pl.bhkv;
+  const int64_t state_bytes = (int64_t)pl.nslots * pl.state_floats * sizeof(float);
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
-    const int64_t off = (int64_t)h0 * n * D;
+    const int64_t off = (int64_t)h0 * n * D;   // query-head tensors
+    const int kv0 = h0 / ratio;                // first key/value head of the batch
+    const int64_t koff = (int64_t)kv0 * n * D;
     float* stS = state;
     float* stR = state + (int64_t)hb * pl.nslots * pl.state_floats;
+    // grouped key/value heads: dk and dv per query head, added up over each group afterwards
+    T* dk_q = dk + off;
+    T* dv_q = dv + off;
+    if (ratio > 1) {
+      char* tmp = reinterpret_cast<char*>(state) + 2 * hb * state_bytes;
+      dk_q = reinterpret_cast<T*>(tmp);
+      dv_q = dk_q + (int64_t)hb * n * D;
+    }
     const float* denh = den + (int64_t)h0 * n * den_stride;
     const float* ch = cvec + (int64_t)h0 * n;
-    // prefix state of (kh, v, 1) and suffix state of (qh, go/den, c)
-    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, scale + bh + h0, nullptr, 0, nullptr, stS, 0, 2, stream)));
+    // prefix state of (kh, v, 1) per key/value head and suffix state of (qh, go/den, c) per query head
+    FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, stS, 0,
+                               2, stream)));
     FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, 3, stream)));
     const dim3 grid(pl.nblk, heads);
     {
       ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
       if constexpr (kBf16Mfma<T>) {
         grad_kernel_bf<D, 0><<<grid, 256, 0, stream>>>(
-            q + off, go + off, denh, den_stride, ch, k + off, v + off, nullptr, 0, scale + h0,
-            scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, pl.chunk, pl.masked,
-            pl.p2, ds->a1, a2);
+            q + off, go + off, denh, den_stride, ch, k + koff, v + koff, nullptr, 0, scale + h0,
+            scale + bh + kv0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, pl.chunk,
+            pl.masked, pl.p2, ds->a1, a2, 1, ratio);
       } else {
         grad_kernel<D, T, 0><<<grid, 256, 0, stream>>>(
-            q + off, go + off, denh, den_stride, ch, k + off, v + off, nullptr, 0, scale + h0,
-            scale + bh + h0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, pl.chunk, pl.masked,
-            pl.p2, ds->a1, a2);
+            q + off, go + off, denh, den_stride, ch, k + koff, v + koff, nullptr, 0, scale + h0,
+            scale + bh + kv0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, pl.chunk,
+            pl.masked, pl.p2, ds->a1, a2, 1, ratio);
       }
     }
     FM_TRY(launch_status("grad_kernel (dq)"));
@@ -348,14 +372,14 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
       if constexpr (kBf16Mfma<T>) {
         grad_kernel_bf<D, 1><<<grid, 256, 0, stream>>>(
-            k + off, v + off, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + h0,
-            scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, pl.chunk,
-            pl.masked, pl.p2, ds->a1, a2);
+            k + koff, v + koff, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + kv0,
+            scale + h0, stR, pl.nslots, dk_q, rpart + (int64_t)(bh + h0) * pl.nblk, n, pl.chunk,
+            pl.masked, pl.p2, ds->a1, a2, ratio, 1);
       } else {
         grad_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
-            k + off, v + off, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + h0,
-            scale + h0, stR, pl.nslots, dk + off, rpart + (int64_t)(bh + h0) * pl.nblk, n, pl.chunk,
-            pl.masked, pl.p2, ds->a1, a2);
+            k + koff, v + koff, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + kv0,
+            scale + h0, stR, pl.nslots, dk_q, rpart + (int64_t)(bh + h0) * pl.nblk, n, pl.chunk,
+            pl.masked, pl.p2, ds->a1, a2, ratio, 1);
       }
     }
     FM_TRY(launch_status("grad_kernel (dk)"));
@@ -363,20 +387,28 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       ScopedKernel sk(FASTMAX_K_BWD_DV, stream);
       if constexpr (kBf16Mfma<T>) {
         apply_kernel_bf<D, 1><<<grid, 256, 0, stream>>>(
-            k + off, q + off, go + off, scale + bh + h0, scale + h0, denh, den_stride, stR, pl.nslots,
-            dv + off, D, nullptr, 0, n, pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
+            k + koff, q + off, go + off, scale + bh + kv0, scale + h0, denh, den_stride, stR, pl.nslots,
+            dv_q, D, nullptr, 0, n, pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2, ratio, 1);
       } else {
         apply_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
-            k + off, q + off, go + off, scale + bh + h0, scale + h0, denh, den_stride, stR, pl.nslots,
-            dv + off, D, nullptr, 0, n, pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2);
+            k + koff, q + off, go + off, scale + bh + kv0, scale + h0, denh, den_stride, stR, pl.nslots,
+            dv_q, D, nullptr, 0, n, pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2, ratio, 1);
       }
     }
     FM_TRY(launch_status("apply_kernel (dv)"));
+    if (ratio > 1) {
+      const int64_t per_head = (int64_t)n * D;
+      const dim3 sgrid((unsigned)((per_head / 4 + 255) / 256), heads / ratio);
+      group_sum_kernel<T><<<sgrid, 256, 0, stream>>>(dk_q, dk + koff, per_head, ratio);
+      group_sum_kernel<T><<<sgrid, 256, 0, stream>>>(dv_q, dv + koff, per_head, ratio);
+      FM_TRY(launch_status("group_sum_kernel"));
+    }
   }
   if (ds->normalize) {
     ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
     norm_fix_kernel<T><<<bh, D, 0, stream>>>(dq, q, scale, arg, rpart, pl.nblk, n, D, ds->lim);
-    norm_fix_kernel<T><<<bh, D, 0, stream>>>(dk, k, scale + bh, arg + bh, rpart + (int64_t)bh * pl.nblk, pl.nblk, n, D, ds->lim);
+    norm_fix_kernel<T><<<bhkv, D, 0, stream>>>(dk, k, scale + bh, arg + bh, rpart + (int64_t)bh * pl.nblk,
+                                               pl.nblk * ratio, n, D, ds->lim);
     FM_TRY(launch_status("norm_fix_kernel"));
   }
   return FASTMAX_OK;
@@ -470,7 +502,7 @@ size_t fastmax_workspace_min_bytes(const fastmax_desc* desc, int pass) {
     return 0;
   }
   const Plan pl = make_plan(desc, pass);
-  return pl.fixed_bytes + pl.per_head_bytes;
+  return pl.fixed_bytes + pl.ratio * pl.per_head_bytes;  // one whole key/value group
 }
 
 size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass) {
@@ -478,7 +510,7 @@ size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass) {
   if (!mn) return 0;
   const Plan pl = make_plan(desc, pass);
   size_t heads = (kWorkspaceBudget - (pl.fixed_bytes < kWorkspaceBudget ? pl.fixed_bytes : 0)) / pl.per_head_bytes;
-  if (heads < 1) heads = 1;
+  if (heads < (size_t)pl.ratio) heads = pl.ratio;
   if (heads > (size_t)pl.bh) heads = pl.bh;
   return pl.fixed_bytes + heads * pl.per_head_bytes;
 }
@@ -550,14 +582,15 @@ int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k, void* 
   int* arg = reinterpret_cast<int*>(static_cast<char*>(workspace) + align256((size_t)2 * bh * sizeof(float)));
   const int64_t per_head = (int64_t)desc->nq * desc->d;
   const dim3 grid((unsigned)((per_head / 4 + 255) / 256), bh);
+  const dim3 kgrid(grid.x, desc->bhkv);
   if (desc->dtype == FASTMAX_F32) {
     FM_TRY(compute_scales<float>(desc, (const float*)q, (const float*)k, scale, arg, st));
     scale_rows_kernel<float><<<grid, 256, 0, st>>>((float*)q, scale, per_head);
-    scale_rows_kernel<float><<<grid, 256, 0, st>>>((float*)k, scale + bh, per_head);
+    scale_rows_kernel<float><<<kgrid, 256, 0, st>>>((float*)k, scale + bh, per_head);
   } else {
     FM_TRY(compute_scales<bf16_t>(desc, (const bf16_t*)q, (const bf16_t*)k, scale, arg, st));
     scale_rows_kernel<bf16_t><<<grid, 256, 0, st>>>((bf16_t*)q, scale, per_head);
-    scale_rows_kernel<bf16_t><<<grid, 256, 0, st>>>((bf16_t*)k, scale + bh, per_head);
+    scale_rows_kernel<bf16_t><<<kgrid, 256, 0, st>>>((bf16_t*)k, scale + bh, per_head);
   }
   return launch_status("scale_rows_kernel");
 }
@@ -580,6 +613,7 @@ int fastmax_state_update(const fastmax_desc* desc, const void* k, const void* v,
   g_err[0] = 0;
   FM_TRY(check_desc(desc));
   if (!k || !v || !state) return fail(FASTMAX_E_NULL, "k, v and state must be non-NULL");
+  if (desc->bhkv != desc->bh) return fail(FASTMAX_E_SHAPE, "the recurrent form needs bhkv == bh (one state per head)");
   if (desc->normalize && !k_scale)
     return fail(FASTMAX_E_NULL, "normalize is set: k_scale (the factor a forward pass reported) is required");
   fastmax_desc d2 = *desc;
@@ -607,6 +641,7 @@ int fastmax_decode_step(const fastmax_desc* desc, const void* q, const void* k, 
   g_err[0] = 0;
   FM_TRY(check_desc(desc));
   if (!q || !k || !v || !state || !o) return fail(FASTMAX_E_NULL, "q, k, v, state and o must be non-NULL");
+  if (desc->bhkv != desc->bh) return fail(FASTMAX_E_SHAPE, "the recurrent form needs bhkv == bh (one state per head)");
   if (desc->nq != 1) return fail(FASTMAX_E_SHAPE, "a decode step takes one token per head (nq = nk = 1), got nq = %d", desc->nq);
   if (desc->normalize && (!q_scale || !k_scale))
     return fail(FASTMAX_E_NULL, "normalize is set: q_scale and k_scale (the factors a forward pass reported) are required");

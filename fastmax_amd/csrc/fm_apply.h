@@ -41,7 +41,8 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
     const float* __restrict__ a2den, int64_t a2den_stride, const float* __restrict__ state,
     int nslots, T* __restrict__ OUT, int64_t ldo, float* __restrict__ den, int64_t den_stride, int n,
-    int chunk, int masked, int p2, float a0, float a1, float a2) {
+    int chunk, int masked, int p2, float a0, float a1, float a2, int xdiv,
+    int adiv) {
   using G = Geo<D>;
   constexpr bool FWD = MODE == 0;
   constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
@@ -58,11 +59,14 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
   const int64_t SS = G::state_floats(p2);
-  const T* Xh = X + (int64_t)head * n * D;
-  const T* A1h = A1 + (int64_t)head * n * D;
-  const T* A2h = A2 + (int64_t)head * n * D;
-  const float* a2dh = a2den ? a2den + (int64_t)head * n * a2den_stride : nullptr;
-  const float xs = xscale[head], a1s = a1scale[head];
+  // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
+  // and the state to head ha = head / adiv (one of the divisors is 1)
+  const int hx = head / xdiv, ha = head / adiv;
+  const T* Xh = X + (int64_t)hx * n * D;
+  const T* A1h = A1 + (int64_t)ha * n * D;
+  const T* A2h = A2 + (int64_t)ha * n * D;
+  const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
+  const float xs = xscale[hx], a1s = a1scale[ha];
 
   {
     RowTile<D, T, 128> xt;
@@ -87,7 +91,7 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
       n_tile = ((cend - 1) >> 5) - tile0 + 1;
     }
   }
-  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
+  const float* sbase = state + ((int64_t)ha * nslots + (masked ? c : 0)) * SS;
   const int nsum = masked ? 1 : nslots;
 
   StateSlab<(D + 1) * LD> slab;
@@ -294,7 +298,8 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
     const float* __restrict__ a2den, int64_t a2den_stride, const float* state,
     int nslots, bf16_t* __restrict__ OUT, int64_t ldo, float* __restrict__ den, int64_t den_stride,
-    int n, int chunk, int masked, int p2, float a0, float a1, float a2) {
+    int n, int chunk, int masked, int p2, float a0, float a1, float a2, int xdiv,
+    int adiv) {
   using G = Geo<D>;
   using T = bf16_t;
   constexpr bool FWD = MODE == 0;
@@ -316,11 +321,14 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
   const int64_t SS = G::state_floats(p2);
-  const T* Xh = X + (int64_t)head * n * D;
-  const T* A1h = A1 + (int64_t)head * n * D;
-  const T* A2h = A2 + (int64_t)head * n * D;
-  const float* a2dh = a2den ? a2den + (int64_t)head * n * a2den_stride : nullptr;
-  const float xs = xscale[head], a1s = a1scale[head];
+  // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
+  // and the state to head ha = head / adiv (one of the divisors is 1)
+  const int hx = head / xdiv, ha = head / adiv;
+  const T* Xh = X + (int64_t)hx * n * D;
+  const T* A1h = A1 + (int64_t)ha * n * D;
+  const T* A2h = A2 + (int64_t)ha * n * D;
+  const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
+  const float xs = xscale[hx], a1s = a1scale[ha];
 
   {
     RowTile<D, T, 128> xt;
@@ -343,7 +351,7 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     }
   }
   // packed state of this block's chunk (masked) or the head's summed state (last slot)
-  const char* sbase = reinterpret_cast<const char*>(state + ((int64_t)head * nslots + (masked ? c : nslots - 1)) * SS);
+  const char* sbase = reinterpret_cast<const char*>(state + ((int64_t)ha * nslots + (masked ? c : nslots - 1)) * SS);
   const uint16_t* fsec = reinterpret_cast<const uint16_t*>(sbase);
   const float* zsec = reinterpret_cast<const float*>(sbase + PG::z_off(p2));
 

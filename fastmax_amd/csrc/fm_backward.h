@@ -42,3 +42,23 @@ __global__ void norm_fix_kernel(T* __restrict__ dx, const T* __restrict__ x,
   const int64_t off = ((int64_t)head * n + arg[head]) * d + c;
   dx[off] = from_f32<T>(to_f32(dx[off]) - fac * to_f32(x[off]));
 }
+
+// ---------------------------------------------------------------------------------------
+// Grouped key/value heads: out[g] = sum of the `ratio` per-query-head gradients of group g
+// (fixed order, fp32 sum).  grid = (ceil(per_head / 1024), groups); per_head = n*d elements.
+// ---------------------------------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(256) void group_sum_kernel(const T* __restrict__ part, T* __restrict__ out,
+                                                        int64_t per_head, int ratio) {
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= per_head) return;
+  const int64_t g = blockIdx.y;
+  float a[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < ratio; ++r) {
+    float t[4];
+    load4(part + (g * ratio + r) * per_head + idx, t);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) a[e] += t[e];
+  }
+  store4(out + g * per_head + idx, a);
+}

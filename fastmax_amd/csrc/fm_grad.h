@@ -37,7 +37,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
     const T* __restrict__ A2, const float* __restrict__ a2den, int64_t a2den_stride,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
     const float* __restrict__ state, int nslots, T* __restrict__ OUT, float* __restrict__ rpart,
-    int n, int chunk, int masked, int p2, float a1, float a2) {
+    int n, int chunk, int masked, int p2, float a1, float a2, int xdiv, int adiv) {
   using G = Geo<D>;
   constexpr bool DQ = MODE == 0;
   constexpr int LD = G::LD, AB = G::AB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
@@ -54,14 +54,18 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
   const int64_t SS = G::state_floats(p2);
-  const T* Xh = X + (int64_t)head * n * D;
-  const T* Yh = Y + (int64_t)head * n * D;
-  const T* A1h = A1 + (int64_t)head * n * D;
-  const T* A2h = A2 + (int64_t)head * n * D;
-  const float* ydh = yden ? yden + (int64_t)head * n * yden_stride : nullptr;
-  const float* a2dh = a2den ? a2den + (int64_t)head * n * a2den_stride : nullptr;
+  // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
+  // and the state to head ha = head / adiv (one of the divisors is 1; c_i, the output and the
+  // normalisation partial are per query head = head)
+  const int hx = head / xdiv, ha = head / adiv;
+  const T* Xh = X + (int64_t)hx * n * D;
+  const T* Yh = Y + (int64_t)hx * n * D;
+  const T* A1h = A1 + (int64_t)ha * n * D;
+  const T* A2h = A2 + (int64_t)ha * n * D;
+  const float* ydh = yden ? yden + (int64_t)hx * n * yden_stride : nullptr;
+  const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
   const float* ch = cvec + (int64_t)head * n;
-  const float xs = xscale[head], a1s = a1scale[head];
+  const float xs = xscale[hx], a1s = a1scale[ha];
   const int xrow = w * 32 + i, tok = tok0 + xrow;
 
   {
@@ -97,7 +101,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
       n_tile = ((cend - 1) >> 5) - tile0 + 1;
     }
   }
-  const float* sbase = state + ((int64_t)head * nslots + (masked ? c : 0)) * SS;
+  const float* sbase = state + ((int64_t)ha * nslots + (masked ? c : 0)) * SS;
   const int nsum = masked ? 1 : nslots;
 
   StateSlab<D * LD> slab;
@@ -308,7 +312,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     const bf16_t* __restrict__ A2, const float* __restrict__ a2den, int64_t a2den_stride,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
     const float* state, int nslots, bf16_t* __restrict__ OUT, float* __restrict__ rpart,
-    int n, int chunk, int masked, int p2, float a1, float a2) {
+    int n, int chunk, int masked, int p2, float a1, float a2, int xdiv, int adiv) {
   using G = Geo<D>;
   using T = bf16_t;
   constexpr bool DQ = MODE == 0;
@@ -329,14 +333,18 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
   const int64_t SS = G::state_floats(p2);
-  const T* Xh = X + (int64_t)head * n * D;
-  const T* Yh = Y + (int64_t)head * n * D;
-  const T* A1h = A1 + (int64_t)head * n * D;
-  const T* A2h = A2 + (int64_t)head * n * D;
-  const float* ydh = yden ? yden + (int64_t)head * n * yden_stride : nullptr;
-  const float* a2dh = a2den ? a2den + (int64_t)head * n * a2den_stride : nullptr;
+  // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
+  // and the state to head ha = head / adiv (one of the divisors is 1; c_i, the output and the
+  // normalisation partial are per query head = head)
+  const int hx = head / xdiv, ha = head / adiv;
+  const T* Xh = X + (int64_t)hx * n * D;
+  const T* Yh = Y + (int64_t)hx * n * D;
+  const T* A1h = A1 + (int64_t)ha * n * D;
+  const T* A2h = A2 + (int64_t)ha * n * D;
+  const float* ydh = yden ? yden + (int64_t)hx * n * yden_stride : nullptr;
+  const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
   const float* ch = cvec + (int64_t)head * n;
-  const float xs = xscale[head], a1s = a1scale[head];
+  const float xs = xscale[hx], a1s = a1scale[ha];
   const int xrow = w * 32 + i, tok = tok0 + xrow;
 
   {
@@ -377,7 +385,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   // packed state of this block's chunk (masked) or the head's summed state (last slot)
   using PG = PackedGeo<D>;
   static_assert(PG::LB == LB && PG::CSL == D * LB, "stage layout = column-packed slab layout");
-  const char* sbase = reinterpret_cast<const char*>(state + ((int64_t)head * nslots + (masked ? c : nslots - 1)) * SS);
+  const char* sbase = reinterpret_cast<const char*>(state + ((int64_t)ha * nslots + (masked ? c : nslots - 1)) * SS);
   const uint16_t* csec = reinterpret_cast<const uint16_t*>(sbase + PG::c_off(p2));
 
   // a C slab is copied as it is: 16-byte pieces global -> registers -> LDS

@@ -29,7 +29,7 @@ typedef struct ihipStream_t* fastmax_stream_t; /* == hipStream_t */
 enum {
   FASTMAX_OK = 0,
   FASTMAX_E_NULL = -1,        /* a required pointer is NULL                         */
-  FASTMAX_E_SHAPE = -2,       /* unsupported bh / n / d / bhkv / nq != nk           */
+  FASTMAX_E_SHAPE = -2,       /* unsupported bh / n / d, bhkv not dividing bh, nq != nk */
   FASTMAX_E_DTYPE = -3,       /* dtype not FASTMAX_F32 / FASTMAX_BF16               */
   FASTMAX_E_PARAM = -4,       /* p not in {1,2}, bad lim / temperature / pitch      */
   FASTMAX_E_WORKSPACE = -5,   /* workspace NULL, misaligned or too small            */
@@ -46,7 +46,9 @@ enum { FASTMAX_PASS_FORWARD = 0, FASTMAX_PASS_BACKWARD = 1 };
  * from the tensors (fastmax_cuda_forward.cu:331-336). */
 typedef struct fastmax_desc {
   int32_t bh;          /* query heads  (b*h)                                             */
-  int32_t bhkv;        /* key/value heads; must equal bh                                 */
+  int32_t bhkv;        /* key/value heads; divides bh: query head i reads key/value head
+                          i / (bh / bhkv)  (fastmax_cuda_forward.cu:38); k, v, dk, dv are
+                          then (bhkv, n, d)                                              */
   int32_t nq;          /* query tokens                                                   */
   int32_t nk;          /* key tokens; must equal nq                                      */
   int32_t d;           /* head dimension: 32 or 64                                        */
@@ -69,7 +71,7 @@ const char* fastmax_version(void);
 const char* fastmax_last_error(void);
 
 /* Checks a descriptor without touching the device.  Replaces the shape reads and the
- * implicit assumptions of fastmax_cuda_forward.cu:331-345 (d == 64, bh == bhkv). */
+ * implicit assumptions of fastmax_cuda_forward.cu:331-345 (d == 64). */
 int fastmax_check_desc(const fastmax_desc* desc);
 
 /* Bytes of device workspace that let a pass run all heads in as few batches as a 16 GiB
@@ -80,11 +82,13 @@ size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass);
 size_t fastmax_workspace_min_bytes(const fastmax_desc* desc, int pass);
 
 /* Forward pass.  Replaces forward_cuda (fastmax_cuda_forward.cu:297-411).
- *   q, k, v     (bh, n, d)             inputs, never modified
+ *   q           (bh, n, d)             input, never modified
+ *   k, v        (bhkv, n, d)           inputs, never modified
  *   o           (bh, n, ldo >= d)      out: attention output, columns [0,d)
  *   den         den[(h*n+i)*den_stride] out: row denominators sum_j f(s_ij); may alias
  *                                      column d of o (see layout contract)
- *   qk_scale    2*bh floats or NULL    out: per-head factors applied to q then k
+ *   qk_scale    2*bh floats or NULL    out: per-head factors applied to q (bh values) then k
+ *                                      (bhkv values, from index bh);
  *                                      (lim / max row norm, 1/temperature, or 1)
  *   qk_argmax   2*bh int32 or NULL     out: row index of the max-norm row per head
  *   workspace   256-byte aligned device memory of workspace_bytes bytes               */
@@ -99,7 +103,7 @@ int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, cons
  *   q, k, v, o, den  as given to / produced by fastmax_forward (q, k un-normalised)
  *   go               (bh, n, d) upstream gradient, never modified (the reference divides it
  *                    in place, fastmax_cuda_backward.cu:874-882,970)
- *   dq, dk, dv       (bh, n, d) out
+ *   dq               (bh, n, d) out;  dk, dv  (bhkv, n, d) out
  *   qk_scale, qk_argmax  values written by fastmax_forward, or NULL to recompute them   */
 int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, const void* v,
                      const void* o, int64_t ldo, const float* den, int64_t den_stride,

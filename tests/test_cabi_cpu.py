@@ -33,7 +33,7 @@ def test_version_and_clean_error(built):
 
 
 @pytest.mark.parametrize("over,code", [
-    (dict(d=48), -2), (dict(d=128), -2), (dict(bh=0), -2), (dict(bhkv=2), -2), (dict(nk=50), -2), (dict(n=0), -2),
+    (dict(d=48), -2), (dict(d=128), -2), (dict(bh=0), -2), (dict(bhkv=3), -2), (dict(bhkv=0), -2), (dict(nk=50), -2), (dict(n=0), -2),
     (dict(dtype=7), -3), (dict(p=3), -4), (dict(p=0), -4), (dict(lim=0.0), -4),
     (dict(normalize=False, temperature=0.0), -4),
 ])
@@ -41,6 +41,17 @@ def test_bad_descriptors(built, over, code):
     assert built.fastmax_check_desc(C.byref(desc(**over))) == code
     assert _cabi.last_error() != ""
     assert built.fastmax_workspace_bytes(C.byref(desc(**over)), _cabi.PASS_FORWARD) == 0
+
+
+def test_grouped_heads_descriptor(built):
+    """bhkv must divide bh (fastmax_cuda_forward.cu:38 maps head i to key/value head i / (bh/bhkv)); the
+    smallest workspace then holds one whole group."""
+    ds1, ds4 = desc(bh=8, bhkv=8, mask=True), desc(bh=8, bhkv=2, mask=True)
+    assert built.fastmax_check_desc(C.byref(ds4)) == 0
+    for pas in (_cabi.PASS_FORWARD, _cabi.PASS_BACKWARD):
+        lo1 = built.fastmax_workspace_min_bytes(C.byref(ds1), pas)
+        lo4 = built.fastmax_workspace_min_bytes(C.byref(ds4), pas)
+        assert lo4 > lo1 > 0
 
 
 def test_bad_p_message_matches_reference_wording(built):
