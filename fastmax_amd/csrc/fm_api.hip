@@ -127,8 +127,9 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
     int zlen = ((pl.n + z - 1) / z + 31) / 32 * 32;
     pl.zlen = zlen;
     pl.nparts = (pl.n + zlen - 1) / zlen;
-    // bf16: one more slot for the summed state in the packed form the consumers read
-    pl.nslots = pl.nparts + (ds->dtype == FASTMAX_BF16 ? 1 : 0);
+    // consumers read one state per head, the last slot: the sum of the partial states (for bf16
+    // inputs in packed form), or the only partial state itself
+    pl.nslots = pl.nparts + ((ds->dtype == FASTMAX_BF16 || pl.nparts > 1) ? 1 : 0);
   }
   pl.state_floats = state_floats_for(pl.d, pl.p2);
   size_t fixed = align256((size_t)2 * pl.bh * sizeof(float)) + align256((size_t)2 * pl.bh * sizeof(int));
@@ -229,7 +230,7 @@ constexpr bool kBf16Mfma<bf16_t> = true;
 template <int D, class T>
 int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float* xscale,
                  const float* yden, int64_t yden_stride, const float* ew, float* state, int reverse,
-                 int sections, hipStream_t stream) {
+                 int sections, hipStream_t stream, bool finish = true) {
   const dim3 grid(pl.gsplit, heads, pl.nparts);
   if (pl.masked && pl.nslots < 2) return FASTMAX_OK;  // a single chunk never needs a state
   ScopedKernel sk(FASTMAX_K_BUILD, stream);
@@ -249,9 +250,16 @@ int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float*
     FM_BUILD(5);
   }
 #undef FM_BUILD
-  if constexpr (kBf16Mfma<T>) {
-    if (!pl.masked)
+  // unmasked: the partial states of a head are summed into its last slot (finish = false leaves
+  // that to the caller)
+  if (!pl.masked && finish) {
+    if constexpr (kBf16Mfma<T>) {
       state_pack_kernel<D><<<dim3(PackedGeo<D>::nslab(pl.p2), heads), 256, 0, stream>>>(state, pl.nslots, pl.nparts, pl.p2);
+    } else if (pl.nparts > 1) {
+      const int64_t ss = pl.state_floats;
+      state_accumulate_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads), 256, 0, stream>>>(
+          state + (int64_t)pl.nparts * ss, (int64_t)pl.nslots * ss, state, pl.nslots, pl.nparts, ss, 0);
+    }
   }
   return launch_status("build_kernel");
 }
@@ -436,9 +444,10 @@ int state_update_impl(const fastmax_desc* ds, const Plan& pl, const T* k, const 
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
     const int64_t off = (int64_t)h0 * n * D;
-    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, kscale + h0, nullptr, 0, nullptr, slots, 0, 0, stream)));
+    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, kscale + h0, nullptr, 0, nullptr, slots, 0, 0, stream,
+                               false)));
     state_accumulate_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads), 256, 0, stream>>>(
-        state + (int64_t)h0 * ss, slots, pl.nslots, pl.nparts, ss, accumulate);
+        state + (int64_t)h0 * ss, ss, slots, pl.nslots, pl.nparts, ss, accumulate);
   }
   return launch_status("state_accumulate_kernel");
 }

@@ -91,14 +91,14 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
       n_tile = ((cend - 1) >> 5) - tile0 + 1;
     }
   }
-  const float* sbase = state + ((int64_t)ha * nslots + (masked ? c : 0)) * SS;
-  const int nsum = masked ? 1 : nslots;
+  // this block's chunk snapshot (masked) or the head's summed state (last slot)
+  const float* sbase = state + ((int64_t)ha * nslots + (masked ? c : nslots - 1)) * SS;
 
   StateSlab<(D + 1) * LD> slab;
   RowTile<D, T, 32> t1, t2;
   auto slab_load = [&](int st) {
     const bool ord2 = p2 && st < NS;
-    slab.load(sbase + (ord2 ? st * D * LD : rows2 * LD), SS, nsum, ord2 ? D * LD : (D + 1) * LD, tid);
+    slab.load(sbase + (ord2 ? st * D * LD : rows2 * LD), ord2 ? D * LD : (D + 1) * LD, tid);
   };
   auto slab_store = [&](int st) {
     if (p2 && st < NS) {

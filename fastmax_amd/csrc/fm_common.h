@@ -260,28 +260,18 @@ struct RowTile {
   }
 };
 
-// A run of `count` floats of a moment state staged global -> registers -> LDS, summed over
-// `nsum` slots (token-split partial states of an unmasked build).
+// A run of `count` floats of a moment state staged global -> registers -> LDS.
 template <int MAXF>
 struct StateSlab {
   static constexpr int NV = ((MAXF + 3) / 4 + 255) / 256;
   float4 v[NV];
 
-  __device__ __forceinline__ void load(const float* src, int64_t slot_stride, int nsum, int count,
-                                       int tid) {
+  __device__ __forceinline__ void load(const float* src, int count, int tid) {
     const int nvec = (count + 3) >> 2;
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
-      float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (idx < nvec) {
-        a = *reinterpret_cast<const float4*>(src + idx * 4);
-        for (int z = 1; z < nsum; ++z) {
-          const float4 b = *reinterpret_cast<const float4*>(src + z * slot_stride + idx * 4);
-          a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
-        }
-      }
-      v[u] = a;
+      v[u] = idx < nvec ? *reinterpret_cast<const float4*>(src + idx * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
   }
   // elements [0, split) are scaled by c_lo, the rest by c_hi

@@ -10,15 +10,16 @@
 #include "fm_common.h"
 
 // state[head] = (accumulate ? state[head] : 0) + sum_{part < nparts} slots[head][part]
+// (state[head] starts at state + head * state_stride floats; it may be a further slot of `slots`)
 // grid = (ceil(state_floats / 1024), heads), 256 threads, one float4 each.
-__global__ __launch_bounds__(256) void state_accumulate_kernel(float* __restrict__ state,
+__global__ __launch_bounds__(256) void state_accumulate_kernel(float* __restrict__ state, int64_t state_stride,
                                                                const float* __restrict__ slots,
                                                                int nslots, int nparts, int64_t ss,
                                                                int accumulate) {
   const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (idx >= ss) return;
   const int head = blockIdx.y;
-  float4* dst = reinterpret_cast<float4*>(state + (int64_t)head * ss + idx);
+  float4* dst = reinterpret_cast<float4*>(state + (int64_t)head * state_stride + idx);
   float4 a = accumulate ? *dst : make_float4(0.f, 0.f, 0.f, 0.f);
   for (int part = 0; part < nparts; ++part) {
     const float4 t = *reinterpret_cast<const float4*>(slots + ((int64_t)head * nslots + part) * ss + idx);

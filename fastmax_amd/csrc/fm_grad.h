@@ -101,14 +101,14 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
       n_tile = ((cend - 1) >> 5) - tile0 + 1;
     }
   }
-  const float* sbase = state + ((int64_t)ha * nslots + (masked ? c : 0)) * SS;
-  const int nsum = masked ? 1 : nslots;
+  // this block's chunk snapshot (masked) or the head's summed state (last slot)
+  const float* sbase = state + ((int64_t)ha * nslots + (masked ? c : nslots - 1)) * SS;
 
   StateSlab<D * LD> slab;
   RowTile<D, T, 32> t1, t2;
   float creg = 0.f;
   auto slab_load = [&](int st) {
-    slab.load(sbase + ((p2 && st < NS) ? st * D * LD : rows2 * LD), SS, nsum, D * LD, tid);
+    slab.load(sbase + ((p2 && st < NS) ? st * D * LD : rows2 * LD), D * LD, tid);
   };
   auto slab_store = [&](int st) {
     const float cf = (p2 && st < NS) ? 2.0f * a2 : a1;
