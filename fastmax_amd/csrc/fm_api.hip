@@ -60,11 +60,11 @@ struct ScopedKernel {
   }
 };
 
-constexpr int kChunkP1 = 128;    // p = 1
-constexpr int kChunk = 256;      // tokens between causal state snapshots (fp32 arithmetic)
-constexpr int kChunkBf16 = 512;  // ... when the contractions run on the bf16 matrix instruction: the
-                                 // moment work is ~8x cheaper there, so snapshot traffic is worth
-                                 // halving at the price of more intra-chunk tiles
+// Tokens between causal state snapshots (a multiple of the 128-token block of the consumers).
+// Longer chunks mean fewer snapshots to write and read but more intra-chunk score tiles; measured
+// at the headline shapes, 384 beats 256 and 512 for p = 2 (fp32 and bf16 alike).
+constexpr int kChunkP1 = 128;  // p = 1: a state is only d+1 rows, a snapshot per block is cheapest
+constexpr int kChunk = 384;
 constexpr size_t kWorkspaceBudget = 16ull << 30;   // what fastmax_workspace_bytes aims for
 
 struct Plan {
@@ -102,10 +102,9 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   if (!pl.p2) {
     pl.rtw = 1;
   } else if (pl.d == 64) {
-    // 3 or 4 row tiles per wave (6 or 5 blocks per head): a block's run time grows with its tile
-    // count and 512 blocks are resident at once, so pick the one with fewer tile-rounds
-    auto cost = [&](int rtw) { return (int64_t)((splits(rtw) * pl.bh + 511) / 512) * rtw; };
-    pl.rtw = cost(4) < cost(3) ? 4 : 3;
+    // 3 row tiles per wave, 6 blocks per head (4 tiles per wave would save a block per head
+    // but does not fit the register file: measured 1.6x slower)
+    pl.rtw = 3;
   } else {
     pl.rtw = 5;
   }
@@ -113,7 +112,7 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   pl.nblk = (pl.n + 127) / 128;
   // p = 1: a state is only (d+1) rows, so a snapshot per 128-token block is cheaper than a longer
   // intra-chunk part
-  pl.chunk = !pl.p2 ? kChunkP1 : ds->dtype == FASTMAX_BF16 ? kChunkBf16 : kChunk;
+  pl.chunk = pl.p2 ? kChunk : kChunkP1;
   if (pl.masked) {
     pl.nslots = (pl.n + pl.chunk - 1) / pl.chunk;
     pl.nparts = 1;
@@ -241,11 +240,7 @@ int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float*
   if (pl.rtw == 1) {
     FM_BUILD(1);
   } else if constexpr (D == 64) {
-    if (pl.rtw == 4) {
-      FM_BUILD(4);
-    } else {
-      FM_BUILD(3);
-    }
+    FM_BUILD(3);
   } else {
     FM_BUILD(5);
   }

@@ -260,6 +260,61 @@ struct RowTile {
   }
 };
 
+// bf16 variant of RowTile<D, bf16_t, ROWS, true> that keeps the rows as loaded (two registers
+// per 4-element piece) until they are stored, so that a 64-row tile costs no more registers
+// than a converted 32-row one.  Only the transposed stores exist.
+template <int D, int ROWS>
+struct RawTileBf {
+  static_assert(256 % ROWS == 0 && (ROWS * D / 4) % 256 == 0, "every thread owns whole pieces of one row");
+  static constexpr int RG = 256 / ROWS;          // 4-channel groups covered per sweep of the block
+  static constexpr int NV = (D / 4) / RG;        // pieces per thread: row tid % ROWS, groups tid / ROWS + u * RG
+  uint2 raw[NV];
+  float rdiv;
+
+  __device__ __forceinline__ void load(const bf16_t* base, int tok0, int n, int tid,
+                                       const float* rowdiv = nullptr, int64_t rowdiv_stride = 0) {
+    const int tok = tok0 + tid % ROWS;
+    const bool live = tok < n;
+    const bf16_t* src = base + (int64_t)(live ? tok : 0) * D + (tid / ROWS) * 4;
+    rdiv = (live && rowdiv) ? rowdiv[(int64_t)tok * rowdiv_stride] : 1.0f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const uint2 t = *reinterpret_cast<const uint2*>(src + u * RG * 4);
+      raw[u] = live ? t : make_uint2(0u, 0u);
+    }
+  }
+  // transposed, converted to fp32 and scaled: dst is [D][ld] floats in LDS
+  __device__ __forceinline__ void store_t(float* dst, int ld, float scale, int tid) const {
+    const float sc = scale / rdiv;
+    float* d0 = dst + (tid / ROWS) * 4 * ld + tid % ROWS;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      d0[(u * RG * 4 + 0) * ld] = bf_lo(raw[u].x) * sc;
+      d0[(u * RG * 4 + 1) * ld] = bf_hi(raw[u].x) * sc;
+      d0[(u * RG * 4 + 2) * ld] = bf_lo(raw[u].y) * sc;
+      d0[(u * RG * 4 + 3) * ld] = bf_hi(raw[u].y) * sc;
+    }
+  }
+  // transposed bf16: dst is [D][ld] 16-bit elements in LDS.  exact: the rows go out as loaded
+  // (no scale, no divisor); otherwise they are scaled in fp32 and rounded again.
+  __device__ __forceinline__ void store_t_bf(uint16_t* dst, int ld, float scale, int tid, bool exact) const {
+    const float sc = scale / rdiv;
+    uint16_t* d0 = dst + (tid / ROWS) * 4 * ld + tid % ROWS;
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      uint32_t p01 = raw[u].x, p23 = raw[u].y;
+      if (!exact) {
+        p01 = pack_bf2(bf_lo(raw[u].x) * sc, bf_hi(raw[u].x) * sc);
+        p23 = pack_bf2(bf_lo(raw[u].y) * sc, bf_hi(raw[u].y) * sc);
+      }
+      d0[(u * RG * 4 + 0) * ld] = (uint16_t)p01;
+      d0[(u * RG * 4 + 1) * ld] = (uint16_t)(p01 >> 16);
+      d0[(u * RG * 4 + 2) * ld] = (uint16_t)p23;
+      d0[(u * RG * 4 + 3) * ld] = (uint16_t)(p23 >> 16);
+    }
+  }
+};
+
 // A run of `count` floats of a moment state staged global -> registers -> LDS.
 template <int MAXF>
 struct StateSlab {

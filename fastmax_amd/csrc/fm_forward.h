@@ -23,18 +23,25 @@ __global__ __launch_bounds__(256) void rowstat_kernel(const T* __restrict__ x, i
   const T* base = x + (int64_t)blockIdx.x * n * d;
   float best = -1.f;
   int bi = 0x7fffffff;
-  for (int i0 = 0; i0 < n; i0 += rpp) {
-    const int i = i0 + rowi;
-    float ss = 0.f;
-    if (i < n) {
-      float v[4];
-      load4(base + (int64_t)i * d + sub * 4, v);
-      ss = v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+  // four row groups per trip, loaded before any of them is reduced (rows past the end are
+  // clamped to the last row: a duplicate cannot change the maximum or its first index)
+  for (int i0 = 0; i0 < n; i0 += 4 * rpp) {
+    float v[4][4];
+    int idx[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * rpp + rowi;
+      idx[u] = i < n ? i : n - 1;
+      load4(base + (int64_t)idx[u] * d + sub * 4, v[u]);
     }
-    for (int off = tpr >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-    if (i < n && ss > best) {
-      best = ss;
-      bi = i;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float ss = v[u][0] * v[u][0] + v[u][1] * v[u][1] + v[u][2] * v[u][2] + v[u][3] * v[u][3];
+      for (int off = tpr >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      if (ss > best || (ss == best && idx[u] < bi)) {
+        best = ss;
+        bi = idx[u];
+      }
     }
   }
   sbest[tid] = best;
@@ -107,7 +114,8 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     float* __restrict__ state, int n, int chunk, int nslots, int masked, int reverse, int p2,
     int zlen, int sections) {
   using G = Geo<D>;
-  constexpr int TS = 32;        // tokens per pipeline step
+  constexpr int TS = 32;  // tokens per pipeline step (64 for bf16 halves the barriers but does not fit the
+                        // register file next to three row tiles of accumulators)
   constexpr int TP = TS + 4;    // pitch of the transposed tiles: 16-byte aligned rows, and the
                                 // 8 lanes of a 128-bit LDS access phase fall in distinct banks
   constexpr int LD = G::LD;
@@ -182,24 +190,27 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   const float* ewh = ew ? ew + (int64_t)head * n : nullptr;
   const float xs = xscale[head];
 
-  RowTile<D, T, TS, true> kx, vy;
+  // a step is staged in halves of 32 tokens (one half when TS == 32), so that only one half's
+  // rows are in registers at a time
+  constexpr int NH = TS / 32;
+  std::conditional_t<BF, RawTileBf<D, 32>, RowTile<D, T, 32, true>> kx, vy;
   float ereg = 0.f;
 
   auto load = [&](int t0, int tend) {
     kx.load(Xh, t0, tend, tid);
     vy.load(Yh, t0, tend, tid, ydh, yden_stride);
-    if (tid < TS) {
+    if (tid < 32) {
       const int tok = t0 + tid;
       ereg = (tok < tend) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
     }
   };
-  auto store = [&](int buf, int t0, int tend) {
-    kx.store_t(Kt[buf], TP, xs, tid);
-    if constexpr (BF) vy.store_t_bf(Vtb[buf], TPB, 1.0f, tid);
-    else vy.store_t(Vt[buf], TP, 1.0f, tid);
-    if (tid < TS) {
-      El[buf][tid] = ereg;
-      Kt[buf][D * TP + tid] = (t0 + tid < tend) ? 1.0f : 0.f;
+  auto store = [&](int buf, int h, int t0, int tend) {
+    kx.store_t(Kt[buf] + 32 * h, TP, xs, tid);
+    if constexpr (BF) vy.store_t_bf(Vtb[buf] + 32 * h, TPB, 1.0f, tid, ydh == nullptr);
+    else vy.store_t(Vt[buf] + 32 * h, TP, 1.0f, tid);
+    if (tid < 32) {
+      El[buf][32 * h + tid] = ereg;
+      Kt[buf][D * TP + 32 * h + tid] = (t0 + tid < tend) ? 1.0f : 0.f;
     }
   };
   // operands of one group of 8 tokens (lane half hh takes tokens 8*grp + 4*hh + u, u = 0..3,
@@ -222,14 +233,15 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       g4.rot[x] = *reinterpret_cast<const float4*>(kb + rotoff[x] + go8);
     }
   };
-  auto compute = [&](int buf) {
+  auto compute = [&](int buf, int h) {
     const float* kb = Kt[buf];
     const float* eb = El[buf];
     GroupOps cur, nxt;
-    fetch(kb, buf, eb, 0, cur);
+    fetch(kb, buf, eb, 4 * h, cur);
 #pragma unroll
-    for (int grp = 0; grp < TS / 8; ++grp) {
-      if (grp + 1 < TS / 8) fetch(kb, buf, eb, grp + 1, nxt);
+    for (int gq = 0; gq < 4; ++gq) {
+      const int grp = 4 * h + gq;
+      if (gq + 1 < 4) fetch(kb, buf, eb, grp + 1, nxt);
       // tiles past the end of the feature list (x >= nx) run on dummy operands and are never stored
 #pragma unroll
       for (int x = 0; x < RTW; ++x) {
@@ -250,15 +262,19 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
         }
         dacc[x] += a0 * cur.e4.x + a1 * cur.e4.y + a2 * cur.e4.z + a3 * cur.e4.w;
       }
-      if (grp + 1 < TS / 8) cur = nxt;
+      if (gq + 1 < 4) cur = nxt;
     }
+  };
+  // order-0 sums of the staged step
+  auto sum0 = [&](int buf) {
+    const float* eb = El[buf];
     if (g == 0 && tid <= D) {
       if (BF && tid < D) {
         const uint16_t* src = Vtb[buf] + tid * TPB;
 #pragma unroll
-        for (int j = 0; j < TS; j += 2) {
-          const uint32_t u = *reinterpret_cast<const uint32_t*>(src + j);
-          s0 += bf_lo(u) + bf_hi(u);
+        for (int j = 0; j < TS; j += 4) {
+          const uint2 u = *reinterpret_cast<const uint2*>(src + j);
+          s0 += (bf_lo(u.x) + bf_hi(u.x)) + (bf_lo(u.y) + bf_hi(u.y));
         }
       } else {
         const float* src = tid < D ? Vt[buf] + tid * TP : eb;
@@ -393,16 +409,23 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   };
 
   if (nsteps > 0) {
-    load(step_tok(0), tend);
-    store(0, step_tok(0), tend);
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      load(step_tok(0) + 32 * h, tend);
+      store(0, h, step_tok(0) + 32 * h, tend);
+    }
   }
   __syncthreads();
   for (int p = 0; p < nsteps; ++p) {
     const bool more = p + 1 < nsteps;
     const int tnext = step_tok(more ? p + 1 : p);
-    if (more) load(tnext, tend);
-    compute(p & 1);
-    if (more) store((p + 1) & 1, tnext, tend);
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      if (more) load(tnext + 32 * h, tend);
+      compute(p & 1, h);
+      if (h == NH - 1) sum0(p & 1);
+      if (more) store((p + 1) & 1, h, tnext + 32 * h, tend);
+    }
     // after the staged tile has been consumed: waiting for loads while stores are pending
     // would wait for the stores too (one in-order counter covers both)
     const int slot = step_slot(p);
