@@ -43,7 +43,7 @@ COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 # FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/headline_causal_fp32_all_kernels.txt
 # (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch x2.0, write x1.0).
 MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD = {
-    "headline": {"build": 3785.0, "fwd_apply": 3502.0, "bwd_dq": 3754.0, "bwd_dk": 3939.0, "bwd_dv": 3582.0},
+    "headline": {"build": 3023.0, "fwd_apply": 2611.0, "bwd_dq": 2863.0, "bwd_dk": 3045.0, "bwd_dv": 2714.0},
 }
 
 
@@ -113,6 +113,9 @@ def main() -> int:
                     help="also run one plain 1 GiB device copy, so that a counter profile of this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--through-module", action="store_true",
+                    help="also time forward + backward through FASTMultiHeadAttention and autograd "
+                         "(allocations and the extension included)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -169,6 +172,29 @@ def main() -> int:
     torch.cuda.synchronize()
     ms_fwd = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    ms_module = None
+    if args.through_module:
+        from fastmax_amd import FASTMultiHeadAttention
+        ops.release_workspaces()
+        mod = FASTMultiHeadAttention()
+        qm, km, vm = (t.view(B, H, N, D).requires_grad_(True) for t in (q, k, v))
+        gom = go.view(B, H, N, D)
+
+        def mstep():
+            o = mod(qm, km, vm, None, cfg["mask"], 0.0, COEF["normalize"], COEF["temperature"], COEF["a0"],
+                    COEF["a1"], COEF["a2"], COEF["lim"], cfg["p"])
+            o.backward(gom)
+            qm.grad = km.grad = vm.grad = None
+
+        for _ in range(args.warmup):
+            mstep()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            mstep()
+        torch.cuda.synchronize()
+        ms_module = (time.perf_counter() - t0) * 1e3 / args.steps
+
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
@@ -218,6 +244,7 @@ def main() -> int:
                                f"B={B} H={H} N={N} D={D} p={cfg['p']} {cfg['dtype']}, normalize lim=1, "
                                "a=(1,1,0.5), q/k/v/grad iid N(0,1) seed 0"},
         "fwd_ms": ms_fwd, "fwd_tokens_per_s": B * N / (ms_fwd * 1e-3),
+        "module_autograd_ms_per_step": ms_module,
         "fwd_tflops": fl["fwd"] * token_heads / (ms_fwd * 1e-3) / 1e12,
         "fwd_bwd_tflops": (fl["fwd"] + fl["bwd"]) * token_heads / (ms_step * 1e-3) / 1e12,
         "mfma_frac_of_peak_fwd_bwd": (fl["fwd"] + fl["bwd"]) * token_heads / (ms_step * 1e-3) / 1e12 / peak,
