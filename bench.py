@@ -113,6 +113,9 @@ def main() -> int:
                     help="also run one plain 1 GiB device copy, so that a counter profile of this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--recompute-states", action="store_true",
+                    help="backward rebuilds the prefix states instead of reading the ones the forward pass "
+                         "kept (saves bhkv * chunks * 592 KB of HBM, costs one more state build)")
     ap.add_argument("--through-module", action="store_true",
                     help="also time forward + backward through FASTMultiHeadAttention and autograd "
                          "(allocations and the extension included)")
@@ -148,8 +151,12 @@ def main() -> int:
         return ops.forward(q, k, v, **kw)
 
     def step():
-        o, den, sc, arg = fwd()
-        return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+        if args.recompute_states:
+            o, den, sc, arg = fwd()
+            return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+        # the forward pass leaves its prefix states behind for the backward pass
+        o, den, sc, arg, saved = ops.forward(q, k, v, save_states=True, **kw)
+        return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, saved_states=saved, **kw)
 
     for _ in range(args.warmup):
         step()
@@ -209,8 +216,10 @@ def main() -> int:
     for i, name in enumerate(_cabi.KERNEL_NAMES):
         if kt.launches[i]:
             kernels[name] = {"ms_per_step": kt.ms[i] / args.steps, "launches_per_step": kt.launches[i] / args.steps}
-    # algorithmic flops each kernel class executes per step (build runs 3x: fwd prefix, bwd prefix, bwd suffix)
-    per_step_flops = {"build": 3 * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
+    # algorithmic flops each kernel class executes per step (builds: fwd prefix, bwd suffix, and the bwd prefix
+    # again when the states are not kept)
+    n_builds = 3 if args.recompute_states else 2
+    per_step_flops = {"build": n_builds * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
                       "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dk": fl["bwd_dk"] * token_heads,
                       "bwd_dv": fl["bwd_dv"] * token_heads}
     dom = max(per_step_flops, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0))
@@ -226,7 +235,7 @@ def main() -> int:
     }
     per_th = MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD.get(args.workload if not args.batch else "", {}).get(dom)
     if per_th is not None:
-        n_states = 3 if dom == "build" else 1
+        n_states = n_builds if dom == "build" else 1
         roofline["traffic"] = per_th * token_heads * n_states / launches  # bytes per launch (profiled, not live)
         roofline["traffic_source"] = "profiles/headline_causal_fp32_all_kernels.txt"
     for name, f in per_step_flops.items():
@@ -242,7 +251,9 @@ def main() -> int:
         "dtype": cfg["dtype"] if cfg["dtype"] == "f32" else "bf16 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": f"{args.workload}: Fastmax {'causal' if cfg['mask'] else 'unmasked'} fwd+bwd, "
                                f"B={B} H={H} N={N} D={D} p={cfg['p']} {cfg['dtype']}, normalize lim=1, "
-                               "a=(1,1,0.5), q/k/v/grad iid N(0,1) seed 0"},
+                               "a=(1,1,0.5), q/k/v/grad iid N(0,1) seed 0; backward "
+                               + ("rebuilds the prefix states" if args.recompute_states
+                                  else "reads the prefix states the forward pass kept")},
         "fwd_ms": ms_fwd, "fwd_tokens_per_s": B * N / (ms_fwd * 1e-3),
         "module_autograd_ms_per_step": ms_module,
         "fwd_tflops": fl["fwd"] * token_heads / (ms_fwd * 1e-3) / 1e12,

@@ -26,6 +26,7 @@ EXPORTS = (
     "fastmax_workspace_min_bytes", "fastmax_forward", "fastmax_backward", "fastmax_normalize_inplace",
     "fastmax_profile_begin", "fastmax_profile_end",
     "fastmax_state_bytes", "fastmax_decode_workspace_bytes", "fastmax_state_update", "fastmax_decode_step",
+    "fastmax_saved_state_bytes", "fastmax_forward_saving", "fastmax_backward_saved",
 )
 
 KERNEL_NAMES = ("rowstat", "build", "fwd_apply", "bwd_prep", "bwd_dq", "bwd_dk", "bwd_dv", "norm_fix")
@@ -78,6 +79,13 @@ def load() -> C.CDLL:
     lib.fastmax_forward.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, sz, vp]
     lib.fastmax_backward.restype = C.c_int
     lib.fastmax_backward.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+    lib.fastmax_saved_state_bytes.restype = sz
+    lib.fastmax_saved_state_bytes.argtypes = [dp]
+    lib.fastmax_forward_saving.restype = C.c_int
+    lib.fastmax_forward_saving.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, sz, vp, sz, vp]
+    lib.fastmax_backward_saved.restype = C.c_int
+    lib.fastmax_backward_saved.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, sz, vp,
+                                           sz, vp]
     lib.fastmax_normalize_inplace.restype = C.c_int
     lib.fastmax_normalize_inplace.argtypes = [dp, vp, vp, vp, sz, vp]
     lib.fastmax_state_bytes.restype = sz

@@ -22,6 +22,21 @@ import torch
 from . import _ext
 
 
+# fraction of the free device memory the saved prefix states of one call may take
+SAVE_STATES_MEMORY_FRACTION = 0.25
+
+
+def _states_fit(k3: torch.Tensor, mask: bool) -> bool:
+    """True when the prefix states of this call (one 592 KB state per key/value head per 384
+    tokens at d = 64, p = 2) take less than SAVE_STATES_MEMORY_FRACTION of the free memory."""
+    heads, n, d = k3.shape
+    rows = (d // 2 + 1) * d + d + 1
+    state_bytes = rows * (d + 4) * 4 + 256
+    slots = (n + 127) // 128 if mask else 8  # upper bounds: the chunk is at least 128 tokens
+    free, _ = torch.cuda.mem_get_info(k3.device)
+    return heads * slots * state_bytes <= SAVE_STATES_MEMORY_FRACTION * free
+
+
 class FASTMultiHeadAttention_Function(torch.autograd.Function):
     """Same call signature as example.py:8 / model.py:22."""
 
@@ -47,8 +62,12 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             # zero channels change neither q.k nor the row norms, and give zero output columns
             q3, k3, v3 = (torch.nn.functional.pad(t, (0, pad)) for t in (q3, k3, v3))
         q3, k3, v3 = q3.contiguous(), k3.contiguous(), v3.contiguous()
-        o, den, scale, arg = ext.forward_ex(q3, k3, v3, bool(mask), bool(normalize), float(temperature),
-                                            float(a0), float(a1), float(a2), float(lim), int(p))
+        # keep the prefix states for the backward pass (it then skips rebuilding them) when a
+        # backward pass will come and the states fit comfortably in free device memory
+        need_grad = any(t.requires_grad for t in (q, k, v))
+        save = need_grad and _states_fit(k3, bool(mask))
+        o, den, scale, arg, saved = ext.forward_ex(q3, k3, v3, bool(mask), bool(normalize), float(temperature),
+                                                   float(a0), float(a1), float(a2), float(lim), int(p), save)
         noise = None
         out = o
         if dropout and dropout > 0.0:
@@ -59,7 +78,8 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             if pad:
                 noise = torch.nn.functional.pad(noise, (0, pad), value=1.0)
             out = o * noise
-        ctx.save_for_backward(q3, k3, v3, o, den, scale, arg, noise if noise is not None else o.new_empty(0))
+        ctx.save_for_backward(q3, k3, v3, o, den, scale, arg, noise if noise is not None else o.new_empty(0),
+                              saved)
         ctx.cfg = (bool(mask), bool(normalize), float(temperature), float(a0), float(a1), float(a2), float(lim), int(p))
         ctx.kshape, ctx.vshape, ctx.pad = k.shape, v.shape, pad
         if pad:
@@ -69,7 +89,7 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         ext = _ext.load()
-        q3, k3, v3, o, den, scale, arg, noise = ctx.saved_tensors
+        q3, k3, v3, o, den, scale, arg, noise, saved = ctx.saved_tensors
         mask, normalize, temperature, a0, a1, a2, lim, p = ctx.cfg
         go = grad_output.reshape(q3.shape[0], q3.shape[1], -1)
         if ctx.pad:
@@ -78,7 +98,7 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
             go = go * noise
         go = go.contiguous()
         dq, dk, dv = ext.backward_ex(q3, k3, v3, o, den, go, scale, arg, mask, normalize, temperature,
-                                     a0, a1, a2, lim, p)
+                                     a0, a1, a2, lim, p, saved)
         if ctx.pad:
             d = grad_output.shape[-1]
             dq, dk, dv = dq[..., :d], dk[..., :d], dv[..., :d]

@@ -64,10 +64,11 @@ fastmax_stream_t current_stream(const torch::Tensor& t) {
   return reinterpret_cast<fastmax_stream_t>(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream());
 }
 
-// (o, den, qk_scale, qk_argmax); o is (bh, n, d)
+// (o, den, qk_scale, qk_argmax, saved_states); o is (bh, n, d).  save_states keeps the prefix
+// states for backward_ex (a uint8 tensor; empty when not asked for)
 std::vector<torch::Tensor> forward_ex(torch::Tensor q, torch::Tensor k, torch::Tensor v, bool mask,
                                       bool normalize, double temperature, double a0, double a1,
-                                      double a2, double lim, int64_t p) {
+                                      double a2, double lim, int64_t p, bool save_states) {
   CHECK_INPUT(q);
   CHECK_INPUT(k);
   CHECK_INPUT(v);
@@ -81,18 +82,29 @@ std::vector<torch::Tensor> forward_ex(torch::Tensor q, torch::Tensor k, torch::T
   auto scale = torch::empty({2 * q.size(0)}, q.options().dtype(torch::kFloat32));
   auto arg = torch::empty({2 * q.size(0)}, q.options().dtype(torch::kInt32));
   size_t wsb = 0;
-  auto ws = workspace(ds, FASTMAX_PASS_FORWARD, q, &wsb);
-  raise_on(fastmax_forward(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ds.d,
-                           den.data_ptr<float>(), 1, scale.data_ptr<float>(), arg.data_ptr<int32_t>(),
-                           ws.data_ptr(), wsb, current_stream(q)));
-  return {o, den, scale, arg};
+  torch::Tensor ws, saved;
+  if (save_states) {
+    const size_t sb = fastmax_saved_state_bytes(&ds);
+    TORCH_CHECK(sb > 0, "fastmax: ", fastmax_last_error());
+    saved = torch::empty({(int64_t)sb}, q.options().dtype(torch::kUInt8));
+    wsb = (size_t)16 * ds.bh + 512;  // the per-head scalars only: the states go to `saved`
+    ws = torch::empty({(int64_t)wsb}, q.options().dtype(torch::kUInt8));
+  } else {
+    saved = torch::empty({0}, q.options().dtype(torch::kUInt8));
+    ws = workspace(ds, FASTMAX_PASS_FORWARD, q, &wsb);
+  }
+  raise_on(fastmax_forward_saving(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ds.d,
+                                  den.data_ptr<float>(), 1, scale.data_ptr<float>(), arg.data_ptr<int32_t>(),
+                                  ws.data_ptr(), wsb, save_states ? saved.data_ptr() : nullptr,
+                                  (size_t)saved.numel(), current_stream(q)));
+  return {o, den, scale, arg, saved};
 }
 
 std::vector<torch::Tensor> backward_ex(torch::Tensor q, torch::Tensor k, torch::Tensor v,
                                        torch::Tensor o, torch::Tensor den, torch::Tensor go,
                                        torch::Tensor scale, torch::Tensor arg, bool mask,
                                        bool normalize, double temperature, double a0, double a1,
-                                       double a2, double lim, int64_t p) {
+                                       double a2, double lim, int64_t p, torch::Tensor saved) {
   CHECK_INPUT(q);
   CHECK_INPUT(k);
   CHECK_INPUT(v);
@@ -116,10 +128,17 @@ std::vector<torch::Tensor> backward_ex(torch::Tensor q, torch::Tensor k, torch::
   auto dv = torch::empty_like(v);
   size_t wsb = 0;
   auto ws = workspace(ds, FASTMAX_PASS_BACKWARD, q, &wsb);
-  raise_on(fastmax_backward(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ds.d,
-                            den.data_ptr<float>(), 1, go.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                            dv.data_ptr(), scale.data_ptr<float>(), arg.data_ptr<int32_t>(),
-                            ws.data_ptr(), wsb, current_stream(q)));
+  const bool have_saved = saved.defined() && saved.numel() > 0;
+  if (have_saved) {
+    TORCH_CHECK(saved.is_cuda() && saved.is_contiguous() && saved.device() == q.device(),
+                "saved_states must be a contiguous tensor on q's device");
+  }
+  raise_on(fastmax_backward_saved(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ds.d,
+                                  den.data_ptr<float>(), 1, go.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                  dv.data_ptr(), scale.data_ptr<float>(), arg.data_ptr<int32_t>(),
+                                  ws.data_ptr(), wsb, have_saved ? saved.data_ptr() : nullptr,
+                                  have_saved ? (size_t)(saved.numel() * saved.element_size()) : 0,
+                                  current_stream(q)));
   return {dq, dk, dv};
 }
 
@@ -198,7 +217,7 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
 PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("forwardpass", &forwardpass, "forwardpass");
   m.def("backwardpass", &backwardpass, "backwardpass");
-  m.def("forward_ex", &forward_ex, "forward returning (o, den, qk_scale, qk_argmax)");
+  m.def("forward_ex", &forward_ex, "forward returning (o, den, qk_scale, qk_argmax, saved_states)");
   m.def("backward_ex", &backward_ex, "backward through the normalisation, returns [dq, dk, dv]");
   m.def("version", []() { return std::string(fastmax_version()); });
 }

@@ -148,8 +148,15 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
 // Heads per launch that fit the workspace.  When several batches are needed the batch is
 // rounded down so that the build grid (gsplit blocks per head, two resident blocks per CU)
 // is a whole number of rounds over the 256 CUs; a ragged last round would idle most of the chip.
-int heads_per_batch(const Plan& pl, size_t ws_bytes) {
-  size_t hb = (ws_bytes - pl.fixed_bytes) / pl.per_head_bytes;
+// (with_saved: the prefix states live in the caller's saved-state buffer, not in the workspace)
+size_t batch_bytes_per_head(const Plan& pl, bool with_saved) {
+  return pl.per_head_bytes - (with_saved ? (size_t)pl.nslots * pl.state_floats * sizeof(float) : 0);
+}
+
+int heads_per_batch(const Plan& pl, size_t ws_bytes, bool with_saved = false) {
+  const size_t per_head = batch_bytes_per_head(pl, with_saved);
+  if (per_head == 0) return pl.bh;
+  size_t hb = (ws_bytes - pl.fixed_bytes) / per_head;
   if (hb >= (size_t)pl.bh) return pl.bh;
   int g = pl.gsplit, m = 512;
   while (g % 2 == 0 && m > 1) {
@@ -181,12 +188,25 @@ int check_desc(const fastmax_desc* ds) {
   return FASTMAX_OK;
 }
 
-int check_ws(const Plan& pl, void* ws, size_t ws_bytes) {
+int check_ws(const Plan& pl, void* ws, size_t ws_bytes, bool with_saved = false) {
   if (!ws) return fail(FASTMAX_E_WORKSPACE, "workspace is NULL");
   if (((uintptr_t)ws) & 255) return fail(FASTMAX_E_WORKSPACE, "workspace is not 256-byte aligned");
-  const size_t need = pl.fixed_bytes + pl.ratio * pl.per_head_bytes;
+  const size_t need = pl.fixed_bytes + pl.ratio * batch_bytes_per_head(pl, with_saved);
   if (ws_bytes < need)
     return fail(FASTMAX_E_WORKSPACE, "workspace of %zu bytes is below the minimum of %zu", ws_bytes, need);
+  return FASTMAX_OK;
+}
+
+size_t saved_bytes_for(const Plan& pl) {
+  return (size_t)pl.bhkv * pl.nslots * pl.state_floats * sizeof(float);
+}
+
+int check_saved(const Plan& pl, const void* saved, size_t saved_bytes) {
+  if (!saved) return FASTMAX_OK;
+  if (((uintptr_t)saved) & 255) return fail(FASTMAX_E_WORKSPACE, "saved-state buffer is not 256-byte aligned");
+  if (saved_bytes < saved_bytes_for(pl))
+    return fail(FASTMAX_E_WORKSPACE, "saved-state buffer of %zu bytes is below the %zu needed", saved_bytes,
+                saved_bytes_for(pl));
   return FASTMAX_OK;
 }
 
@@ -262,12 +282,14 @@ int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float*
 template <int D, class T>
 int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k, const T* v, T* o,
                  int64_t ldo, float* den, int64_t den_stride, float* scale_out, int32_t* arg_out,
-                 char* ws, size_t ws_bytes, hipStream_t stream) {
+                 char* ws, size_t ws_bytes, float* saved, hipStream_t stream) {
   const int bh = pl.bh, n = pl.n;
   float* scale = reinterpret_cast<float*>(ws);
   int* arg = reinterpret_cast<int*>(ws + align256((size_t)2 * bh * sizeof(float)));
-  float* state = reinterpret_cast<float*>(ws + pl.fixed_bytes);
-  const int hb = heads_per_batch(pl, ws_bytes);
+  // the prefix states go to the workspace (one head batch at a time) or, when the caller keeps
+  // them for the backward pass, straight into its buffer (all heads)
+  const int hb = heads_per_batch(pl, ws_bytes, saved != nullptr);
+  const int64_t head_floats = (int64_t)pl.nslots * pl.state_floats;
 
   FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
   if (scale_out) hipMemcpyAsync(scale_out, scale, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);
@@ -279,8 +301,10 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
     const int64_t off = (int64_t)h0 * n * D;             // query-head tensors
     const int kv0 = h0 / ratio;                          // first key/value head of the batch
     const int64_t koff = (int64_t)kv0 * n * D;
+    float* state = saved ? saved + kv0 * head_floats : reinterpret_cast<float*>(ws + pl.fixed_bytes);
+    // (bf16: a saved state is also read by the dq kernel, which needs the column-packed section)
     FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr,
-                               state, 0, 1, stream)));
+                               state, 0, saved ? 3 : 1, stream)));
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       const dim3 agrid(pl.nblk, heads);
@@ -305,7 +329,7 @@ template <int D, class T>
 int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k, const T* v,
                   const T* o, int64_t ldo, const float* den, int64_t den_stride, const T* go, T* dq,
                   T* dk, T* dv, const float* scale_in, const int32_t* arg_in, char* ws,
-                  size_t ws_bytes, hipStream_t stream) {
+                  size_t ws_bytes, const float* saved, hipStream_t stream) {
   const int bh = pl.bh, n = pl.n;
   char* p = ws;
   float* scale = reinterpret_cast<float*>(p);
@@ -316,7 +340,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
   p += align256((size_t)bh * n * sizeof(float));
   float* rpart = reinterpret_cast<float*>(p);
   float* state = reinterpret_cast<float*>(ws + pl.fixed_bytes);
-  const int hb = heads_per_batch(pl, ws_bytes);
+  const int hb = heads_per_batch(pl, ws_bytes, saved != nullptr);
 
   if (scale_in && arg_in) {
     hipMemcpyAsync(scale, scale_in, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);
@@ -339,21 +363,23 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     const int64_t off = (int64_t)h0 * n * D;   // query-head tensors
     const int kv0 = h0 / ratio;                // first key/value head of the batch
     const int64_t koff = (int64_t)kv0 * n * D;
-    float* stS = state;
-    float* stR = state + (int64_t)hb * pl.nslots * pl.state_floats;
+    // prefix states: the ones the forward pass saved, or rebuilt into the workspace
+    const float* stS = saved ? saved + (int64_t)kv0 * pl.nslots * pl.state_floats : state;
+    float* stR = saved ? state : state + (int64_t)hb * pl.nslots * pl.state_floats;
     // grouped key/value heads: dk and dv per query head, added up over each group afterwards
     T* dk_q = dk + off;
     T* dv_q = dv + off;
     if (ratio > 1) {
-      char* tmp = reinterpret_cast<char*>(state) + 2 * hb * state_bytes;
+      char* tmp = reinterpret_cast<char*>(state) + (saved ? 1 : 2) * hb * state_bytes;
       dk_q = reinterpret_cast<T*>(tmp);
       dv_q = dk_q + (int64_t)hb * n * D;
     }
     const float* denh = den + (int64_t)h0 * n * den_stride;
     const float* ch = cvec + (int64_t)h0 * n;
     // prefix state of (kh, v, 1) per key/value head and suffix state of (qh, go/den, c) per query head
-    FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, stS, 0,
-                               2, stream)));
+    if (!saved)
+      FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state,
+                                 0, 2, stream)));
     FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, 3, stream)));
     const dim3 grid(pl.nblk, heads);
     {
@@ -519,22 +545,29 @@ size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass) {
   return pl.fixed_bytes + heads * pl.per_head_bytes;
 }
 
-int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
-                    int64_t ldo, float* den, int64_t den_stride, float* qk_scale,
-                    int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
-                    fastmax_stream_t stream) {
+size_t fastmax_saved_state_bytes(const fastmax_desc* desc) {
+  g_err[0] = 0;
+  if (check_desc(desc) != FASTMAX_OK) return 0;
+  return saved_bytes_for(make_plan(desc, FASTMAX_PASS_FORWARD));
+}
+
+int fastmax_forward_saving(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
+                           int64_t ldo, float* den, int64_t den_stride, float* qk_scale,
+                           int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                           void* saved_states, size_t saved_bytes, fastmax_stream_t stream) {
   g_err[0] = 0;
   FM_TRY(check_desc(desc));
   if (!q || !k || !v || !o || !den) return fail(FASTMAX_E_NULL, "q, k, v, o and den must be non-NULL");
   if (ldo < desc->d) return fail(FASTMAX_E_PARAM, "ldo = %lld < d = %d", (long long)ldo, desc->d);
   if (den_stride < 1) return fail(FASTMAX_E_PARAM, "den_stride = %lld < 1", (long long)den_stride);
   const Plan pl = make_plan(desc, FASTMAX_PASS_FORWARD);
-  FM_TRY(check_ws(pl, workspace, workspace_bytes));
+  FM_TRY(check_ws(pl, workspace, workspace_bytes, saved_states != nullptr));
+  FM_TRY(check_saved(pl, saved_states, saved_bytes));
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 #define FM_FWD(DD, TT)                                                                             \
   return forward_impl<DD, TT>(desc, pl, (const TT*)q, (const TT*)k, (const TT*)v, (TT*)o, ldo, den, \
-                              den_stride, qk_scale, qk_argmax, ws, workspace_bytes, st)
+                              den_stride, qk_scale, qk_argmax, ws, workspace_bytes, (float*)saved_states, st)
   if (desc->dtype == FASTMAX_F32) {
     if (desc->d == 64) FM_FWD(64, float);
     FM_FWD(32, float);
@@ -544,11 +577,19 @@ int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, cons
 #undef FM_FWD
 }
 
-int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, const void* v,
-                     const void* o, int64_t ldo, const float* den, int64_t den_stride,
-                     const void* go, void* dq, void* dk, void* dv, const float* qk_scale,
-                     const int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
-                     fastmax_stream_t stream) {
+int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
+                    int64_t ldo, float* den, int64_t den_stride, float* qk_scale,
+                    int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                    fastmax_stream_t stream) {
+  return fastmax_forward_saving(desc, q, k, v, o, ldo, den, den_stride, qk_scale, qk_argmax, workspace,
+                                workspace_bytes, nullptr, 0, stream);
+}
+
+int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                           const void* o, int64_t ldo, const float* den, int64_t den_stride,
+                           const void* go, void* dq, void* dk, void* dv, const float* qk_scale,
+                           const int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                           const void* saved_states, size_t saved_bytes, fastmax_stream_t stream) {
   g_err[0] = 0;
   FM_TRY(check_desc(desc));
   if (!q || !k || !v || !o || !den || !go || !dq || !dk || !dv)
@@ -556,13 +597,14 @@ int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, con
   if (ldo < desc->d) return fail(FASTMAX_E_PARAM, "ldo = %lld < d = %d", (long long)ldo, desc->d);
   if (den_stride < 1) return fail(FASTMAX_E_PARAM, "den_stride = %lld < 1", (long long)den_stride);
   const Plan pl = make_plan(desc, FASTMAX_PASS_BACKWARD);
-  FM_TRY(check_ws(pl, workspace, workspace_bytes));
+  FM_TRY(check_ws(pl, workspace, workspace_bytes, saved_states != nullptr));
+  FM_TRY(check_saved(pl, saved_states, saved_bytes));
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 #define FM_BWD(DD, TT)                                                                              \
   return backward_impl<DD, TT>(desc, pl, (const TT*)q, (const TT*)k, (const TT*)v, (const TT*)o, ldo, \
                                den, den_stride, (const TT*)go, (TT*)dq, (TT*)dk, (TT*)dv, qk_scale,  \
-                               qk_argmax, ws, workspace_bytes, st)
+                               qk_argmax, ws, workspace_bytes, (const float*)saved_states, st)
   if (desc->dtype == FASTMAX_F32) {
     if (desc->d == 64) FM_BWD(64, float);
     FM_BWD(32, float);
@@ -570,6 +612,15 @@ int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, con
   if (desc->d == 64) FM_BWD(64, bf16_t);
   FM_BWD(32, bf16_t);
 #undef FM_BWD
+}
+
+int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                     const void* o, int64_t ldo, const float* den, int64_t den_stride,
+                     const void* go, void* dq, void* dk, void* dv, const float* qk_scale,
+                     const int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                     fastmax_stream_t stream) {
+  return fastmax_backward_saved(desc, q, k, v, o, ldo, den, den_stride, go, dq, dk, dv, qk_scale, qk_argmax,
+                                workspace, workspace_bytes, nullptr, 0, stream);
 }
 
 int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k, void* workspace,

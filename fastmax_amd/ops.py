@@ -51,8 +51,10 @@ def _desc(q, k, mask, normalize, p, lim, temperature, a0, a1, a2):
 
 
 def forward(q, k, v, *, mask=False, normalize=False, lim=1.0, temperature=1.0, a0=1.0, a1=1.0, a2=0.5,
-            p=2, denominator_column: bool = False, workspace_bytes: Optional[int] = None):
-    """Returns (o, den, qk_scale, qk_argmax).
+            p=2, denominator_column: bool = False, workspace_bytes: Optional[int] = None,
+            save_states: bool = False):
+    """Returns (o, den, qk_scale, qk_argmax), plus the saved prefix states (a uint8 tensor to hand
+    to backward(saved_states=...), which then skips rebuilding them) when save_states is set.
 
     denominator_column=True gives the reference extension's layout: o is (bh, n, d+1) with the
     row denominators in column d (fastmax_cuda_forward.cu:353); den is then a view of it.
@@ -65,7 +67,12 @@ def forward(q, k, v, *, mask=False, normalize=False, lim=1.0, temperature=1.0, a
     if v.shape != k.shape:
         raise RuntimeError("fastmax: k and v must have the same shape")
     with torch.cuda.device(q.device):
-        nbytes = workspace_bytes or lib.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD)
+        saved = None
+        if save_states:
+            saved = torch.empty(lib.fastmax_saved_state_bytes(C.byref(ds)), dtype=torch.uint8, device=q.device)
+            nbytes = workspace_bytes or (64 * bh + 4096)  # only the per-head scalars live in the workspace
+        else:
+            nbytes = workspace_bytes or lib.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD)
         ws = _workspace(q.device, nbytes, 0)
         if denominator_column:
             if q.dtype != torch.float32:
@@ -80,16 +87,21 @@ def forward(q, k, v, *, mask=False, normalize=False, lim=1.0, temperature=1.0, a
         scale = torch.empty(2 * bh, dtype=torch.float32, device=q.device)
         arg = torch.empty(2 * bh, dtype=torch.int32, device=q.device)
         stream = torch.cuda.current_stream(q.device).cuda_stream
-        _cabi.check(lib.fastmax_forward(C.byref(ds), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
-                                        ldo, den_ptr, den_stride, scale.data_ptr(), arg.data_ptr(),
-                                        ws.data_ptr(), nbytes, stream))
+        _cabi.check(lib.fastmax_forward_saving(
+            C.byref(ds), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ldo, den_ptr, den_stride,
+            scale.data_ptr(), arg.data_ptr(), ws.data_ptr(), nbytes,
+            saved.data_ptr() if saved is not None else None, saved.numel() if saved is not None else 0, stream))
+    if save_states:
+        return o, den, scale, arg, saved
     return o, den, scale, arg
 
 
 def backward(q, k, v, o, den, go, *, mask=False, normalize=False, lim=1.0, temperature=1.0, a0=1.0,
              a1=1.0, a2=0.5, p=2, qk_scale: Optional[torch.Tensor] = None,
-             qk_argmax: Optional[torch.Tensor] = None, workspace_bytes: Optional[int] = None):
-    """Returns (dq, dk, dv).  o may be (bh,n,d) or (bh,n,d+1); den any strided (bh,n) fp32 view."""
+             qk_argmax: Optional[torch.Tensor] = None, workspace_bytes: Optional[int] = None,
+             saved_states: Optional[torch.Tensor] = None):
+    """Returns (dq, dk, dv).  o may be (bh,n,d) or (bh,n,d+1); den any strided (bh,n) fp32 view.
+    saved_states: what forward(save_states=True) returned for the same inputs."""
     _check_inputs(q, k, v, go)
     lib = _cabi.load()
     bh, n, d = q.shape
@@ -106,11 +118,13 @@ def backward(q, k, v, o, den, go, *, mask=False, normalize=False, lim=1.0, tempe
         dk = torch.empty_like(k)
         dv = torch.empty_like(v)
         stream = torch.cuda.current_stream(q.device).cuda_stream
-        _cabi.check(lib.fastmax_backward(
+        _cabi.check(lib.fastmax_backward_saved(
             C.byref(ds), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), o.stride(1), den.data_ptr(),
             den.stride(1), go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
             qk_scale.data_ptr() if qk_scale is not None else None,
-            qk_argmax.data_ptr() if qk_argmax is not None else None, ws.data_ptr(), nbytes, stream))
+            qk_argmax.data_ptr() if qk_argmax is not None else None, ws.data_ptr(), nbytes,
+            saved_states.data_ptr() if saved_states is not None else None,
+            saved_states.numel() if saved_states is not None else 0, stream))
     return dq, dk, dv
 
 

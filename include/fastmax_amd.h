@@ -111,6 +111,29 @@ int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, con
                      const float* qk_scale, const int32_t* qk_argmax,
                      void* workspace, size_t workspace_bytes, fastmax_stream_t stream);
 
+/* Keeping the prefix states for the backward pass (no counterpart in the reference, whose
+ * backward re-walks the sequence, fastmax_cuda_backward.cu:26-882).  The backward pass needs
+ * the same prefix states S of (k, v) the forward pass built; fastmax_backward rebuilds them
+ * (one of its three state builds).  A caller with memory to spare passes a buffer of
+ * fastmax_saved_state_bytes(desc) bytes (256-byte aligned; bhkv * slots * state bytes, 16 GB
+ * at bh = 1024, n = 10000, d = 64, p = 2) to fastmax_forward_saving, keeps it untouched, and
+ * hands it to fastmax_backward_saved, which then skips that build.  With saved_states == NULL
+ * the two calls are fastmax_forward / fastmax_backward.  When a buffer is given the workspace
+ * need not hold the prefix states: 16*bh + 512 bytes suffice for fastmax_forward_saving, and
+ * fastmax_backward_saved needs one state per head less. */
+size_t fastmax_saved_state_bytes(const fastmax_desc* desc);
+int fastmax_forward_saving(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                           void* o, int64_t ldo, float* den, int64_t den_stride,
+                           float* qk_scale, int32_t* qk_argmax,
+                           void* workspace, size_t workspace_bytes,
+                           void* saved_states, size_t saved_bytes, fastmax_stream_t stream);
+int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                           const void* o, int64_t ldo, const float* den, int64_t den_stride,
+                           const void* go, void* dq, void* dk, void* dv,
+                           const float* qk_scale, const int32_t* qk_argmax,
+                           void* workspace, size_t workspace_bytes,
+                           const void* saved_states, size_t saved_bytes, fastmax_stream_t stream);
+
 /* In-place q <- lim*q/max||q_n||, k likewise: the side effect the reference's forward has
  * on its inputs (calc_norms/find_max/apply_norm, fastmax_cuda_forward.cu:223-269,368-382,
  * with the PyTorch path's definition of the norm, example.py:105-108).  Only the legacy

@@ -301,3 +301,28 @@ def test_legacy_extension_entry_points(built):
         ext.forwardpass(qd.transpose(0, 1), kd, vd, qd, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
     with pytest.raises(RuntimeError, match="p must be 1 or 2"):
         ext.forwardpass(qd, kd, vd, qd, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 3)
+
+
+@pytest.mark.parametrize("bh,bhkv,n,d,mask,p,dtype", [
+    (4, 4, 900, 64, True, 2, torch.float32), (4, 4, 700, 64, False, 2, torch.float32),
+    (6, 2, 500, 32, True, 2, torch.float32), (4, 4, 1000, 64, True, 2, torch.bfloat16),
+    (4, 2, 300, 64, False, 2, torch.bfloat16), (3, 3, 400, 64, True, 1, torch.float32),
+])
+def test_saved_prefix_states_give_the_same_gradients(built, bh, bhkv, n, d, mask, p, dtype):
+    """forward(save_states) + backward(saved_states) skips one state build and must reproduce the
+    recomputing backward bit for bit (same kernels, same data)."""
+    from fastmax_amd import ops
+
+    q, _, _, go = O.seeded_inputs((bh, n, d), seed=51, dtype=dtype)
+    _, k, v, _ = O.seeded_inputs((bhkv, n, d), seed=52, dtype=dtype)
+    qd, kd, vd, god = (t.cuda() for t in (q, k, v, go))
+    kw = dict(mask=mask, normalize=True, p=p)
+    o, den, sc, arg = ops.forward(qd, kd, vd, **kw)
+    ref = ops.backward(qd, kd, vd, o, den, god, qk_scale=sc, qk_argmax=arg, **kw)
+    o2, den2, sc2, arg2, saved = ops.forward(qd, kd, vd, save_states=True, **kw)
+    assert torch.equal(o, o2) and torch.equal(den, den2)
+    got = ops.backward(qd, kd, vd, o2, den2, god, qk_scale=sc2, qk_argmax=arg2, saved_states=saved, **kw)
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
+    with pytest.raises(Exception, match="saved-state buffer"):
+        ops.backward(qd, kd, vd, o2, den2, god, saved_states=saved[: saved.numel() // 2], **kw)
