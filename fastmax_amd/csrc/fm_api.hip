@@ -284,16 +284,15 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
                  int64_t ldo, float* den, int64_t den_stride, float* scale_out, int32_t* arg_out,
                  char* ws, size_t ws_bytes, float* saved, hipStream_t stream) {
   const int bh = pl.bh, n = pl.n;
-  float* scale = reinterpret_cast<float*>(ws);
-  int* arg = reinterpret_cast<int*>(ws + align256((size_t)2 * bh * sizeof(float)));
+  // per-head factors and arg-max rows: straight into the caller's arrays when it wants them
+  float* scale = scale_out ? scale_out : reinterpret_cast<float*>(ws);
+  int* arg = arg_out ? arg_out : reinterpret_cast<int*>(ws + align256((size_t)2 * bh * sizeof(float)));
   // the prefix states go to the workspace (one head batch at a time) or, when the caller keeps
   // them for the backward pass, straight into its buffer (all heads)
   const int hb = heads_per_batch(pl, ws_bytes, saved != nullptr);
   const int64_t head_floats = (int64_t)pl.nslots * pl.state_floats;
 
   FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
-  if (scale_out) hipMemcpyAsync(scale_out, scale, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);
-  if (arg_out) hipMemcpyAsync(arg_out, arg, (size_t)2 * bh * sizeof(int), hipMemcpyDeviceToDevice, stream);
 
   const int ratio = pl.ratio;
   for (int h0 = 0; h0 < bh; h0 += hb) {
@@ -332,9 +331,12 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
                   size_t ws_bytes, const float* saved, hipStream_t stream) {
   const int bh = pl.bh, n = pl.n;
   char* p = ws;
-  float* scale = reinterpret_cast<float*>(p);
+  const bool given = scale_in && arg_in;  // the forward pass's values: read in place
+  const float* scale = given ? scale_in : reinterpret_cast<float*>(p);
+  float* scale_ws = reinterpret_cast<float*>(p);
   p += align256((size_t)2 * bh * sizeof(float));
-  int* arg = reinterpret_cast<int*>(p);
+  const int* arg = given ? arg_in : reinterpret_cast<int*>(p);
+  int* arg_ws = reinterpret_cast<int*>(p);
   p += align256((size_t)2 * bh * sizeof(int));
   float* cvec = reinterpret_cast<float*>(p);
   p += align256((size_t)bh * n * sizeof(float));
@@ -342,12 +344,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
   float* state = reinterpret_cast<float*>(ws + pl.fixed_bytes);
   const int hb = heads_per_batch(pl, ws_bytes, saved != nullptr);
 
-  if (scale_in && arg_in) {
-    hipMemcpyAsync(scale, scale_in, (size_t)2 * bh * sizeof(float), hipMemcpyDeviceToDevice, stream);
-    hipMemcpyAsync(arg, arg_in, (size_t)2 * bh * sizeof(int), hipMemcpyDeviceToDevice, stream);
-  } else {
-    FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
-  }
+  if (!given) FM_TRY(compute_scales<T>(ds, q, k, scale_ws, arg_ws, stream));
   {
     const int64_t rows = (int64_t)bh * n;
     const int rpp = 256 / (D / 4);
