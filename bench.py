@@ -233,6 +233,13 @@ def main() -> int:
         "frac": achieved / peak, "traffic": None,
         "flops_per_launch": per_step_flops[dom] / launches, "avg_launch_ms": dom_ms / launches,
     }
+    # what the build kernel really executes (the pair symmetry halves the order-2 rows): row-tile
+    # slots per head x 32 rows x d columns MACs per token
+    if dom == "build" and cfg["p"] == 2:
+        slots = {64: 72, 32: 20}[D]  # 6 blocks x 4 waves x 3 tiles; 1 block x 4 waves x 5 tiles
+        executed = 2.0 * slots * 32 * D * token_heads * n_builds / (dom_ms * 1e-3) / 1e12
+        roofline["executed_tflops"] = executed
+        roofline["executed_frac"] = executed / peak
     per_th = MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD.get(args.workload if not args.batch else "", {}).get(dom)
     if per_th is not None:
         n_states = n_builds if dom == "build" else 1
