@@ -151,11 +151,13 @@ def fastmax_bruteforce(q, k, v, mask=False, normalize=False, a0=1.0, a1=1.0, a2=
     k = k.double()
     v = v.double()
     B, H, N, D = q.shape
+    NK = k.shape[2]          # NK > N: the first NK - N keys are visible to every query
+    shift = NK - N           # (fastmax_cuda_forward.cu:109-150)
     out = torch.zeros(B, H, N, D, dtype=torch.float64)
     for b in range(B):
         for h in range(H):
             qq = [[float(q[b, h, i, c]) for c in range(D)] for i in range(N)]
-            kk = [[float(k[b, h, i, c]) for c in range(D)] for i in range(N)]
+            kk = [[float(k[b, h, i, c]) for c in range(D)] for i in range(NK)]
             if normalize:
                 mq = max(math.sqrt(sum(x * x for x in row)) for row in qq)
                 mk = max(math.sqrt(sum(x * x for x in row)) for row in kk)
@@ -164,8 +166,8 @@ def fastmax_bruteforce(q, k, v, mask=False, normalize=False, a0=1.0, a1=1.0, a2=
             for i in range(N):
                 num = [0.0] * D
                 den = 0.0
-                for j in range(N):
-                    if mask and j > i:
+                for j in range(NK):
+                    if mask and j > i + shift:
                         continue
                     s = sum(qq[i][c] * kk[j][c] for c in range(D))
                     f = a0 + a1 * s + (a2 * s * s if p == 2 else 0.0)

@@ -160,3 +160,23 @@ def test_three_d_layout_matches_four_d():
     d3 = O.fastmax_grads_closed(*(t.reshape(6, 7, 4) for t in (q, k, v, go)), **kw)
     for a, b in zip(d4, d3):
         torch.testing.assert_close(a.reshape(6, 7, 4), b)
+
+
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("normalize", [False, True])
+def test_key_prefix_dense_equals_bruteforce(mask, normalize):
+    """nk > nq: the first nk - nq keys are visible to every query (fastmax_cuda_forward.cu:109-150)."""
+    q, _, _, _ = O.seeded_inputs((2, 2, 3, 2), seed=61, dtype=torch.float64)
+    _, k, v, _ = O.seeded_inputs((2, 2, 5, 2), seed=62, dtype=torch.float64)
+    a = O.fastmax_dense(q, k, v, mask=mask, normalize=normalize)
+    b = O.fastmax_bruteforce(q, k, v, mask=mask, normalize=normalize)
+    assert torch.allclose(a, b, rtol=1e-11, atol=1e-12)
+
+
+def test_key_prefix_is_the_tail_of_a_longer_causal_pass():
+    """Without the (non-causal) normaliser, queries nk-nq.. of a full causal pass see exactly
+    what the prefix form shows them."""
+    q, k, v, _ = O.seeded_inputs((1, 2, 9, 4), seed=63, dtype=torch.float64)
+    full = O.fastmax_dense(q, k, v, mask=True, normalize=False)
+    tail = O.fastmax_dense(q[:, :, 4:], k, v, mask=True, normalize=False)
+    assert torch.allclose(full[:, :, 4:], tail, rtol=1e-12, atol=1e-13)

@@ -326,3 +326,28 @@ def test_saved_prefix_states_give_the_same_gradients(built, bh, bhkv, n, d, mask
         assert torch.equal(a, b)
     with pytest.raises(Exception, match="saved-state buffer"):
         ops.backward(qd, kd, vd, o2, den2, god, saved_states=saved[: saved.numel() // 2], **kw)
+
+
+@pytest.mark.parametrize("nq,nk,d,mask,p,a0", [(200, 330, 64, True, 2, 1.0), (130, 131, 32, True, 2, 1.0),
+                                               (100, 400, 64, False, 2, 1.0), (257, 300, 64, True, 1, 1.0),
+                                               (150, 260, 64, True, 2, 0.0)])
+def test_module_key_prefix(built, nq, nk, d, mask, p, a0):
+    """k, v longer than q: the first nk - nq keys are visible to every query
+    (fastmax_cuda_forward.cu:109-150); a0 = 0 makes the padding rows' denominators vanish."""
+    from fastmax_amd import FASTMultiHeadAttention
+
+    b, h = 1, 3
+    q, _, _, go = O.seeded_inputs((b, h, nq, d), seed=71)
+    _, k, v, _ = O.seeded_inputs((b, h, nk, d), seed=72)
+    a1, a2 = (1.0, 0.5) if a0 else (0.3, 1.0)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = FASTMultiHeadAttention()(qd, kd, vd, None, mask, 0.0, True, 1.0, a0, a1, a2, 1.0, p)
+    assert o.shape == q.shape
+    o.backward(go.cuda())
+    ro, rdq, rdk, rdv = O.dense_truth(q, k, v, go, mask=mask, normalize=True, a0=a0, a1=a1, a2=a2, p=p)
+    for name, got, ref in (("o", o, ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+        assert got.shape == ref.shape
+        assert torch.isfinite(got).all()
+        assert_close(name, got, ref, 1e-4)
+    with pytest.raises(ValueError, match="fewer keys"):
+        FASTMultiHeadAttention()(kd, qd, qd, None, mask, 0.0, True)
