@@ -59,8 +59,8 @@ def test_golden_vectors(ops, name):
 @pytest.mark.parametrize("d", [32, 64])
 @pytest.mark.parametrize("mask", [False, True])
 @pytest.mark.parametrize("p", [1, 2])
-@pytest.mark.parametrize("n", [1, 31, 128, 257, 700])
-def test_shapes_fp32(ops, d, mask, p, n):
+@pytest.mark.parametrize("n", [1, 31, 128, 257, 383, 384, 385, 700, 769])  # around the 128-token block and
+def test_shapes_fp32(ops, d, mask, p, n):                                  # the 384-token chunk
     run_case(ops, (3, n, d), seed=n + d, mask=mask, normalize=True, p=p)
 
 
@@ -102,6 +102,8 @@ def test_temperature_divides_keys_when_not_normalising(ops):
 def test_bf16_inputs(ops, mask):
     run_case(ops, (2, 600, 64), dtype=torch.bfloat16, seed=11, mask=mask, normalize=True, p=2)
     run_case(ops, (2, 300, 32), dtype=torch.bfloat16, seed=12, mask=mask, normalize=True, p=1)
+    for n in (1, 33, 384, 385, 1153):
+        run_case(ops, (3, n, 64), dtype=torch.bfloat16, seed=13 + n, mask=mask, normalize=True, p=2)
 
 
 def test_deterministic_and_independent_of_head_batching(ops, built):
