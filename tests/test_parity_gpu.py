@@ -102,7 +102,7 @@ def test_temperature_divides_keys_when_not_normalising(ops):
 def test_bf16_inputs(ops, mask):
     run_case(ops, (2, 600, 64), dtype=torch.bfloat16, seed=11, mask=mask, normalize=True, p=2)
     run_case(ops, (2, 300, 32), dtype=torch.bfloat16, seed=12, mask=mask, normalize=True, p=1)
-    for n in (1, 33, 384, 385, 1153):
+    for n in (33, 384, 385, 1153):  # (n = 1 has zero true dq, dk: nothing to compare a bf16 result with)
         run_case(ops, (3, n, 64), dtype=torch.bfloat16, seed=13 + n, mask=mask, normalize=True, p=2)
 
 
