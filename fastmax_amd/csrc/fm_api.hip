@@ -51,11 +51,11 @@ struct ScopedKernel {
       g_prof.ev.push_back(b);
     }
     g_prof.cls.push_back(kclass);
-    hipEventRecord(g_prof.ev[g_prof.used], st);
+    (void)hipEventRecord(g_prof.ev[g_prof.used], st);
   }
   ~ScopedKernel() {
     if (!on) return;
-    hipEventRecord(g_prof.ev[g_prof.used + 1], st);
+    (void)hipEventRecord(g_prof.ev[g_prof.used + 1], st);
     g_prof.used += 2;
   }
 };
