@@ -418,45 +418,54 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     }
   };
 
-  // one slab: B operands are 64-bit reads of [feature group][column][4 features], fetched one
-  // group ahead of the MFMAs that use them
+  // one slab: B operands are 64-bit reads of [feature group][column][4 features]; two feature
+  // groups (8 features per lane half) make one k = 16 MFMA.  Operands are fetched one step ahead
+  // of the MFMAs that use them.
   auto slab_compute = [&](const uint16_t* sl, auto tag) {
     constexpr bool ORD2 = decltype(tag)::value;
     constexpr int NB = FWD ? CB + 1 : CB;
+    constexpr int NM = H2 / 8;  // MFMA steps per column tile
     const uint16_t* brow = sl + (hh * (H2 / 4) * NCF + i) * 4;
     const uint16_t* erow = sl + (hh * (H2 / 4) * NCF + D) * 4;
-    auto fetch = [&](int g4, uint2 (&b)[NB]) {
+    auto fetch = [&](int m, uint2 (&b)[2 * NB]) {
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) b[cb] = *reinterpret_cast<const uint2*>(brow + (g4 * NCF + cb * 32) * 4);
-      if (FWD) b[NB - 1] = *reinterpret_cast<const uint2*>(erow + g4 * NCF * 4);
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+          b[2 * cb + u] = *reinterpret_cast<const uint2*>(brow + ((2 * m + u) * NCF + cb * 32) * 4);
+        if (FWD) b[2 * (NB - 1) + u] = *reinterpret_cast<const uint2*>(erow + (2 * m + u) * NCF * 4);
+      }
     };
     auto feat = [&](int g4) {
       const int t = 4 * g4;
-      return ORD2 ? pack_bf4(Xr[t] * Wn[t], Xr[t + 1] * Wn[t + 1], Xr[t + 2] * Wn[t + 2], Xr[t + 3] * Wn[t + 3])
-                  : pack_bf4(Xr[t] * a1, Xr[t + 1] * a1, Xr[t + 2] * a1, Xr[t + 3] * a1);
+      return ORD2 ? pack_bf4u(Xr[t] * Wn[t], Xr[t + 1] * Wn[t + 1], Xr[t + 2] * Wn[t + 2], Xr[t + 3] * Wn[t + 3])
+                  : pack_bf4u(Xr[t] * a1, Xr[t + 1] * a1, Xr[t + 2] * a1, Xr[t + 3] * a1);
     };
-    uint2 bc[NB], bn[NB];
+    uint2 bc[2 * NB], bn[2 * NB];
     fetch(0, bc);
-    s4v apc = feat(0), apn = apc;
+    uint2 alo = feat(0), ahi = feat(1), nlo = alo, nhi = ahi;
 #pragma unroll
-    for (int g4 = 0; g4 < H2 / 4; ++g4) {
-      if (g4 + 1 < H2 / 4) {
-        fetch(g4 + 1, bn);
-        apn = feat(g4 + 1);
+    for (int m = 0; m < NM; ++m) {
+      if (m + 1 < NM) {
+        fetch(m + 1, bn);
+        nlo = feat(2 * m + 2);
+        nhi = feat(2 * m + 3);
       }
+      const bf8v ap = as_bf8(alo, ahi);
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA_BF(apc, as_s4v(bc[cb]), acc[cb]);
-      if (FWD) accd = FM_MFMA_BF(apc, as_s4v(bc[NB - 1]), accd);
-      // interleave: each MFMA is followed by one of the next group's LDS reads and two of its VALU ops
+      for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA_BF16(ap, as_bf8(bc[2 * cb], bc[2 * cb + 1]), acc[cb]);
+      if (FWD) accd = FM_MFMA_BF16(ap, as_bf8(bc[2 * (NB - 1)], bc[2 * (NB - 1) + 1]), accd);
+      // interleave: each MFMA is followed by two of the next step's LDS reads and four of its VALU ops
 #pragma unroll
       for (int x = 0; x < NB; ++x) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
       }
 #pragma unroll
-      for (int x = 0; x < NB; ++x) bc[x] = bn[x];
-      apc = apn;
+      for (int x = 0; x < 2 * NB; ++x) bc[x] = bn[x];
+      alo = nlo;
+      ahi = nhi;
     }
   };
 
@@ -510,10 +519,10 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   }
 
   if (n_tile > 0) {
-    s4v Xp[H2 / 4];
+    uint2 Xp[H2 / 4];
 #pragma unroll
-    for (int g4 = 0; g4 < H2 / 4; ++g4) Xp[g4] = pack_bf4(Xr[4 * g4], Xr[4 * g4 + 1], Xr[4 * g4 + 2], Xr[4 * g4 + 3]);
-    const s4v ones = as_s4v(make_uint2(0x3f803f80u, 0x3f803f80u));
+    for (int g4 = 0; g4 < H2 / 4; ++g4) Xp[g4] = pack_bf4u(Xr[4 * g4], Xr[4 * g4 + 1], Xr[4 * g4 + 2], Xr[4 * g4 + 3]);
+    const bf8v ones = as_bf8(make_uint2(0x3f803f80u, 0x3f803f80u), make_uint2(0x3f803f80u, 0x3f803f80u));
     const int mine = (tok0 >> 5) + w;
     for (int kk = 0; kk < n_tile; ++kk) {
       const int buf = (n_state + kk) & 1;
@@ -526,8 +535,10 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
 #pragma unroll
         for (int r = 0; r < 16; ++r) sc[r] = 0.f;
 #pragma unroll
-        for (int g4 = 0; g4 < H2 / 4; ++g4)
-          sc = FM_MFMA_BF(as_s4v(*reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 4 * g4)), Xp[g4], sc);
+        for (int m = 0; m < H2 / 8; ++m)
+          sc = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 8 * m),
+                                   *reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 8 * m + 4)),
+                            as_bf8(Xp[2 * m], Xp[2 * m + 1]), sc);
         const bool diag = tl == mine;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -536,13 +547,19 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
           if (diag && (FWD ? trow(r, hh) > i : trow(r, hh) < i)) f = 0.f;
           sc[r] = f;
         }
+        // accumulator rows 8m..8m+7 of this lane half (tokens 16m + 4hh + {0..3} and + 8) are the
+        // eight k slots of one MFMA; the transposed value tile supplies the same tokens
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const s4v pp = pack_bf4(sc[4 * j], sc[4 * j + 1], sc[4 * j + 2], sc[4 * j + 3]);
+        for (int m = 0; m < 2; ++m) {
+          const bf8v pp = as_bf8(pack_bf4u(sc[8 * m], sc[8 * m + 1], sc[8 * m + 2], sc[8 * m + 3]),
+                                 pack_bf4u(sc[8 * m + 4], sc[8 * m + 5], sc[8 * m + 6], sc[8 * m + 7]));
 #pragma unroll
-          for (int cb = 0; cb < CB; ++cb)
-            acc[cb] = FM_MFMA_BF(pp, as_s4v(*reinterpret_cast<const uint2*>(l2 + (cb * 32 + i) * TPB + 8 * j + 4 * hh)), acc[cb]);
-          if (FWD) accd = FM_MFMA_BF(pp, ones, accd);
+          for (int cb = 0; cb < CB; ++cb) {
+            const uint16_t* vrow = l2 + (cb * 32 + i) * TPB + 16 * m + 4 * hh;
+            acc[cb] = FM_MFMA_BF16(pp, as_bf8(*reinterpret_cast<const uint2*>(vrow),
+                                              *reinterpret_cast<const uint2*>(vrow + 8)), acc[cb]);
+          }
+          if (FWD) accd = FM_MFMA_BF16(pp, ones, accd);
         }
       }
       if (kk + 1 < n_tile) tiles_store(buf ^ 1);

@@ -25,6 +25,12 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 typedef short s4v __attribute__((ext_vector_type(4)));
 typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
 #define FM_MFMA_BF(a, b, c) __builtin_amdgcn_mfma_f32_32x32x8bf16_1k((a), (b), (c), 0, 0, 0)
+// v_mfma_f32_32x32x16_bf16: eight bf16 per lane, k = 8*(l/32) + {0..7}; issues at the rate of
+// the k = 8 form (measured ~35 cycles), i.e. twice its throughput.  Because the k index of A and
+// B may be permuted together, two k = 8 operand pairs (each the four k-slots of a lane) are
+// simply concatenated: slots 0..3 from the first pair, 4..7 from the second.
+typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
+#define FM_MFMA_BF16(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
 
 __device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
   const bf2v p = {(__bf16)lo, (__bf16)hi};  // round to nearest even (v_cvt_pk_bf16_f32)
@@ -35,6 +41,13 @@ __device__ __forceinline__ s4v pack_bf4(float a, float b, float c, float d) {
   return __builtin_bit_cast(s4v, u);
 }
 __device__ __forceinline__ s4v as_s4v(uint2 u) { return __builtin_bit_cast(s4v, u); }
+__device__ __forceinline__ bf8v as_bf8(uint2 lo, uint2 hi) {
+  const uint4 u = make_uint4(lo.x, lo.y, hi.x, hi.y);
+  return __builtin_bit_cast(bf8v, u);
+}
+__device__ __forceinline__ uint2 pack_bf4u(float a, float b, float c, float d) {
+  return make_uint2(pack_bf2(a, b), pack_bf2(c, d));
+}
 __device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 

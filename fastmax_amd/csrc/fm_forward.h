@@ -237,6 +237,9 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     const float* kb = Kt[buf];
     const float* eb = El[buf];
     GroupOps cur, nxt;
+    // BF: the packed operands of an even group wait for the odd group that follows, and the two
+    // go into one k = 16 MFMA
+    uint2 ap_even[RTW], vb_even[BF ? CB : 1];
     fetch(kb, buf, eb, 4 * h, cur);
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
@@ -248,9 +251,14 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
         const float a0 = cur.own[x].x * cur.rot[x].x, a1 = cur.own[x].y * cur.rot[x].y;
         const float a2 = cur.own[x].z * cur.rot[x].z, a3 = cur.own[x].w * cur.rot[x].w;
         if constexpr (BF) {
-          const s4v ap = pack_bf4(a0, a1, a2, a3);
+          const uint2 ap = pack_bf4u(a0, a1, a2, a3);
+          if ((gq & 1) == 0) {
+            ap_even[x] = ap;
+          } else {
 #pragma unroll
-          for (int cb = 0; cb < CB; ++cb) acc[x][cb] = FM_MFMA_BF(ap, as_s4v(cur.vb[cb]), acc[x][cb]);
+            for (int cb = 0; cb < CB; ++cb)
+              acc[x][cb] = FM_MFMA_BF16(as_bf8(ap_even[x], ap), as_bf8(vb_even[cb], cur.vb[cb]), acc[x][cb]);
+          }
         } else {
 #pragma unroll
           for (int cb = 0; cb < CB; ++cb) {
@@ -261,6 +269,12 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
           }
         }
         dacc[x] += a0 * cur.e4.x + a1 * cur.e4.y + a2 * cur.e4.z + a3 * cur.e4.w;
+      }
+      if constexpr (BF) {
+        if ((gq & 1) == 0) {
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) vb_even[cb] = cur.vb[cb];
+        }
       }
       if (gq + 1 < 4) cur = nxt;
     }

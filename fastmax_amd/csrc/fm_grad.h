@@ -359,13 +359,14 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   __syncthreads();
   // own token of this lane = row xrow: its half of y, packed (A operand of the state
   // contraction, B operand of g.v)
-  s4v Yp[H2 / 4];
+  uint2 Yp[H2 / 4];
 #pragma unroll
   for (int g4 = 0; g4 < H2 / 4; ++g4)
-    Yp[g4] = as_s4v(*reinterpret_cast<const uint2*>(&Sb[0][0] + xrow * LB + hh * H2 + 4 * g4));
+    Yp[g4] = *reinterpret_cast<const uint2*>(&Sb[0][0] + xrow * LB + hh * H2 + 4 * g4);
   const float c_own = (DQ && tok < n) ? ch[tok] : 0.f;
   const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
-  const s4v yxp = pack_bf4(yxhi, yx - yxhi, yxhi, yx - yxhi);  // pairs with (e_hi, e_hi, e_lo, e_lo)
+  // pairs with (e_hi, e_hi, e_lo, e_lo); the upper four k slots of that MFMA are empty
+  const bf8v yxp = as_bf8(pack_bf4u(yxhi, yx - yxhi, yxhi, yx - yxhi), make_uint2(0u, 0u));
   __syncthreads();
 
   const bool no_state = masked && (DQ ? c == 0 : c == nc - 1);
@@ -446,8 +447,8 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
 #pragma unroll
     for (int r = 0; r < 16; ++r) t[r] = 0.f;
 #pragma unroll
-    for (int g4 = 0; g4 < H2 / 4; ++g4) t = FM_MFMA_BF(Yp[g4], as_s4v(b[g4]), t);
-    return FM_MFMA_BF(yxp, as_s4v(b[H2 / 4]), t);
+    for (int m = 0; m < H2 / 8; ++m) t = FM_MFMA_BF16(as_bf8(Yp[2 * m], Yp[2 * m + 1]), as_bf8(b[2 * m], b[2 * m + 1]), t);
+    return FM_MFMA_BF16(yxp, as_bf8(b[H2 / 4], make_uint2(0u, 0u)), t);
   };
   const float* xtok = Xl + (w * 32 + 4 * hh) * LD;
   auto xat = [&](int r, int col) { return xtok[((r >> 2) * 8 + (r & 3)) * LD + col]; };
@@ -515,11 +516,11 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   }
 
   if (n_tile > 0) {
-    s4v Xp[H2 / 4];
+    uint2 Xp[H2 / 4];
 #pragma unroll
     for (int g4 = 0; g4 < H2 / 4; ++g4) {
       const float4 x4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + hh * H2 + 4 * g4);
-      Xp[g4] = pack_bf4(x4.x, x4.y, x4.z, x4.w);
+      Xp[g4] = pack_bf4u(x4.x, x4.y, x4.z, x4.w);
     }
     const int mine = (tok0 >> 5) + w;
     const float twoa2 = 2.0f * a2;
@@ -535,9 +536,13 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
 #pragma unroll
         for (int r = 0; r < 16; ++r) sc[r] = gv[r] = 0.f;
 #pragma unroll
-        for (int g4 = 0; g4 < H2 / 4; ++g4) {
-          sc = FM_MFMA_BF(as_s4v(*reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 4 * g4)), Xp[g4], sc);
-          gv = FM_MFMA_BF(as_s4v(*reinterpret_cast<const uint2*>(l2 + i * LB + hh * H2 + 4 * g4)), Yp[g4], gv);
+        for (int m = 0; m < H2 / 8; ++m) {
+          const uint16_t* r1 = l1 + i * LB + hh * H2 + 8 * m;
+          const uint16_t* r2 = l2 + i * LB + hh * H2 + 8 * m;
+          sc = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(r1), *reinterpret_cast<const uint2*>(r1 + 4)),
+                            as_bf8(Xp[2 * m], Xp[2 * m + 1]), sc);
+          gv = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(r2), *reinterpret_cast<const uint2*>(r2 + 4)),
+                            as_bf8(Yp[2 * m], Yp[2 * m + 1]), gv);
         }
         const bool diag = tl == mine;
 #pragma unroll
@@ -548,11 +553,16 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
           sc[r] = wv;
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const s4v wp = pack_bf4(sc[4 * j], sc[4 * j + 1], sc[4 * j + 2], sc[4 * j + 3]);
+        for (int m = 0; m < 2; ++m) {
+          // accumulator rows 8m..8m+7 of this lane half = tokens 16m + 4hh + {0..3} and + 8
+          const bf8v wp = as_bf8(pack_bf4u(sc[8 * m], sc[8 * m + 1], sc[8 * m + 2], sc[8 * m + 3]),
+                                 pack_bf4u(sc[8 * m + 4], sc[8 * m + 5], sc[8 * m + 6], sc[8 * m + 7]));
 #pragma unroll
-          for (int ab = 0; ab < AB; ++ab)
-            out[ab] = FM_MFMA_BF(wp, as_s4v(*reinterpret_cast<const uint2*>(l1t + (ab * 32 + i) * TPB + 8 * j + 4 * hh)), out[ab]);
+          for (int ab = 0; ab < AB; ++ab) {
+            const uint16_t* trw = l1t + (ab * 32 + i) * TPB + 16 * m + 4 * hh;
+            out[ab] = FM_MFMA_BF16(wp, as_bf8(*reinterpret_cast<const uint2*>(trw), *reinterpret_cast<const uint2*>(trw + 8)),
+                                   out[ab]);
+          }
         }
       }
       if (kk + 1 < n_tile) tiles_store(buf ^ 1);
