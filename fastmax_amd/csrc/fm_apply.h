@@ -281,7 +281,7 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
 
 // ---------------------------------------------------------------------------------------
 // bf16 variant of apply_kernel (bf16 inputs and outputs): same decomposition, but every
-// contraction runs on v_mfma_f32_32x32x8_bf16 with fp32 accumulation.  Features are formed in
+// contraction runs on v_mfma_f32_32x32x16_bf16 with fp32 accumulation.  Features are formed in
 // fp32 from the fp32-scaled inputs and rounded when packed.  The state arrives in the packed
 // bf16 form (PackedGeo): a feature-packed slab is copied to LDS as it is and the four features
 // of a lane's k-slots are one 64-bit LDS read; the order-2 slabs carry their pair weights, a2

@@ -17,14 +17,12 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 
 #define FM_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
 
-// bf16 matrix instruction used when the inputs are bf16: v_mfma_f32_32x32x8_bf16, fp32 accumulate.
-//   A (32 x 8): row l%32, k = 4*(l/32) + {0,1,2,3}  -> four bf16 per lane (s4v)
+// bf16 matrix instructions (fp32 accumulate).  Operands are built in the k = 8 layout,
+//   A (32 x 8): row l%32, k = 4*(l/32) + {0,1,2,3}  -> four bf16 per lane
 //   B (8 x 32): col l%32, k = 4*(l/32) + {0,1,2,3}
 //   D (32 x 32): as for the fp32 instruction
-// One of these replaces four fp32 MFMAs whose k indices were 2*u + l/32, u = 0..3.
-typedef short s4v __attribute__((ext_vector_type(4)));
+// where one operand pair replaces four fp32 MFMAs whose k indices were 2*u + l/32, u = 0..3.
 typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
-#define FM_MFMA_BF(a, b, c) __builtin_amdgcn_mfma_f32_32x32x8bf16_1k((a), (b), (c), 0, 0, 0)
 // v_mfma_f32_32x32x16_bf16: eight bf16 per lane, k = 8*(l/32) + {0..7}; issues at the rate of
 // the k = 8 form (measured ~35 cycles), i.e. twice its throughput.  Because the k index of A and
 // B may be permuted together, two k = 8 operand pairs (each the four k-slots of a lane) are
@@ -36,11 +34,6 @@ __device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
   const bf2v p = {(__bf16)lo, (__bf16)hi};  // round to nearest even (v_cvt_pk_bf16_f32)
   return __builtin_bit_cast(uint32_t, p);
 }
-__device__ __forceinline__ s4v pack_bf4(float a, float b, float c, float d) {
-  const uint2 u = make_uint2(pack_bf2(a, b), pack_bf2(c, d));
-  return __builtin_bit_cast(s4v, u);
-}
-__device__ __forceinline__ s4v as_s4v(uint2 u) { return __builtin_bit_cast(s4v, u); }
 __device__ __forceinline__ bf8v as_bf8(uint2 lo, uint2 hi) {
   const uint4 u = make_uint4(lo.x, lo.y, hi.x, hi.y);
   return __builtin_bit_cast(bf8v, u);
@@ -145,8 +138,8 @@ struct Geo {
 // Packed bf16 form of a state, used when the inputs are bf16 (it occupies the same
 // state_floats slot as the fp32 form).  A "slab" is the D feature rows of one shift s
 // (order 2; rows carry their pair weight: x2 for 0 < s < D/2) or the D order-1 rows (slab
-// NS, or slab 0 when p == 1).  Each slab is stored twice, in the two operand layouts of
-// v_mfma_f32_32x32x8_bf16, so that consumers stage it with plain 16-byte copies:
+// NS, or slab 0 when p == 1).  Each slab is stored twice, in the two operand layouts of the
+// bf16 matrix instruction, so that consumers stage it with plain 16-byte copies:
 //   F, feature-packed  [a/4][column 0..D (+1 pad)][a%4]   contraction over features (apply)
 //   C, column-packed   [a][LB = D+4]                        contraction over columns (grad);
 //      columns D..D+3 hold the extra column as (hi, hi, lo, lo) bf16 pairs

@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 
 // ---------------------------------------------------------------------------------------
 // bf16 variant of grad_kernel (bf16 inputs and outputs): every contraction runs on
-// v_mfma_f32_32x32x8_bf16 with fp32 accumulation.  The state arrives in the packed bf16 form
+// v_mfma_f32_32x32x16_bf16 with fp32 accumulation.  The state arrives in the packed bf16 form
 // (PackedGeo): a column-packed slab ([row][column], unweighted, extra column split into hi + lo
 // parts) is copied to LDS as it is; 2*a2 multiplies the accumulated order-2 credits and a1 the
 // order-1 tile.  The token's extended value vector is packed once, so a 32-row tile costs
