@@ -1,5 +1,5 @@
-// Forward-side kernels: per-head row-norm statistics, the moment-state build (used by
-// both passes) and the forward apply.
+// Per-head row-norm statistics and the moment-state build (used by both passes; the kernels
+// that consume the states are in fm_apply.h and fm_grad.h).
 #pragma once
 #include <type_traits>
 
