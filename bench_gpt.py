@@ -42,9 +42,9 @@ def apply_rope(x, cos, sin):
 
 
 class Block(nn.Module):
-    def __init__(self, d_model, n_head, d_mlp, attn, p):
+    def __init__(self, d_model, n_head, d_mlp, attn, p, fused_rope):
         super().__init__()
-        self.n_head, self.hs, self.p = n_head, d_model // n_head, p
+        self.n_head, self.hs, self.p, self.fused_rope = n_head, d_model // n_head, p, fused_rope
         self.ln1 = nn.LayerNorm(d_model)
         self.qkv = nn.Linear(d_model, 3 * d_model)
         self.proj = nn.Linear(d_model, d_model)
@@ -55,20 +55,28 @@ class Block(nn.Module):
 
     def forward(self, x, cos, sin):
         B, T, C = x.shape
-        q, k, v = self.qkv(self.ln1(x)).view(B, T, 3, self.n_head, self.hs).permute(2, 0, 3, 1, 4)
-        q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+        qkv = self.qkv(self.ln1(x))
+        if self.fused_rope:
+            # one HBM pass: split of the projection (packed per head as [q, k, v], the reference's
+            # group-major layout with one query per group, model.py:474-497), RoPE on q and k,
+            # contiguous (B, H, T, hs) outputs
+            from fastmax_amd import qkv_rope_split
+            q, k, v = qkv_rope_split(qkv, cos, sin, self.n_head, 1, self.hs)
+        else:
+            q, k, v = qkv.view(B, T, self.n_head, 3, self.hs).permute(3, 0, 2, 1, 4)
+            q, k = apply_rope(q, cos, sin).contiguous(), apply_rope(k, cos, sin).contiguous()
+            v = v.contiguous()
         # same call as reference model.py:575: mask, no dropout, normalize, lim 1, a = (1, 1, 0.5)
-        y = self.attn(q.contiguous(), k.contiguous(), v.contiguous(), None, True, 0.0, True, 1.0, 1.0, 1.0, 0.5,
-                      1.0, self.p)
+        y = self.attn(q, k, v, None, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, self.p)
         x = x + self.proj(y.transpose(1, 2).reshape(B, T, C))
         return x + self.out(F.gelu(self.fc(self.ln2(x))))
 
 
 class MiniGPT(nn.Module):
-    def __init__(self, vocab, d_model, n_layer, n_head, d_mlp, seq, attn, p):
+    def __init__(self, vocab, d_model, n_layer, n_head, d_mlp, seq, attn, p, fused_rope):
         super().__init__()
         self.wte = nn.Embedding(vocab, d_model)
-        self.blocks = nn.ModuleList(Block(d_model, n_head, d_mlp, attn, p) for _ in range(n_layer))
+        self.blocks = nn.ModuleList(Block(d_model, n_head, d_mlp, attn, p, fused_rope) for _ in range(n_layer))
         self.ln_f = nn.LayerNorm(d_model)
         self.lm_head = nn.Linear(d_model, vocab, bias=False)
         self.seq, self.hs = seq, d_model // n_head
@@ -132,6 +140,9 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--seq", type=int, default=2048)
     ap.add_argument("--pytorch-attention", action="store_true", help="use_custom_gradient=False path")
+    ap.add_argument("--unfused-rope", action="store_true",
+                    help="split the projection, apply RoPE and make q, k, v contiguous with PyTorch ops "
+                         "(the reference's chain, model.py:474-497, 812-825, 572-574) instead of the fused kernel")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         print("bench_gpt.py: no GPU visible", file=sys.stderr)
@@ -141,7 +152,7 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
     attn = TimedAttention(FASTMultiHeadAttention(use_custom_gradient=not args.pytorch_attention))
-    model = MiniGPT(50304, 768, args.layers, 12, 3072, args.seq, attn, args.p).to(dev)
+    model = MiniGPT(50304, 768, args.layers, 12, 3072, args.seq, attn, args.p, not args.unfused_rope).to(dev)
     opt = torch.optim.AdamW(model.parameters(), lr=3e-4, weight_decay=0.1)
     gen = torch.Generator(device=dev).manual_seed(0)
     idx = torch.randint(0, 50304, (args.batch, args.seq + 1), device=dev, generator=gen)
@@ -174,7 +185,8 @@ def main() -> int:
         "dtype": "bf16 autocast (attention: bf16 in/out, bf16 matrix instructions, fp32 accumulate)", "data": "synthetic",
         "config": {"workload": f"{args.layers} layers, d_model 768, 12 heads x 64, MLP 3072 GELU, RoPE, vocab 50304, "
                                f"seq {args.seq}, batch {args.batch}, p={args.p}, AdamW",
-                   "attention": "pytorch function" if args.pytorch_attention else "hip kernels"},
+                   "attention": "pytorch function" if args.pytorch_attention else "hip kernels",
+                   "qkv split + rope": "pytorch ops" if args.unfused_rope else "fused hip kernel"},
         "loss_first_last": [losses[0], losses[-1]], "steps": args.steps, "warmup": args.warmup,
     }))
     return 0 if all(math.isfinite(v) for v in losses) else 1

@@ -7,6 +7,7 @@ mirrors the reference's operator API; the C ABI underneath is include/fastmax_am
 from .attention import (FASTMultiHeadAttention, FASTMultiHeadAttention_Function, fastmax_custom,
                         fastmax_function)
 from ._ext import install_as_fastmax_cuda
+from .rope import qkv_rope_split
 
 __all__ = ["FASTMultiHeadAttention", "FASTMultiHeadAttention_Function", "fastmax_custom",
-           "fastmax_function", "install_as_fastmax_cuda"]
+           "fastmax_function", "install_as_fastmax_cuda", "qkv_rope_split"]

@@ -26,7 +26,7 @@ EXPORTS = (
     "fastmax_workspace_min_bytes", "fastmax_forward", "fastmax_backward", "fastmax_normalize_inplace",
     "fastmax_profile_begin", "fastmax_profile_end",
     "fastmax_state_bytes", "fastmax_decode_workspace_bytes", "fastmax_state_update", "fastmax_decode_step",
-    "fastmax_saved_state_bytes", "fastmax_forward_saving", "fastmax_backward_saved",
+    "fastmax_saved_state_bytes", "fastmax_forward_saving", "fastmax_backward_saved", "fastmax_qkv_rope",
 )
 
 KERNEL_NAMES = ("rowstat", "build", "fwd_apply", "bwd_prep", "bwd_dq", "bwd_dk", "bwd_dv", "norm_fix")
@@ -43,6 +43,11 @@ class FastmaxDesc(C.Structure):
         ("p", C.c_int32), ("lim", C.c_float), ("temperature", C.c_float),
         ("a0", C.c_float), ("a1", C.c_float), ("a2", C.c_float),
     ]
+
+
+class RopeDesc(C.Structure):
+    _fields_ = [("b", C.c_int32), ("t", C.c_int32), ("groups", C.c_int32), ("q_per_kv", C.c_int32),
+                ("hs", C.c_int32), ("rope_n", C.c_int32), ("dtype", C.c_int32)]
 
 
 class FastmaxError(RuntimeError):
@@ -86,6 +91,8 @@ def load() -> C.CDLL:
     lib.fastmax_backward_saved.restype = C.c_int
     lib.fastmax_backward_saved.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, sz, vp,
                                            sz, vp]
+    lib.fastmax_qkv_rope.restype = C.c_int
+    lib.fastmax_qkv_rope.argtypes = [C.POINTER(RopeDesc), C.c_int, vp, vp, vp, vp, vp, vp, vp]
     lib.fastmax_normalize_inplace.restype = C.c_int
     lib.fastmax_normalize_inplace.argtypes = [dp, vp, vp, vp, sz, vp]
     lib.fastmax_state_bytes.restype = sz

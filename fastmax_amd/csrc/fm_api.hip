@@ -13,6 +13,7 @@
 #include "fm_decode.h"
 #include "fm_forward.h"
 #include "fm_grad.h"
+#include "fm_rope.h"
 
 namespace {
 
@@ -712,6 +713,33 @@ int fastmax_decode_step(const fastmax_desc* desc, const void* q, const void* k, 
   if (desc->d == 64) FM_DEC(64, bf16_t);
   FM_DEC(32, bf16_t);
 #undef FM_DEC
+}
+
+int fastmax_qkv_rope(const fastmax_rope_desc* desc, int grad, void* qkv, const float* cos, const float* sin,
+                     void* q, void* k, void* v, fastmax_stream_t stream) {
+  g_err[0] = 0;
+  if (!desc) return fail(FASTMAX_E_NULL, "desc is NULL");
+  if (!qkv || !q || !k || !v) return fail(FASTMAX_E_NULL, "qkv, q, k and v must be non-NULL");
+  if (desc->dtype != FASTMAX_F32 && desc->dtype != FASTMAX_BF16)
+    return fail(FASTMAX_E_DTYPE, "dtype %d is neither FASTMAX_F32 nor FASTMAX_BF16", desc->dtype);
+  if (desc->b < 1 || desc->t < 1 || desc->groups < 1 || desc->q_per_kv < 1 || desc->hs < 4 || desc->hs % 4)
+    return fail(FASTMAX_E_SHAPE, "b, t, groups, q_per_kv must be positive and hs a positive multiple of 4");
+  if (desc->rope_n < 0 || desc->rope_n > desc->hs || desc->rope_n % 8)
+    return fail(FASTMAX_E_SHAPE, "rope_n = %d must be a multiple of 8 in [0, hs]", desc->rope_n);
+  if (desc->rope_n > 0 && (!cos || !sin)) return fail(FASTMAX_E_NULL, "cos and sin must be non-NULL when rope_n > 0");
+  const RopeShape sh{desc->b, desc->t, desc->groups, desc->q_per_kv, desc->hs, desc->rope_n};
+  const int64_t total = (int64_t)sh.b * sh.t * sh.groups * (sh.qpk + 2) * (sh.hs / 4);
+  if (total >= ((int64_t)1 << 39)) return fail(FASTMAX_E_SHAPE, "tensor too large");
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (desc->dtype == FASTMAX_F32) {
+    if (grad) qkv_rope_kernel<float, true><<<blocks, 256, 0, st>>>(sh, (float*)qkv, cos, sin, (float*)q, (float*)k, (float*)v);
+    else qkv_rope_kernel<float, false><<<blocks, 256, 0, st>>>(sh, (float*)qkv, cos, sin, (float*)q, (float*)k, (float*)v);
+  } else {
+    if (grad) qkv_rope_kernel<bf16_t, true><<<blocks, 256, 0, st>>>(sh, (bf16_t*)qkv, cos, sin, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v);
+    else qkv_rope_kernel<bf16_t, false><<<blocks, 256, 0, st>>>(sh, (bf16_t*)qkv, cos, sin, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v);
+  }
+  return launch_status("qkv_rope_kernel");
 }
 
 }  // extern "C"

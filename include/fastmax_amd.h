@@ -168,6 +168,23 @@ int fastmax_decode_step(const fastmax_desc* desc, const void* q, const void* k, 
                         float* den, int64_t den_stride, void* workspace, size_t workspace_bytes,
                         fastmax_stream_t stream);
 
+/* Caller-side helper of a GPT block (no kernel of the reference does this; it replaces the
+ * chain of PyTorch ops at model.py:474-497 -- view the fused projection as
+ * (b, t, groups, q_per_kv + 2, hs), permute, split -- then model.py:812-825 apply_rope on the
+ * first rope_n channels of q and k, then the .contiguous() calls at model.py:572-574).
+ *   grad == 0: qkv (b, t, groups*(q_per_kv+2)*hs) in;  q (b, groups*q_per_kv, t, hs),
+ *              k, v (b, groups, t, hs) out, q and k rotated:
+ *              y = x*cos + (-x2, x1)*sin on channels [0, rope_n), x1/x2 = its halves
+ *   grad != 0: the adjoint: q, k, v hold the gradients of the three outputs (in), qkv receives
+ *              the gradient of the projection (out)
+ * cos, sin: (t, rope_n) fp32, rope_n a multiple of 8 (0: no rotation, they may be NULL). */
+typedef struct fastmax_rope_desc {
+  int32_t b, t, groups, q_per_kv, hs, rope_n;
+  int32_t dtype;       /* FASTMAX_F32 or FASTMAX_BF16 */
+} fastmax_rope_desc;
+int fastmax_qkv_rope(const fastmax_rope_desc* desc, int grad, void* qkv, const float* cos, const float* sin,
+                     void* q, void* k, void* v, fastmax_stream_t stream);
+
 /* Kernel timing aid (no counterpart in the reference, which only wall-clocks whole calls,
  * test_fastmax.py:351-356).  Between begin and end every kernel the calling thread launches
  * through this library is bracketed by two HIP events on the caller's stream; end waits for

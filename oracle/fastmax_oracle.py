@@ -276,3 +276,35 @@ def dense_truth(q, k, v, go: Optional[torch.Tensor], **kw):
         return o, den
     o, dq, dk, dv = fastmax_grads_autograd(fastmax_dense, q64, k64, v64, go.detach().cpu().double(), **kw)
     return o, dq, dk, dv
+
+
+# --------------------------------------------------------------------------------------
+# caller side of a GPT block: split of the fused projection + rotary embedding
+# (reference: model.py:474-497 view/permute/split, model.py:812-825 apply_rope,
+#  model.py:694-760 build_rope_cache with condense_ratio 1 and no extra_config)
+# --------------------------------------------------------------------------------------
+def rope_cache(seq_len: int, n_elem: int, base: float = 10000.0, dtype=torch.float64):
+    theta = 1.0 / (base ** (torch.arange(0, n_elem, 2, dtype=dtype) / n_elem))
+    idx = torch.outer(torch.arange(seq_len, dtype=dtype), theta).repeat(1, 2)
+    return torch.cos(idx), torch.sin(idx)
+
+
+def apply_rope(x, cos, sin):
+    hs = x.size(-1)
+    x1, x2 = x[..., : hs // 2], x[..., hs // 2:]
+    rotated = torch.cat((-x2, x1), dim=-1)
+    return x * cos + rotated * sin
+
+
+def qkv_rope_split(qkv, cos, sin, groups: int, q_per_kv: int, hs: int, rope_n: int):
+    """qkv (B, T, groups*(q_per_kv+2)*hs) -> q (B, groups*q_per_kv, T, hs), k, v (B, groups, T, hs)."""
+    B, T, _ = qkv.shape
+    x = qkv.view(B, T, groups, q_per_kv + 2, hs).permute(0, 2, 3, 1, 4)
+    q, k, v = x.split((q_per_kv, 1, 1), dim=2)
+    q = q.reshape(B, groups * q_per_kv, T, hs)
+    k = k.reshape(B, groups, T, hs)
+    v = v.reshape(B, groups, T, hs)
+    if rope_n:
+        q = torch.cat((apply_rope(q[..., :rope_n], cos, sin), q[..., rope_n:]), dim=-1)
+        k = torch.cat((apply_rope(k[..., :rope_n], cos, sin), k[..., rope_n:]), dim=-1)
+    return q, k, v

@@ -15,8 +15,8 @@ def test_small_gpt_gradients_match_pytorch_path(built, p):
 
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-    ref_model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 300, FASTMultiHeadAttention(use_custom_gradient=False), p).to(dev)
-    hip_model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 300, FASTMultiHeadAttention(use_custom_gradient=True), p).to(dev)
+    ref_model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 300, FASTMultiHeadAttention(use_custom_gradient=False), p, False).to(dev)
+    hip_model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 300, FASTMultiHeadAttention(use_custom_gradient=True), p, True).to(dev)
     hip_model.load_state_dict(ref_model.state_dict())
     idx = torch.randint(0, 512, (2, 301), device=dev, generator=torch.Generator(device=dev).manual_seed(1))
     x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
@@ -38,7 +38,7 @@ def test_bf16_autocast_step_runs_and_learns(built):
 
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-    model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 256, FASTMultiHeadAttention(), 2).to(dev)
+    model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 256, FASTMultiHeadAttention(), 2, True).to(dev)
     opt = torch.optim.AdamW(model.parameters(), lr=1e-3)
     idx = torch.randint(0, 512, (4, 257), device=dev, generator=torch.Generator(device=dev).manual_seed(2))
     x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()

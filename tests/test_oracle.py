@@ -180,3 +180,32 @@ def test_key_prefix_is_the_tail_of_a_longer_causal_pass():
     full = O.fastmax_dense(q, k, v, mask=True, normalize=False)
     tail = O.fastmax_dense(q[:, :, 4:], k, v, mask=True, normalize=False)
     assert torch.allclose(full[:, :, 4:], tail, rtol=1e-12, atol=1e-13)
+
+
+def test_rope_is_a_rotation_and_identity_at_position_zero():
+    """apply_rope rotates channel pairs (c, c + hs/2): norms are kept, position 0 is the identity,
+    and relative positions are what q.k sees (the defining property of the rotary embedding)."""
+    hs, T = 16, 12
+    cos, sin = O.rope_cache(T, hs)
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(2, 3, T, hs, generator=g, dtype=torch.float64)
+    y = O.apply_rope(x, cos, sin)
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), rtol=1e-12)
+    assert torch.allclose(y[:, :, 0], x[:, :, 0], rtol=0, atol=1e-15)
+    # <rope(a, m), rope(b, n)> depends on m - n only
+    a, b = x[0, 0, 0], x[0, 1, 0]
+    ra = torch.stack([O.apply_rope(a, cos[m], sin[m]) for m in range(T)])
+    rb = torch.stack([O.apply_rope(b, cos[m], sin[m]) for m in range(T)])
+    assert torch.allclose(ra[5] @ rb[2], ra[9] @ rb[6], rtol=1e-12)
+    assert torch.allclose(ra[3] @ rb[3], a @ b, rtol=1e-12)
+
+
+def test_qkv_split_places_heads_as_the_reference_view_does():
+    """Group-major packing (model.py:474-497): per group q_per_kv queries, then one key, one value."""
+    B, T, G, Q, hs = 2, 3, 2, 3, 8
+    qkv = torch.arange(B * T * G * (Q + 2) * hs, dtype=torch.float64).view(B, T, -1)
+    q, k, v = O.qkv_rope_split(qkv, None, None, G, Q, hs, 0)
+    assert q.shape == (B, G * Q, T, hs) and k.shape == v.shape == (B, G, T, hs)
+    row = qkv[1, 2].view(G, Q + 2, hs)
+    assert torch.equal(q[1, 1 * Q + 2, 2], row[1, 2]) and torch.equal(k[1, 0, 2], row[0, Q])
+    assert torch.equal(v[1, 1, 2], row[1, Q + 1])
