@@ -151,6 +151,14 @@ def fastmax_function(q, k, v, mask=0, dropout_rate=0.0, normalize=0, temperature
         return drop(x), None
 
     b, h, n, d = q.shape
+    if k.shape[1] != h:  # grouped key/value heads: query head i reads head i // (h / h_kv)
+        if h % k.shape[1]:
+            raise ValueError(f"{k.shape[1]} key/value heads do not divide {h} query heads")
+        k = k.repeat_interleave(h // k.shape[1], dim=1)
+        v = v.repeat_interleave(h // v.shape[1], dim=1)
+    lead = k.shape[2] - n  # key prefix: the first nk - nq keys are visible to every query
+    if lead < 0:
+        raise ValueError(f"k, v have {k.shape[2]} tokens but q has {n}: fewer keys than queries is not supported")
     if not mask:
         k1, k2 = feats(k)
         q1, q2 = feats(q)
@@ -168,6 +176,17 @@ def fastmax_function(q, k, v, mask=0, dropout_rate=0.0, normalize=0, temperature
     s2 = v.new_zeros(b, h, d * d, d) if p == 2 else None
     z2 = v.new_zeros(b, h, d * d, 1) if p == 2 else None
     count = 0
+    if lead:  # the prefix keys go into the running state before the first query
+        kp, vp = k[:, :, :lead], v[:, :, :lead]
+        k1, k2 = feats(kp)
+        s0 = s0 + vp.sum(-2, keepdim=True)
+        s1 = s1 + k1.transpose(-1, -2) @ vp
+        z1 = z1 + k1.sum(-2).unsqueeze(-1)
+        if p == 2:
+            s2 = s2 + k2.transpose(-1, -2) @ vp
+            z2 = z2 + k2.sum(-2).unsqueeze(-1)
+        count = lead
+        k, v = k[:, :, lead:], v[:, :, lead:]
     for t0 in range(0, n, chunk):
         qc, kc, vc = q[:, :, t0:t0 + chunk], k[:, :, t0:t0 + chunk], v[:, :, t0:t0 + chunk]
         c = qc.shape[2]

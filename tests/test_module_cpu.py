@@ -110,3 +110,20 @@ def test_ops_reject_cpu_and_bad_dtype(built):
     t = torch.zeros(2, 3, 32)
     with pytest.raises(RuntimeError, match="GPU"):
         ops.forward(t, t, t)
+
+
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("p", [1, 2])
+def test_pytorch_path_grouped_heads_and_key_prefix(mask, p):
+    """The PyTorch function takes the shapes the kernels take: fewer key/value heads
+    (fastmax_cuda_forward.cu:38) and a key prefix nk > nq (fastmax_cuda_forward.cu:109-150)."""
+    from fastmax_amd import fastmax_function
+
+    q, _, _, _ = O.seeded_inputs((2, 4, 21, 8), seed=91, dtype=torch.float64)
+    _, k, v, _ = O.seeded_inputs((2, 2, 30, 8), seed=92, dtype=torch.float64)
+    got = fastmax_function(q, k, v, mask, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, p, chunk=8)
+    ke, ve = k.repeat_interleave(2, dim=1), v.repeat_interleave(2, dim=1)
+    ref = O.fastmax_dense(q, ke, ve, mask=mask, normalize=True, p=p)
+    assert torch.allclose(got, ref, rtol=1e-10, atol=1e-12)
+    with pytest.raises(ValueError, match="fewer keys"):
+        fastmax_function(ke, q, q, mask)
