@@ -13,6 +13,7 @@
 #include "fm_decode.h"
 #include "fm_forward.h"
 #include "fm_grad.h"
+#include "fm_linear.h"
 #include "fm_rope.h"
 
 namespace {
@@ -88,6 +89,14 @@ int64_t state_floats_for(int d, int p2) {
 
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
+// Causal p = 1 at d = 64 runs as one sequential scan per head (fm_linear.h: one wave per head, the
+// state never leaves its registers) once there are enough heads to fill the chip's 1024 SIMDs
+// about half way; below that the chunked kernels, which split a head over many blocks, win.
+#ifndef FM_LINEAR_MIN_HEADS
+#define FM_LINEAR_MIN_HEADS 512
+#endif
+bool use_linear_scan(const Plan& pl);
+
 Plan make_plan(const fastmax_desc* ds, int pass) {
   Plan pl;
   pl.d = ds->d;
@@ -144,6 +153,10 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   if (pass == FASTMAX_PASS_BACKWARD && pl.ratio > 1)
     pl.per_head_bytes += 2 * (size_t)pl.n * pl.d * (ds->dtype == FASTMAX_BF16 ? 2 : 4);
   return pl;
+}
+
+bool use_linear_scan(const Plan& pl) {
+  return !pl.p2 && pl.masked && pl.d == 64 && pl.ratio == 1 && pl.bh >= FM_LINEAR_MIN_HEADS;
 }
 
 // Heads per launch that fit the workspace.  When several batches are needed the batch is
@@ -295,6 +308,20 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
 
   FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
 
+  if constexpr (D == 64) {
+    if (use_linear_scan(pl)) {
+      ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
+      // (pairs of output columns go out as one store when the row pitch keeps them aligned)
+      if (ldo % 2 == 0)
+        lin::linear_fwd_kernel<T, true><<<bh, 64, 0, stream>>>(q, k, v, scale, scale + bh, o, ldo, den, den_stride, n,
+                                                                ds->a0, ds->a1);
+      else
+        lin::linear_fwd_kernel<T, false><<<bh, 64, 0, stream>>>(q, k, v, scale, scale + bh, o, ldo, den, den_stride, n,
+                                                                 ds->a0, ds->a1);
+      return launch_status("linear_fwd_kernel");
+    }
+  }
+
   const int ratio = pl.ratio;
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
@@ -352,6 +379,40 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
     bwd_prep_kernel<T><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
     FM_TRY(launch_status("bwd_prep_kernel"));
+  }
+  if constexpr (D == 64) {
+    if (use_linear_scan(pl)) {
+      const float* qs = scale;
+      const float* ks = scale + bh;
+      // one normalisation partial per head, shared by q and k:
+      // sum_i dq_hat_i . q_hat_i = sum_ij W_ij s_ij = sum_j dk_hat_j . k_hat_j
+      float* rq = rpart;
+      {
+        ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
+        if (ds->normalize)
+          lin::linear_dq_kernel<T, true><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, k, v, qs, ks, dq, rq, n, ds->a1);
+        else
+          lin::linear_dq_kernel<T, false><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, k, v, qs, ks, dq, rq, n, ds->a1);
+      }
+      FM_TRY(launch_status("linear_dq_kernel"));
+      {
+        ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
+        lin::linear_dk_kernel<T><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, v, qs, ks, dk, n, ds->a1);
+      }
+      FM_TRY(launch_status("linear_dk_kernel"));
+      {
+        ScopedKernel sk(FASTMAX_K_BWD_DV, stream);
+        lin::linear_dv_kernel<T><<<bh, 64, 0, stream>>>(go, den, den_stride, q, k, qs, ks, dv, n, ds->a0, ds->a1);
+      }
+      FM_TRY(launch_status("linear_dv_kernel"));
+      if (ds->normalize) {
+        ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
+        norm_fix_kernel<T><<<bh, D, 0, stream>>>(dq, q, qs, arg, rq, 1, n, D, ds->lim);
+        norm_fix_kernel<T><<<bh, D, 0, stream>>>(dk, k, ks, arg + bh, rq, 1, n, D, ds->lim);
+        FM_TRY(launch_status("norm_fix_kernel"));
+      }
+      return FASTMAX_OK;
+    }
   }
   const float a2 = pl.p2 ? ds->a2 : 0.f;
   const int ratio = pl.ratio, bhkv = pl.bhkv;
