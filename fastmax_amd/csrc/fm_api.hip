@@ -95,7 +95,7 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 #ifndef FM_LINEAR_MIN_HEADS
 #define FM_LINEAR_MIN_HEADS 512
 #endif
-bool use_linear_scan(const Plan& pl);
+bool use_linear_scan(const fastmax_desc* ds, const Plan& pl);
 
 Plan make_plan(const fastmax_desc* ds, int pass) {
   Plan pl;
@@ -155,8 +155,10 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   return pl;
 }
 
-bool use_linear_scan(const Plan& pl) {
-  return !pl.p2 && pl.masked && pl.d == 64 && pl.ratio == 1 && pl.bh >= FM_LINEAR_MIN_HEADS;
+bool use_linear_scan(const fastmax_desc* ds, const Plan& pl) {
+  // (its kernels keep the weights divided by a1, and every tile is a full 32 rows)
+  return !pl.p2 && pl.masked && pl.d == 64 && pl.ratio == 1 && pl.n >= 32 && ds->a1 != 0.f &&
+         pl.bh >= FM_LINEAR_MIN_HEADS;
 }
 
 // Heads per launch that fit the workspace.  When several batches are needed the batch is
@@ -309,7 +311,7 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
 
   if constexpr (D == 64) {
-    if (use_linear_scan(pl)) {
+    if (use_linear_scan(ds, pl)) {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       // (pairs of output columns go out as one store when the row pitch keeps them aligned)
       if (ldo % 2 == 0)
@@ -381,7 +383,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     FM_TRY(launch_status("bwd_prep_kernel"));
   }
   if constexpr (D == 64) {
-    if (use_linear_scan(pl)) {
+    if (use_linear_scan(ds, pl)) {
       const float* qs = scale;
       const float* ks = scale + bh;
       // one normalisation partial per head, shared by q and k:
@@ -390,9 +392,9 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       {
         ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
         if (ds->normalize)
-          lin::linear_dq_kernel<T, true><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, k, v, qs, ks, dq, rq, n, ds->a1);
+          lin::linear_dq_kernel<T, true><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, k, v, qs, ks, dq, rq, n, ds->a0, ds->a1);
         else
-          lin::linear_dq_kernel<T, false><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, k, v, qs, ks, dq, rq, n, ds->a1);
+          lin::linear_dq_kernel<T, false><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, k, v, qs, ks, dq, rq, n, ds->a0, ds->a1);
       }
       FM_TRY(launch_status("linear_dq_kernel"));
       {

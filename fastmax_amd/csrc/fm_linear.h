@@ -13,17 +13,38 @@
 // bf16 inputs take the same path (fp32 matrix instruction, half the memory traffic).
 //
 // Operand layouts (lane l: i = l % 32, hh = l / 32; trow(t, hh) = row of accumulator register t):
-//   token-major   X^tok[g*8 + e]  = X[tile row i][16 g + 8 hh + e]      (8 contiguous channels x 4)
-//   channel-major X^ch[c][t]      = X[tile row trow(t, hh)][2 i + c]    (2 contiguous channels x 16)
-// A state tile (rc, cc) holds State[2 m + rc][2 n' + cc] at accumulator (row m, column n'), so
-// register t of a lane holds state row 2 trow(t, hh) + rc = 16 (t/4) + 8 hh + 2 (t%4) + rc, which
-// is exactly the channel of token-major element (t/4)*8 + 2 (t%4) + rc: a token-major operand and
-// the state's registers contract against each other with no data movement.  (The k index of an
-// MFMA and the order of output rows / columns may be permuted freely as long as both operands,
-// respectively the final store, agree.)
+//   channel-major X^ch[c][t] = X[tile row trow(t, hh)][chan(c, i)], c = 0, 1: the lane's two channels
+//   token-major   X^tok[e]   = X[tile row i][channel of e], 32 of the row's 64 channels per lane half
+// A state tile (rc, cc) holds State[chan(rc, m)][chan(cc, n')] at accumulator (row m, column n'),
+// and the token-major element tok_of(t, rc) is the channel chan(rc, trow(t, hh)) of the state row
+// that register t of the lane holds in tile row-class rc: a token-major operand and the state's
+// registers contract against each other with no data movement.  (The k index of an MFMA and the
+// order of output rows / columns may be permuted freely as long as both operands, respectively
+// the final store, agree.)  Two channel maps, chosen so that every load is one full instruction:
+//   fp32: chan(c, i) = 32 c + i (4-byte loads, a half-wave reads 128 contiguous bytes; 32-bit
+//         destinations keep the loop-carried operand registers free of pairing constraints);
+//         token-major loads are 16 bytes at channel 32 rc + 8 g + 4 hh -> elements rc*16 + 4 g + u
+//   bf16: chan(c, i) = 2 i + c (one 4-byte load gives both); token-major loads are 16 bytes =
+//         8 channels at 16 g + 8 hh -> elements 8 g + e
 //
-// Rows past the end of the sequence are read from the last valid row (clamped) and kept out of
-// the results by the masks / zeroed factors named at each use.
+// Every tile is a full 32-row tile (the sequence has at least 32 tokens): when the length is
+// not a multiple of 32, the last tile of a scan is moved back so that it ends at the sequence's
+// end (a forward scan's last tile is rows [n-32, n); a reverse scan runs its tiles down from the
+// end and its last one is rows [0, 32)).  The rows it shares with the tile before it are already
+// in the state and already written; they are masked out of the weights, the state update and
+// the stores.  So all loads are unclamped, with one per-lane offset and immediates, and the hot
+// loop has a single straight path.
+//
+// Order of work in a loop iteration (tile m): fold tile m-1 into the state (its channel-major
+// operands are still in registers) -> load tile m's channel-major operands into those registers
+// -> score tile and own rows x state with the token-major operands -> load tile m+1's
+// token-major operands into those registers -> weights -> intra-tile product -> store.  Every
+// load is thus issued right after the last use of the registers it replaces and at least a
+// third of an iteration before its first use, and only the token-major loads are still in flight
+// at the loop's back edge (where the compiler waits for whatever is outstanding).  The state
+// update of the last tile is never needed.  Per-row and per-head factors are applied to the
+// accumulators, not to the operands: the weights are kept divided by a1' (resp. by 1/den_i) so
+// that the state product and the intra-tile product share one accumulator (hence a1 != 0).
 #pragma once
 #include "fm_common.h"
 
@@ -36,91 +57,145 @@ constexpr int D = 64;
 // ranges), where their latency is fully exposed.  Nothing may be moved across FM_PIN().
 #define FM_PIN() __builtin_amdgcn_sched_barrier(0)
 
+// Channel maps (see above).
 template <class T>
-__device__ __forceinline__ void ld8(const T* p, float* x);
+struct Map;
 template <>
-__device__ __forceinline__ void ld8<float>(const float* p, float* x) {
-  const float4 a = *reinterpret_cast<const float4*>(p);
-  const float4 b = *reinterpret_cast<const float4*>(p + 4);
-  x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
-  x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
-}
+struct Map<float> {
+  static constexpr bool PAIR = false;
+  static constexpr bool CLOSED_R = true;
+  __device__ static constexpr int chan(int c, int i) { return 32 * c + i; }
+  __device__ static constexpr int tok_of(int t, int rc) { return rc * 16 + t; }
+};
 template <>
-__device__ __forceinline__ void ld8<bf16_t>(const bf16_t* p, float* x) {
-  const uint4 u = *reinterpret_cast<const uint4*>(p);
-  x[0] = bf_lo(u.x); x[1] = bf_hi(u.x); x[2] = bf_lo(u.y); x[3] = bf_hi(u.y);
-  x[4] = bf_lo(u.z); x[5] = bf_hi(u.z); x[6] = bf_lo(u.w); x[7] = bf_hi(u.w);
-}
-__device__ __forceinline__ void ld2(const float* p, float& a, float& b) {
-  const float2 t = *reinterpret_cast<const float2*>(p);
-  a = t.x; b = t.y;
-}
-__device__ __forceinline__ void ld2(const bf16_t* p, float& a, float& b) {
-  const uint32_t u = *reinterpret_cast<const uint32_t*>(p);
-  a = bf_lo(u); b = bf_hi(u);
-}
-// (aligned: the pair may be written as one 8- or 4-byte store)
-template <bool ALIGNED>
-__device__ __forceinline__ void st2(float* p, float a, float b) {
-  if constexpr (ALIGNED) {
-    *reinterpret_cast<float2*>(p) = make_float2(a, b);
-  } else {
-    p[0] = a; p[1] = b;
-  }
-}
-template <bool ALIGNED>
-__device__ __forceinline__ void st2(bf16_t* p, float a, float b) {
-  if constexpr (ALIGNED) {
-    *reinterpret_cast<uint32_t*>(p) = pack_bf2(a, b);
-  } else {
-    p[0] = from_f32<bf16_t>(a); p[1] = from_f32<bf16_t>(b);
-  }
-}
+struct Map<bf16_t> {
+  static constexpr bool PAIR = true;
+  static constexpr bool CLOSED_R = false;   // (see linear_dq_kernel)
+  __device__ static constexpr int chan(int c, int i) { return 2 * i + c; }
+  __device__ static constexpr int tok_of(int t, int rc) { return (t >> 2) * 8 + 2 * (t & 3) + rc; }
+};
 
 // Tile operands are addressed as (uniform pointer to the tile's first row) + (per-lane element
-// offset, constant from tile to tile) so that the loads take a scalar base and an immediate.
-// token-major operand of the tile starting at row `base` of one head (hp)
+// offset, the same for every tile) so that the loads take a scalar base and an immediate.
 template <class T>
-__device__ __forceinline__ void load_tok(const T* hp, int base, int n, int i, int hh, float (&x)[32]) {
-  const T* tp = hp + (int64_t)base * D;
-  const int last = n - 1 - base;                       // last valid row of the tile
-  const int off = (i < last ? i : last) * D + 8 * hh;  // (rows past the end read the last valid row)
+struct Lane {
+  int l, i, hh;
+  int tok;   // token-major: row i, first channel of the lane half
+  int ch;    // channel-major: row 4 hh, channel chan(0, i)
+  __device__ __forceinline__ Lane() {
+    l = threadIdx.x; i = l & 31; hh = l >> 5;
+    tok = i * D + (Map<T>::PAIR ? 8 : 4) * hh;
+    ch = 4 * hh * D + Map<T>::chan(0, i);
+  }
+};
+
+__device__ __forceinline__ void load_tok(const float* hp, int base, const Lane<float>& L, float (&x)[32]) {
+  const float* tp = hp + (int64_t)base * D;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) ld8<T>(tp + (off + 16 * g), &x[8 * g]);
+  for (int rc = 0; rc < 2; ++rc)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const float4 a = *reinterpret_cast<const float4*>(tp + (L.tok + 32 * rc + 8 * g));
+      float* y = &x[rc * 16 + 4 * g];
+      y[0] = a.x; y[1] = a.y; y[2] = a.z; y[3] = a.w;
+    }
+}
+__device__ __forceinline__ void load_tok(const bf16_t* hp, int base, const Lane<bf16_t>& L, float (&x)[32]) {
+  const bf16_t* tp = hp + (int64_t)base * D;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const uint4 u = *reinterpret_cast<const uint4*>(tp + (L.tok + 16 * g));
+    float* y = &x[8 * g];
+    y[0] = bf_lo(u.x); y[1] = bf_hi(u.x); y[2] = bf_lo(u.y); y[3] = bf_hi(u.y);
+    y[4] = bf_lo(u.z); y[5] = bf_hi(u.z); y[6] = bf_lo(u.w); y[7] = bf_hi(u.w);
+  }
+}
+__device__ __forceinline__ void load_ch(const float* hp, int base, const Lane<float>& L, float (&x)[2][16]) {
+  const float* tp = hp + (int64_t)base * D;
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    x[0][t] = tp[L.ch + (8 * (t >> 2) + (t & 3)) * D];
+    x[1][t] = tp[L.ch + (8 * (t >> 2) + (t & 3)) * D + 32];
+  }
+}
+__device__ __forceinline__ void load_ch(const bf16_t* hp, int base, const Lane<bf16_t>& L, float (&x)[2][16]) {
+  const bf16_t* tp = hp + (int64_t)base * D;
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    const uint32_t u = *reinterpret_cast<const uint32_t*>(tp + (L.ch + (8 * (t >> 2) + (t & 3)) * D));
+    x[0][t] = bf_lo(u);
+    x[1][t] = bf_hi(u);
+  }
 }
 
-// channel-major operand; roff[t] = element offset of the lane's pair in row trow(t, hh) of a tile
-// (row_offsets: rows past the tile's last valid row read that row).  The offsets live in
-// registers and are only recomputed for a ragged last tile, so the hot loop has one load path.
-__device__ __forceinline__ void row_offsets(int last, int i, int hh, int (&roff)[16]) {
-#pragma unroll
-  for (int t = 0; t < 16; ++t) roff[t] = (trow(t, hh) < last ? trow(t, hh) : last) * D + 2 * i;
+// x[c][t] -> row trow(t, hh) of the tile, columns chan(c, i), for the tile rows in [lo, hi)
+// (ALIGNED, bf16 only: the row pitch keeps the lane's channel pair 4-byte aligned)
+template <bool ALIGNED>
+__device__ __forceinline__ void store_row(float* rp, const Lane<float>& L, float a, float b) {
+  rp[L.i] = a;
+  rp[32 + L.i] = b;
 }
-template <class T>
-__device__ __forceinline__ void load_ch(const T* hp, int base, const int (&roff)[16], float (&x)[2][16]) {
-  const T* tp = hp + (int64_t)base * D;
-#pragma unroll
-  for (int t = 0; t < 16; ++t) ld2(tp + roff[t], x[0][t], x[1][t]);
+template <bool ALIGNED>
+__device__ __forceinline__ void store_row(bf16_t* rp, const Lane<bf16_t>& L, float a, float b) {
+  if constexpr (ALIGNED) {
+    *reinterpret_cast<uint32_t*>(rp + 2 * L.i) = pack_bf2(a, b);
+  } else {
+    rp[2 * L.i] = from_f32<bf16_t>(a);
+    rp[2 * L.i + 1] = from_f32<bf16_t>(b);
+  }
 }
-
-// one value per tile row, lane i of either half holding row i (clamped like the operands)
-__device__ __forceinline__ float load_lane(const float* hp, int64_t stride, int base, int n, int i) {
-  const int last = n - 1 - base;
-  return hp[(int64_t)(base + (i < last ? i : last)) * stride];
+template <bool ALIGNED, class T>
+__device__ __forceinline__ void store_tile(T* hp, int ld, int base, int lo, int hi, const Lane<T>& L,
+                                           const float (&x)[2][16]) {
+  T* tp = hp + (int64_t)base * ld;
+  if (lo == 0 && hi == 32) {
+#pragma unroll
+    for (int t = 0; t < 16; ++t) store_row<ALIGNED>(tp + trow(t, L.hh) * ld, L, x[0][t], x[1][t]);
+  } else {
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+      if (trow(t, L.hh) >= lo && trow(t, L.hh) < hi) store_row<ALIGNED>(tp + trow(t, L.hh) * ld, L, x[0][t], x[1][t]);
+  }
 }
 
 __device__ __forceinline__ float half_swap_add(float x) { return x + __shfl_xor(x, 32, 64); }
 __device__ __forceinline__ float rcp(float x) { return __builtin_amdgcn_rcpf(x); }  // 1 ulp
 
-// token-major element that contracts against register t of state tile row-class rc
-__device__ __forceinline__ constexpr int tok_of(int t, int rc) { return (t >> 2) * 8 + 2 * (t & 3) + rc; }
+// A 64-vector over channels, held as (chan(0, i), chan(1, i)) by the lanes of either half, goes
+// through LDS to be dotted with a token-major operand: returns the lane half's part of x . vec.
+template <class T>
+__device__ __forceinline__ void vec_put(float* lds64, const Lane<T>& L, float v0, float v1) {
+  if (L.l < 32) {
+    lds64[Map<T>::chan(0, L.i)] = v0;
+    lds64[Map<T>::chan(1, L.i)] = v1;
+  }
+}
+template <class T>
+__device__ __forceinline__ float vec_dot(const float* lds64, const Lane<T>& L, const float (&x)[32]) {
+  float s = 0.f;
+  if constexpr (Map<T>::PAIR) {
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+      const float4 u = *reinterpret_cast<const float4*>(&lds64[16 * (g >> 1) + 8 * L.hh + 4 * (g & 1)]);
+      s += x[4 * g] * u.x + x[4 * g + 1] * u.y + x[4 * g + 2] * u.z + x[4 * g + 3] * u.w;
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {   // g = rc * 4 + (group of four rows)
+      const float4 u = *reinterpret_cast<const float4*>(&lds64[32 * (g >> 2) + 8 * (g & 3) + 4 * L.hh]);
+      s += x[4 * g] * u.x + x[4 * g + 1] * u.y + x[4 * g + 2] * u.z + x[4 * g + 3] * u.w;
+    }
+  }
+  return s;
+}
 
 // ---- the matrix phases of a tile (all kernels of this file share them) ----------------------
 
 // Score tile P (rows = rows of `a`, columns = rows of `b`, contraction over the 64 channels) and
-// own rows x running state, O[own row][2n+cc] = sum_ch own[ch] State[ch][2n+cc] (the state's
-// accumulator registers are the B operand).  The three accumulation chains are independent and
-// issued interleaved.
+// own rows x running state, O[own row][chan(cc, n)] = sum_ch own[ch] State[ch][chan(cc, n)] (the
+// state's accumulator registers are the B operand).  The three accumulation chains are
+// independent and issued interleaved.
+template <class T>
 __device__ __forceinline__ void score_and_state(const float (&a)[32], const float (&b)[32],
                                                 const float (&own)[32], const f16v (&S)[2][2], f16v& P,
                                                 f16v (&O)[2]) {
@@ -131,12 +206,12 @@ __device__ __forceinline__ void score_and_state(const float (&a)[32], const floa
 #pragma unroll
     for (int rc = 0; rc < 2; ++rc) {
       P = FM_MFMA(a[2 * t + rc], b[2 * t + rc], P);
-      O[0] = FM_MFMA(own[tok_of(t, rc)], S[rc][0][t], O[0]);
-      O[1] = FM_MFMA(own[tok_of(t, rc)], S[rc][1][t], O[1]);
+      O[0] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][0][t], O[0]);
+      O[1] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][1][t], O[1]);
     }
 }
 
-// State[2m+rc][2n+cc] += sum over the tile's rows of ua[row][2m+rc] * ub[row][2n+cc]
+// State[chan(rc, m)][chan(cc, n)] += sum over the tile's rows of ua[row][chan(rc, m)] * ub[row][chan(cc, n)]
 __device__ __forceinline__ void state_update(f16v (&S)[2][2], const float (&ua)[2][16], const float (&ub)[2][16]) {
 #pragma unroll
   for (int t = 0; t < 16; ++t) {
@@ -147,8 +222,8 @@ __device__ __forceinline__ void state_update(f16v (&S)[2][2], const float (&ua)[
   }
 }
 
-// O[own row][2n+cc] += sum over streamed rows of W[streamed][own] * ub[streamed][2n+cc]; the
-// weights are fed from their accumulator registers as the A operand
+// O[own row][chan(cc, n)] += sum over streamed rows of W[streamed][own] * ub[streamed][chan(cc, n)];
+// the weights are fed from their accumulator registers as the A operand
 __device__ __forceinline__ void weight_product(const f16v& W, const float (&ub)[2][16], f16v (&O)[2]) {
 #pragma unroll
   for (int t = 0; t < 16; ++t) {
@@ -158,11 +233,12 @@ __device__ __forceinline__ void weight_product(const f16v& W, const float (&ub)[
 }
 
 // x[t] = v[trow(t, hh)] for a value v held per lane (lane i of either half = tile row i)
-__device__ __forceinline__ void rows_from_lanes(float v, float* lds32, int l, int hh, float (&x)[16]) {
-  if (l < 32) lds32[l] = v;
+template <class T>
+__device__ __forceinline__ void rows_from_lanes(float v, float* lds32, const Lane<T>& L, float (&x)[16]) {
+  if (L.l < 32) lds32[L.l] = v;
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const float4 u = *reinterpret_cast<const float4*>(&lds32[8 * g + 4 * hh]);
+    const float4 u = *reinterpret_cast<const float4*>(&lds32[8 * g + 4 * L.hh]);
     x[4 * g] = u.x; x[4 * g + 1] = u.y; x[4 * g + 2] = u.z; x[4 * g + 3] = u.w;
   }
 }
@@ -171,34 +247,6 @@ __device__ __forceinline__ float wave_sum(float x) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off, 64);
   return x;
-}
-
-// x[c][t] -> row trow(t, hh) of the tile, columns 2i + c (rows past the end are skipped)
-template <bool ALIGNED, class T>
-__device__ __forceinline__ void store_tile(T* hp, int ld, int base, int n, int i, int hh, const float (&x)[2][16]) {
-  T* tp = hp + (int64_t)base * ld;
-  if (base + 32 <= n) {
-#pragma unroll
-    for (int t = 0; t < 16; ++t) st2<ALIGNED>(tp + (trow(t, hh) * ld + 2 * i), x[0][t], x[1][t]);
-  } else {
-#pragma unroll
-    for (int t = 0; t < 16; ++t)
-      if (base + trow(t, hh) < n) st2<ALIGNED>(tp + (trow(t, hh) * ld + 2 * i), x[0][t], x[1][t]);
-  }
-}
-
-// sum over the tile's valid rows of x . y (both in the output layout)
-__device__ __forceinline__ float tile_dot(const float (&x)[2][16], const float (&y)[2][16], int base, int n, int hh) {
-  float s = 0.f;
-  if (base + 32 <= n) {
-#pragma unroll
-    for (int t = 0; t < 16; ++t) s += x[0][t] * y[0][t] + x[1][t] * y[1][t];
-  } else {
-#pragma unroll
-    for (int t = 0; t < 16; ++t)
-      if (base + trow(t, hh) < n) s += x[0][t] * y[0][t] + x[1][t] * y[1][t];
-  }
-  return s;
 }
 
 __device__ __forceinline__ void zero_state(f16v (&S)[2][2]) {
@@ -210,12 +258,38 @@ __device__ __forceinline__ void zero_state(f16v (&S)[2][2]) {
       for (int t = 0; t < 16; ++t) S[a][b][t] = 0.f;
 }
 
+// rows of a channel-major operand outside [lo, hi) -> 0 (the shared rows of a moved-back tile)
+__device__ __forceinline__ void keep_rows(float (&x)[2][16], int lo, int hi, int hh) {
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    const bool in = trow(t, hh) >= lo && trow(t, hh) < hi;
+    x[0][t] = in ? x[0][t] : 0.f;
+    x[1][t] = in ? x[1][t] : 0.f;
+  }
+}
+
+// per-lane sums over the tile's rows of a channel-major operand: s[c] = sum_rows x[row][chan(c, i)]
+__device__ __forceinline__ void column_sums(const float (&x)[2][16], float (&s)[2]) {
+  float a = 0.f, b = 0.f;
+#pragma unroll
+  for (int t = 0; t < 16; ++t) a += x[0][t], b += x[1][t];
+  s[0] = half_swap_add(a);
+  s[1] = half_swap_add(b);
+}
+
+// Tiles of a forward scan: tile tt covers rows [fbase, fbase + 32), fbase = min(32 tt, n - 32);
+// its first 32 tt - fbase rows were already part of tile tt - 1.
+__device__ __forceinline__ int fbase(int tt, int n) { return 32 * tt < n - 32 ? 32 * tt : n - 32; }
+// Tiles of a reverse scan: tile tt covers rows [rbase, rbase + 32), rbase = max(n - 32 (tt + 1), 0);
+// only its first n - 32 tt - rbase rows are new.
+__device__ __forceinline__ int rbase(int tt, int n) { return n - 32 * (tt + 1) > 0 ? n - 32 * (tt + 1) : 0; }
+
 // ---------------------------------------------------------------------------------------
 // Forward: o_i = [a0 sum_{j<=i} v_j + a1' sum_{j<=i} (q_i.k_j) v_j] / [a0 (i+1) + a1' q_i . sum_{j<=i} k_j]
-// with a1' = a1 * qscale * kscale (the normaliser folded into the coefficient, which is applied
-// to the query rows as they are loaded; the state is built from the raw keys).
-// State: S1[a][c] = sum k_j[a] v_j[c], s1[a] = sum k_j[a], s0[c] = sum v_j[c].
-// grid = heads, block = one wave.
+// with a1' = a1 * qscale * kscale (the normaliser folded into the coefficient; the state is built
+// from the raw keys).  State: S1[a][c] = sum k_j[a] v_j[c], s1[a] = sum k_j[a], s0[c] = sum v_j[c].
+// The weights are kept as f(s)/a1' = a0/a1' + q_i.k_j, so one accumulator takes q_i S1 and the
+// intra-tile product.  grid = heads, block = one wave; n >= 32, a1 != 0.
 // ---------------------------------------------------------------------------------------
 template <class T, bool ALIGNED>
 __global__ __launch_bounds__(64) void linear_fwd_kernel(const T* __restrict__ q, const T* __restrict__ k,
@@ -226,114 +300,95 @@ __global__ __launch_bounds__(64) void linear_fwd_kernel(const T* __restrict__ q,
                                                         int64_t den_stride, int n, float a0, float a1) {
   __shared__ __attribute__((aligned(16))) float s1l[D];
   __shared__ __attribute__((aligned(16))) float denl[32];
-  const int head = blockIdx.x, l = threadIdx.x, i = l & 31, hh = l >> 5;
+  const Lane<T> L;
+  const int head = blockIdx.x;
   const T* qh = q + (int64_t)head * n * D;
   const T* kh = k + (int64_t)head * n * D;
   const T* vh = v + (int64_t)head * n * D;
   T* oh = o + (int64_t)head * n * ldo;
   float* dh = den + (int64_t)head * n * den_stride;
   const float a1s = a1 * qscale[head] * kscale[head];
+  const float a0r = a0 / a1s;
 
   f16v S1[2][2];
   zero_state(S1);
   float s0[2] = {0.f, 0.f}, s1[2] = {0.f, 0.f};
-  if (l < 32) *reinterpret_cast<float2*>(&s1l[2 * l]) = make_float2(0.f, 0.f);
-
-  float qt[32], kt[32], kc[2][16], vc[2][16];
-  int roff[16];
-  row_offsets(n - 1, i, hh, roff);
-  load_tok<T>(kh, 0, n, i, hh, kt);
-  load_tok<T>(qh, 0, n, i, hh, qt);
-  load_ch<T>(kh, 0, roff, kc);
-  load_ch<T>(vh, 0, roff, vc);
+  float qt[32], kt[32], kc[2][16] = {}, vc[2][16] = {};   // (tile "-1" is empty)
+  load_tok(kh, 0, L, kt);
+  load_tok(qh, 0, L, qt);
 
   const int ntiles = (n + 31) >> 5;
-  for (int tile = 0; tile < ntiles; ++tile) {
-    const int base = tile << 5;
-    // the next tile is fetched while this one is worked on (after the last tile: this one again,
-    // unused, so that the loop has a single straight path); a ragged next tile needs new offsets
-    const int nb = tile + 1 < ntiles ? base + 32 : base;
-    if (n - 1 - nb < 31) row_offsets(n - 1 - nb, i, hh, roff);
-#pragma unroll
-    for (int e = 0; e < 32; ++e) qt[e] *= a1s;
+  for (int tt = 0; tt < ntiles; ++tt) {
+    const int base = fbase(tt, n), skip = 32 * tt - base;
+    // (after the last tile the "next" one is this one again, unused: one straight path)
+    const int nb = tt + 1 < ntiles ? fbase(tt + 1, n) : base;
+
+    // the previous tile joins the state
+    state_update(S1, kc, vc);
+    {
+      float ks[2], vs[2];
+      column_sums(kc, ks);
+      column_sums(vc, vs);
+      s1[0] += ks[0]; s1[1] += ks[1];
+      s0[0] += vs[0]; s0[1] += vs[1];
+      vec_put<T>(s1l, L, s1[0], s1[1]);
+    }
+    FM_PIN();
+    load_ch(kh, base, L, kc);
+    load_ch(vh, base, L, vc);
+    FM_PIN();
 
     // transposed score tile (rows = keys of the tile, columns = queries); own rows x state
     f16v P, O[2];
-    score_and_state(kt, qt, qt, S1, P, O);
+    score_and_state<T>(kt, qt, qt, S1, P, O);
+    // q_i . s1 (the lane's 32 channels, then the other half's)
+    const float qs = half_swap_add(vec_dot<T>(s1l, L, qt));
     FM_PIN();
-    load_tok<T>(kh, nb, n, i, hh, kt);
+    load_tok(kh, nb, L, kt);
+    load_tok(qh, nb, L, qt);
     FM_PIN();
 
-    // weights f(s) of the visible keys (key <= query; a key past the end is only ever "visible"
-    // to queries past the end) and their sum
+    // weights f(s)/a1' of the visible keys and their sum
     float dsum = 0.f;
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
-      const float w = trow(t, hh) <= i ? a0 + P[t] : 0.f;
+      const int r = trow(t, L.hh);
+      const float w = (r <= L.i && r >= skip) ? a0r + P[t] : 0.f;
       P[t] = w;
       dsum += w;
     }
-    dsum = half_swap_add(dsum);
-    // a1' q_i . s1 (the lane's 32 channels, then the other half's)
-    float qs = 0.f;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const float4 u0 = *reinterpret_cast<const float4*>(&s1l[16 * g + 8 * hh]);
-      const float4 u1 = *reinterpret_cast<const float4*>(&s1l[16 * g + 8 * hh + 4]);
-      qs += qt[8 * g] * u0.x + qt[8 * g + 1] * u0.y + qt[8 * g + 2] * u0.z + qt[8 * g + 3] * u0.w +
-            qt[8 * g + 4] * u1.x + qt[8 * g + 5] * u1.y + qt[8 * g + 6] * u1.z + qt[8 * g + 7] * u1.w;
-    }
-    const float den_i = dsum + a0 * (float)base + half_swap_add(qs);   // query base + i
-    FM_PIN();
-    load_tok<T>(qh, nb, n, i, hh, qt);
-    FM_PIN();
-
-    // state update (rows past the end only reach a state nobody reads: this is the last tile)
-    const float s0a[2] = {a0 * s0[0], a0 * s0[1]};   // order-0 term of this tile's rows
-    state_update(S1, kc, vc);
-    {
-      float ks[2] = {0.f, 0.f}, vs[2] = {0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int t = 0; t < 16; ++t) ks[c] += kc[c][t], vs[c] += vc[c][t];
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        s1[c] += half_swap_add(ks[c]);
-        s0[c] += half_swap_add(vs[c]);
-      }
-      if (l < 32) *reinterpret_cast<float2*>(&s1l[2 * l]) = make_float2(s1[0], s1[1]);
-    }
-    FM_PIN();
-    load_ch<T>(kh, nb, roff, kc);
-    FM_PIN();
+    // query base + i sees the 32 tt keys of the state and the tile's visible ones
+    const float den_i = a1s * (half_swap_add(dsum) + qs) + a0 * (float)(32 * tt);
 
     // intra-tile part: weights x values
     weight_product(P, vc, O);
-    FM_PIN();
-    load_ch<T>(vh, nb, roff, vc);
-    FM_PIN();
 
     // denominators move from "lane = token" to the row order of the output registers
-    if (l < 32 && base + l < n) dh[(int64_t)(base + l) * den_stride] = den_i;
-    float inv[16];
-    rows_from_lanes(rcp(den_i), denl, l, hh, inv);
-    float x[2][16];
+    if (L.l < 32 && L.l >= skip) dh[(int64_t)(base + L.l) * den_stride] = den_i;
+    float inv[16], x[2][16];
+    rows_from_lanes(rcp(den_i), denl, L, inv);
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int t = 0; t < 16; ++t) x[c][t] = (O[c][t] + s0a[c]) * inv[t];
-    store_tile<ALIGNED, T>(oh, (int)ldo, base, n, i, hh, x);
+      for (int t = 0; t < 16; ++t) x[c][t] = (a1s * O[c][t] + a0 * s0[c]) * inv[t];
+    store_tile<ALIGNED, T>(oh, (int)ldo, base, skip, 32, L, x);
   }
 }
 
 // ---------------------------------------------------------------------------------------
 // Backward.  g_i = go_i / den_i, c_i = g_i . o_i (cvec), a1' as above.  Gradients with respect to
-// the raw inputs (the normaliser's factor folded in), plus, when NORM, rpart[head] =
-// sum_rows dx_hat . x_hat for the normalisation chain rule.
+// the raw inputs (the normaliser's factor folded in).
 //
 // dq_i = a1' [ sum_{j<=i} (g_i.v_j - c_i) k_j ]:  forward scan, state T[c][a] = sum v_j[c] k_j[a],
-//        s1[a] = sum k_j[a];  dq_i = a1' [ g_i T - c_i s1 + intra-tile part ].
+//        s1[a] = sum k_j[a];  dq_i = a1' [ g_i T - c_i s1 + intra-tile part ].  The weights are kept
+// multiplied by den_i, go_i.v_j - c_i den_i, so that one accumulator takes go_i T and the
+// intra-tile product; 1/den_i scales its rows at the end.
+// When NORM, rpart[head] = sum_i dq_hat_i . q_hat_i for the normalisation chain rule (the same
+// number serves k: sum_j dk_hat_j . k_hat_j = sum_ij W_ij s_ij as well).  With f linear it has
+// a closed form that needs no q: a1 sum_j s_ij = den_i - a0 (i+1) and a1 sum_j s_ij g_i.v_j =
+// c_i den_i - a0 g_i . V_i, V_i = sum_{j<=i} v_j, give  sum_ij W_ij s_ij = a0 sum_i [c_i (i+1) - g_i . V_i].
+// That rests on o_i = num_i / den_i holding to working precision, so it is used for fp32 only;
+// with bf16 tensors (o rounded to 8 bits) the partial is formed directly as sum_i dq_i . q_i.
 // ---------------------------------------------------------------------------------------
 template <class T, bool NORM>
 __global__ __launch_bounds__(64) void linear_dq_kernel(const T* __restrict__ go, const float* __restrict__ den,
@@ -342,94 +397,110 @@ __global__ __launch_bounds__(64) void linear_dq_kernel(const T* __restrict__ go,
                                                        const T* __restrict__ v,
                                                        const float* __restrict__ qscale,
                                                        const float* __restrict__ kscale, T* __restrict__ dq,
-                                                       float* __restrict__ rpart, int n, float a1) {
+                                                       float* __restrict__ rpart, int n, float a0, float a1) {
   __shared__ __attribute__((aligned(16))) float cl[32];
-  const int head = blockIdx.x, l = threadIdx.x, i = l & 31, hh = l >> 5;
+  __shared__ __attribute__((aligned(16))) float dl[32];
+  __shared__ __attribute__((aligned(16))) float s0l[D];
+  const Lane<T> L;
+  const int head = blockIdx.x;
   const T* gh = go + (int64_t)head * n * D;
-  const T* qh = q + (int64_t)head * n * D;
   const T* kh = k + (int64_t)head * n * D;
   const T* vh = v + (int64_t)head * n * D;
   const float* dh = den + (int64_t)head * n * den_stride;
   const float* ch = cvec + (int64_t)head * n;
   T* oh = dq + (int64_t)head * n * D;
   const float a1s = a1 * qscale[head] * kscale[head];
+  constexpr bool CLOSED = NORM && Map<T>::CLOSED_R, DIRECT = NORM && !Map<T>::CLOSED_R;
+  const T* qh = q + (int64_t)head * n * D;
 
   f16v S[2][2];
   zero_state(S);
-  float s1[2] = {0.f, 0.f}, rs = 0.f;
-
-  float gt[32], vt[32], vc[2][16], kc[2][16], qc[2][16];
-  int roff[16];
-  row_offsets(n - 1, i, hh, roff);
-  load_tok<T>(vh, 0, n, i, hh, vt);
-  load_tok<T>(gh, 0, n, i, hh, gt);
-  float den_l = load_lane(dh, den_stride, 0, n, i), c_l = load_lane(ch, 1, 0, n, i);
-  load_ch<T>(vh, 0, roff, vc);
-  load_ch<T>(kh, 0, roff, kc);
+  float s1[2] = {0.f, 0.f}, s0[2] = {0.f, 0.f}, rs = 0.f;
+  float gt[32], vt[32], vc[2][16] = {}, kc[2][16] = {};   // (tile "-1" is empty)
+  float qc[2][16];
+  load_tok(vh, 0, L, vt);
+  load_tok(gh, 0, L, gt);
+  float den_l = dh[(int64_t)L.i * den_stride], c_l = ch[L.i];
 
   const int ntiles = (n + 31) >> 5;
-  for (int tile = 0; tile < ntiles; ++tile) {
-    const int base = tile << 5;
-    if (NORM) load_ch<T>(qh, base, roff, qc);   // only for the normalisation partial at the end
-    const int nb = tile + 1 < ntiles ? base + 32 : base;   // next tile (see linear_fwd_kernel)
-    if (n - 1 - nb < 31) row_offsets(n - 1 - nb, i, hh, roff);
-    {
-      const float inv = rcp(den_l);
-#pragma unroll
-      for (int e = 0; e < 32; ++e) gt[e] *= inv;
-    }
-    const float c_cur = c_l;
-    // rows = keys, columns = queries: g_i . v_j; own rows x state
-    f16v W, O[2];
-    score_and_state(vt, gt, gt, S, W, O);
-    FM_PIN();
-    load_tok<T>(vh, nb, n, i, hh, vt);
-    load_tok<T>(gh, nb, n, i, hh, gt);
-    den_l = load_lane(dh, den_stride, nb, n, i);
-    c_l = load_lane(ch, 1, nb, n, i);
-    FM_PIN();
-#pragma unroll
-    for (int t = 0; t < 16; ++t) W[t] = trow(t, hh) <= i ? W[t] - c_cur : 0.f;
-    float cT[16];
-    rows_from_lanes(c_cur, cl, l, hh, cT);
+  for (int tt = 0; tt < ntiles; ++tt) {
+    const int base = fbase(tt, n), skip = 32 * tt - base;
+    const int nb = tt + 1 < ntiles ? fbase(tt + 1, n) : base;   // next tile (see linear_fwd_kernel)
+    const float den_cur = den_l, c_cur = c_l, inv_l = rcp(den_l);
 
-    const float s1old[2] = {s1[0], s1[1]};
+    // the previous tile joins the state
     state_update(S, vc, kc);
     {
-      float ks[2] = {0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int t = 0; t < 16; ++t) ks[c] += kc[c][t];
-      s1[0] += half_swap_add(ks[0]);
-      s1[1] += half_swap_add(ks[1]);
+      float ks[2];
+      column_sums(kc, ks);
+      s1[0] += ks[0]; s1[1] += ks[1];
+      if (CLOSED) {
+        float vs[2];
+        column_sums(vc, vs);
+        s0[0] += vs[0]; s0[1] += vs[1];
+        vec_put<T>(s0l, L, s0[0], s0[1]);
+      }
     }
     FM_PIN();
-    load_ch<T>(vh, nb, roff, vc);
+    load_ch(vh, base, L, vc);
+    load_ch(kh, base, L, kc);
+    if (DIRECT) load_ch(qh, base, L, qc);
     FM_PIN();
 
+    // rows = keys, columns = queries: go_i . v_j; own rows (go) x state
+    f16v W, O[2];
+    score_and_state<T>(vt, gt, gt, S, W, O);
+    float gv = 0.f;
+    if (CLOSED) gv = half_swap_add(vec_dot<T>(s0l, L, gt));   // go_i . (sum of the state's v_j)
+    FM_PIN();
+    load_tok(vh, nb, L, vt);
+    load_tok(gh, nb, L, gt);
+    den_l = dh[(int64_t)(nb + L.i) * den_stride];
+    c_l = ch[nb + L.i];
+    FM_PIN();
+    {
+      const float cd = c_cur * den_cur;
+      float psum = 0.f;
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        const int r = trow(t, L.hh);
+        const bool vis = r <= L.i && r >= skip;
+        psum += vis ? W[t] : 0.f;
+        W[t] = vis ? W[t] - cd : 0.f;
+      }
+      if (CLOSED) {
+        const float ri = c_cur * (float)(base + L.i + 1) - inv_l * (half_swap_add(psum) + gv);
+        rs += (L.l < 32 && L.i >= skip) ? ri : 0.f;
+      }
+    }
+    float cT[16], inv[16];
+    rows_from_lanes(c_cur, cl, L, cT);
+    rows_from_lanes(inv_l, dl, L, inv);
+
     weight_product(W, kc, O);
-    FM_PIN();
-    load_ch<T>(kh, nb, roff, kc);
-    FM_PIN();
 
     float x[2][16];
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int t = 0; t < 16; ++t) x[c][t] = a1s * (O[c][t] - cT[t] * s1old[c]);
-    store_tile<true, T>(oh, D, base, n, i, hh, x);
-    if (NORM) rs += tile_dot(x, qc, base, n, hh);
+      for (int t = 0; t < 16; ++t) x[c][t] = a1s * (inv[t] * O[c][t] - cT[t] * s1[c]);
+    store_tile<true, T>(oh, D, base, skip, 32, L, x);
+    if (DIRECT) {
+#pragma unroll
+      for (int t = 0; t < 16; ++t)
+        rs += trow(t, L.hh) >= skip ? x[0][t] * qc[0][t] + x[1][t] * qc[1][t] : 0.f;
+    }
   }
   if (NORM) {
     rs = wave_sum(rs);
-    if (l == 0) rpart[head] = rs;
+    if (L.l == 0) rpart[head] = CLOSED ? a0 * rs : rs;
   }
 }
 
 // ---------------------------------------------------------------------------------------
 // dv_j = sum_{i>=j} f(s_ij) g_i:  reverse scan, state R[a][c] = sum q_i[a] g_i[c], r0[c] = sum g_i[c];
-//        dv_j = a0 r0 + a1' k_j R + intra-tile part.  Rows past the end enter with g = 0.
+//        dv_j = a0 r0 + a1' [ k_j R + intra-tile part with the weights f(s)/a1' ].  Rows of a
+// moved-back tile that are already in the state enter with g = 0.
 // ---------------------------------------------------------------------------------------
 template <class T>
 __global__ __launch_bounds__(64) void linear_dv_kernel(const T* __restrict__ go, const float* __restrict__ den,
@@ -439,88 +510,77 @@ __global__ __launch_bounds__(64) void linear_dv_kernel(const T* __restrict__ go,
                                                        const float* __restrict__ kscale, T* __restrict__ dv,
                                                        int n, float a0, float a1) {
   __shared__ __attribute__((aligned(16))) float dl[32];
-  const int head = blockIdx.x, l = threadIdx.x, i = l & 31, hh = l >> 5;
+  const Lane<T> L;
+  const int head = blockIdx.x;
   const T* gh = go + (int64_t)head * n * D;
   const T* qh = q + (int64_t)head * n * D;
   const T* kh = k + (int64_t)head * n * D;
   const float* dh = den + (int64_t)head * n * den_stride;
   T* oh = dv + (int64_t)head * n * D;
   const float a1s = a1 * qscale[head] * kscale[head];
+  const float a0r = a0 / a1s;
 
   f16v S[2][2];
   zero_state(S);
   float r0[2] = {0.f, 0.f};
 
   const int ntiles = (n + 31) >> 5;
-  const int b0 = (ntiles - 1) << 5;
-  float qt[32], kt[32], qc[2][16], gc[2][16];
-  int roff[16];
-  row_offsets(n - 1 - b0, i, hh, roff);   // the last tile may be ragged; it is the first one here
-  load_tok<T>(qh, b0, n, i, hh, qt);
-  load_tok<T>(kh, b0, n, i, hh, kt);
-  float den_l = load_lane(dh, den_stride, b0, n, i);
-  load_ch<T>(qh, b0, roff, qc);
-  load_ch<T>(gh, b0, roff, gc);
-  if (ntiles > 1) row_offsets(31, i, hh, roff);   // every other tile is full
+  float qt[32], kt[32], qc[2][16] = {}, gc[2][16] = {};   // (tile "-1" is empty)
+  load_tok(qh, n - 32, L, qt);
+  load_tok(kh, n - 32, L, kt);
+  float den_l = dh[(int64_t)(n - 32 + L.i) * den_stride];
 
-  for (int tile = ntiles - 1; tile >= 0; --tile) {
-    const int base = tile << 5;
-    const int nb = tile > 0 ? base - 32 : base;   // next tile (see linear_fwd_kernel)
-#pragma unroll
-    for (int e = 0; e < 32; ++e) kt[e] *= a1s;
-    const float inv_l = base + i < n ? rcp(den_l) : 0.f;
-    // rows = queries, columns = keys; own rows x state
-    f16v P, O[2];
-    score_and_state(qt, kt, kt, S, P, O);
+  for (int tt = 0; tt < ntiles; ++tt) {
+    const int base = rbase(tt, n), hi = n - 32 * tt - base;      // tile rows [0, hi) are new
+    const int nb = tt + 1 < ntiles ? rbase(tt + 1, n) : base;    // next tile (see linear_fwd_kernel)
+    const float inv_l = L.i < hi ? rcp(den_l) : 0.f;
+
+    // the previous tile (its g rows already divided by den) joins the state
+    state_update(S, qc, gc);
+    {
+      float gs[2];
+      column_sums(gc, gs);
+      r0[0] += gs[0]; r0[1] += gs[1];
+    }
     FM_PIN();
-    load_tok<T>(qh, nb, n, i, hh, qt);
-    load_tok<T>(kh, nb, n, i, hh, kt);
-    den_l = load_lane(dh, den_stride, nb, n, i);
+    load_ch(qh, base, L, qc);
+    load_ch(gh, base, L, gc);
+    FM_PIN();
+
+    // rows = queries, columns = keys; own rows (k) x state
+    f16v P, O[2];
+    score_and_state<T>(qt, kt, kt, S, P, O);
+    FM_PIN();
+    load_tok(qh, nb, L, qt);
+    load_tok(kh, nb, L, kt);
+    den_l = dh[(int64_t)(nb + L.i) * den_stride];
     FM_PIN();
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
-      const int r = trow(t, hh);
-      P[t] = (r >= i && base + r < n) ? a0 + P[t] : 0.f;
+      const int r = trow(t, L.hh);
+      P[t] = (r >= L.i && r < hi) ? a0r + P[t] : 0.f;
     }
     float inv[16];
-    rows_from_lanes(inv_l, dl, l, hh, inv);
-    const float r0a[2] = {a0 * r0[0], a0 * r0[1]};
-    {
-      float gs[2] = {0.f, 0.f};
+    rows_from_lanes(inv_l, dl, L, inv);
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < 2; ++c)
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
-          gc[c][t] *= inv[t];
-          gs[c] += gc[c][t];
-        }
-      state_update(S, qc, gc);
-      r0[0] += half_swap_add(gs[0]);
-      r0[1] += half_swap_add(gs[1]);
-    }
-    FM_PIN();
-    load_ch<T>(qh, nb, roff, qc);
-    FM_PIN();
+      for (int t = 0; t < 16; ++t) gc[c][t] *= inv[t];
 
     weight_product(P, gc, O);
-    FM_PIN();
-    load_ch<T>(gh, nb, roff, gc);
-    FM_PIN();
 
     float x[2][16];
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int t = 0; t < 16; ++t) x[c][t] = O[c][t] + r0a[c];
-    store_tile<true, T>(oh, D, base, n, i, hh, x);
+      for (int t = 0; t < 16; ++t) x[c][t] = a1s * O[c][t] + a0 * r0[c];
+    store_tile<true, T>(oh, D, base, 0, hi, L, x);
   }
 }
 
 // ---------------------------------------------------------------------------------------
 // dk_j = a1' [ sum_{i>=j} (g_i.v_j - c_i) q_i ]:  reverse scan, state Rt[c][a] = sum g_i[c] q_i[a],
 //        r1[a] = sum c_i q_i[a];  dk_j = a1' [ v_j Rt - r1 + intra-tile part ].
-// (No normalisation partial here: sum_j dk_hat_j . k_hat_j = sum_ij W_ij s_ij = sum_i dq_hat_i . q_hat_i,
-// the dq kernel's.)
 // ---------------------------------------------------------------------------------------
 template <class T>
 __global__ __launch_bounds__(64) void linear_dk_kernel(const T* __restrict__ go, const float* __restrict__ den,
@@ -531,7 +591,8 @@ __global__ __launch_bounds__(64) void linear_dk_kernel(const T* __restrict__ go,
                                                        int n, float a1) {
   __shared__ __attribute__((aligned(16))) float dl[32];
   __shared__ __attribute__((aligned(16))) float cl[32];
-  const int head = blockIdx.x, l = threadIdx.x, i = l & 31, hh = l >> 5;
+  const Lane<T> L;
+  const int head = blockIdx.x;
   const T* gh = go + (int64_t)head * n * D;
   const T* qh = q + (int64_t)head * n * D;
   const T* vh = v + (int64_t)head * n * D;
@@ -542,76 +603,68 @@ __global__ __launch_bounds__(64) void linear_dk_kernel(const T* __restrict__ go,
 
   f16v S[2][2];
   zero_state(S);
-  float r1[2] = {0.f, 0.f};
+  float r1[2] = {0.f, 0.f}, r1next[2] = {0.f, 0.f};
 
   const int ntiles = (n + 31) >> 5;
-  const int b0 = (ntiles - 1) << 5;
-  float gt[32], vt[32], gc[2][16], qc[2][16];
-  int roff[16];
-  row_offsets(n - 1 - b0, i, hh, roff);   // the last tile may be ragged; it is the first one here
-  load_tok<T>(gh, b0, n, i, hh, gt);
-  load_tok<T>(vh, b0, n, i, hh, vt);
-  float den_l = load_lane(dh, den_stride, b0, n, i), c_l = load_lane(ch, 1, b0, n, i);
-  load_ch<T>(gh, b0, roff, gc);
-  load_ch<T>(qh, b0, roff, qc);
-  if (ntiles > 1) row_offsets(31, i, hh, roff);   // every other tile is full
+  float gt[32], vt[32], gc[2][16] = {}, qc[2][16] = {};   // (tile "-1" is empty)
+  load_tok(gh, n - 32, L, gt);
+  load_tok(vh, n - 32, L, vt);
+  float den_l = dh[(int64_t)(n - 32 + L.i) * den_stride], c_l = ch[n - 32 + L.i];
 
-  for (int tile = ntiles - 1; tile >= 0; --tile) {
-    const int base = tile << 5;
-    const int nb = tile > 0 ? base - 32 : base;   // next tile (see linear_fwd_kernel)
-    const bool inside = base + i < n;
-    const float inv_l = inside ? rcp(den_l) : 0.f;
-    const float c_cur = inside ? c_l : 0.f;
-#pragma unroll
-    for (int e = 0; e < 32; ++e) gt[e] *= inv_l;
-
-    // rows = queries, columns = keys: g_i . v_j; own rows x state
-    f16v W, O[2];
-    score_and_state(gt, vt, vt, S, W, O);
-    FM_PIN();
-    load_tok<T>(gh, nb, n, i, hh, gt);
-    load_tok<T>(vh, nb, n, i, hh, vt);
-    den_l = load_lane(dh, den_stride, nb, n, i);
-    c_l = load_lane(ch, 1, nb, n, i);
-    FM_PIN();
+  for (int tt = 0; tt < ntiles; ++tt) {
+    const int base = rbase(tt, n), hi = n - 32 * tt - base;      // tile rows [0, hi) are new
+    const int nb = tt + 1 < ntiles ? rbase(tt + 1, n) : base;    // next tile (see linear_fwd_kernel)
+    const bool fresh = L.i < hi;
+    const float inv_l = fresh ? rcp(den_l) : 0.f;
+    const float c_cur = fresh ? c_l : 0.f;
     float inv[16], cT[16];
-    rows_from_lanes(inv_l, dl, l, hh, inv);
-    rows_from_lanes(c_cur, cl, l, hh, cT);
+    rows_from_lanes(inv_l, dl, L, inv);
+    rows_from_lanes(c_cur, cl, L, cT);
+
+    // the previous tile (its g rows already divided by den) joins the state
+    state_update(S, gc, qc);
+    r1[0] += r1next[0];
+    r1[1] += r1next[1];
+    FM_PIN();
+    load_ch(gh, base, L, gc);
+    load_ch(qh, base, L, qc);
+    FM_PIN();
+
+    // rows = queries, columns = keys: go_i . v_j; own rows (v) x state
+    f16v W, O[2];
+    score_and_state<T>(gt, vt, vt, S, W, O);
+    FM_PIN();
+    load_tok(gh, nb, L, gt);
+    load_tok(vh, nb, L, vt);
+    den_l = dh[(int64_t)(nb + L.i) * den_stride];
+    c_l = ch[nb + L.i];
+    FM_PIN();
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
-      const int r = trow(t, hh);
-      W[t] = (r >= i && base + r < n) ? W[t] - cT[t] : 0.f;
+      const int r = trow(t, L.hh);
+      W[t] = (r >= L.i && r < hi) ? W[t] * inv[t] - cT[t] : 0.f;
     }
-
-    const float r1old[2] = {r1[0], r1[1]};
     {
-      float cs[2] = {0.f, 0.f};
+      float ca = 0.f, cb = 0.f;
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
-#pragma unroll
-        for (int t = 0; t < 16; ++t) {
-          gc[c][t] *= inv[t];
-          cs[c] += cT[t] * qc[c][t];
-        }
-      state_update(S, gc, qc);
-      r1[0] += half_swap_add(cs[0]);
-      r1[1] += half_swap_add(cs[1]);
+      for (int t = 0; t < 16; ++t) {
+        gc[0][t] *= inv[t];
+        gc[1][t] *= inv[t];
+        ca += cT[t] * qc[0][t];
+        cb += cT[t] * qc[1][t];
+      }
+      r1next[0] = half_swap_add(ca);
+      r1next[1] = half_swap_add(cb);
     }
-    FM_PIN();
-    load_ch<T>(gh, nb, roff, gc);
-    FM_PIN();
 
     weight_product(W, qc, O);
-    FM_PIN();
-    load_ch<T>(qh, nb, roff, qc);
-    FM_PIN();
 
     float x[2][16];
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int t = 0; t < 16; ++t) x[c][t] = a1s * (O[c][t] - r1old[c]);
-    store_tile<true, T>(oh, D, base, n, i, hh, x);
+      for (int t = 0; t < 16; ++t) x[c][t] = a1s * (O[c][t] - r1[c]);
+    store_tile<true, T>(oh, D, base, 0, hi, L, x);
   }
 }
 
