@@ -39,12 +39,16 @@ WORKLOADS = {
 }
 COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 
-# HBM bytes per token-head moved by each kernel class at the headline workload, from the
-# FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/headline_causal_fp32_all_kernels.txt
+# HBM bytes per token-head moved by each kernel class, from the FETCH_SIZE / WRITE_SIZE counter
+# runs summarised under profiles/ (one file per workload, TRAFFIC_SOURCE)
 # (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch x2.0, write x1.0).
 MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD = {
     "headline": {"build": 3023.0, "fwd_apply": 2611.0, "bwd_dq": 2863.0, "bwd_dk": 3045.0, "bwd_dv": 2714.0},
+    # profiles/headline_p1_causal_fp32_scan_kernels.txt (algorithmic: 1024 B per token-head and kernel)
+    "headline-p1": {"fwd_apply": 1167.0, "bwd_dq": 1174.0, "bwd_dk": 1181.0, "bwd_dv": 1176.0},
 }
+TRAFFIC_SOURCE = {"headline": "profiles/headline_causal_fp32_all_kernels.txt",
+                  "headline-p1": "profiles/headline_p1_causal_fp32_scan_kernels.txt"}
 
 
 def algorithmic_flops(d: int, p: int) -> dict:
@@ -240,11 +244,21 @@ def main() -> int:
         executed = 2.0 * slots * 32 * D * token_heads * n_builds / (dom_ms * 1e-3) / 1e12
         roofline["executed_tflops"] = executed
         roofline["executed_frac"] = executed / peak
+    if cfg["p"] == 1:
+        # p = 1 is HBM-bound (about 19 flop per byte): price the slowest kernel against the bytes it must
+        # move -- three (bh, n, d) tensors read and one written per kernel (forward: q, k, v -> o; dq: grad,
+        # k, v -> dq; dk: grad, q, v -> dk; dv: grad, q, k -> dv); the per-token scalars are negligible
+        es = 4 if cfg["dtype"] == "f32" else 2
+        bytes_per_launch = 4.0 * D * es * token_heads / launches
+        gbs = bytes_per_launch / (dom_ms / launches * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": gbs / PEAK_HBM_GBS, "traffic": None, "bytes_per_launch": bytes_per_launch,
+                    "avg_launch_ms": dom_ms / launches}
     per_th = MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD.get(args.workload if not args.batch else "", {}).get(dom)
     if per_th is not None:
         n_states = n_builds if dom == "build" else 1
         roofline["traffic"] = per_th * token_heads * n_states / launches  # bytes per launch (profiled, not live)
-        roofline["traffic_source"] = "profiles/headline_causal_fp32_all_kernels.txt"
+        roofline["traffic_source"] = TRAFFIC_SOURCE[args.workload]
     for name, f in per_step_flops.items():
         if name in kernels:
             kernels[name]["algorithmic_tflops"] = f / (kernels[name]["ms_per_step"] * 1e-3) / 1e12
@@ -259,7 +273,8 @@ def main() -> int:
         "config": {"workload": f"{args.workload}: Fastmax {'causal' if cfg['mask'] else 'unmasked'} fwd+bwd, "
                                f"B={B} H={H} N={N} D={D} p={cfg['p']} {cfg['dtype']}, normalize lim=1, "
                                "a=(1,1,0.5), q/k/v/grad iid N(0,1) seed 0; backward "
-                               + ("rebuilds the prefix states" if args.recompute_states
+                               + ("keeps every state in registers (one scan per head)" if "build" not in kernels
+                                  else "rebuilds the prefix states" if args.recompute_states
                                   else "reads the prefix states the forward pass kept")},
         "fwd_ms": ms_fwd, "fwd_tokens_per_s": B * N / (ms_fwd * 1e-3),
         "module_autograd_ms_per_step": ms_module,
