@@ -78,6 +78,7 @@ struct Plan {
                        // inputs add one slot that receives their sum in packed form
   int chunk;           // tokens between causal state snapshots
   int nblk;            // 128-token blocks per head
+  bool scan;           // causal p = 1 as one scan per head (fm_linear.h): no states in memory
   int64_t state_floats;
   size_t fixed_bytes;     // scale/argmax/cvec/rpart
   size_t per_head_bytes;  // states of one head
@@ -152,6 +153,8 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   // grouped key/value heads, backward: dk and dv are formed per query head and then added up
   if (pass == FASTMAX_PASS_BACKWARD && pl.ratio > 1)
     pl.per_head_bytes += 2 * (size_t)pl.n * pl.d * (ds->dtype == FASTMAX_BF16 ? 2 : 4);
+  pl.scan = use_linear_scan(ds, pl);
+  if (pl.scan) pl.per_head_bytes = 0;
   return pl;
 }
 
@@ -166,6 +169,7 @@ bool use_linear_scan(const fastmax_desc* ds, const Plan& pl) {
 // is a whole number of rounds over the 256 CUs; a ragged last round would idle most of the chip.
 // (with_saved: the prefix states live in the caller's saved-state buffer, not in the workspace)
 size_t batch_bytes_per_head(const Plan& pl, bool with_saved) {
+  if (pl.scan) return 0;
   return pl.per_head_bytes - (with_saved ? (size_t)pl.nslots * pl.state_floats * sizeof(float) : 0);
 }
 
@@ -214,6 +218,7 @@ int check_ws(const Plan& pl, void* ws, size_t ws_bytes, bool with_saved = false)
 }
 
 size_t saved_bytes_for(const Plan& pl) {
+  if (pl.scan) return 256;   // nothing to keep; a token size, so that 0 still means "bad descriptor"
   return (size_t)pl.bhkv * pl.nslots * pl.state_floats * sizeof(float);
 }
 
@@ -311,7 +316,7 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
 
   if constexpr (D == 64) {
-    if (use_linear_scan(ds, pl)) {
+    if (pl.scan) {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       // (pairs of output columns go out as one store when the row pitch keeps them aligned)
       if (ldo % 2 == 0)
@@ -383,7 +388,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     FM_TRY(launch_status("bwd_prep_kernel"));
   }
   if constexpr (D == 64) {
-    if (use_linear_scan(ds, pl)) {
+    if (pl.scan) {
       const float* qs = scale;
       const float* ks = scale + bh;
       // one normalisation partial per head, shared by q and k:
@@ -600,6 +605,7 @@ size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass) {
   const size_t mn = fastmax_workspace_min_bytes(desc, pass);
   if (!mn) return 0;
   const Plan pl = make_plan(desc, pass);
+  if (!pl.per_head_bytes) return mn;
   size_t heads = (kWorkspaceBudget - (pl.fixed_bytes < kWorkspaceBudget ? pl.fixed_bytes : 0)) / pl.per_head_bytes;
   if (heads < (size_t)pl.ratio) heads = pl.ratio;
   if (heads > (size_t)pl.bh) heads = pl.bh;

@@ -120,7 +120,10 @@ int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, con
  * hands it to fastmax_backward_saved, which then skips that build.  With saved_states == NULL
  * the two calls are fastmax_forward / fastmax_backward.  When a buffer is given the workspace
  * need not hold the prefix states: 16*bh + 512 bytes suffice for fastmax_forward_saving, and
- * fastmax_backward_saved needs one state per head less. */
+ * fastmax_backward_saved needs one state per head less.  (Causal p = 1 at d = 64 with at
+ * least 512 heads runs as one register-resident scan per head that keeps no state in memory:
+ * there the size is a token 256 bytes, the buffer is left untouched and the workspace only
+ * holds per-head and per-token scalars.) */
 size_t fastmax_saved_state_bytes(const fastmax_desc* desc);
 int fastmax_forward_saving(const fastmax_desc* desc, const void* q, const void* k, const void* v,
                            void* o, int64_t ldo, float* den, int64_t den_stride,

@@ -79,6 +79,21 @@ def test_workspace_sizes(built):
     assert built.fastmax_workspace_bytes(C.byref(ds), 9) == 0  # unknown pass
 
 
+def test_scan_path_needs_no_state_memory(built):
+    """Causal p = 1, d = 64, >= 512 heads, n >= 32, a1 != 0 runs as one register-resident scan
+    per head: the workspace holds only the per-head and per-token scalars."""
+    ds = desc(bh=1024, n=10000, mask=True, p=1)
+    fwd = built.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD)
+    bwd = built.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_BACKWARD)
+    assert fwd == built.fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_FORWARD) == 2 * 4096 * 2
+    blocks = (10000 + 127) // 128
+    assert bwd == 2 * 8192 + 1024 * 10000 * 4 + 2 * 1024 * blocks * 4
+    assert built.fastmax_saved_state_bytes(C.byref(ds)) == 256
+    for other in (desc(bh=511, n=10000, mask=True, p=1), desc(bh=1024, n=31, mask=True, p=1),
+                  desc(bh=1024, n=10000, mask=True, p=1, a1=0.0), desc(bh=1024, n=10000, mask=False, p=1)):
+        assert built.fastmax_workspace_min_bytes(C.byref(other), _cabi.PASS_FORWARD) > 2 * 8192
+
+
 def test_forward_rejects_before_touching_device(built):
     ds = desc()
     f = built.fastmax_forward
