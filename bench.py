@@ -32,6 +32,7 @@ WORKLOADS = {
     "headline": dict(B=64, H=16, N=10000, D=64, mask=True, p=2, dtype="f32"),
     "headline-unmasked": dict(B=64, H=16, N=10000, D=64, mask=False, p=2, dtype="f32"),
     "headline-p1": dict(B=64, H=16, N=10000, D=64, mask=True, p=1, dtype="f32"),
+    "headline-unmasked-p1": dict(B=64, H=16, N=10000, D=64, mask=False, p=1, dtype="f32"),
     "c1": dict(B=8, H=8, N=1024, D=32, mask=False, p=2, dtype="f32"),
     "c2": dict(B=64, H=8, N=1000, D=32, mask=True, p=2, dtype="f32"),
     "c4": dict(B=16, H=32, N=16384, D=64, mask=True, p=2, dtype="bf16"),
@@ -245,11 +246,19 @@ def main() -> int:
         roofline["executed_tflops"] = executed
         roofline["executed_frac"] = executed / peak
     if cfg["p"] == 1:
-        # p = 1 is HBM-bound (about 19 flop per byte): price the slowest kernel against the bytes it must
-        # move -- three (bh, n, d) tensors read and one written per kernel (forward: q, k, v -> o; dq: grad,
-        # k, v -> dq; dk: grad, q, v -> dk; dv: grad, q, k -> dv); the per-token scalars are negligible
+        # p = 1 is HBM-bound (about 19 flop per byte): price the slowest kernel against the (bh, n, d)
+        # tensors it must move; the per-token scalars and the (d+1) x (d+1) states are negligible.
+        #   causal (one scan per head and kernel): three read, one written -- forward: q, k, v -> o;
+        #     dq: grad, k, v -> dq; dk: grad, q, v -> dk; dv: grad, q, k -> dv
+        #   unmasked (state of the whole sequence, then one pass over the rows): build k, v (or q, grad);
+        #     forward q -> o; dq grad -> dq; dk v -> dk; dv k -> dv: two tensors each
         es = 4 if cfg["dtype"] == "f32" else 2
-        bytes_per_launch = 4.0 * D * es * token_heads / launches
+        tensors = 4 if "build" not in kernels else 2
+        dom = max(per_step_flops, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0)
+                  / kernels.get(n, {}).get("launches_per_step", 1.0))
+        dom_ms = kernels[dom]["ms_per_step"]
+        launches = kernels[dom]["launches_per_step"]
+        bytes_per_launch = float(tensors) * D * es * token_heads
         gbs = bytes_per_launch / (dom_ms / launches * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": gbs / PEAK_HBM_GBS, "traffic": None, "bytes_per_launch": bytes_per_launch,
