@@ -124,6 +124,8 @@ def main() -> int:
     ap.add_argument("--through-module", action="store_true",
                     help="also time forward + backward through FASTMultiHeadAttention and autograd "
                          "(allocations and the extension included)")
+    ap.add_argument("--hip-graph", action="store_true",
+                    help="also time replays of the step captured in a HIP graph (launch-bound small shapes)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -183,6 +185,25 @@ def main() -> int:
         fwd()
     torch.cuda.synchronize()
     ms_fwd = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    ms_graph = None
+    if args.hip_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        ms_graph = (time.perf_counter() - t0) * 1e3 / args.steps
+        del graph
 
     ms_module = None
     if args.through_module:
@@ -287,6 +308,7 @@ def main() -> int:
                                   else "reads the prefix states the forward pass kept")},
         "fwd_ms": ms_fwd, "fwd_tokens_per_s": B * N / (ms_fwd * 1e-3),
         "module_autograd_ms_per_step": ms_module,
+        "hip_graph_replay_ms_per_step": ms_graph,
         "fwd_tflops": fl["fwd"] * token_heads / (ms_fwd * 1e-3) / 1e12,
         "fwd_bwd_tflops": (fl["fwd"] + fl["bwd"]) * token_heads / (ms_step * 1e-3) / 1e12,
         "mfma_frac_of_peak_fwd_bwd": (fl["fwd"] + fl["bwd"]) * token_heads / (ms_step * 1e-3) / 1e12 / peak,
