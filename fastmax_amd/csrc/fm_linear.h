@@ -31,9 +31,9 @@
 // not a multiple of 32, the last tile of a scan is moved back so that it ends at the sequence's
 // end (a forward scan's last tile is rows [n-32, n); a reverse scan runs its tiles down from the
 // end and its last one is rows [0, 32)).  The rows it shares with the tile before it are already
-// in the state and already written; they are masked out of the weights, the state update and
-// the stores.  So all loads are unclamped, with one per-lane offset and immediates, and the hot
-// loop has a single straight path.
+// in the state and already written; they are masked out of the weights and the stores (and a
+// scan's last tile never joins the state).  So all loads are unclamped, with one per-lane offset
+// and immediates, and the hot loop has a single straight path.
 //
 // Order of work in a loop iteration (tile m): fold tile m-1 into the state (its channel-major
 // operands are still in registers) -> load tile m's channel-major operands into those registers
@@ -256,16 +256,6 @@ __device__ __forceinline__ void zero_state(f16v (&S)[2][2]) {
     for (int b = 0; b < 2; ++b)
 #pragma unroll
       for (int t = 0; t < 16; ++t) S[a][b][t] = 0.f;
-}
-
-// rows of a channel-major operand outside [lo, hi) -> 0 (the shared rows of a moved-back tile)
-__device__ __forceinline__ void keep_rows(float (&x)[2][16], int lo, int hi, int hh) {
-#pragma unroll
-  for (int t = 0; t < 16; ++t) {
-    const bool in = trow(t, hh) >= lo && trow(t, hh) < hi;
-    x[0][t] = in ? x[0][t] : 0.f;
-    x[1][t] = in ? x[1][t] : 0.f;
-  }
 }
 
 // per-lane sums over the tile's rows of a channel-major operand: s[c] = sum_rows x[row][chan(c, i)]
