@@ -380,13 +380,6 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
   const int hb = heads_per_batch(pl, ws_bytes, saved != nullptr);
 
   if (!given) FM_TRY(compute_scales<T>(ds, q, k, scale_ws, arg_ws, stream));
-  {
-    const int64_t rows = (int64_t)bh * n;
-    const int rpp = 256 / (D / 4);
-    ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
-    bwd_prep_kernel<T><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
-    FM_TRY(launch_status("bwd_prep_kernel"));
-  }
   if constexpr (D == 64) {
     if (pl.scan) {
       const float* qs = scale;
@@ -394,12 +387,27 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       // one normalisation partial per head, shared by q and k:
       // sum_i dq_hat_i . q_hat_i = sum_ij W_ij s_ij = sum_j dk_hat_j . k_hat_j
       float* rq = rpart;
+      // the dq kernel forms c_i itself when the forward output has plain rows; otherwise the
+      // separate pass does
+      const bool prep_in_dq = ldo == D;
+      if (!prep_in_dq) {
+        const int64_t rows = (int64_t)bh * n;
+        const int rpp = 256 / (D / 4);
+        ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
+        bwd_prep_kernel<T><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
+        FM_TRY(launch_status("bwd_prep_kernel"));
+      }
       {
         ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
-        if (ds->normalize)
-          lin::linear_dq_kernel<T, true><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, k, v, qs, ks, dq, rq, n, ds->a0, ds->a1);
-        else
-          lin::linear_dq_kernel<T, false><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, q, k, v, qs, ks, dq, rq, n, ds->a0, ds->a1);
+#define FM_DQ(NORM, PREP)                                                                                   \
+  lin::linear_dq_kernel<T, NORM, PREP><<<bh, 64, 0, stream>>>(go, den, den_stride, cvec, o, q, k, v, qs, ks, dq, rq, \
+                                                              n, ds->a0, ds->a1)
+        if (ds->normalize) {
+          if (prep_in_dq) FM_DQ(true, true); else FM_DQ(true, false);
+        } else {
+          if (prep_in_dq) FM_DQ(false, true); else FM_DQ(false, false);
+        }
+#undef FM_DQ
       }
       FM_TRY(launch_status("linear_dq_kernel"));
       {
@@ -420,6 +428,13 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       }
       return FASTMAX_OK;
     }
+  }
+  {
+    const int64_t rows = (int64_t)bh * n;
+    const int rpp = 256 / (D / 4);
+    ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
+    bwd_prep_kernel<T><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
+    FM_TRY(launch_status("bwd_prep_kernel"));
   }
   const float a2 = pl.p2 ? ds->a2 : 0.f;
   const int ratio = pl.ratio, bhkv = pl.bhkv;

@@ -379,11 +379,14 @@ __global__ __launch_bounds__(64) void linear_fwd_kernel(const T* __restrict__ q,
 // c_i den_i - a0 g_i . V_i, V_i = sum_{j<=i} v_j, give  sum_ij W_ij s_ij = a0 sum_i [c_i (i+1) - g_i . V_i].
 // That rests on o_i = num_i / den_i holding to working precision, so it is used for fp32 only;
 // with bf16 tensors (o rounded to 8 bits) the partial is formed directly as sum_i dq_i . q_i.
+// PREP: c_i is not read from cvec but formed from the forward output (rows of pitch D) and
+// written to cvec for the dk kernel, which saves the separate pass over grad and o.
 // ---------------------------------------------------------------------------------------
-template <class T, bool NORM>
+template <class T, bool NORM, bool PREP>
 __global__ __launch_bounds__(64) void linear_dq_kernel(const T* __restrict__ go, const float* __restrict__ den,
-                                                       int64_t den_stride, const float* __restrict__ cvec,
-                                                       const T* __restrict__ q, const T* __restrict__ k,
+                                                       int64_t den_stride, float* __restrict__ cvec,
+                                                       const T* __restrict__ o, const T* __restrict__ q,
+                                                       const T* __restrict__ k,
                                                        const T* __restrict__ v,
                                                        const float* __restrict__ qscale,
                                                        const float* __restrict__ kscale, T* __restrict__ dq,
@@ -397,7 +400,8 @@ __global__ __launch_bounds__(64) void linear_dq_kernel(const T* __restrict__ go,
   const T* kh = k + (int64_t)head * n * D;
   const T* vh = v + (int64_t)head * n * D;
   const float* dh = den + (int64_t)head * n * den_stride;
-  const float* ch = cvec + (int64_t)head * n;
+  float* ch = cvec + (int64_t)head * n;
+  const T* fh = PREP ? o + (int64_t)head * n * D : nullptr;   // forward output, rows of pitch D
   T* oh = dq + (int64_t)head * n * D;
   const float a1s = a1 * qscale[head] * kscale[head];
   constexpr bool CLOSED = NORM && Map<T>::CLOSED_R, DIRECT = NORM && !Map<T>::CLOSED_R;
@@ -407,16 +411,25 @@ __global__ __launch_bounds__(64) void linear_dq_kernel(const T* __restrict__ go,
   zero_state(S);
   float s1[2] = {0.f, 0.f}, s0[2] = {0.f, 0.f}, rs = 0.f;
   float gt[32], vt[32], vc[2][16] = {}, kc[2][16] = {};   // (tile "-1" is empty)
-  float qc[2][16];
+  float qc[2][16], ot[32];
   load_tok(vh, 0, L, vt);
   load_tok(gh, 0, L, gt);
-  float den_l = dh[(int64_t)L.i * den_stride], c_l = ch[L.i];
+  if (PREP) load_tok(fh, 0, L, ot);
+  float den_l = dh[(int64_t)L.i * den_stride], c_l = PREP ? 0.f : ch[L.i];
 
   const int ntiles = (n + 31) >> 5;
   for (int tt = 0; tt < ntiles; ++tt) {
     const int base = fbase(tt, n), skip = 32 * tt - base;
     const int nb = tt + 1 < ntiles ? fbase(tt + 1, n) : base;   // next tile (see linear_fwd_kernel)
-    const float den_cur = den_l, c_cur = c_l, inv_l = rcp(den_l);
+    const float den_cur = den_l, inv_l = rcp(den_l);
+    float c_cur = c_l;
+    if (PREP) {   // c_i = (go_i . o_i) / den_i, formed here and left behind for the dk kernel
+      float d = 0.f;
+#pragma unroll
+      for (int e = 0; e < 32; ++e) d += gt[e] * ot[e];
+      c_cur = half_swap_add(d) * inv_l;
+      if (L.l < 32 && L.i >= skip) ch[base + L.i] = c_cur;
+    }
 
     // the previous tile joins the state
     state_update(S, vc, kc);
@@ -445,8 +458,9 @@ __global__ __launch_bounds__(64) void linear_dq_kernel(const T* __restrict__ go,
     FM_PIN();
     load_tok(vh, nb, L, vt);
     load_tok(gh, nb, L, gt);
+    if (PREP) load_tok(fh, nb, L, ot);
     den_l = dh[(int64_t)(nb + L.i) * den_stride];
-    c_l = ch[nb + L.i];
+    if (!PREP) c_l = ch[nb + L.i];
     FM_PIN();
     {
       const float cd = c_cur * den_cur;

@@ -81,6 +81,13 @@ def test_denominator_column_layout(ops):
     o2, den2, _, _ = ops.forward(q, k, v, denominator_column=True, **kw)
     assert torch.equal(o2[..., :64], o1)
     assert torch.equal(o2[..., 64], den1.reshape(o2[..., 64].shape))
+    # backward from either layout (with plain rows the dq kernel forms c_i = g_i . o_i itself,
+    # with the d+1 pitch a separate pass does): same gradients up to the rounding of 1/den
+    go = go
+    g1 = ops.backward(q, k, v, o1, den1, go, **kw)
+    g2 = ops.backward(q, k, v, o2[..., :64], den2, go, **kw)
+    for name, a, b in zip(("dq", "dk", "dv"), g1, g2):
+        assert_close(name, a, b, 2e-6)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
