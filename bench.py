@@ -45,8 +45,9 @@ COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 # (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch x2.0, write x1.0).
 MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD = {
     "headline": {"build": 3023.0, "fwd_apply": 2611.0, "bwd_dq": 2863.0, "bwd_dk": 3045.0, "bwd_dv": 2714.0},
-    # profiles/headline_p1_causal_fp32_scan_kernels.txt (algorithmic: 1024 B per token-head and kernel)
-    "headline-p1": {"fwd_apply": 1167.0, "bwd_dq": 1174.0, "bwd_dk": 1181.0, "bwd_dv": 1176.0},
+    # profiles/headline_p1_causal_fp32_scan_kernels.txt (algorithmic: 1024 B per token-head and kernel,
+    # 1280 B for dq, which also reads the forward output)
+    "headline-p1": {"fwd_apply": 1166.0, "bwd_dq": 1499.0, "bwd_dk": 1182.0, "bwd_dv": 1181.0},
 }
 TRAFFIC_SOURCE = {"headline": "profiles/headline_causal_fp32_all_kernels.txt",
                   "headline-p1": "profiles/headline_p1_causal_fp32_scan_kernels.txt"}
@@ -270,7 +271,8 @@ def main() -> int:
         # p = 1 is HBM-bound (about 19 flop per byte): price the slowest kernel against the (bh, n, d)
         # tensors it must move; the per-token scalars and the (d+1) x (d+1) states are negligible.
         #   causal (one scan per head and kernel): three read, one written -- forward: q, k, v -> o;
-        #     dq: grad, k, v -> dq; dk: grad, q, v -> dk; dv: grad, q, k -> dv
+        #     dq: grad, k, v (and o, when it forms c_i itself: no bwd_prep launch) -> dq; dk: grad, q, v -> dk;
+        #     dv: grad, q, k -> dv
         #   unmasked (state of the whole sequence, then one pass over the rows): build k, v (or q, grad);
         #     forward q -> o; dq grad -> dq; dk v -> dk; dv k -> dv: two tensors each
         es = 4 if cfg["dtype"] == "f32" else 2
@@ -279,6 +281,8 @@ def main() -> int:
                   / kernels.get(n, {}).get("launches_per_step", 1.0))
         dom_ms = kernels[dom]["ms_per_step"]
         launches = kernels[dom]["launches_per_step"]
+        if tensors == 4 and dom == "bwd_dq" and "bwd_prep" not in kernels:
+            tensors = 5
         bytes_per_launch = float(tensors) * D * es * token_heads
         gbs = bytes_per_launch / (dom_ms / launches * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
