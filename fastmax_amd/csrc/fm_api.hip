@@ -79,6 +79,7 @@ struct Plan {
   int chunk;           // tokens between causal state snapshots
   int nblk;            // 128-token blocks per head
   bool scan;           // causal p = 1 as one scan per head (fm_linear.h): no states in memory
+  bool rowpass;        // unmasked p = 1: states from the build kernel, one pass over the rows per output
   int64_t state_floats;
   size_t fixed_bytes;     // scale/argmax/cvec/rpart
   size_t per_head_bytes;  // states of one head
@@ -155,6 +156,7 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
     pl.per_head_bytes += 2 * (size_t)pl.n * pl.d * (ds->dtype == FASTMAX_BF16 ? 2 : 4);
   pl.scan = use_linear_scan(ds, pl);
   if (pl.scan) pl.per_head_bytes = 0;
+  pl.rowpass = !pl.p2 && !pl.masked && pl.d == 64 && pl.ratio == 1 && pl.n >= 32;
   return pl;
 }
 
@@ -300,6 +302,16 @@ int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float*
   return launch_status("build_kernel");
 }
 
+// Unmasked p = 1 row passes read the head's state in fp32: the partial states of the token splits are
+// summed into slot nparts (with a single split, slot 0 is the state).  Returns that slot.
+inline int finish_state_fp32(const Plan& pl, int heads, float* state, hipStream_t stream) {
+  if (pl.nparts == 1) return 0;
+  const int64_t ss = pl.state_floats;
+  state_accumulate_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads), 256, 0, stream>>>(
+      state + (int64_t)pl.nparts * ss, (int64_t)pl.nslots * ss, state, pl.nslots, pl.nparts, ss, 0);
+  return pl.nparts;
+}
+
 template <int D, class T>
 int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k, const T* v, T* o,
                  int64_t ldo, float* den, int64_t den_stride, float* scale_out, int32_t* arg_out,
@@ -337,6 +349,23 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
     const int64_t koff = (int64_t)kv0 * n * D;
     float* state = saved ? saved + kv0 * head_floats : reinterpret_cast<float*>(ws + pl.fixed_bytes);
     // (bf16: a saved state is also read by the dq kernel, which needs the column-packed section)
+    if constexpr (D == 64) {
+      if (pl.rowpass) {
+        FM_TRY((launch_build<D, T>(pl, heads, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state, 0, 0,
+                                   stream, false)));
+        const int slot = finish_state_fp32(pl, heads, state, stream);
+        ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
+        const dim3 rgrid((n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE, heads);
+#define FM_ROWFWD(AL)                                                                                          \
+  lin::linear_rowpass_kernel<T, lin::ROWPASS_FWD, false, AL><<<rgrid, 64, 0, stream>>>(                          \
+      q + off, state + (int64_t)slot * pl.state_floats, head_floats, scale + h0, nullptr, den_stride, nullptr, \
+      nullptr, o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, nullptr, n, ds->a0, ds->a1)
+        if (ldo % 2 == 0) FM_ROWFWD(true); else FM_ROWFWD(false);
+#undef FM_ROWFWD
+        FM_TRY(launch_status("linear_rowpass_kernel (forward)"));
+        continue;
+      }
+    }
     FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr,
                                state, 0, saved ? 3 : 1, stream)));
     {
@@ -457,6 +486,51 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     }
     const float* denh = den + (int64_t)h0 * n * den_stride;
     const float* ch = cvec + (int64_t)h0 * n;
+    if constexpr (D == 64) {
+      if (pl.rowpass) {
+        // states of the whole sequence in fp32 (S as the forward pass left it when it was kept), then one
+        // pass over the rows per gradient
+        const int64_t ss = pl.state_floats, hf = (int64_t)pl.nslots * ss;
+        int slot = pl.nparts > 1 ? pl.nparts : 0;
+        if (!saved) {
+          FM_TRY((launch_build<D, T>(pl, heads, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state, 0, 0,
+                                     stream, false)));
+          slot = finish_state_fp32(pl, heads, state, stream);
+        }
+        FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, 0, stream,
+                                   false)));
+        finish_state_fp32(pl, heads, stR, stream);
+        const int nrb = (n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE;
+        const dim3 rgrid(nrb, heads);
+        {
+          ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
+          if (ds->normalize)
+            lin::linear_rowpass_kernel<T, lin::ROWPASS_DQ, true, true><<<rgrid, 64, 0, stream>>>(
+                go + off, stS + slot * ss, hf, scale + h0, denh, den_stride, ch, q + off, dq + off, D, nullptr,
+                rpart + (int64_t)h0 * nrb, n, ds->a0, ds->a1);
+          else
+            lin::linear_rowpass_kernel<T, lin::ROWPASS_DQ, false, true><<<rgrid, 64, 0, stream>>>(
+                go + off, stS + slot * ss, hf, scale + h0, denh, den_stride, ch, q + off, dq + off, D, nullptr,
+                nullptr, n, ds->a0, ds->a1);
+        }
+        FM_TRY(launch_status("linear_rowpass_kernel (dq)"));
+        {
+          ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
+          lin::linear_rowpass_kernel<T, lin::ROWPASS_DK, false, true><<<rgrid, 64, 0, stream>>>(
+              v + koff, stR + slot * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dk + off, D, nullptr,
+              nullptr, n, ds->a0, ds->a1);
+        }
+        FM_TRY(launch_status("linear_rowpass_kernel (dk)"));
+        {
+          ScopedKernel sk(FASTMAX_K_BWD_DV, stream);
+          lin::linear_rowpass_kernel<T, lin::ROWPASS_DV, false, true><<<rgrid, 64, 0, stream>>>(
+              k + koff, stR + slot * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dv + off, D, nullptr,
+              nullptr, n, ds->a0, ds->a1);
+        }
+        FM_TRY(launch_status("linear_rowpass_kernel (dv)"));
+        continue;
+      }
+    }
     // prefix state of (kh, v, 1) per key/value head and suffix state of (qh, go/den, c) per query head
     if (!saved)
       FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state,
@@ -514,7 +588,14 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       FM_TRY(launch_status("group_sum_kernel"));
     }
   }
-  if (ds->normalize) {
+  if (ds->normalize && pl.rowpass) {
+    // one partial per row block of the dq pass; sum_j dk_hat_j . k_hat_j is the same number
+    const int nrb = (n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE;
+    ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
+    norm_fix_kernel<T><<<bh, D, 0, stream>>>(dq, q, scale, arg, rpart, nrb, n, D, ds->lim);
+    norm_fix_kernel<T><<<bh, D, 0, stream>>>(dk, k, scale + bh, arg + bh, rpart, nrb, n, D, ds->lim);
+    FM_TRY(launch_status("norm_fix_kernel"));
+  } else if (ds->normalize) {
     ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
     norm_fix_kernel<T><<<bh, D, 0, stream>>>(dq, q, scale, arg, rpart, pl.nblk, n, D, ds->lim);
     norm_fix_kernel<T><<<bhkv, D, 0, stream>>>(dk, k, scale + bh, arg + bh, rpart + (int64_t)bh * pl.nblk,

@@ -672,6 +672,159 @@ __global__ __launch_bounds__(64) void linear_dk_kernel(const T* __restrict__ go,
   }
 }
 
+// =======================================================================================
+// Unmasked p = 1 at head dimension 64: every row sees the state of the whole sequence, so after
+// the state is built (the chunked build kernel: token-split partial states, summed) each output
+// is one pass over the rows: out[row] = f(own[row] x State).  A wave loads the 64 x 64 state once
+// into the registers that serve as the B operand (see the layouts above) and walks ROWS_PER_WAVE
+// rows in tiles of 32, 64 matrix instructions per tile.  State layout in memory: rows of LD = 68
+// floats, row a < 64 = [State[a][0..63], vec1[a], pad], row 64 = [vec0[0..63], count, pad]
+// (the moment state of the chunked kernels for p = 1), built from the SCALED x of its first
+// factor:  S  = sum k^_j (x) [v_j, 1]      (k^ = kscale k;  vec1 = sum k^, vec0 = sum v)
+//          R  = sum q^_i (x) [g_i, c_i]    (q^ = qscale q;  vec1 = sum c_i q^_i, vec0 = sum g_i)
+//   FWD: own = q, S:    o_i  = (a0 vec0 + a1 qs q_i S) / den_i,  den_i = a0 n + a1 qs q_i . vec1
+//   DV:  own = k, R:    dv_j = a0 vec0 + a1 ks k_j R
+//   DQ:  own = grad, S^T: dq_i = a1 qs (go_i S^T / den_i - c_i vec1)
+//   DK:  own = v, R^T:  dk_j = a1 ks (v_j R^T - vec1)
+// (qs, ks: the per-head normaliser factors; gradients are with respect to the raw inputs).
+// DQ with NORM also leaves the normalisation partial of its rows in rpart[head * gridDim.x + block]
+// (closed form a0 sum_i [c_i n - g_i . vec0] for fp32, sum_i dq_i . q_i for bf16; see linear_dq_kernel).
+// grid = (ceil(n / ROWS_PER_WAVE), heads), block = one wave; n >= 32.
+// =======================================================================================
+constexpr int ROWS_PER_WAVE = 256;
+constexpr int SLD = 68;   // row pitch of the state in memory
+enum { ROWPASS_FWD = 0, ROWPASS_DV = 1, ROWPASS_DQ = 2, ROWPASS_DK = 3 };
+
+template <class T>
+__device__ __forceinline__ void state_only(const float (&own)[32], const f16v (&S)[2][2], f16v (&O)[2]) {
+#pragma unroll
+  for (int t = 0; t < 16; ++t) O[0][t] = 0.f, O[1][t] = 0.f;
+#pragma unroll
+  for (int t = 0; t < 16; ++t)
+#pragma unroll
+    for (int rc = 0; rc < 2; ++rc) {
+      O[0] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][0][t], O[0]);
+      O[1] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][1][t], O[1]);
+    }
+}
+
+template <class T, int MODE, bool NORM, bool ALIGNED>
+__global__ __launch_bounds__(64, 2) void linear_rowpass_kernel(const T* __restrict__ own, const float* __restrict__ state,
+                                                            int64_t state_stride, const float* __restrict__ xscale,
+                                                            const float* __restrict__ den_in, int64_t den_stride,
+                                                            const float* __restrict__ cvec, const T* __restrict__ xraw,
+                                                            T* __restrict__ out, int64_t ldo, float* __restrict__ den_out,
+                                                            float* __restrict__ rpart, int n, float a0, float a1) {
+  __shared__ __attribute__((aligned(16))) float vl[D];
+  __shared__ __attribute__((aligned(16))) float al[32];
+  __shared__ __attribute__((aligned(16))) float bl[32];
+  constexpr bool FWD = MODE == ROWPASS_FWD, DQ = MODE == ROWPASS_DQ, DK = MODE == ROWPASS_DK;
+  constexpr bool TRANSPOSED = DQ || DK;
+  constexpr bool CLOSED = DQ && NORM && Map<T>::CLOSED_R, DIRECT = DQ && NORM && !Map<T>::CLOSED_R;
+  const Lane<T> L;
+  const int head = blockIdx.y, r0 = blockIdx.x * ROWS_PER_WAVE;
+  const int r1 = r0 + ROWS_PER_WAVE < n ? r0 + ROWS_PER_WAVE : n;
+  const T* xh = own + (int64_t)head * n * D;
+  const float* st = state + (int64_t)head * state_stride;
+  T* oh = out + (int64_t)head * n * ldo;
+  const float fac = a1 * xscale[head];
+
+  // the state as B operand: register t of tile (rc, cc) = M[chan(rc, trow)][chan(cc, i)], M = State or its transpose
+  f16v S[2][2];
+#pragma unroll
+  for (int rc = 0; rc < 2; ++rc)
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        const int row = Map<T>::chan(rc, trow(t, L.hh)), col = Map<T>::chan(cc, L.i);
+        S[rc][cc][t] = TRANSPOSED ? st[col * SLD + row] : st[row * SLD + col];
+      }
+  // the vector that enters per output column (vec0 for FWD / DV, vec1 for DQ / DK)
+  float vcol[2];
+#pragma unroll
+  for (int cc = 0; cc < 2; ++cc) {
+    const int col = Map<T>::chan(cc, L.i);
+    vcol[cc] = TRANSPOSED ? st[col * SLD + D] : st[D * SLD + col];
+  }
+  // the vector that is dotted with the own rows: vec1 for the denominators, vec0 for the closed-form partial
+  if (FWD) vec_put<T>(vl, L, st[Map<T>::chan(0, L.i) * SLD + D], st[Map<T>::chan(1, L.i) * SLD + D]);
+  if (CLOSED) vec_put<T>(vl, L, st[D * SLD + Map<T>::chan(0, L.i)], st[D * SLD + Map<T>::chan(1, L.i)]);
+  const float* dh = den_in ? den_in + (int64_t)head * n * den_stride : nullptr;
+  const float* ch = cvec ? cvec + (int64_t)head * n : nullptr;
+  float* dout = den_out ? den_out + (int64_t)head * n * den_stride : nullptr;
+  const T* qh = DIRECT ? xraw + (int64_t)head * n * D : nullptr;
+
+  // tiles of this wave's rows: tile tt covers [base, base + 32), base = min(r0 + 32 tt, n - 32); only a
+  // sequence's very last tile can be moved back, its first `skip` rows belong to the tile before
+  const int ntiles = (r1 - r0 + 31) >> 5;
+  auto tile_base = [&](int tt) { return r0 + 32 * tt < n - 32 ? r0 + 32 * tt : n - 32; };
+  float xt[32], qc[2][16];
+  load_tok(xh, tile_base(0), L, xt);
+  float den_l = DQ ? dh[(int64_t)(tile_base(0) + L.i) * den_stride] : 0.f;
+  float c_l = DQ ? ch[tile_base(0) + L.i] : 0.f;
+  float rs = 0.f;
+  for (int tt = 0; tt < ntiles; ++tt) {
+    const int base = tile_base(tt), skip = r0 + 32 * tt - base;
+    const int nb = tt + 1 < ntiles ? tile_base(tt + 1) : base;
+    if (DIRECT) load_ch(qh, base, L, qc);
+    f16v O[2];
+    state_only<T>(xt, S, O);
+    float dot = 0.f;
+    if (FWD || CLOSED) dot = half_swap_add(vec_dot<T>(vl, L, xt));
+    const float den_cur = den_l, c_cur = c_l;
+    FM_PIN();
+    load_tok(xh, nb, L, xt);
+    if (DQ) {
+      den_l = dh[(int64_t)(nb + L.i) * den_stride];
+      c_l = ch[nb + L.i];
+    }
+    FM_PIN();
+
+    float x[2][16];
+    if (FWD) {
+      const float den_i = a0 * (float)n + fac * dot;
+      if (L.l < 32 && L.i >= skip) dout[(int64_t)(base + L.i) * den_stride] = den_i;
+      float inv[16];
+      rows_from_lanes(rcp(den_i), al, L, inv);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 16; ++t) x[c][t] = (fac * O[c][t] + a0 * vcol[c]) * inv[t];
+    } else if (DQ) {
+      const float inv_l = rcp(den_cur);
+      float inv[16], cT[16];
+      rows_from_lanes(inv_l, al, L, inv);
+      rows_from_lanes(c_cur, bl, L, cT);
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 16; ++t) x[c][t] = fac * (inv[t] * O[c][t] - cT[t] * vcol[c]);
+      if (CLOSED) rs += (L.l < 32 && L.i >= skip) ? c_cur * (float)n - inv_l * dot : 0.f;
+      if (DIRECT) {
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+          rs += trow(t, L.hh) >= skip ? x[0][t] * qc[0][t] + x[1][t] * qc[1][t] : 0.f;
+      }
+    } else if (DK) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 16; ++t) x[c][t] = fac * (O[c][t] - vcol[c]);
+    } else {
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 16; ++t) x[c][t] = fac * O[c][t] + a0 * vcol[c];
+    }
+    store_tile<ALIGNED, T>(oh, (int)ldo, base, skip, 32, L, x);
+  }
+  if (DQ && NORM) {
+    rs = wave_sum(rs);
+    if (L.l == 0) rpart[(int64_t)head * gridDim.x + blockIdx.x] = CLOSED ? a0 * rs : rs;
+  }
+}
+
 #undef FM_PIN
 
 }  // namespace lin
