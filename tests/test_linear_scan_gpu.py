@@ -159,6 +159,15 @@ def test_unmasked_variants(ops):
     check_whole(ops, 3, 290, seed=23, scale=0.1, mask=False, normalize=False, p=1)
     check_whole(ops, 4, 600, dtype=torch.bfloat16, seed=24, mask=False, normalize=True, p=1)
     check_whole(ops, 600, 40, seed=25, mask=False, normalize=True, p=1)
+    # kernel semantics of the reference: k /= temperature (fastmax_cuda_forward.cu:212-221,366)
+    q, k, v, go = O.seeded_inputs((4, 150, 64), seed=27)
+    q, k = 0.1 * q, 0.1 * k
+    T = 0.6
+    kw = dict(mask=False, normalize=False, p=1)
+    o, den, dq, dk, dv = fwd_bwd(ops, q.cuda(), k.cuda(), v.cuda(), go.cuda(), temperature=T, **kw)
+    ro, rdq, rdk, rdv = O.dense_truth(q, k / T, v, go, **kw)
+    for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk / T), ("dv", dv, rdv)):
+        assert_close(name, got, ref, 1e-4)
 
 
 def test_unmasked_denominator_column_saved_states_and_small_workspace(ops):
