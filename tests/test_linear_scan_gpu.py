@@ -195,3 +195,20 @@ def test_unmasked_denominator_column_saved_states_and_small_workspace(ops):
     for a, b in zip(g1, g4):
         assert torch.equal(a, b)
     ops.release_workspaces()
+
+
+@pytest.mark.parametrize("mask", [True, False])
+def test_p1_equals_p2_with_a2_zero_at_length(ops, mask):
+    """p = 1 is p = 2 with a2 = 0 (example.py:167-193 against 125-160): the scan / row-pass kernels
+    against the chunked p = 2 kernels, which share no code with them, on a long sequence."""
+    n = 20001
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v, go = (torch.randn((BH, n, 64), device="cuda", generator=g) for _ in range(4))
+    one = fwd_bwd(ops, q, k, v, go, mask=mask, normalize=True, p=1)
+    for s in (slice(0, 3), slice(509, 512)):
+        ref = fwd_bwd(ops, *(t[s].contiguous() for t in (q, k, v, go)), mask=mask, normalize=True, p=2, a2=0.0)
+        for name, a, b in zip(("o", "den", "dq", "dk", "dv"), one, ref):
+            assert_close(f"{name}[{s.start}:]", a[s].reshape(b.shape), b, 2e-5)
+    del q, k, v, go, one
+    ops.release_workspaces()
+    torch.cuda.empty_cache()
