@@ -165,9 +165,11 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
       if (FWD) bt.dd[e] = base[e * LD + D];
     }
   };
-  // one slab; ORD2 = false is the order-1 sweep (feature = x[a] itself)
-  auto slab_compute = [&](const float* sl, auto tag) {
+  // one slab; ORD2 = false is the order-1 sweep (feature = x[a] itself).  WO = position of the
+  // window: Wn[WO + x] is the partner of channel x for the current shift
+  auto slab_compute = [&](const float* sl, auto tag, auto wo) __attribute__((always_inline)) {
     constexpr bool ORD2 = decltype(tag)::value;
+    constexpr int WO = decltype(wo)::value;
     Batch cur, nxt;
     batch_fetch(sl, 0, cur);
 #pragma unroll
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
       if (t0 + KB < H2) batch_fetch(sl, t0 + KB, nxt);
 #pragma unroll
       for (int e = 0; e < KB; ++e) {
-        const float a = ORD2 ? Xr[t0 + e] * Wn[t0 + e] : Xr[t0 + e];
+        const float a = ORD2 ? Xr[t0 + e] * Wn[WO + t0 + e] : Xr[t0 + e];
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA(a, cur.b[e][cb], acc[cb]);
         if (FWD) dn += a * cur.dd[e];
@@ -184,21 +186,14 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
       if (t0 + KB < H2) cur = nxt;
     }
   };
-
-  for (int st = 0; st < n_state; ++st) {
+  // one pipeline step: fetch slab st+1, work on slab st, stage slab st+1 (or the first streamed tile)
+  auto slab_iter = [&](int st, auto tag, auto wo) __attribute__((always_inline)) {
+    constexpr bool ORD2 = decltype(tag)::value;
+    __builtin_amdgcn_sched_barrier(0);   // (keeps the unrolled steps from being interleaved: register pressure)
     slab_load(st + 1 < n_state ? st + 1 : st);
     const float* sl = Sl[st & 1];
-    if (p2 && st < NS) {
-      // window of rotated partners for shift st: reloaded every fourth shift, slid by one otherwise
-      if ((st & 3) == 0) {
-        window_load(st);
-      } else {
-#pragma unroll
-        for (int x = 0; x < H2 + 3; ++x) Wn[x] = Wn[x + 1];
-      }
-      slab_compute(sl, std::true_type{});
-    } else {
-      slab_compute(sl, std::false_type{});
+    slab_compute(sl, tag, wo);
+    if (!ORD2) {
       const float* s0 = sl + D * LD;  // order 0 rides at the end of the order-1 slab
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) {
@@ -211,6 +206,54 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
     if (st + 1 < n_state) slab_store(st + 1);
     else if (n_tile > 0) tiles_store((st + 1) & 1);
     __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  if constexpr (FWD) {
+    // (the forward pass also carries the denominator sums; with them the unrolled form below does not
+    // fit the register file, so its window is slid by one register per shift instead)
+    for (int st = 0; st < n_state; ++st) {
+      slab_load(st + 1 < n_state ? st + 1 : st);
+      const float* sl = Sl[st & 1];
+      if (p2 && st < NS) {
+        if ((st & 3) == 0) {
+          window_load(st);
+        } else {
+#pragma unroll
+          for (int x = 0; x < H2 + 3; ++x) Wn[x] = Wn[x + 1];
+        }
+        slab_compute(sl, std::true_type{}, std::integral_constant<int, 0>{});
+      } else {
+        slab_compute(sl, std::false_type{}, std::integral_constant<int, 0>{});
+        const float* s0 = sl + D * LD;  // order 0 rides at the end of the order-1 slab
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+          const float z = s0[cb * 32 + i];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[cb][r] += z;
+        }
+        if (hh == 0) dn += s0[D];
+      }
+      if (st + 1 < n_state) slab_store(st + 1);
+      else if (n_tile > 0) tiles_store((st + 1) & 1);
+      __syncthreads();
+    }
+  } else if (n_state > 1) {
+    // p = 2: shifts 0 .. NS-1, then the order-1 slab.  The window of rotated partners is loaded
+    // every fourth shift and read at a compile-time position in between (no register moves).
+    static_assert((NS - 1) % 4 == 0, "shifts come in groups of four plus the last one");
+    for (int st = 0; st < NS - 1; st += 4) {
+      window_load(st);
+      slab_iter(st, std::true_type{}, std::integral_constant<int, 0>{});
+      slab_iter(st + 1, std::true_type{}, std::integral_constant<int, 1>{});
+      slab_iter(st + 2, std::true_type{}, std::integral_constant<int, 2>{});
+      slab_iter(st + 3, std::true_type{}, std::integral_constant<int, 3>{});
+    }
+    window_load(NS - 1);
+    slab_iter(NS - 1, std::true_type{}, std::integral_constant<int, 0>{});
+    slab_iter(NS, std::false_type{}, std::integral_constant<int, 0>{});
+  } else if (n_state == 1) {
+    slab_iter(0, std::false_type{}, std::integral_constant<int, 0>{});
   }
 
   const int mine = (tok0 >> 5) + w;
