@@ -252,8 +252,10 @@ int compute_scales(const fastmax_desc* ds, const T* q, const T* k, float* scale,
   const int bh = ds->bh, bhkv = ds->bhkv;
   ScopedKernel sk(FASTMAX_K_ROWSTAT, stream);
   if (ds->normalize) {
-    rowstat_kernel<T><<<bh, 256, 0, stream>>>(q, ds->nq, ds->d, ds->lim, scale, arg);
-    rowstat_kernel<T><<<bhkv, 256, 0, stream>>>(k, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
+    if (bh >= 512) rowstat_kernel<T, 256><<<bh, 256, 0, stream>>>(q, ds->nq, ds->d, ds->lim, scale, arg);
+    else rowstat_kernel<T, 1024><<<bh, 1024, 0, stream>>>(q, ds->nq, ds->d, ds->lim, scale, arg);
+    if (bhkv >= 512) rowstat_kernel<T, 256><<<bhkv, 256, 0, stream>>>(k, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
+    else rowstat_kernel<T, 1024><<<bhkv, 1024, 0, stream>>>(k, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
   } else {
     fill_scale_kernel<<<(bh + 255) / 256, 256, 0, stream>>>(scale, arg, bh, 1.0f);
     fill_scale_kernel<<<(bhkv + 255) / 256, 256, 0, stream>>>(scale + bh, arg + bh, bhkv, 1.0f / ds->temperature);

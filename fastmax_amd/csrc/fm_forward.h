@@ -9,16 +9,17 @@
 // Per-head normaliser: scale[h] = lim / max_i ||x_i||_2 and the row that attains the max
 // (first one on ties).  Replaces calc_norms / find_max of the reference
 // (fastmax_cuda_forward.cu:223-253) with the PyTorch path's definition (example.py:105-108).
-// One block per head; d/4 threads share a row.
+// One block of NT threads per head; d/4 threads share a row.  (NT = 1024 when there are too few
+// heads to fill the chip with 256-thread blocks: four times the loads in flight per head.)
 // ---------------------------------------------------------------------------------------
-template <class T>
-__global__ __launch_bounds__(256) void rowstat_kernel(const T* __restrict__ x, int n, int d,
-                                                      float lim, float* __restrict__ scale_out,
-                                                      int* __restrict__ arg_out) {
-  __shared__ float sbest[256];
-  __shared__ int sarg[256];
+template <class T, int NT>
+__global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, int n, int d,
+                                                     float lim, float* __restrict__ scale_out,
+                                                     int* __restrict__ arg_out) {
+  __shared__ float sbest[NT];
+  __shared__ int sarg[NT];
   const int tid = threadIdx.x;
-  const int tpr = d >> 2, rpp = 256 / tpr;
+  const int tpr = d >> 2, rpp = NT / tpr;
   const int sub = tid % tpr, rowi = tid / tpr;
   const T* base = x + (int64_t)blockIdx.x * n * d;
   float best = -1.f;
@@ -47,7 +48,7 @@ __global__ __launch_bounds__(256) void rowstat_kernel(const T* __restrict__ x, i
   sbest[tid] = best;
   sarg[tid] = bi;
   __syncthreads();
-  for (int off = 128; off > 0; off >>= 1) {
+  for (int off = NT / 2; off > 0; off >>= 1) {
     if (tid < off) {
       const float ob = sbest[tid + off];
       const int oi = sarg[tid + off];
