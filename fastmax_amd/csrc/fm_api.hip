@@ -895,17 +895,20 @@ int fastmax_qkv_rope(const fastmax_rope_desc* desc, int grad, void* qkv, const f
     return fail(FASTMAX_E_SHAPE, "rope_n = %d must be a multiple of 8 in [0, hs]", desc->rope_n);
   if (desc->rope_n > 0 && (!cos || !sin)) return fail(FASTMAX_E_NULL, "cos and sin must be non-NULL when rope_n > 0");
   const RopeShape sh{desc->b, desc->t, desc->groups, desc->q_per_kv, desc->hs, desc->rope_n};
-  const int64_t total = (int64_t)sh.b * sh.t * sh.groups * (sh.qpk + 2) * (sh.hs / 4);
+  const bool wide = sh.hs % 16 == 0 && sh.rn % 16 == 0;   // 16-channel units, 16-byte accesses
+  const int64_t total = (int64_t)sh.b * sh.t * sh.groups * (sh.qpk + 2) * (wide ? sh.hs / 16 : sh.hs / 4);
   if (total >= ((int64_t)1 << 39)) return fail(FASTMAX_E_SHAPE, "tensor too large");
   const unsigned blocks = (unsigned)((total + 255) / 256);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+#define FM_ROPE(KERNEL, T, G) KERNEL<T, G><<<blocks, 256, 0, st>>>(sh, (T*)qkv, cos, sin, (T*)q, (T*)k, (T*)v)
   if (desc->dtype == FASTMAX_F32) {
-    if (grad) qkv_rope_kernel<float, true><<<blocks, 256, 0, st>>>(sh, (float*)qkv, cos, sin, (float*)q, (float*)k, (float*)v);
-    else qkv_rope_kernel<float, false><<<blocks, 256, 0, st>>>(sh, (float*)qkv, cos, sin, (float*)q, (float*)k, (float*)v);
+    if (wide) { if (grad) FM_ROPE(qkv_rope16_kernel, float, true); else FM_ROPE(qkv_rope16_kernel, float, false); }
+    else { if (grad) FM_ROPE(qkv_rope_kernel, float, true); else FM_ROPE(qkv_rope_kernel, float, false); }
   } else {
-    if (grad) qkv_rope_kernel<bf16_t, true><<<blocks, 256, 0, st>>>(sh, (bf16_t*)qkv, cos, sin, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v);
-    else qkv_rope_kernel<bf16_t, false><<<blocks, 256, 0, st>>>(sh, (bf16_t*)qkv, cos, sin, (bf16_t*)q, (bf16_t*)k, (bf16_t*)v);
+    if (wide) { if (grad) FM_ROPE(qkv_rope16_kernel, bf16_t, true); else FM_ROPE(qkv_rope16_kernel, bf16_t, false); }
+    else { if (grad) FM_ROPE(qkv_rope_kernel, bf16_t, true); else FM_ROPE(qkv_rope_kernel, bf16_t, false); }
   }
+#undef FM_ROPE
   return launch_status("qkv_rope_kernel");
 }
 

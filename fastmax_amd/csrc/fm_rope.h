@@ -75,3 +75,81 @@ __global__ __launch_bounds__(256) void qkv_rope_kernel(RopeShape s, T* __restric
     }
   }
 }
+
+// Wider variant for hs % 16 == 0 and rn % 16 == 0 (the usual head sizes): a unit is 16 channels --
+// a rotary unit covers [8u, 8u+8) and their partners [8u + rn/2, ...), a copy unit 16 contiguous
+// channels at or beyond rn -- so every thread of a row has work and every access is 16 bytes
+// (bf16) or two of them (fp32).
+__device__ __forceinline__ void load8(const float* p, float (&o)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float (&o)[8]) {
+  const uint4 u = *reinterpret_cast<const uint4*>(p);
+  o[0] = bf_lo(u.x); o[1] = bf_hi(u.x); o[2] = bf_lo(u.y); o[3] = bf_hi(u.y);
+  o[4] = bf_lo(u.z); o[5] = bf_hi(u.z); o[6] = bf_lo(u.w); o[7] = bf_hi(u.w);
+}
+__device__ __forceinline__ void store8(float* p, const float (&v)[8]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float (&v)[8]) {
+  *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3]), pack_bf2(v[4], v[5]), pack_bf2(v[6], v[7]));
+}
+
+template <class T, bool GRAD>
+__global__ __launch_bounds__(256) void qkv_rope16_kernel(RopeShape s, T* __restrict__ qkv,
+                                                         const float* __restrict__ cosv,
+                                                         const float* __restrict__ sinv, T* __restrict__ q,
+                                                         T* __restrict__ k, T* __restrict__ v) {
+  const int upr = s.hs / 16;  // units per row
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t total = (int64_t)s.b * s.t * s.groups * (s.qpk + 2) * upr;
+  if (idx >= total) return;
+  const int u = (int)(idx % upr);
+  int64_t r = idx / upr;
+  const int slot = (int)(r % (s.qpk + 2));
+  r /= (s.qpk + 2);
+  const int g = (int)(r % s.groups);
+  r /= s.groups;
+  const int t = (int)(r % s.t);
+  const int b = (int)(r / s.t);
+  T* src = qkv + ((((int64_t)b * s.t + t) * s.groups + g) * (s.qpk + 2) + slot) * s.hs;
+  T* dst;
+  if (slot < s.qpk) dst = q + (((int64_t)b * s.groups * s.qpk + g * s.qpk + slot) * s.t + t) * s.hs;
+  else if (slot == s.qpk) dst = k + (((int64_t)b * s.groups + g) * s.t + t) * s.hs;
+  else dst = v + (((int64_t)b * s.groups + g) * s.t + t) * s.hs;
+  T* from = GRAD ? dst : src;
+  T* to = GRAD ? src : dst;
+  const int rn = slot <= s.qpk ? s.rn : 0;
+  const int nrot = rn / 16;  // rotary units
+  if (u < nrot) {
+    const int c = 8 * u, h = rn / 2;
+    float x1[8], x2[8], c1[8], s1[8], c2[8], s2[8], y1[8], y2[8];
+    load8(from + c, x1);
+    load8(from + c + h, x2);
+    load8(cosv + (int64_t)t * rn + c, c1);
+    load8(sinv + (int64_t)t * rn + c, s1);
+    load8(cosv + (int64_t)t * rn + c + h, c2);
+    load8(sinv + (int64_t)t * rn + c + h, s2);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if (GRAD) {  // dx1 = dy1 c1 + dy2 s2,  dx2 = dy2 c2 - dy1 s1
+        y1[e] = x1[e] * c1[e] + x2[e] * s2[e];
+        y2[e] = x2[e] * c2[e] - x1[e] * s1[e];
+      } else {     // y1 = x1 c1 - x2 s1,  y2 = x2 c2 + x1 s2
+        y1[e] = x1[e] * c1[e] - x2[e] * s1[e];
+        y2[e] = x2[e] * c2[e] + x1[e] * s2[e];
+      }
+    }
+    store8(to + c, y1);
+    store8(to + c + h, y2);
+  } else {
+    const int c = rn + 16 * (u - nrot);
+    float x[8], y[8];
+    load8(from + c, x);
+    load8(from + c + 8, y);
+    store8(to + c, x);
+    store8(to + c + 8, y);
+  }
+}

@@ -14,6 +14,9 @@ pytestmark = pytest.mark.gpu
     (2, 37, 3, 1, 64, 64, torch.float32, 1e-6), (1, 130, 2, 4, 64, 16, torch.float32, 1e-6),
     (2, 50, 4, 2, 32, 32, torch.float32, 1e-6), (1, 9, 1, 1, 64, 0, torch.float32, 1e-7),
     (2, 64, 12, 1, 64, 64, torch.bfloat16, 1e-2),
+    # rn or hs not a multiple of 16: the kernel with 4-channel units
+    (1, 20, 2, 2, 64, 8, torch.float32, 1e-6), (1, 33, 2, 1, 40, 24, torch.float32, 1e-6),
+    (1, 33, 2, 1, 40, 24, torch.bfloat16, 1e-2),
 ])
 def test_qkv_rope_split_forward_and_gradient(built, B, T, G, Q, hs, rn, dtype, tol):
     from fastmax_amd import qkv_rope_split
