@@ -20,6 +20,8 @@ Differences from the reference, all deliberate:
 from __future__ import annotations
 
 
+import math
+
 import torch
 
 from . import _ext
@@ -232,3 +234,30 @@ class FASTMultiHeadAttention(torch.nn.Module):
 
 
 fastmax_custom = FASTMultiHeadAttention()
+
+
+class FASTMultiHeadAttentionRPE(FASTMultiHeadAttention):
+    """The other calling convention of the reference (README.md:12-25, test_fastmax.py:242-249):
+    `rpe_matrix` sits between `drop_noise` and `mask`.  The relative positional encoding is
+    switched off in the reference's kernels (README.md:16) and its PyTorch function never sees
+    the matrix (test_fastmax.py:249), so it is accepted and not used here either."""
+
+    def forward(self, q, k, v, drop_noise=None, rpe_matrix=None, mask=False, dropout=0.0, normalize=False,
+                temperature=1.0, a0=1.0, a1=1.0, a2=0.5, lim=1.0, p=2):
+        return super().forward(q, k, v, drop_noise, mask, dropout, normalize, temperature, a0, a1, a2, lim, p)
+
+
+def rpe_matrix_creator(n, d, device, dtype, structured=False, is_zero=True):
+    """The (2n-1, d) relative-position table of test_fastmax.py:251-280.  structured: row i holds
+    the offset r = n-1-i (n-1 down to -(n-1)), even channels sin(r w_c), odd channels cos(r w_c)
+    with w_c = 10000^(-2c/d) for the channel pair c; otherwise zeros (is_zero) or N(0, 1) draws."""
+    if not structured:
+        if is_zero:
+            return torch.zeros(2 * n - 1, d, device=device, dtype=dtype)
+        return torch.normal(0, 1, size=(2 * n - 1, d), device=device, dtype=dtype)
+    offsets = torch.arange(n - 1, -n, -1, device=device, dtype=dtype).unsqueeze(1)
+    w = torch.exp(torch.arange(0, d, 2, device=device, dtype=dtype) * (-math.log(10000.0) / d))
+    table = torch.zeros(2 * n - 1, d, device=device, dtype=dtype)
+    table[:, 0::2] = torch.sin(offsets * w)
+    table[:, 1::2] = torch.cos(offsets * w)
+    return table

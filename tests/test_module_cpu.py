@@ -127,3 +127,30 @@ def test_pytorch_path_grouped_heads_and_key_prefix(mask, p):
     assert torch.allclose(got, ref, rtol=1e-10, atol=1e-12)
     with pytest.raises(ValueError, match="fewer keys"):
         fastmax_function(ke, q, q, mask)
+
+
+def test_rpe_calling_convention_and_table():
+    """README.md:12-25 / test_fastmax.py:242-280: rpe_matrix between drop_noise and mask (accepted,
+    unused: the reference's kernels have it switched off and its PyTorch function never gets it),
+    and the (2n-1, d) table: offsets n-1 .. -(n-1), sin on even and cos on odd channels."""
+    import math
+
+    from fastmax_amd import FASTMultiHeadAttentionRPE, rpe_matrix_creator
+
+    sig = inspect.signature(FASTMultiHeadAttentionRPE.forward)
+    assert list(sig.parameters) == ["self", "q", "k", "v", "drop_noise", "rpe_matrix", "mask", "dropout", "normalize",
+                                    "temperature", "a0", "a1", "a2", "lim", "p"]
+    n, d = 5, 8
+    t = rpe_matrix_creator(n, d, "cpu", torch.float64, structured=True)
+    assert t.shape == (2 * n - 1, d)
+    for row, off in ((0, n - 1), (n - 1, 0), (n, -1), (2 * n - 2, -(n - 1))):
+        for c in range(d // 2):
+            w = 10000.0 ** (-2.0 * c / d)
+            assert abs(float(t[row, 2 * c]) - math.sin(off * w)) < 1e-12
+            assert abs(float(t[row, 2 * c + 1]) - math.cos(off * w)) < 1e-12
+    assert torch.equal(rpe_matrix_creator(n, d, "cpu", torch.float32), torch.zeros(2 * n - 1, d))
+    assert rpe_matrix_creator(n, d, "cpu", torch.float32, is_zero=False).abs().sum() > 0
+    q, k, v, _ = O.seeded_inputs((1, 2, 6, 4), seed=5, dtype=torch.float64)
+    a = FASTMultiHeadAttentionRPE(use_custom_gradient=False)(q, k, v, None, t, True, 0.0, True)
+    b = FASTMultiHeadAttention(use_custom_gradient=False)(q, k, v, None, True, 0.0, True)
+    assert torch.equal(a, b)
