@@ -142,10 +142,18 @@ std::vector<torch::Tensor> backward_ex(torch::Tensor q, torch::Tensor k, torch::
   return {dq, dk, dv};
 }
 
+// `lead` rows of zeros in front of a (bh, n, w) tensor.
+torch::Tensor lead_rows(const torch::Tensor& t, int64_t lead) {
+  return torch::cat({torch::zeros({t.size(0), lead, t.size(2)}, t.options()), t}, 1);
+}
+
 // Reference signature and side effects (fastmax_cuda.cpp:17-24, fastmax_cuda_forward.cu:366-399):
 // k is divided by temperature and q, k are normalised IN PLACE, so that the caller's saved
-// q, k are the ones backwardpass expects; the result is (bh, n, d+1) with the row denominators
+// q, k are the ones backwardpass expects; the result is (bh, nq, d+1) with the row denominators
 // in column d; dropout > 0 multiplies the output by 1 + dropout * drop_noise.
+// k, v longer than q (fastmax_cuda_forward.cu:109-150: the first nk - nq keys are visible to
+// every query): the pass runs on q with nk - nq zero rows in front, which see only those keys,
+// do not move the row-norm maximum and are cut from the result.
 torch::Tensor forwardpass(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor drop_noise,
                           bool mask, double dropout, bool normalize, double temperature, double a0,
                           double a1, double a2, double lim, int64_t p) {
@@ -155,22 +163,29 @@ torch::Tensor forwardpass(torch::Tensor q, torch::Tensor k, torch::Tensor v, tor
   check_same(q, k, "k");
   check_same(q, v, "v");
   TORCH_CHECK(q.scalar_type() == torch::kFloat32, "forwardpass takes float32 tensors (use forward_ex for bfloat16)");
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3, "q, k, v must be (b*h, n, d)");
   TORCH_CHECK(k.sizes() == v.sizes(), "k and v must have the same shape");
-  fastmax_desc ds = make_desc(q, k, mask, normalize, 1.0, a0, a1, a2, lim, p);
+  const int64_t lead = k.size(1) - q.size(1);
+  TORCH_CHECK(lead >= 0, "k, v have ", k.size(1), " tokens but q has ", q.size(1),
+              ": fewer keys than queries is not supported");
   const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+  torch::Tensor qp = lead ? lead_rows(q, lead) : q;
+  fastmax_desc ds = make_desc(qp, k, mask, normalize, 1.0, a0, a1, a2, lim, p);
   const fastmax_stream_t stream = current_stream(q);
   if (temperature != 1.0) k.div_(temperature);
   if (normalize) {
     auto nws = torch::empty({16 * (int64_t)ds.bh + 1024}, q.options().dtype(torch::kUInt8));
-    raise_on(fastmax_normalize_inplace(&ds, q.data_ptr(), k.data_ptr(), nws.data_ptr(), (size_t)nws.numel(), stream));
+    raise_on(fastmax_normalize_inplace(&ds, qp.data_ptr(), k.data_ptr(), nws.data_ptr(), (size_t)nws.numel(), stream));
     ds.normalize = 0;
+    if (lead) q.copy_(qp.narrow(1, lead, q.size(1)));
   }
   const int64_t d = q.size(2);
-  auto o = torch::empty({q.size(0), q.size(1), d + 1}, q.options());
+  auto o = torch::empty({qp.size(0), qp.size(1), d + 1}, q.options());
   size_t wsb = 0;
   auto ws = workspace(ds, FASTMAX_PASS_FORWARD, q, &wsb);
-  raise_on(fastmax_forward(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d + 1,
+  raise_on(fastmax_forward(&ds, qp.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d + 1,
                            o.data_ptr<float>() + d, d + 1, nullptr, nullptr, ws.data_ptr(), wsb, stream));
+  if (lead) o = o.narrow(1, lead, q.size(1)).contiguous();
   if (dropout > 0.0) {
     TORCH_CHECK(drop_noise.defined() && drop_noise.sizes() == q.sizes(), "drop_noise must be shaped like q");
     o.narrow(2, 0, d).mul_(drop_noise * dropout + 1.0);
@@ -194,12 +209,24 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
   check_same(q, o, "o");
   check_same(q, grad_output, "grad_output");
   TORCH_CHECK(q.scalar_type() == torch::kFloat32, "backwardpass takes float32 tensors (use backward_ex for bfloat16)");
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3, "q, k, v must be (b*h, n, d)");
   const int64_t d = q.size(2);
   TORCH_CHECK(o.dim() == 3 && o.size(0) == q.size(0) && o.size(1) == q.size(1) && o.size(2) == d + 1,
               "o must be the (bh, n, d+1) tensor forwardpass returned");
   TORCH_CHECK(grad_output.sizes() == q.sizes(), "grad_output must be shaped like q");
-  const fastmax_desc ds = make_desc(q, k, mask, false, 1.0, a0, a1, a2, 1.0, p);
+  const int64_t lead = k.size(1) - q.size(1);
+  TORCH_CHECK(lead >= 0, "k, v have ", k.size(1), " tokens but q has ", q.size(1),
+              ": fewer keys than queries is not supported");
   const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+  if (lead) {
+    // key prefix: zero query rows in front with a zero upstream gradient add nothing to dk, dv;
+    // their denominator column is set to 1 so that 0 / den stays 0 whatever a0 is
+    q = lead_rows(q, lead);
+    grad_output = lead_rows(grad_output, lead);
+    o = lead_rows(o, lead);
+    o.narrow(1, 0, lead).select(2, d).fill_(1.0);
+  }
+  const fastmax_desc ds = make_desc(q, k, mask, false, 1.0, a0, a1, a2, 1.0, p);
   auto dq = torch::empty_like(q);
   auto dk = torch::empty_like(k);
   auto dv = torch::empty_like(v);
@@ -209,6 +236,7 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
                             o.data_ptr<float>() + d, d + 1, grad_output.data_ptr(), dq.data_ptr(),
                             dk.data_ptr(), dv.data_ptr(), nullptr, nullptr, ws.data_ptr(), wsb,
                             current_stream(q)));
+  if (lead) dq = dq.narrow(1, lead, dq.size(1) - lead).contiguous();
   return {dq, dk, dv};
 }
 

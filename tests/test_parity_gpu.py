@@ -338,6 +338,36 @@ def test_legacy_extension_entry_points(built):
         ext.forwardpass(qd, kd, vd, qd, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 3)
 
 
+@pytest.mark.parametrize("mask,a0", [(True, 1.0), (False, 1.0), (True, 0.0)])
+def test_legacy_entry_points_with_a_key_prefix(built, mask, a0):
+    """forwardpass / backwardpass with k, v longer than q: the first nk - nq keys are visible to
+    every query (fastmax_cuda_forward.cu:109-150, fastmax_cuda_backward.cu:900-1006)."""
+    from fastmax_amd import _ext
+
+    ext = _ext.load()
+    nq, nk, d = 210, 345, 64
+    a1, a2 = (1.0, 0.5) if a0 else (0.3, 1.0)
+    q, _, _, go = O.seeded_inputs((4, nq, d), seed=29)
+    _, k, v, _ = O.seeded_inputs((4, nk, d), seed=30)
+    qd, kd, vd, god = (t.cuda() for t in (q, k, v, go))
+    o = ext.forwardpass(qd, kd, vd, torch.zeros_like(qd), mask, 0.0, True, 1.0, a0, a1, a2, 1.0, 2)
+    assert o.shape == (4, nq, d + 1) and o.is_contiguous()
+    qh, kh = O.normalize_qk(q[None].double(), k[None].double(), 1.0)
+    assert_close("q normalised in place", qd, qh[0], 1e-6)
+    assert_close("k normalised in place", kd, kh[0], 1e-6)
+    ro, rden = O.dense_truth(q, k, v, None, mask=mask, normalize=True, a0=a0, a1=a1, a2=a2)
+    assert_close("o", o[:, :, :d], ro, 1e-4)
+    assert_close("den column", o[:, :, d], rden, 1e-4)
+    dq, dk, dv = ext.backwardpass(qd, kd, vd, o, god, mask, a0, a1, a2, 2)
+    _, rdq, rdk, rdv = O.dense_truth(qh[0], kh[0], v, go, mask=mask, normalize=False, a0=a0, a1=a1, a2=a2)
+    for name, got, ref in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert got.shape == ref.shape and got.is_contiguous()
+        assert torch.isfinite(got).all()
+        assert_close(name, got, ref, 1e-4)
+    with pytest.raises(RuntimeError, match="fewer keys"):
+        ext.forwardpass(kd, qd, qd, kd, mask, 0.0, True, 1.0, a0, a1, a2, 1.0, 2)
+
+
 @pytest.mark.parametrize("bh,bhkv,n,d,mask,p,dtype", [
     (4, 4, 900, 64, True, 2, torch.float32), (4, 4, 700, 64, False, 2, torch.float32),
     (6, 2, 500, 32, True, 2, torch.float32), (4, 4, 1000, 64, True, 2, torch.bfloat16),
