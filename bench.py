@@ -44,7 +44,7 @@ COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 # runs summarised under profiles/ (one file per workload, TRAFFIC_SOURCE)
 # (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch x2.0, write x1.0).
 MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD = {
-    "headline": {"build": 3023.0, "fwd_apply": 2611.0, "bwd_dq": 2863.0, "bwd_dk": 3045.0, "bwd_dv": 2714.0},
+    "headline": {"build": 3039.0, "fwd_apply": 2611.0, "bwd_dq": 2857.0, "bwd_dk": 3039.0, "bwd_dv": 2787.0},
     # profiles/headline_p1_causal_fp32_scan_kernels.txt (algorithmic: 1024 B per token-head and kernel,
     # 1280 B for dq, which also reads the forward output)
     "headline-p1": {"fwd_apply": 1166.0, "bwd_dq": 1499.0, "bwd_dk": 1182.0, "bwd_dv": 1181.0},
