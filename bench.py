@@ -37,6 +37,7 @@ WORKLOADS = {
     "c2": dict(B=64, H=8, N=1000, D=32, mask=True, p=2, dtype="f32"),
     "c4": dict(B=16, H=32, N=16384, D=64, mask=True, p=2, dtype="bf16"),
     "c5-layer": dict(B=8, H=12, N=2048, D=64, mask=True, p=2, dtype="bf16"),  # one layer of the GPT step
+    "c5-layer-p1": dict(B=8, H=12, N=2048, D=64, mask=True, p=1, dtype="bf16"),  # at the order model.py:569 sets
 }
 COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 
