@@ -203,6 +203,69 @@ def test_linearity_in_values_and_adjoint_identity(ops):
 
 
 # ------------------------------------------------------------------ configurations of record
+@pytest.mark.parametrize("seed", [11, 12])
+def test_random_configurations(ops, seed):
+    """A seeded sweep over shapes (lengths around the tile, block and chunk boundaries, grouped
+    heads, both head dims, enough heads for the p = 1 scan kernels), coefficients, lim,
+    temperature, dtype, kept states and minimum workspaces, each against the fp64 dense form.
+    Coefficients and scales keep f(s) positive, so that no case is ill-conditioned."""
+    import ctypes as C
+    import random
+
+    from fastmax_amd import _cabi
+
+    rng = random.Random(seed)
+    lengths = [1, 2, 31, 32, 33, 64, 65, 127, 128, 129, 255, 257, 383, 384, 385, 511, 513, 769, 1153]
+    for case in range(60):
+        d, p, mask = rng.choice([32, 64, 64]), rng.choice([1, 2]), rng.random() < 0.6
+        dtype = torch.bfloat16 if rng.random() < 0.3 else torch.float32
+        normalize = rng.random() < 0.7
+        bhkv, ratio, n = rng.choice([1, 2, 3, 4, 6]), rng.choice([1, 1, 2, 3]), rng.choice(lengths)
+        if p == 1 and d == 64 and rng.random() < 0.4:
+            bhkv, ratio, n = 512 + rng.choice([0, 1, 7]), 1, rng.choice([32, 33, 40, 64, 100, 129])
+        bh = bhkv * ratio
+        if n < 31:
+            # with one or two visible keys g.v_j - c_i all but cancels, and the 8-bit rounding of a
+            # bf16 o (inside c_i = g_i.o_i) is then no longer small against dq, dk
+            dtype = torch.float32
+        a0, a1, a2 = rng.choice([1.0, 1.5, 2.0]), rng.choice([1.0, 0.5, 0.8]), rng.choice([0.5, 1.0, 0.25])
+        lim = rng.choice([1.0, 0.5]) if normalize else 1.0
+        temperature = 1.0 if normalize else rng.choice([1.0, 2.0, 0.5])
+        scale = 1.0 if normalize else 0.08   # |q.k|/T stays well below a0/a1
+        save, small_ws = rng.random() < 0.4, rng.random() < 0.3
+        g = torch.Generator().manual_seed(seed * 100003 + case)
+        q = (torch.randn(bh, n, d, generator=g) * scale).to(dtype)
+        k = (torch.randn(bhkv, n, d, generator=g) * scale).to(dtype)
+        v = torch.randn(bhkv, n, d, generator=g).to(dtype)
+        go = torch.randn(bh, n, d, generator=g).to(dtype)
+        kw = dict(mask=mask, normalize=normalize, lim=lim, temperature=temperature, a0=a0, a1=a1, a2=a2, p=p)
+        what = f"case {case}: bh={bh} bhkv={bhkv} n={n} d={d} {dtype} save={save} small_ws={small_ws} {kw}"
+        print(what, flush=True)
+        # truth: keys divided by the temperature, key/value heads repeated per query head
+        truth_kw = {key: val for key, val in kw.items() if key != "temperature"}
+        kt = k.double() if normalize else k.double() / temperature
+        ro, rdq, rdk, rdv = O.dense_truth(q.double(), kt.repeat_interleave(ratio, 0),
+                                          v.double().repeat_interleave(ratio, 0), go.double(), **truth_kw)
+        rdk = rdk.view(bhkv, ratio, n, d).sum(1) / (1.0 if normalize else temperature)
+        rdv = rdv.view(bhkv, ratio, n, d).sum(1)
+        qd, kd, vd, god = (t.cuda() for t in (q, k, v, go))
+        wsf = wsb = None
+        if small_ws:
+            ds = ops._desc(qd, kd, mask, normalize, p, lim, temperature, a0, a1, a2)
+            wsf = _cabi.load().fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_FORWARD)
+            wsb = _cabi.load().fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_BACKWARD)
+        saved = None
+        if save:
+            o, den, sc, arg, saved = ops.forward(qd, kd, vd, save_states=True, **kw)
+        else:
+            o, den, sc, arg = ops.forward(qd, kd, vd, workspace_bytes=wsf, **kw)
+        dq, dk, dv = ops.backward(qd, kd, vd, o, den, god, workspace_bytes=wsb, saved_states=saved, **kw)
+        atol = 1e-6   # a single token has o = v whatever q and k are: its dq, dk are zero
+        for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+            assert torch.isfinite(got.float()).all(), what
+            assert_close(f"{what} / {name}", got.float(), ref, TOL[dtype], atol=atol)
+
+
 def test_config1_unmasked_b8_h8_n1024_d32(ops):
     run_case(ops, (64, 1024, 32), seed=0, mask=False, normalize=True, p=2)
 
