@@ -334,6 +334,12 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
 // lane, which leaves den[row] in every lane that holds that row of the output.
 // Lane half hh owns features/channels 32*hh + t as in the fp32 kernel; MFMA g of a sweep takes
 // t = 4g..4g+3 from both halves.
+// Pipeline of the state part: slabs go global -> LDS directly (no staging registers), two slabs
+// ahead, into four buffers; a step is two slabs and one barrier; the window of rotated partner
+// channels is read at compile-time positions (four unrolled shifts per window load); within a
+// slab all B operands are requested first, the features are formed while they travel, and the
+// matrix instructions then run back to back.  Streamed tiles of the intra-chunk part are
+// fetched two tiles ahead.
 // ---------------------------------------------------------------------------------------
 template <int D, int MODE>
 __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
@@ -353,9 +359,20 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   constexpr int TPB = 36;              // pitch of the transposed 32-token value tile
   constexpr int NCF = PG::NCF, FSL = PG::FSL;
   constexpr int SLB1 = 32 * LB + D * TPB;  // both 32-token tiles
-  constexpr int SLB = ((FSL > SLB1 ? FSL : SLB1) + 7) / 8 * 8;
+  // A slab travels global -> LDS without passing through registers (global_load_lds_dwordx4: lane
+  // l of a wave delivers its 16 bytes at a wave-uniform LDS base + 16 l), two slabs ahead of its
+  // use, into one of four buffers (four separate arrays: the compiler's bookkeeping of outstanding
+  // transfers is per LDS object).  A buffer is a whole number of 64-piece wave transfers.
+  constexpr int NPC = FSL / 8;                       // 16-byte pieces of a slab
+  constexpr int NPCR = (NPC + 63) / 64 * 64;
+  constexpr int NVS = (NPC + 255) / 256;             // transfers per wave and slab
+  constexpr int SLB = (NPCR * 8 > SLB1 ? NPCR * 8 : (SLB1 + 7) / 8 * 8);
   __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
-  __shared__ __attribute__((aligned(16))) uint16_t Sb[2][SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb0[SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb1[SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb2[SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb3[SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sjunk[512];   // where transfers nobody needs end up
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
@@ -398,40 +415,42 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   const uint16_t* fsec = reinterpret_cast<const uint16_t*>(sbase);
   const float* zsec = reinterpret_cast<const float*>(sbase + PG::z_off(p2));
 
-  // an F slab is copied as it is: 16-byte pieces global -> registers -> LDS
-  // (no branches: threads past the end wrap round and copy an early piece a second time, so that
-  // every load is issued up front and stays in flight under the MFMAs)
-  constexpr int NPC = FSL / 8, NVS = (NPC + 255) / 256;
-  static_assert(NVS <= 3, "three named pieces per thread (an indexed array would live in scratch)");
-  uint4 sv0, sv1, sv2;
-  RowTile<D, T, 32> t1, t2;
-  auto slab_load = [&](int st) {
-    const uint4* src = reinterpret_cast<const uint4*>(fsec + st * FSL);
-    sv0 = src[tid % NPC];
-    if constexpr (NVS > 1) sv1 = src[(tid + 256) % NPC];
-    if constexpr (NVS > 2) sv2 = src[(tid + 512) % NPC];
+  // Transfers of slab st into `buf` (wave-uniform).  No branches: pieces past the slab's end wrap
+  // round at the source, and a wave transfer that lies wholly past the end, or a slab past the
+  // last one, is sent to Sjunk.
+  auto slab_dma = [&](int st, uint16_t* buf) __attribute__((always_inline)) {
+    const bool live = st < n_state;
+    const uint16_t* src = fsec + (live ? st : 0) * FSL;
+#pragma unroll
+    for (int r = 0; r < NVS; ++r) {
+      const int first = r * 256 + w * 64;
+      uint16_t* dst = (live && first < NPCR) ? buf + first * 8 : Sjunk;
+      __builtin_amdgcn_global_load_lds(src + ((first + l) % NPC) * 8,
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
   };
-  auto slab_store = [&](int st) {
-    uint4* dst = reinterpret_cast<uint4*>(Sb[st & 1]);
-    dst[tid % NPC] = sv0;
-    if constexpr (NVS > 1) dst[(tid + 256) % NPC] = sv1;
-    if constexpr (NVS > 2) dst[(tid + 512) % NPC] = sv2;
+  // streamed tiles travel through registers (they are scaled, and one of them transposed, on the
+  // way), two tiles ahead of their use: two sets of registers that take turns
+  RowTile<D, T, 32> t1a, t2a, t1b, t2b;
+  auto tiles_load = [&](int kk, auto& u1, auto& u2) __attribute__((always_inline)) {
+    u1.load(A1h, (tile0 + kk) * 32, n, tid);
+    u2.load(A2h, (tile0 + kk) * 32, n, tid, a2dh, a2den_stride);
   };
-  auto tiles_load = [&](int kk) {
-    t1.load(A1h, (tile0 + kk) * 32, n, tid);
-    t2.load(A2h, (tile0 + kk) * 32, n, tid, a2dh, a2den_stride);
-  };
-  auto tiles_store = [&](int buf) {
-    t1.store_bf(Sb[buf], LB, a1s, tid);
-    t2.store_t_bf(Sb[buf] + 32 * LB, TPB, 1.0f, tid);
+  auto tiles_store = [&](int buf, auto& u1, auto& u2) __attribute__((always_inline)) {
+    uint16_t* tb = buf ? Sb1 : Sb0;
+    u1.store_bf(tb, LB, a1s, tid);
+    u2.store_t_bf(tb + 32 * LB, TPB, 1.0f, tid);
   };
 
-  if (n_tile > 0) tiles_load(0);
+  if (n_tile > 0) {
+    tiles_load(0, t1a, t2a);
+    tiles_load(n_tile > 1 ? 1 : 0, t1b, t2b);
+  }
   if (n_state > 0) {
-    slab_load(0);
-    slab_store(0);
+    slab_dma(0, Sb0);
+    slab_dma(1, Sb1);
   } else if (n_tile > 0) {
-    tiles_store(0);
+    tiles_store(0, t1a, t2a);
   }
   __syncthreads();
 
@@ -464,51 +483,52 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   // one slab: B operands are 64-bit reads of [feature group][column][4 features]; two feature
   // groups (8 features per lane half) make one k = 16 MFMA.  Operands are fetched one step ahead
   // of the MFMAs that use them.
-  auto slab_compute = [&](const uint16_t* sl, auto tag) {
+  auto slab_compute = [&](const uint16_t* sl, auto tag, auto wo) __attribute__((always_inline)) {
     constexpr bool ORD2 = decltype(tag)::value;
+    constexpr int WO = decltype(wo)::value;   // Wn[WO + t] is the partner of channel t for this shift
     constexpr int NB = FWD ? CB + 1 : CB;
     constexpr int NM = H2 / 8;  // MFMA steps per column tile
     const uint16_t* brow = sl + (hh * (H2 / 4) * NCF + i) * 4;
     const uint16_t* erow = sl + (hh * (H2 / 4) * NCF + D) * 4;
+    // (the two halves of an operand are read next to each other, so that they pair into one
+    // two-address LDS read whose four destination registers are the operand)
     auto fetch = [&](int m, uint2 (&b)[2 * NB]) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
+        for (int u = 0; u < 2; ++u)
           b[2 * cb + u] = *reinterpret_cast<const uint2*>(brow + ((2 * m + u) * NCF + cb * 32) * 4);
-        if (FWD) b[2 * (NB - 1) + u] = *reinterpret_cast<const uint2*>(erow + (2 * m + u) * NCF * 4);
+      }
+      if (FWD) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+          b[2 * (NB - 1) + u] = *reinterpret_cast<const uint2*>(erow + (2 * m + u) * NCF * 4);
       }
     };
     auto feat = [&](int g4) {
       const int t = 4 * g4;
-      return ORD2 ? pack_bf4u(Xr[t] * Wn[t], Xr[t + 1] * Wn[t + 1], Xr[t + 2] * Wn[t + 2], Xr[t + 3] * Wn[t + 3])
+      return ORD2 ? pack_bf4u(Xr[t] * Wn[WO + t], Xr[t + 1] * Wn[WO + t + 1], Xr[t + 2] * Wn[WO + t + 2],
+                              Xr[t + 3] * Wn[WO + t + 3])
                   : pack_bf4u(Xr[t] * a1, Xr[t + 1] * a1, Xr[t + 2] * a1, Xr[t + 3] * a1);
     };
-    uint2 bc[2 * NB], bn[2 * NB];
-    fetch(0, bc);
-    uint2 alo = feat(0), ahi = feat(1), nlo = alo, nhi = ahi;
+    // all B operands of the slab are requested first, the features are formed while they are on
+    // their way, then the matrix instructions run back to back
+    uint2 b[NM][2 * NB], a[NM][2];
+#pragma unroll
+    for (int m = 0; m < NM; ++m) fetch(m, b[m]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
-      if (m + 1 < NM) {
-        fetch(m + 1, bn);
-        nlo = feat(2 * m + 2);
-        nhi = feat(2 * m + 3);
-      }
-      const bf8v ap = as_bf8(alo, ahi);
+      a[m][0] = feat(2 * m);
+      a[m][1] = feat(2 * m + 1);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA_BF16(ap, as_bf8(bc[2 * cb], bc[2 * cb + 1]), acc[cb]);
-      if (FWD) accd = FM_MFMA_BF16(ap, as_bf8(bc[2 * (NB - 1)], bc[2 * (NB - 1) + 1]), accd);
-      // interleave: each MFMA is followed by two of the next step's LDS reads and four of its VALU ops
+    for (int m = 0; m < NM; ++m) {
+      const bf8v ap = as_bf8(a[m][0], a[m][1]);
 #pragma unroll
-      for (int x = 0; x < NB; ++x) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-      }
-#pragma unroll
-      for (int x = 0; x < 2 * NB; ++x) bc[x] = bn[x];
-      alo = nlo;
-      ahi = nhi;
+      for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA_BF16(ap, as_bf8(b[m][2 * cb], b[m][2 * cb + 1]), acc[cb]);
+      if (FWD) accd = FM_MFMA_BF16(ap, as_bf8(b[m][2 * (NB - 1)], b[m][2 * (NB - 1) + 1]), accd);
     }
   };
 
@@ -519,46 +539,68 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   for (int cb = 0; cb < CB; ++cb) zc[cb] = n_state > 0 ? a0 * zsec[cb * 32 + i] : 0.f;
   if (FWD && n_state > 0) zd = a0 * zsec[D];
 
-  auto slab_step = [&](int st) {
-    const uint16_t* sl = Sb[st & 1];
-    if (p2 && st < NS) {
-      if ((st & 3) == 0) {
-        window_load(st);
-      } else {
+  // One pipeline step = two slabs and one barrier: start the transfers of slabs st+2, st+3 into the
+  // buffers the previous step read from (every wave is past them: it has passed the barrier),
+  // work on slabs st and st+1, wait for the wave's own transfers, barrier (which covers the other
+  // waves').  After the last slab the first streamed tile is staged instead.
+  auto order0 = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int x = 0; x < H2 + 3; ++x) Wn[x] = Wn[x + 1];
-      }
-      slab_compute(sl, std::true_type{});
-      if (st == NS - 1) {
+    for (int r = 0; r < 16; ++r) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-#pragma unroll
-          for (int cb = 0; cb < CB; ++cb) acc[cb][r] *= a2;
-          accd[r] *= a2;
-        }
-      }
-    } else {
-      slab_compute(sl, std::false_type{});
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) acc[cb][r] += zc[cb];
-        if (FWD) accd[r] += zd;
-      }
+      for (int cb = 0; cb < CB; ++cb) acc[cb][r] += zc[cb];
+      if (FWD) accd[r] += zd;
     }
   };
-  // the last slab is peeled off so that load and store of the next slab are unconditional in
-  // the loop (a load whose only use sits in a branch is moved there and waited for at once)
-  for (int st = 0; st + 1 < n_state; ++st) {
-    slab_load(st + 1);
-    slab_step(st);
-    slab_store(st + 1);
-    __syncthreads();
-  }
-  if (n_state > 0) {
-    slab_step(n_state - 1);
-    if (n_tile > 0) tiles_store(n_state & 1);
-    __syncthreads();
+  auto step_begin = [&](int st, uint16_t* ahead0, uint16_t* ahead1) __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);   // (keeps the unrolled steps apart: register pressure)
+    slab_dma(st + 2, ahead0);
+    slab_dma(st + 3, ahead1);
+  };
+  auto step_end = [&](bool last) __attribute__((always_inline)) {
+    if (!last) {
+      FM_WAIT_VM(0);
+      __builtin_amdgcn_s_barrier();
+    } else {
+      if (n_tile > 0) tiles_store(n_state & 1, t1a, t2a);
+      __syncthreads();
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using W0 = std::integral_constant<int, 0>;
+  if (n_state > 1) {
+    // p = 2: shifts 0 .. NS-1, then the order-1 slab.  The window of rotated partners is loaded
+    // every fourth shift and read at a compile-time position in between (no register moves).
+    static_assert((NS - 1) % 4 == 0, "shifts come in groups of four plus the last one");
+    for (int st = 0; st < NS - 1; st += 4) {
+      window_load(st);
+      step_begin(st, Sb2, Sb3);
+      slab_compute(Sb0, std::true_type{}, W0{});
+      __builtin_amdgcn_sched_barrier(0);
+      slab_compute(Sb1, std::true_type{}, std::integral_constant<int, 1>{});
+      step_end(false);
+      step_begin(st + 2, Sb0, Sb1);
+      slab_compute(Sb2, std::true_type{}, std::integral_constant<int, 2>{});
+      __builtin_amdgcn_sched_barrier(0);
+      slab_compute(Sb3, std::true_type{}, std::integral_constant<int, 3>{});
+      step_end(false);
+    }
+    window_load(NS - 1);
+    step_begin(NS - 1, Sb2, Sb3);   // (nothing left to bring in: these go to Sjunk)
+    slab_compute(Sb0, std::true_type{}, W0{});
+    // the order-2 slabs carry their pair weights; a2 multiplies their sum
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) acc[cb][r] *= a2;
+      if (FWD) accd[r] *= a2;
+    }
+    slab_compute(Sb1, std::false_type{}, W0{});
+    order0();
+    step_end(true);
+  } else if (n_state == 1) {
+    slab_compute(Sb0, std::false_type{}, W0{});
+    order0();
+    step_end(true);
   }
 
   if (n_tile > 0) {
@@ -567,13 +609,15 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     for (int g4 = 0; g4 < H2 / 4; ++g4) Xp[g4] = pack_bf4u(Xr[4 * g4], Xr[4 * g4 + 1], Xr[4 * g4 + 2], Xr[4 * g4 + 3]);
     const bf8v ones = as_bf8(make_uint2(0x3f803f80u, 0x3f803f80u), make_uint2(0x3f803f80u, 0x3f803f80u));
     const int mine = (tok0 >> 5) + w;
-    for (int kk = 0; kk < n_tile; ++kk) {
+    // tile kk is in LDS, tile kk+1 in the registers `nx`; the registers `ld` that carried tile kk are
+    // free and take tile kk+2
+    auto tile_iter = [&](int kk, auto& ld1, auto& ld2, auto& nx1, auto& nx2) __attribute__((always_inline)) {
       const int buf = (n_state + kk) & 1;
-      tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
+      tiles_load(kk + 2 < n_tile ? kk + 2 : n_tile - 1, ld1, ld2);
       const int tl = tile0 + kk;
       if (FWD ? tl <= mine : tl >= mine) {
-        const uint16_t* l1 = Sb[buf];
-        const uint16_t* l2 = Sb[buf] + 32 * LB;
+        const uint16_t* l1 = buf ? Sb1 : Sb0;
+        const uint16_t* l2 = l1 + 32 * LB;
         f16v sc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) sc[r] = 0.f;
@@ -605,8 +649,12 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
           if (FWD) accd = FM_MFMA_BF16(pp, ones, accd);
         }
       }
-      if (kk + 1 < n_tile) tiles_store(buf ^ 1);
+      if (kk + 1 < n_tile) tiles_store(buf ^ 1, nx1, nx2);
       __syncthreads();
+    };
+    for (int kk = 0; kk < n_tile; kk += 2) {
+      tile_iter(kk, t1a, t2a, t1b, t2b);
+      if (kk + 1 < n_tile) tile_iter(kk + 1, t1b, t2b, t1a, t2a);
     }
   }
 

@@ -29,6 +29,10 @@ typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
 // simply concatenated: slots 0..3 from the first pair, 4..7 from the second.
 typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
 #define FM_MFMA_BF16(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
+// wait until at most n vector-memory operations of this wave are outstanding (they complete in
+// order), leaving the other counters alone: s_waitcnt simm16 = vmcnt[3:0] | expcnt << 4 |
+// lgkmcnt << 8 | vmcnt[5:4] << 14
+#define FM_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 
 __device__ __forceinline__ uint32_t pack_bf2(float lo, float hi) {
   const bf2v p = {(__bf16)lo, (__bf16)hi};  // round to nearest even (v_cvt_pk_bf16_f32)
