@@ -618,14 +618,33 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
       if (FWD ? tl <= mine : tl >= mine) {
         const uint16_t* l1 = buf ? Sb1 : Sb0;
         const uint16_t* l2 = l1 + 32 * LB;
-        f16v sc;
+        // every LDS operand of the tile is requested first; the scores accumulate in two
+        // independent chains
+        uint2 ka[H2 / 8][2], vb[2][CB][2];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+        for (int m = 0; m < H2 / 8; ++m) {
+          ka[m][0] = *reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 8 * m);
+          ka[m][1] = *reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 8 * m + 4);
+        }
 #pragma unroll
-        for (int m = 0; m < H2 / 8; ++m)
-          sc = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 8 * m),
-                                   *reinterpret_cast<const uint2*>(l1 + i * LB + hh * H2 + 8 * m + 4)),
-                            as_bf8(Xp[2 * m], Xp[2 * m + 1]), sc);
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) {
+            const uint16_t* vrow = l2 + (cb * 32 + i) * TPB + 16 * m + 4 * hh;
+            vb[m][cb][0] = *reinterpret_cast<const uint2*>(vrow);
+            vb[m][cb][1] = *reinterpret_cast<const uint2*>(vrow + 8);
+          }
+        f16v sc, sc1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = sc1[r] = 0.f;
+        static_assert((H2 / 8) % 2 == 0, "score steps come in pairs");
+#pragma unroll
+        for (int m = 0; m < H2 / 8; m += 2) {
+          sc = FM_MFMA_BF16(as_bf8(ka[m][0], ka[m][1]), as_bf8(Xp[2 * m], Xp[2 * m + 1]), sc);
+          sc1 = FM_MFMA_BF16(as_bf8(ka[m + 1][0], ka[m + 1][1]), as_bf8(Xp[2 * m + 2], Xp[2 * m + 3]), sc1);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] += sc1[r];
         const bool diag = tl == mine;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -641,11 +660,7 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
           const bf8v pp = as_bf8(pack_bf4u(sc[8 * m], sc[8 * m + 1], sc[8 * m + 2], sc[8 * m + 3]),
                                  pack_bf4u(sc[8 * m + 4], sc[8 * m + 5], sc[8 * m + 6], sc[8 * m + 7]));
 #pragma unroll
-          for (int cb = 0; cb < CB; ++cb) {
-            const uint16_t* vrow = l2 + (cb * 32 + i) * TPB + 16 * m + 4 * hh;
-            acc[cb] = FM_MFMA_BF16(pp, as_bf8(*reinterpret_cast<const uint2*>(vrow),
-                                              *reinterpret_cast<const uint2*>(vrow + 8)), acc[cb]);
-          }
+          for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA_BF16(pp, as_bf8(vb[m][cb][0], vb[m][cb][1]), acc[cb]);
           if (FWD) accd = FM_MFMA_BF16(pp, ones, accd);
         }
       }

@@ -10,6 +10,7 @@
 // contraction (k=0/1 then stand for rows trow(r,0)/trow(r,1)); the kernels use that to chain
 // score tiles into value/gradient tiles without going through memory.
 #pragma once
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -174,30 +175,48 @@ struct RowTile {
   static constexpr int VPR = D / 4;
   static constexpr int TOTAL = ROWS * VPR;
   static constexpr int NV = (TOTAL + 255) / 256;
-  float v[NV][4];
+  // The pieces stay as loaded (and the divisors unread) until a store converts, masks and scales
+  // them: nothing in load() consumes what it fetches, and it has no branch, so the loads of a
+  // tile can stay in flight under whatever work separates load() from the store.  Rows >= n are
+  // fetched from row n-1 (a valid address) and zeroed by the store.
+  using Raw = typename std::conditional<std::is_same<T, float>::value, float4, uint2>::type;
+  Raw raw[NV];
+  float rdiv[NV];  // per-row divisors fetched by load(), applied by the stores
+  bool live[NV];
   __device__ __forceinline__ static int row_of(int idx) { return ROWFAST ? idx % ROWS : idx / VPR; }
   __device__ __forceinline__ static int c4_of(int idx) { return ROWFAST ? idx / ROWS : idx % VPR; }
-
-  float rdiv[NV];  // per-row divisors fetched by load(), applied by the stores
+  __device__ __forceinline__ static void unpack(const float4& r, float (&o)[4]) {
+    o[0] = r.x; o[1] = r.y; o[2] = r.z; o[3] = r.w;
+  }
+  __device__ __forceinline__ static void unpack(const uint2& r, float (&o)[4]) {
+    o[0] = __uint_as_float(r.x << 16);
+    o[1] = __uint_as_float(r.x & 0xffff0000u);
+    o[2] = __uint_as_float(r.y << 16);
+    o[3] = __uint_as_float(r.y & 0xffff0000u);
+  }
+  // piece u converted, times `scale` over the row's divisor; zero for a row past the end
+  __device__ __forceinline__ void piece(int u, float scale, float (&o)[4]) const {
+    const float sc = live[u] ? scale / rdiv[u] : 0.f;
+    unpack(raw[u], o);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = live[u] ? o[e] * sc : 0.f;
+  }
 
   // rows tok0.. of one head (base points at the head's first row); rows >= n read as zero.
-  // rowdiv, when given, makes the stores divide every row by rowdiv[tok * rowdiv_stride]; the
-  // division is deferred to the store so that no load has to be waited for here.
+  // rowdiv, when given, makes the stores divide every row by rowdiv[tok * rowdiv_stride].
   __device__ __forceinline__ void load(const T* base, int tok0, int n, int tid,
                                        const float* rowdiv = nullptr, int64_t rowdiv_stride = 0) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
-      const int row = row_of(idx), c4 = c4_of(idx);
+      const bool in = idx < TOTAL;
+      const int row = in ? row_of(idx) : 0, c4 = in ? c4_of(idx) : 0;
       const int tok = tok0 + row;
+      live[u] = in && tok < n;
+      const int tk = tok < n ? tok : n - 1;
+      raw[u] = *reinterpret_cast<const Raw*>(base + (int64_t)tk * D + c4 * 4);
       rdiv[u] = 1.0f;
-      if (idx < TOTAL && tok < n) {
-        load4(base + (int64_t)tok * D + c4 * 4, v[u]);
-        if (rowdiv) rdiv[u] = rowdiv[(int64_t)tok * rowdiv_stride];
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[u][e] = 0.f;
-      }
+      if (rowdiv) rdiv[u] = rowdiv[(int64_t)tk * rowdiv_stride];
     }
   }
   // dst is [ROWS][ld] floats in LDS, 16-byte aligned, ld a multiple of 4
@@ -207,9 +226,9 @@ struct RowTile {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
       if (idx < TOTAL) {
-        const float sc = scale / rdiv[u];
-        *reinterpret_cast<float4*>(dst + row * ld + c4 * 4) =
-            make_float4(v[u][0] * sc, v[u][1] * sc, v[u][2] * sc, v[u][3] * sc);
+        float x[4];
+        piece(u, scale, x);
+        *reinterpret_cast<float4*>(dst + row * ld + c4 * 4) = make_float4(x[0], x[1], x[2], x[3]);
       }
     }
   }
@@ -220,9 +239,10 @@ struct RowTile {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
       if (idx < TOTAL) {
-        const float sc = scale / rdiv[u];
+        float x[4];
+        piece(u, scale, x);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dst[row * ld + c4 * 4 + e] = v[u][e] * sc;
+        for (int e = 0; e < 4; ++e) dst[row * ld + c4 * 4 + e] = x[e];
       }
     }
   }
@@ -233,8 +253,9 @@ struct RowTile {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
       if (idx < TOTAL) {
-        const float sc = scale / rdiv[u];
-        const uint32_t p01 = pack_bf2(v[u][0] * sc, v[u][1] * sc), p23 = pack_bf2(v[u][2] * sc, v[u][3] * sc);
+        float x[4];
+        piece(u, scale, x);
+        const uint32_t p01 = pack_bf2(x[0], x[1]), p23 = pack_bf2(x[2], x[3]);
         dst[(c4 * 4 + 0) * ld + row] = (uint16_t)p01;
         dst[(c4 * 4 + 1) * ld + row] = (uint16_t)(p01 >> 16);
         dst[(c4 * 4 + 2) * ld + row] = (uint16_t)p23;
@@ -249,9 +270,9 @@ struct RowTile {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
       if (idx < TOTAL) {
-        const float sc = scale / rdiv[u];
-        *reinterpret_cast<uint2*>(dst + row * ld + c4 * 4) =
-            make_uint2(pack_bf2(v[u][0] * sc, v[u][1] * sc), pack_bf2(v[u][2] * sc, v[u][3] * sc));
+        float x[4];
+        piece(u, scale, x);
+        *reinterpret_cast<uint2*>(dst + row * ld + c4 * 4) = make_uint2(pack_bf2(x[0], x[1]), pack_bf2(x[2], x[3]));
       }
     }
   }
@@ -262,9 +283,10 @@ struct RowTile {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
       if (idx < TOTAL) {
-        const float sc = scale / rdiv[u];
+        float x[4];
+        piece(u, scale, x);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dst[(c4 * 4 + e) * ld + row] = v[u][e] * sc;
+        for (int e = 0; e < 4; ++e) dst[(c4 * 4 + e) * ld + row] = x[e];
       }
     }
   }
