@@ -33,6 +33,7 @@ WORKLOADS = {
     "headline-unmasked": dict(B=64, H=16, N=10000, D=64, mask=False, p=2, dtype="f32"),
     "headline-p1": dict(B=64, H=16, N=10000, D=64, mask=True, p=1, dtype="f32"),
     "headline-unmasked-p1": dict(B=64, H=16, N=10000, D=64, mask=False, p=1, dtype="f32"),
+    "headline-p1-bf16": dict(B=64, H=16, N=10000, D=64, mask=True, p=1, dtype="bf16"),
     "c1": dict(B=8, H=8, N=1024, D=32, mask=False, p=2, dtype="f32"),
     "c2": dict(B=64, H=8, N=1000, D=32, mask=True, p=2, dtype="f32"),
     "c4": dict(B=16, H=32, N=16384, D=64, mask=True, p=2, dtype="bf16"),

@@ -128,6 +128,36 @@ __device__ __forceinline__ void load_ch(const bf16_t* hp, int base, const Lane<b
   }
 }
 
+// A channel-major operand whose conversion is put off until ready(): with bf16 tensors the 16
+// loaded dwords stay as they are (half the registers of the 32 floats, and nothing consumes them
+// while they travel); with fp32 tensors the loads are the floats.
+template <class T>
+struct ChOperand;
+template <>
+struct ChOperand<float> {
+  float x[2][16] = {};
+  __device__ __forceinline__ void load(const float* hp, int base, const Lane<float>& L) { load_ch(hp, base, L, x); }
+  __device__ __forceinline__ void ready() {}
+};
+template <>
+struct ChOperand<bf16_t> {
+  float x[2][16] = {};
+  uint32_t raw[16] = {};
+  __device__ __forceinline__ void load(const bf16_t* hp, int base, const Lane<bf16_t>& L) {
+    const bf16_t* tp = hp + (int64_t)base * D;
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+      raw[t] = *reinterpret_cast<const uint32_t*>(tp + (L.ch + (8 * (t >> 2) + (t & 3)) * D));
+  }
+  __device__ __forceinline__ void ready() {
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      x[0][t] = bf_lo(raw[t]);
+      x[1][t] = bf_hi(raw[t]);
+    }
+  }
+};
+
 // x[c][t] -> row trow(t, hh) of the tile, columns chan(c, i), for the tile rows in [lo, hi)
 // (ALIGNED, bf16 only: the row pitch keeps the lane's channel pair 4-byte aligned)
 template <bool ALIGNED>
@@ -303,7 +333,8 @@ __global__ __launch_bounds__(64) void linear_fwd_kernel(const T* __restrict__ q,
   f16v S1[2][2];
   zero_state(S1);
   float s0[2] = {0.f, 0.f}, s1[2] = {0.f, 0.f};
-  float qt[32], kt[32], kc[2][16] = {}, vc[2][16] = {};   // (tile "-1" is empty)
+  float qt[32], kt[32];
+  ChOperand<T> kc, vc;   // (tile "-1" is empty)
   load_tok(kh, 0, L, kt);
   load_tok(qh, 0, L, qt);
 
@@ -314,18 +345,19 @@ __global__ __launch_bounds__(64) void linear_fwd_kernel(const T* __restrict__ q,
     const int nb = tt + 1 < ntiles ? fbase(tt + 1, n) : base;
 
     // the previous tile joins the state
-    state_update(S1, kc, vc);
+    kc.ready();
+    state_update(S1, kc.x, vc.x);
     {
       float ks[2], vs[2];
-      column_sums(kc, ks);
-      column_sums(vc, vs);
+      column_sums(kc.x, ks);
+      column_sums(vc.x, vs);
       s1[0] += ks[0]; s1[1] += ks[1];
       s0[0] += vs[0]; s0[1] += vs[1];
       vec_put<T>(s1l, L, s1[0], s1[1]);
     }
     FM_PIN();
-    load_ch(kh, base, L, kc);
-    load_ch(vh, base, L, vc);
+    kc.load(kh, base, L);
+    vc.load(vh, base, L);
     FM_PIN();
 
     // transposed score tile (rows = keys of the tile, columns = queries); own rows x state
@@ -351,7 +383,8 @@ __global__ __launch_bounds__(64) void linear_fwd_kernel(const T* __restrict__ q,
     const float den_i = a1s * (half_swap_add(dsum) + qs) + a0 * (float)(32 * tt);
 
     // intra-tile part: weights x values
-    weight_product(P, vc, O);
+    vc.ready();
+    weight_product(P, vc.x, O);
 
     // denominators move from "lane = token" to the row order of the output registers
     if (L.l < 32 && L.l >= skip) dh[(int64_t)(base + L.l) * den_stride] = den_i;
