@@ -269,19 +269,17 @@ constexpr bool kBf16Mfma = false;
 template <>
 constexpr bool kBf16Mfma<bf16_t> = true;
 
-// sections (bf16 inputs, masked): which packed layouts the consumers of this state read --
-// 1 = feature-packed (apply kernels), 2 = column-packed (grad kernels)
 template <int D, class T>
 int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float* xscale,
                  const float* yden, int64_t yden_stride, const float* ew, float* state, int reverse,
-                 int sections, hipStream_t stream, bool finish = true) {
+                 hipStream_t stream, bool finish = true) {
   const dim3 grid(pl.gsplit, heads, pl.nparts);
   if (pl.masked && pl.nslots < 2) return FASTMAX_OK;  // a single chunk never needs a state
   ScopedKernel sk(FASTMAX_K_BUILD, stream);
 #define FM_BUILD(RTW)                                                                            \
   build_kernel<D, T, RTW, kBf16Mfma<T>><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, yden_stride, ew, state, \
                                                     pl.n, pl.chunk, pl.nslots, pl.masked, reverse, \
-                                                    pl.p2, pl.zlen, sections)
+                                                    pl.p2, pl.zlen)
   if (pl.rtw == 1) {
     FM_BUILD(1);
   } else if constexpr (D == 64) {
@@ -353,7 +351,7 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
     // (bf16: a saved state is also read by the dq kernel, which needs the column-packed section)
     if constexpr (D == 64) {
       if (pl.rowpass) {
-        FM_TRY((launch_build<D, T>(pl, heads, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state, 0, 0,
+        FM_TRY((launch_build<D, T>(pl, heads, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state, 0,
                                    stream, false)));
         const int slot = finish_state_fp32(pl, heads, state, stream);
         ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
@@ -369,7 +367,7 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
       }
     }
     FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr,
-                               state, 0, saved ? 3 : 1, stream)));
+                               state, 0, stream)));
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       const dim3 agrid(pl.nblk, heads);
@@ -495,11 +493,11 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
         const int64_t ss = pl.state_floats, hf = (int64_t)pl.nslots * ss;
         int slot = pl.nparts > 1 ? pl.nparts : 0;
         if (!saved) {
-          FM_TRY((launch_build<D, T>(pl, heads, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state, 0, 0,
+          FM_TRY((launch_build<D, T>(pl, heads, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state, 0,
                                      stream, false)));
           slot = finish_state_fp32(pl, heads, state, stream);
         }
-        FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, 0, stream,
+        FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, stream,
                                    false)));
         finish_state_fp32(pl, heads, stR, stream);
         const int nrb = (n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE;
@@ -536,8 +534,8 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     // prefix state of (kh, v, 1) per key/value head and suffix state of (qh, go/den, c) per query head
     if (!saved)
       FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state,
-                                 0, 2, stream)));
-    FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, 3, stream)));
+                                 0, stream)));
+    FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, stream)));
     const dim3 grid(pl.nblk, heads);
     {
       ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
@@ -629,7 +627,7 @@ int state_update_impl(const fastmax_desc* ds, const Plan& pl, const T* k, const 
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
     const int64_t off = (int64_t)h0 * n * D;
-    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, kscale + h0, nullptr, 0, nullptr, slots, 0, 0, stream,
+    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, kscale + h0, nullptr, 0, nullptr, slots, 0, stream,
                                false)));
     state_accumulate_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads), 256, 0, stream>>>(
         state + (int64_t)h0 * ss, ss, slots, pl.nslots, pl.nparts, ss, accumulate);

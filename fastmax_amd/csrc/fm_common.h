@@ -89,6 +89,18 @@ __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) {
   return o;
 }
 
+// Transposing 64-bit LDS read of 16-bit elements (gfx950): in every group of 16 lanes, lane L
+// receives, for k = 0..3, element L % 4 of the 8-byte word whose address lane 4 k + L / 4 of the
+// group supplied.  So if the 16 lanes address a 4 x 4 arrangement of words, word (r, k) by lane
+// 4 k + r, lane L gets one element of each word of its row L / 4: a 4 x 4 transpose of 16-bit
+// elements between "four lanes x one word" and "one lane x four words".
+typedef short fm_v4s __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint2 lds_read_tr16(const uint16_t* p) {
+  const fm_v4s r = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) fm_v4s*)(const_cast<uint16_t*>(p)));
+  return __builtin_bit_cast(uint2, r);
+}
+
 // four consecutive elements <-> four floats
 __device__ __forceinline__ void load4(const float* p, float (&o)[4]) {
   const float4 t = *reinterpret_cast<const float4*>(p);
@@ -140,27 +152,25 @@ struct Geo {
   static constexpr int SLABF = (SLAB + 3) / 4 * 4;
 };
 
-// Packed bf16 form of a state, used when the inputs are bf16 (it occupies the same
-// state_floats slot as the fp32 form).  A "slab" is the D feature rows of one shift s
-// (order 2; rows carry their pair weight: x2 for 0 < s < D/2) or the D order-1 rows (slab
-// NS, or slab 0 when p == 1).  Each slab is stored twice, in the two operand layouts of the
-// bf16 matrix instruction, so that consumers stage it with plain 16-byte copies:
-//   F, feature-packed  [a/4][column 0..D (+1 pad)][a%4]   contraction over features (apply)
-//   C, column-packed   [a][LB = D+4]                        contraction over columns (grad);
-//      columns D..D+3 hold the extra column as (hi, hi, lo, lo) bf16 pairs
-// followed by the order-0 row as D+1 floats.  Column D is the extra (denominator) column.
+// Packed bf16 form of a state, used when the inputs are bf16 (it occupies the front of the same
+// state_floats slot as the fp32 form).  A "slab" is the D feature rows of one shift s (order 2;
+// rows carry their pair weight: x2 for 0 < s < D/2) or the D order-1 rows (slab NS, or slab 0
+// when p == 1), stored feature-packed,
+//   [a/4][column 0..D+3][a%4]
+// i.e. 8-byte words of four consecutive rows, which is the B operand layout of the bf16 matrix
+// instruction for a contraction over features (apply kernels: plain 64-bit LDS reads); for a
+// contraction over columns (grad kernels) the same words are read through the transposing LDS
+// load (lds_read_tr16).  Consumers stage a slab with plain 16-byte copies.  Columns D..D+3 hold
+// the extra (denominator) column split into hi + lo bf16 parts as (hi, hi, lo, lo), because in the
+// grad kernels that term nearly cancels the value columns' sum.  The slabs are followed by the
+// order-0 row as D+1 floats.
 template <int D>
 struct PackedGeo {
   using G = Geo<D>;
-  static constexpr int NCF = D + 2;
-  static constexpr int FSL = (D / 4) * NCF * 4;  // bf16 elements of an F slab (a multiple of 128)
-  static constexpr int LB = D + 4;
-  static constexpr int CSL = D * LB;             // bf16 elements of a C slab (a multiple of 128)
+  static constexpr int NCF = D + 4;
+  static constexpr int FSL = (D / 4) * NCF * 4;  // bf16 elements of a slab (a multiple of 128)
   __host__ __device__ static constexpr int nslab(int p2) { return (p2 ? G::NS : 0) + 1; }
-  __host__ __device__ static constexpr int64_t c_off(int p2) { return ((int64_t)nslab(p2) * FSL * 2 + 255) / 256 * 256; }
-  __host__ __device__ static constexpr int64_t z_off(int p2) {
-    return c_off(p2) + ((int64_t)nslab(p2) * CSL * 2 + 255) / 256 * 256;
-  }
+  __host__ __device__ static constexpr int64_t z_off(int p2) { return ((int64_t)nslab(p2) * FSL * 2 + 255) / 256 * 256; }
   __host__ __device__ static constexpr int64_t bytes(int p2) { return z_off(p2) + (D + 1) * 4; }
   static_assert(bytes(1) <= G::state_floats(1) * 4 && bytes(0) <= G::state_floats(0) * 4,
                 "the packed form must fit the fp32 state slot");

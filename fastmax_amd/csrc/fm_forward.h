@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     const T* __restrict__ X, const T* __restrict__ Y, const float* __restrict__ xscale,
     const float* __restrict__ yden, int64_t yden_stride, const float* __restrict__ ew,
     float* __restrict__ state, int n, int chunk, int nslots, int masked, int reverse, int p2,
-    int zlen, int sections) {
+    int zlen) {
   using G = Geo<D>;
   constexpr int TS = 32;  // tokens per pipeline step (64 for bf16 halves the barriers but does not fit the
                         // register file next to three row tiles of accumulators)
@@ -324,20 +324,18 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     if (g == 0 && tid <= D) st[(unsigned)((rows2 + D) * LD + tid)] = s0;
   };
 
-  // BF, masked: the snapshot goes out in the packed bf16 form (PackedGeo): section F when
-  // sections & 1, section C when sections & 2, and the fp32 order-0 row.
+  // BF, masked: the snapshot goes out in the packed bf16 form (PackedGeo) with the fp32 order-0 row.
   auto snapshot_packed = [&](int slot) {
     using PG = PackedGeo<D>;
     char* sb = reinterpret_cast<char*>(state + ((int64_t)head * nslots + slot) * SS);  // uniform
     uint16_t* fsec = reinterpret_cast<uint16_t*>(sb);
-    uint16_t* csec = reinterpret_cast<uint16_t*>(sb + PG::c_off(p2));
 #pragma unroll
     for (int x = 0; x < RTW; ++x) {
       if (x < nx) {
         const int slab = rowbase[x] / D, arow = rowbase[x] % D;
         const bool dbl = rowbase[x] < rows2 && slab != 0 && slab != G::H2;  // pair weight 2
         const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
-        if (sections & 1) {
+        {
           const float wgt = dbl ? 2.0f : 1.0f;
           uint16_t* fx = fsec + (unsigned)(slab * PG::FSL + (arow >> 2) * PG::NCF * 4);
           const unsigned lo = (unsigned)((hh * PG::NCF + cbase * 32 + i) * 4);
@@ -349,25 +347,11 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
               *reinterpret_cast<uint2*>(fx + lo + (unsigned)((2 * j * PG::NCF + cb * 32) * 4)) =
                   make_uint2(pack_bf2(a[4 * j] * wgt, a[4 * j + 1] * wgt), pack_bf2(a[4 * j + 2] * wgt, a[4 * j + 3] * wgt));
             }
-          if (hh == 0 && cbase == 0) fx[(unsigned)(((i >> 2) * PG::NCF + D) * 4 + (i & 3))] = (uint16_t)pack_bf2(ds * wgt, 0.f);
-        }
-        if (sections & 2) {
-          uint16_t* cx = csec + (unsigned)(slab * PG::CSL + arow * PG::LB);
-          const unsigned lo = (unsigned)(4 * hh * PG::LB + cbase * 32 + i);
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; e += 2)
-#pragma unroll
-              for (int cb = 0; cb < CB; ++cb) {
-                const uint32_t u = pack_bf2(acc[x][cb][4 * j + e], acc[x][cb][4 * j + e + 1]);
-                cx[lo + (unsigned)((8 * j + e) * PG::LB + cb * 32)] = (uint16_t)u;
-                cx[lo + (unsigned)((8 * j + e + 1) * PG::LB + cb * 32)] = (uint16_t)(u >> 16);
-              }
-          if (hh == 0 && cbase == 0) {
-            const float ehi = bf_lo(pack_bf2(ds, 0.f));
-            *reinterpret_cast<uint2*>(cx + (unsigned)(i * PG::LB + D)) =
-                make_uint2(pack_bf2(ehi, ehi), pack_bf2(ds - ehi, ds - ehi));
+          if (hh == 0 && cbase == 0) {   // the extra column, split into hi + lo parts: columns D..D+3 = (hi, hi, lo, lo)
+            const float ew = ds * wgt, ehi = bf_lo(pack_bf2(ew, 0.f));
+            const uint16_t h16 = (uint16_t)pack_bf2(ehi, 0.f), l16 = (uint16_t)pack_bf2(ew - ehi, 0.f);
+            uint16_t* ex = fx + (unsigned)(((i >> 2) * PG::NCF + D) * 4 + (i & 3));
+            ex[0] = h16; ex[4] = h16; ex[8] = l16; ex[12] = l16;
           }
         }
       }
@@ -477,22 +461,21 @@ __global__ __launch_bounds__(256) void state_pack_kernel(float* __restrict__ sta
   __syncthreads();
   char* sb = reinterpret_cast<char*>(state + ((int64_t)head * nslots + nslots - 1) * SS);
   uint16_t* fsec = reinterpret_cast<uint16_t*>(sb) + slab * PG::FSL;
-  uint16_t* csec = reinterpret_cast<uint16_t*>(sb + PG::c_off(p2)) + slab * PG::CSL;
   const float wgt = (!ord1 && slab != 0 && slab != G::H2) ? 2.0f : 1.0f;
   for (int idx = tid; idx < (D / 4) * (D + 1); idx += 256) {
     const int tg = idx / (D + 1), col = idx % (D + 1);
     const float* f = Sl + 4 * tg * LD + col;
-    *reinterpret_cast<uint2*>(fsec + (tg * PG::NCF + col) * 4) =
-        make_uint2(pack_bf2(f[0] * wgt, f[LD] * wgt), pack_bf2(f[2 * LD] * wgt, f[3 * LD] * wgt));
-  }
-  for (int idx = tid; idx < D * (D / 4); idx += 256) {
-    const int a = idx / (D / 4), c4 = (idx % (D / 4)) * 4;
-    const float4 t = *reinterpret_cast<const float4*>(Sl + a * LD + c4);
-    *reinterpret_cast<uint2*>(csec + a * PG::LB + c4) = make_uint2(pack_bf2(t.x, t.y), pack_bf2(t.z, t.w));
-  }
-  if (tid < D) {
-    const float e = Sl[tid * LD + D], ehi = bf_lo(pack_bf2(e, 0.f));
-    *reinterpret_cast<uint2*>(csec + tid * PG::LB + D) = make_uint2(pack_bf2(ehi, ehi), pack_bf2(e - ehi, e - ehi));
+    const float f0 = f[0] * wgt, f1 = f[LD] * wgt, f2 = f[2 * LD] * wgt, f3 = f[3 * LD] * wgt;
+    uint2* dst = reinterpret_cast<uint2*>(fsec + (tg * PG::NCF + col) * 4);
+    if (col < D) {
+      *dst = make_uint2(pack_bf2(f0, f1), pack_bf2(f2, f3));
+    } else {   // the extra column, split into hi + lo parts: columns D..D+3 = (hi, hi, lo, lo)
+      const float h0 = bf_lo(pack_bf2(f0, 0.f)), h1 = bf_lo(pack_bf2(f1, 0.f));
+      const float h2 = bf_lo(pack_bf2(f2, 0.f)), h3 = bf_lo(pack_bf2(f3, 0.f));
+      const uint2 hi = make_uint2(pack_bf2(h0, h1), pack_bf2(h2, h3));
+      const uint2 lo = make_uint2(pack_bf2(f0 - h0, f1 - h1), pack_bf2(f2 - h2, f3 - h3));
+      dst[0] = hi; dst[1] = hi; dst[2] = lo; dst[3] = lo;
+    }
   }
   if (ord1 && tid <= D) reinterpret_cast<float*>(sb + PG::z_off(p2))[tid] = Sl[D * LD + tid];
 }

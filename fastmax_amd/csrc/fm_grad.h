@@ -299,11 +299,14 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 // ---------------------------------------------------------------------------------------
 // bf16 variant of grad_kernel (bf16 inputs and outputs): every contraction runs on
 // v_mfma_f32_32x32x16_bf16 with fp32 accumulation.  The state arrives in the packed bf16 form
-// (PackedGeo): a column-packed slab ([row][column], unweighted, extra column split into hi + lo
-// parts) is copied to LDS as it is; 2*a2 multiplies the accumulated order-2 credits and a1 the
-// order-1 tile.  The token's extended value vector is packed once, so a 32-row tile costs
-// D/8 + 1 MFMAs; the credits are the fp32 register/LDS work of the fp32 kernel.  Streamed tiles are staged as bf16, the first
-// one in both orientations (rows for the scores, transposed for the product with W).
+// (PackedGeo): a feature-packed slab ([row / 4][column][row % 4], rows carrying their pair weights,
+// extra column split into hi + lo parts) is copied to LDS as it is and read through the
+// transposing LDS load, which hands every lane = row four consecutive columns per 64-bit piece;
+// the two slabs of pair weight 1 are doubled after their contraction, a2 multiplies the
+// accumulated order-2 credits and a1 the order-1 tile.  The token's extended value vector is
+// packed once, so a 32-row tile costs D/8 + 1 MFMAs; the credits are the fp32 register/LDS work
+// of the fp32 kernel.  Streamed tiles are staged as bf16, the first one in both orientations
+// (rows for the scores, transposed for the product with W).
 // ---------------------------------------------------------------------------------------
 template <int D, int MODE>
 __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
@@ -385,20 +388,21 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   }
   // packed state of this block's chunk (masked) or the head's summed state (last slot)
   using PG = PackedGeo<D>;
-  static_assert(PG::LB == LB && PG::CSL == D * LB, "stage layout = column-packed slab layout");
+  constexpr int NCF = PG::NCF;
+  static_assert(PG::FSL <= SLB, "a feature-packed slab must fit a stage buffer");
   const char* sbase = reinterpret_cast<const char*>(state + ((int64_t)ha * nslots + (masked ? c : nslots - 1)) * SS);
-  const uint16_t* csec = reinterpret_cast<const uint16_t*>(sbase + PG::c_off(p2));
+  const uint16_t* fsec = reinterpret_cast<const uint16_t*>(sbase);
 
   // a C slab is copied as it is: 16-byte pieces global -> registers -> LDS
   // (no branches: threads past the end wrap round and copy an early piece a second time, so that
   // every load is issued up front and stays in flight under the MFMAs)
-  constexpr int NPC = PG::CSL / 8, NVS = (NPC + 255) / 256;
+  constexpr int NPC = PG::FSL / 8, NVS = (NPC + 255) / 256;
   static_assert(NVS <= 3, "three named pieces per thread (an indexed array would live in scratch)");
   uint4 sv0, sv1, sv2;
   RowTile<D, T, 32> t1, t2;
   float creg = 0.f;
   auto slab_load = [&](int st) {
-    const uint4* src = reinterpret_cast<const uint4*>(csec + st * PG::CSL);
+    const uint4* src = reinterpret_cast<const uint4*>(fsec + st * PG::FSL);
     sv0 = src[tid % NPC];
     if constexpr (NVS > 1) sv1 = src[(tid + 256) % NPC];
     if constexpr (NVS > 2) sv2 = src[(tid + 512) % NPC];
@@ -437,12 +441,18 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   }
   __syncthreads();
 
+  // The slab is feature-packed, [row / 4][column][row % 4]; the B operand of the contraction over
+  // columns wants, per lane = row, four consecutive columns per 64-bit piece: the transposing LDS
+  // read delivers exactly that when, in every group of 16 lanes (16 consecutive rows), lane J
+  // addresses the word of row group J % 4 and column J / 4 of the piece.
+  const int trj = l & 15;
+  const int troff = (((i >> 4) * 4 + (trj & 3)) * NCF + (trj >> 2)) * 4;   // + (ab * 8 * NCF + column) * 4
   auto chain = [&](const uint16_t* sl, int ab) {
-    const uint16_t* ar = sl + (ab * 32 + i) * LB;
+    const uint16_t* ar = sl + ab * 8 * NCF * 4 + troff;
     uint2 b[H2 / 4 + 1];
 #pragma unroll
-    for (int g4 = 0; g4 < H2 / 4; ++g4) b[g4] = *reinterpret_cast<const uint2*>(ar + hh * H2 + 4 * g4);
-    b[H2 / 4] = *reinterpret_cast<const uint2*>(ar + D);  // extra column and its zero padding
+    for (int g4 = 0; g4 < H2 / 4; ++g4) b[g4] = lds_read_tr16(ar + (hh * H2 + 4 * g4) * 4);
+    b[H2 / 4] = lds_read_tr16(ar + D * 4);  // extra column as (hi, hi, lo, lo)
     f16v t;
 #pragma unroll
     for (int r = 0; r < 16; ++r) t[r] = 0.f;
@@ -467,6 +477,14 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     for (int ab = 0; ab < AB; ++ab) tt[ab] = chain(sl, ab);
     if (p2 && st < NS) {
       const int s = st;
+      // the order-2 slabs carry their pair weights (2, except shifts 0 and D/2): bring those two up
+      // to the others, the common factor goes into the final scale
+      if (s == 0 || s == H2) {
+#pragma unroll
+        for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tt[ab][r] *= 2.0f;
+      }
 #pragma unroll
       for (int ab = 0; ab < AB; ++ab) {
         const int rc = (ab * 32 + i + s) & (D - 1);
@@ -488,11 +506,11 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
             out[ab][r] += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, v)));
           }
       }
-      if (st == NS - 1) {  // the order-2 slabs are stored raw: f'(s) contributes 2*a2 to their sum
+      if (st == NS - 1) {  // f'(s) contributes 2*a2 to the order-2 sum, the pair weight 2 is already in
 #pragma unroll
         for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) out[ab][r] *= 2.0f * a2;
+          for (int r = 0; r < 16; ++r) out[ab][r] *= a2;
       }
     } else {
 #pragma unroll
