@@ -220,7 +220,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     float4 own[RTW], rot[RTW], vv[BF ? 1 : CB], e4;
     uint2 vb[BF ? CB : 1];
   };
-  auto fetch = [&](const float* kb, int buf, const float* eb, int grp, GroupOps& g4) {
+  auto fetch = [&](const float* kb, int buf, const float* eb, int grp, GroupOps& g4) __attribute__((always_inline)) {
     const int go8 = 8 * grp;
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
@@ -234,7 +234,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       g4.rot[x] = *reinterpret_cast<const float4*>(kb + rotoff[x] + go8);
     }
   };
-  auto compute = [&](int buf, int h) {
+  auto compute = [&](int buf, int h) __attribute__((always_inline)) {
     const float* kb = Kt[buf];
     const float* eb = El[buf];
     GroupOps cur, nxt;
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     }
   };
   // order-0 sums of the staged step
-  auto sum0 = [&](int buf) {
+  auto sum0 = [&](int buf) __attribute__((always_inline)) {
     const float* eb = El[buf];
     if (g == 0 && tid <= D) {
       if (BF && tid < D) {
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   };
   // lane part of a snapshot address: row 4*hh (+ 8j + e per register), column i (+ 32*cb)
   const unsigned lane_off = (unsigned)(4 * hh * LD + cbase * 32 + i);
-  auto snapshot = [&](int slot) {
+  auto snapshot = [&](int slot) __attribute__((always_inline)) {
     float* st = state + ((int64_t)head * nslots + slot) * SS;  // uniform: scalar base + 32-bit lane offsets
 #pragma unroll
     for (int x = 0; x < RTW; ++x) {
@@ -325,7 +325,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   };
 
   // BF, masked: the snapshot goes out in the packed bf16 form (PackedGeo) with the fp32 order-0 row.
-  auto snapshot_packed = [&](int slot) {
+  auto snapshot_packed = [&](int slot) __attribute__((always_inline)) {
     using PG = PackedGeo<D>;
     char* sb = reinterpret_cast<char*>(state + ((int64_t)head * nslots + slot) * SS);  // uniform
     uint16_t* fsec = reinterpret_cast<uint16_t*>(sb);
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     }
     if (g == 0 && tid <= D) reinterpret_cast<float*>(sb + PG::z_off(p2))[tid] = s0;
   };
-  auto emit = [&](int slot) {
+  auto emit = [&](int slot) __attribute__((always_inline)) {
     if constexpr (BF) {
       if (masked) {
         snapshot_packed(slot);
@@ -407,29 +407,77 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     return (q + 1) % spc == 0 ? nc - 3 - q / spc : -1;
   };
 
-  if (nsteps > 0) {
-#pragma unroll
-    for (int h = 0; h < NH; ++h) {
-      load(step_tok(0) + 32 * h, tend);
-      store(0, h, step_tok(0) + 32 * h, tend);
+  if constexpr (BF) {
+    // bf16: the tiles are requested two steps before they are staged (two sets of registers that
+    // take turns; the requests are unconditional, the last ones repeat the last step and are not
+    // used), so that a step's global latency and the drain of a snapshot's stores -- which the
+    // same in-order counter makes later loads wait for -- are spread over two steps of work.
+    static_assert(NH == 1, "one 32-token half per step");
+    std::conditional_t<BF, RawTileBf<D, 32>, RowTile<D, T, 32, true>> kx2, vy2;
+    float ereg2 = 0.f;
+    auto load_into = [&](auto& k_, auto& v_, float& e_, int t0) __attribute__((always_inline)) {
+      k_.load(Xh, t0, tend, tid);
+      v_.load(Yh, t0, tend, tid, ydh, yden_stride);
+      if (tid < 32) {
+        const int tok = t0 + tid;
+        e_ = (tok < tend) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
+      }
+    };
+    auto store_from = [&](auto& k_, auto& v_, float e_, int buf, int t0) __attribute__((always_inline)) {
+      k_.store_t(Kt[buf], TP, xs, tid);
+      v_.store_t_bf(Vtb[buf], TPB, 1.0f, tid, ydh == nullptr);
+      if (tid < 32) {
+        El[buf][tid] = e_;
+        Kt[buf][D * TP + tid] = (t0 + tid < tend) ? 1.0f : 0.f;
+      }
+    };
+    auto step = [&](int p, auto& lk, auto& lv, float& le, auto& sk, auto& sv, float se) __attribute__((always_inline)) {
+      __builtin_amdgcn_sched_barrier(0);
+      const int pl2 = p + 2 < nsteps ? p + 2 : nsteps - 1;
+      load_into(lk, lv, le, step_tok(pl2));
+      compute(p & 1, 0);
+      sum0(p & 1);
+      if (p + 1 < nsteps) store_from(sk, sv, se, (p + 1) & 1, step_tok(p + 1));
+      const int slot = step_slot(p);
+      if (slot >= 0) emit(slot);
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    if (nsteps > 0) {
+      load_into(kx, vy, ereg, step_tok(0));
+      store_from(kx, vy, ereg, 0, step_tok(0));
+      load_into(kx2, vy2, ereg2, step_tok(nsteps > 1 ? 1 : 0));
     }
-  }
-  __syncthreads();
-  for (int p = 0; p < nsteps; ++p) {
-    const bool more = p + 1 < nsteps;
-    const int tnext = step_tok(more ? p + 1 : p);
-#pragma unroll
-    for (int h = 0; h < NH; ++h) {
-      if (more) load(tnext + 32 * h, tend);
-      compute(p & 1, h);
-      if (h == NH - 1) sum0(p & 1);
-      if (more) store((p + 1) & 1, h, tnext + 32 * h, tend);
-    }
-    // after the staged tile has been consumed: waiting for loads while stores are pending
-    // would wait for the stores too (one in-order counter covers both)
-    const int slot = step_slot(p);
-    if (slot >= 0) emit(slot);
     __syncthreads();
+    for (int p = 0; p < nsteps; p += 2) {
+      step(p, kx, vy, ereg, kx2, vy2, ereg2);
+      if (p + 1 < nsteps) step(p + 1, kx2, vy2, ereg2, kx, vy, ereg);
+    }
+  } else {
+    if (nsteps > 0) {
+  #pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        load(step_tok(0) + 32 * h, tend);
+        store(0, h, step_tok(0) + 32 * h, tend);
+      }
+    }
+    __syncthreads();
+    for (int p = 0; p < nsteps; ++p) {
+      const bool more = p + 1 < nsteps;
+      const int tnext = step_tok(more ? p + 1 : p);
+  #pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        if (more) load(tnext + 32 * h, tend);
+        compute(p & 1, h);
+        if (h == NH - 1) sum0(p & 1);
+        if (more) store((p + 1) & 1, h, tnext + 32 * h, tend);
+      }
+      // after the staged tile has been consumed: waiting for loads while stores are pending
+      // would wait for the stores too (one in-order counter covers both)
+      const int slot = step_slot(p);
+      if (slot >= 0) emit(slot);
+      __syncthreads();
+    }
   }
   if (!masked && nsteps == 0) emit(zsplit);  // an empty token split still owns its slot
 }
