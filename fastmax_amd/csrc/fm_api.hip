@@ -88,6 +88,11 @@ struct Plan {
 int64_t state_floats_for(int d, int p2) {
   return d == 64 ? Geo<64>::state_floats(p2) : Geo<32>::state_floats(p2);
 }
+// floats per state slot of a pass: causal bf16 passes keep packed states only
+int64_t slot_floats_for(int d, int p2, bool packed) {
+  if (!packed) return state_floats_for(d, p2);
+  return d == 64 ? PackedGeo<64>::slot_floats(p2) : PackedGeo<32>::slot_floats(p2);
+}
 
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
@@ -142,7 +147,7 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
     // inputs in packed form), or the only partial state itself
     pl.nslots = pl.nparts + ((ds->dtype == FASTMAX_BF16 || pl.nparts > 1) ? 1 : 0);
   }
-  pl.state_floats = state_floats_for(pl.d, pl.p2);
+  pl.state_floats = slot_floats_for(pl.d, pl.p2, pl.masked && ds->dtype == FASTMAX_BF16);
   size_t fixed = align256((size_t)2 * pl.bh * sizeof(float)) + align256((size_t)2 * pl.bh * sizeof(int));
   if (pass == FASTMAX_PASS_BACKWARD) {
     fixed += align256((size_t)pl.bh * pl.n * sizeof(float));            // c_i

@@ -380,7 +380,7 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
-  const int64_t SS = G::state_floats(p2);
+  const int64_t SS = masked ? PackedGeo<D>::slot_floats(p2) : G::state_floats(p2);   // slot pitch
   // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
   // and the state to head ha = head / adiv (one of the divisors is 1)
   const int hx = head / xdiv, ha = head / adiv;

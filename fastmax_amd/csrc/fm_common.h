@@ -172,6 +172,9 @@ struct PackedGeo {
   __host__ __device__ static constexpr int nslab(int p2) { return (p2 ? G::NS : 0) + 1; }
   __host__ __device__ static constexpr int64_t z_off(int p2) { return ((int64_t)nslab(p2) * FSL * 2 + 255) / 256 * 256; }
   __host__ __device__ static constexpr int64_t bytes(int p2) { return z_off(p2) + (D + 1) * 4; }
+  // floats between the packed states of consecutive slots (causal scans only: an unmasked state
+  // sits in the last of the fp32 slots its partial sums were built in)
+  __host__ __device__ static constexpr int64_t slot_floats(int p2) { return (bytes(p2) + 255) / 256 * 64; }
   static_assert(bytes(1) <= G::state_floats(1) * 4 && bytes(0) <= G::state_floats(0) * 4,
                 "the packed form must fit the fp32 state slot");
 };

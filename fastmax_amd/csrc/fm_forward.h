@@ -143,7 +143,8 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   const int g = lid % gridDim.x, head = (lid / gridDim.x) % gridDim.y, zsplit = lid / (gridDim.x * gridDim.y);
   const int rows2 = G::rows2(p2);
   const int rt2 = p2 ? G::NS * G::AB : 0, rt_total = rt2 + G::AB;
-  const int64_t SS = G::state_floats(p2);
+  // slot pitch: causal bf16 scans write packed states only, which are about half the fp32 size
+  const int64_t SS = (BF && masked) ? PackedGeo<D>::slot_floats(p2) : G::state_floats(p2);
 
   // per owned row tile: LDS offsets of the lane's own channel row and of its rotated partner
   int ownoff[RTW], rotoff[RTW], rowbase[RTW];
