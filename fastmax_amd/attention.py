@@ -33,10 +33,13 @@ SAVE_STATES_MEMORY_FRACTION = 0.25
 
 def _states_fit(k3: torch.Tensor, mask: bool) -> bool:
     """True when the prefix states of this call (one 592 KB state per key/value head per 384
-    tokens at d = 64, p = 2) take less than SAVE_STATES_MEMORY_FRACTION of the free memory."""
+    tokens at d = 64, p = 2; half of that for causal bf16 passes, whose states are kept packed)
+    take less than SAVE_STATES_MEMORY_FRACTION of the free memory."""
     heads, n, d = k3.shape
     rows = (d // 2 + 1) * d + d + 1
     state_bytes = rows * (d + 4) * 4 + 256
+    if mask and k3.dtype == torch.bfloat16:
+        state_bytes = state_bytes // 2 + 512
     slots = (n + 127) // 128 if mask else 8  # upper bounds: the chunk is at least 128 tokens
     free, _ = torch.cuda.mem_get_info(k3.device)
     return heads * slots * state_bytes <= SAVE_STATES_MEMORY_FRACTION * free
