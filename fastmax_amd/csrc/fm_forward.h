@@ -9,17 +9,40 @@
 // Per-head normaliser: scale[h] = lim / max_i ||x_i||_2 and the row that attains the max
 // (first one on ties).  Replaces calc_norms / find_max of the reference
 // (fastmax_cuda_forward.cu:223-253) with the PyTorch path's definition (example.py:105-108).
-// One block of NT threads per head; d/4 threads share a row.  (NT = 1024 when there are too few
+// One block of NT threads per head; a row is shared by d/4 (fp32) or d/8 (bf16) threads, 16 bytes each.  (NT = 1024 when there are too few
 // heads to fill the chip with 256-thread blocks: four times the loads in flight per head.)
 // ---------------------------------------------------------------------------------------
+// a thread's piece of a row: 16 bytes = 4 fp32 or 8 bf16 elements
+template <class T>
+struct RowPiece;
+template <>
+struct RowPiece<float> {
+  static constexpr int N = 4;
+  __device__ __forceinline__ static float sumsq(const float* p) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    return t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w;
+  }
+};
+template <>
+struct RowPiece<bf16_t> {
+  static constexpr int N = 8;
+  __device__ __forceinline__ static float sumsq(const bf16_t* p) {
+    const uint4 t = *reinterpret_cast<const uint4*>(p);
+    const float a0 = bf_lo(t.x), a1 = bf_hi(t.x), a2 = bf_lo(t.y), a3 = bf_hi(t.y);
+    const float a4 = bf_lo(t.z), a5 = bf_hi(t.z), a6 = bf_lo(t.w), a7 = bf_hi(t.w);
+    return (a0 * a0 + a1 * a1 + a2 * a2 + a3 * a3) + (a4 * a4 + a5 * a5 + a6 * a6 + a7 * a7);
+  }
+};
+
 template <class T, int NT>
 __global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, int n, int d,
                                                      float lim, float* __restrict__ scale_out,
                                                      int* __restrict__ arg_out) {
   __shared__ float sbest[NT];
   __shared__ int sarg[NT];
+  constexpr int EPT = RowPiece<T>::N;
   const int tid = threadIdx.x;
-  const int tpr = d >> 2, rpp = NT / tpr;
+  const int tpr = d / EPT, rpp = NT / tpr;
   const int sub = tid % tpr, rowi = tid / tpr;
   const T* base = x + (int64_t)blockIdx.x * n * d;
   float best = -1.f;
@@ -27,17 +50,17 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, in
   // four row groups per trip, loaded before any of them is reduced (rows past the end are
   // clamped to the last row: a duplicate cannot change the maximum or its first index)
   for (int i0 = 0; i0 < n; i0 += 4 * rpp) {
-    float v[4][4];
+    float ssq[4];
     int idx[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int i = i0 + u * rpp + rowi;
       idx[u] = i < n ? i : n - 1;
-      load4(base + (int64_t)idx[u] * d + sub * 4, v[u]);
+      ssq[u] = RowPiece<T>::sumsq(base + (int64_t)idx[u] * d + sub * EPT);
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      float ss = v[u][0] * v[u][0] + v[u][1] * v[u][1] + v[u][2] * v[u][2] + v[u][3] * v[u][3];
+      float ss = ssq[u];
       for (int off = tpr >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
       if (ss > best || (ss == best && idx[u] < bi)) {
         best = ss;
