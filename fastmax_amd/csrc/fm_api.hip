@@ -393,6 +393,22 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   return FASTMAX_OK;
 }
 
+// c_i = go_i . o_i / den_i for every token: 16-byte accesses when the rows of o allow it
+template <int D, class T>
+int launch_bwd_prep(const T* go, const T* o, int64_t ldo, const float* den, int64_t den_stride, float* cvec,
+                    int64_t rows, hipStream_t stream) {
+  ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
+  const bool vec = (ldo * sizeof(T)) % 16 == 0 && ((uintptr_t)o & 15) == 0 && ((uintptr_t)go & 15) == 0;
+  if (vec) {
+    const int rpp = 256 / (D * (int)sizeof(T) / 16);
+    bwd_prep_kernel<T, true><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
+  } else {
+    const int rpp = 256 / (D / 4);
+    bwd_prep_kernel<T, false><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
+  }
+  return launch_status("bwd_prep_kernel");
+}
+
 template <int D, class T>
 int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k, const T* v,
                   const T* o, int64_t ldo, const float* den, int64_t den_stride, const T* go, T* dq,
@@ -425,11 +441,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       // separate pass does
       const bool prep_in_dq = ldo == D;
       if (!prep_in_dq) {
-        const int64_t rows = (int64_t)bh * n;
-        const int rpp = 256 / (D / 4);
-        ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
-        bwd_prep_kernel<T><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
-        FM_TRY(launch_status("bwd_prep_kernel"));
+        FM_TRY((launch_bwd_prep<D, T>(go, o, ldo, den, den_stride, cvec, (int64_t)bh * n, stream)));
       }
       {
         ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
@@ -464,11 +476,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
     }
   }
   {
-    const int64_t rows = (int64_t)bh * n;
-    const int rpp = 256 / (D / 4);
-    ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
-    bwd_prep_kernel<T><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
-    FM_TRY(launch_status("bwd_prep_kernel"));
+    FM_TRY((launch_bwd_prep<D, T>(go, o, ldo, den, den_stride, cvec, (int64_t)bh * n, stream)));
   }
   const float a2 = pl.p2 ? ds->a2 : 0.f;
   const int ratio = pl.ratio, bhkv = pl.bhkv;

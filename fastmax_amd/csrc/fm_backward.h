@@ -1,25 +1,41 @@
 // Small backward-side kernels: the per-token scalar c_i and the normalisation chain rule.
 #pragma once
+#include <type_traits>
+
 #include "fm_common.h"
 
-// c_i = (go_i . o_i) / den_i, one value per token.  d/4 threads share a row.
-template <class T>
+// c_i = (go_i . o_i) / den_i, one value per token.  A row is shared by d/4 threads, or, VEC, by
+// d/8 threads for bf16 rows: 16 bytes per thread and tensor (VEC needs rows of o that start on a
+// 16-byte boundary; otherwise o is read element by element, e.g. from the (d+1)-column layout).
+template <class T, bool VEC>
 __global__ __launch_bounds__(256) void bwd_prep_kernel(const T* __restrict__ go,
                                                        const T* __restrict__ o, int64_t ldo,
                                                        const float* __restrict__ den,
                                                        int64_t den_stride, float* __restrict__ cvec,
                                                        int64_t rows, int d) {
-  const int tpr = d >> 2, rpp = 256 / tpr;
+  constexpr int EPT = VEC ? (std::is_same<T, float>::value ? 4 : 8) : 4;
+  const int tpr = d / EPT, rpp = 256 / tpr;
   const int sub = threadIdx.x % tpr;
   const int64_t row = (int64_t)blockIdx.x * rpp + threadIdx.x / tpr;
   float s = 0.f;
   if (row < rows) {
-    float a[4], b[4];
-    load4(go + row * d + sub * 4, a);
-    const T* orow = o + row * ldo + sub * 4;
+    const T* grow = go + row * d + sub * EPT;
+    const T* orow = o + row * ldo + sub * EPT;
+    if constexpr (VEC && !std::is_same<T, float>::value) {
+      const uint4 a = *reinterpret_cast<const uint4*>(grow), b = *reinterpret_cast<const uint4*>(orow);
+      s = (bf_lo(a.x) * bf_lo(b.x) + bf_hi(a.x) * bf_hi(b.x) + bf_lo(a.y) * bf_lo(b.y) + bf_hi(a.y) * bf_hi(b.y)) +
+          (bf_lo(a.z) * bf_lo(b.z) + bf_hi(a.z) * bf_hi(b.z) + bf_lo(a.w) * bf_lo(b.w) + bf_hi(a.w) * bf_hi(b.w));
+    } else {
+      float a[4], b[4];
+      load4(grow, a);
+      if constexpr (VEC) {
+        load4(orow, b);
+      } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) b[e] = to_f32(orow[e]);
-    s = a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+        for (int e = 0; e < 4; ++e) b[e] = to_f32(orow[e]);
+      }
+      s = a[0] * b[0] + a[1] * b[1] + a[2] * b[2] + a[3] * b[3];
+    }
   }
   for (int off = tpr >> 1; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
   if (row < rows && sub == 0) cvec[row] = s / den[row * den_stride];
