@@ -350,28 +350,6 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   const float xs = xscale[hx], a1s = a1scale[ha];
   const int xrow = w * 32 + i, tok = tok0 + xrow;
 
-  {
-    RowTile<D, T, 128> t;
-    t.load(Xh, tok0, n, tid);
-    t.store(Xl, LD, xs, tid);
-    t.load(Yh, tok0, n, tid, ydh, yden_stride);
-    // the own y rows only pass through LDS to reach their lanes: [128][LB] bf16 fits one stage pair
-    static_assert(128 * LB <= 2 * SLB, "own-row staging must fit the stage buffers");
-    t.store_bf(&Sb[0][0], LB, 1.0f, tid);
-  }
-  __syncthreads();
-  // own token of this lane = row xrow: its half of y, packed (A operand of the state
-  // contraction, B operand of g.v)
-  uint2 Yp[H2 / 4];
-#pragma unroll
-  for (int g4 = 0; g4 < H2 / 4; ++g4)
-    Yp[g4] = *reinterpret_cast<const uint2*>(&Sb[0][0] + xrow * LB + hh * H2 + 4 * g4);
-  const float c_own = (DQ && tok < n) ? ch[tok] : 0.f;
-  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
-  // pairs with (e_hi, e_hi, e_lo, e_lo); the upper four k slots of that MFMA are empty
-  const bf8v yxp = as_bf8(pack_bf4u(yxhi, yx - yxhi, yxhi, yx - yxhi), make_uint2(0u, 0u));
-  __syncthreads();
-
   const bool no_state = masked && (DQ ? c == 0 : c == nc - 1);
   const int n_state = no_state ? 0 : (p2 ? NS : 0) + 1;
   int n_tile = 0, tile0 = 0;
@@ -432,9 +410,34 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
 #pragma unroll
     for (int r = 0; r < 16; ++r) out[ab][r] = 0.f;
 
+  // Everything the block needs first is requested before anything is waited for (one memory
+  // latency instead of three in a row): the first slab, the first streamed tile, c of the own
+  // token, the own rows.
   if (n_tile > 0) tiles_load(0);
+  if (n_state > 0) slab_load(0);
+  const float c_ld = DQ ? ch[tok < n ? tok : n - 1] : 0.f;
+  {
+    RowTile<D, T, 128> t, u;
+    t.load(Xh, tok0, n, tid);
+    u.load(Yh, tok0, n, tid, ydh, yden_stride);
+    t.store(Xl, LD, xs, tid);
+    // the own y rows only pass through LDS to reach their lanes: [128][LB] bf16 fits one stage pair
+    static_assert(128 * LB <= 2 * SLB, "own-row staging must fit the stage buffers");
+    u.store_bf(&Sb[0][0], LB, 1.0f, tid);
+  }
+  __syncthreads();
+  // own token of this lane = row xrow: its half of y, packed (A operand of the state
+  // contraction, B operand of g.v)
+  uint2 Yp[H2 / 4];
+#pragma unroll
+  for (int g4 = 0; g4 < H2 / 4; ++g4)
+    Yp[g4] = *reinterpret_cast<const uint2*>(&Sb[0][0] + xrow * LB + hh * H2 + 4 * g4);
+  const float c_own = (DQ && tok < n) ? c_ld : 0.f;
+  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
+  // pairs with (e_hi, e_hi, e_lo, e_lo); the upper four k slots of that MFMA are empty
+  const bf8v yxp = as_bf8(pack_bf4u(yxhi, yx - yxhi, yxhi, yx - yxhi), make_uint2(0u, 0u));
+  __syncthreads();
   if (n_state > 0) {
-    slab_load(0);
     slab_store(0);
   } else if (n_tile > 0) {
     tiles_store(0);
