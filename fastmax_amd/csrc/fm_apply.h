@@ -68,11 +68,10 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
   const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
   const float xs = xscale[hx], a1s = a1scale[ha];
 
-  {
-    RowTile<D, T, 128> xt;
-    xt.load(Xh, tok0, n, tid);
-    xt.store(Xl, LD, xs, tid);
-  }
+  // (the own rows are requested here and staged after the first slab and streamed tile have been
+  // requested too: one memory latency at the start of a block instead of two in a row)
+  RowTile<D, T, 128> xt;
+  xt.load(Xh, tok0, n, tid);
 
   // the state is all zero for the first chunk in scan order
   const bool no_state = masked && (FWD ? c == 0 : c == nc - 1);
@@ -118,8 +117,9 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
   };
 
   if (n_tile > 0) tiles_load(0);
+  if (n_state > 0) slab_load(0);
+  xt.store(Xl, LD, xs, tid);
   if (n_state > 0) {
-    slab_load(0);
     slab_store(0);
   } else if (n_tile > 0) {
     tiles_store(0);

@@ -68,25 +68,6 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   const float xs = xscale[hx], a1s = a1scale[ha];
   const int xrow = w * 32 + i, tok = tok0 + xrow;
 
-  {
-    RowTile<D, T, 128> t;
-    t.load(Xh, tok0, n, tid);
-    t.store(Xl, LD, xs, tid);
-    t.load(Yh, tok0, n, tid, ydh, yden_stride);
-    t.store(Sl, LD, 1.0f, tid);
-  }
-  __syncthreads();
-  // own token of this lane = row xrow: its half of y (A operand of the state contraction, B of g.v)
-  float Yr[H2];
-#pragma unroll
-  for (int t = 0; t < H2; t += 4) {
-    const float4 y4 = *reinterpret_cast<const float4*>(Sl + xrow * LD + hh * H2 + t);
-    Yr[t] = y4.x; Yr[t + 1] = y4.y; Yr[t + 2] = y4.z; Yr[t + 3] = y4.w;
-  }
-  const float c_own = (DQ && tok < n) ? ch[tok] : 0.f;
-  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f;
-  __syncthreads();
-
   const bool no_state = masked && (DQ ? c == 0 : c == nc - 1);
   const int n_state = no_state ? 0 : (p2 ? NS : 0) + 1;
   int n_tile = 0, tile0 = 0;
@@ -133,9 +114,31 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) out[ab][r] = 0.f;
 
+  // Everything the block needs first is requested before anything is waited for (one memory
+  // latency instead of three in a row): the first slab, the first streamed tile, c of the own
+  // token, the own rows.
   if (n_tile > 0) tiles_load(0);
+  if (n_state > 0) slab_load(0);
+  const float c_ld = DQ ? ch[tok < n ? tok : n - 1] : 0.f;
+  {
+    RowTile<D, T, 128> t, u;
+    t.load(Xh, tok0, n, tid);
+    u.load(Yh, tok0, n, tid, ydh, yden_stride);
+    t.store(Xl, LD, xs, tid);
+    u.store(Sl, LD, 1.0f, tid);
+  }
+  __syncthreads();
+  // own token of this lane = row xrow: its half of y (A operand of the state contraction, B of g.v)
+  float Yr[H2];
+#pragma unroll
+  for (int t = 0; t < H2; t += 4) {
+    const float4 y4 = *reinterpret_cast<const float4*>(Sl + xrow * LD + hh * H2 + t);
+    Yr[t] = y4.x; Yr[t + 1] = y4.y; Yr[t + 2] = y4.z; Yr[t + 3] = y4.w;
+  }
+  const float c_own = (DQ && tok < n) ? c_ld : 0.f;
+  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f;
+  __syncthreads();
   if (n_state > 0) {
-    slab_load(0);
     slab_store(0);
   } else if (n_tile > 0) {
     tiles_store(0);
