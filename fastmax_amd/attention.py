@@ -63,6 +63,8 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
         if d > 64:
             raise ValueError(f"head dimension {d} is not supported (kernels exist for d <= 64)")
         pad = (32 if d <= 32 else 64) - d
+        if k.shape[-1] != d or v.shape[-1] != d:
+            raise ValueError(f"q, k and v must share the head dimension (got {d}, {k.shape[-1]}, {v.shape[-1]})")
         q3 = q.reshape(-1, q.shape[-2], d)
         k3 = k.reshape(-1, k.shape[-2], d)
         v3 = v.reshape(-1, v.shape[-2], d)

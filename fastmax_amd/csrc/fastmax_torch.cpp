@@ -28,6 +28,7 @@ void raise_on(int rc) { TORCH_CHECK(rc == FASTMAX_OK, "fastmax: ", fastmax_last_
 fastmax_desc make_desc(const torch::Tensor& q, const torch::Tensor& k, bool mask, bool normalize,
                        double temperature, double a0, double a1, double a2, double lim, int64_t p) {
   TORCH_CHECK(q.dim() == 3 && k.dim() == 3, "q, k, v must be (b*h, n, d)");
+  TORCH_CHECK(k.size(2) == q.size(2), "k has head dimension ", k.size(2), " but q has ", q.size(2));
   TORCH_CHECK(q.scalar_type() == torch::kFloat32 || q.scalar_type() == torch::kBFloat16,
               "q must be float32 or bfloat16");
   fastmax_desc ds;

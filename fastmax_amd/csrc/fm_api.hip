@@ -192,6 +192,7 @@ int heads_per_batch(const Plan& pl, size_t ws_bytes, bool with_saved = false) {
   }
   if (hb >= (size_t)m) hb = hb / m * m;
   hb = hb / pl.ratio * pl.ratio;  // whole key/value groups
+  if (hb < (size_t)pl.ratio) hb = pl.ratio;  // (check_ws made sure one group fits)
   return (int)hb;
 }
 

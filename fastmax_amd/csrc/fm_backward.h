@@ -44,18 +44,21 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const T* __restrict__ go,
 // ---------------------------------------------------------------------------------------
 // Chain rule through x_hat = lim * x / max_n ||x_n||: the scaling by lim/M is already in dx;
 // the max-norm row i* additionally gets  dx[i*] -= (sum dx_hat.x_hat) * x[i*] / M^2.
-// One block per head; blockDim.x = d.
+// One block per head; blockDim.x = d.  A row index outside [0, n) (only a caller-supplied
+// qk_argmax can hold one) leaves the head untouched.
 // ---------------------------------------------------------------------------------------
 template <class T>
 __global__ void norm_fix_kernel(T* __restrict__ dx, const T* __restrict__ x,
                                 const float* __restrict__ scale, const int* __restrict__ arg,
                                 const float* __restrict__ rpart, int nblk, int n, int d, float lim) {
   const int head = blockIdx.x, c = threadIdx.x;
+  const int row = arg[head];
+  if (row < 0 || row >= n) return;
   float r = 0.f;
   for (int b = 0; b < nblk; ++b) r += rpart[(int64_t)head * nblk + b];
   const float s = scale[head];
   const float fac = r * s * s / (lim * lim);
-  const int64_t off = ((int64_t)head * n + arg[head]) * d + c;
+  const int64_t off = ((int64_t)head * n + row) * d + c;
   dx[off] = from_f32<T>(to_f32(dx[off]) - fac * to_f32(x[off]));
 }
 

@@ -45,8 +45,16 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, in
   const int tpr = d / EPT, rpp = NT / tpr;
   const int sub = tid % tpr, rowi = tid / tpr;
   const T* base = x + (int64_t)blockIdx.x * n * d;
+  // A NaN row norm wins over every number (the maximum of the reference's path propagates NaN,
+  // example.py:105-108), so the head's scale becomes NaN and the reported row is always a row
+  // of the tensor: first NaN row if there is one, else first row of maximal norm.
+  auto better = [](float ss, int idx, float best, int bi) {
+    const bool ssnan = ss != ss, bnan = best != best;
+    if (ssnan) return !bnan || idx < bi;
+    return !bnan && (ss > best || (ss == best && idx < bi));
+  };
   float best = -1.f;
-  int bi = 0x7fffffff;
+  int bi = 0;
   // four row groups per trip, loaded before any of them is reduced (rows past the end are
   // clamped to the last row: a duplicate cannot change the maximum or its first index)
   for (int i0 = 0; i0 < n; i0 += 4 * rpp) {
@@ -62,7 +70,7 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, in
     for (int u = 0; u < 4; ++u) {
       float ss = ssq[u];
       for (int off = tpr >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
-      if (ss > best || (ss == best && idx[u] < bi)) {
+      if (better(ss, idx[u], best, bi)) {
         best = ss;
         bi = idx[u];
       }
@@ -75,7 +83,7 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, in
     if (tid < off) {
       const float ob = sbest[tid + off];
       const int oi = sarg[tid + off];
-      if (ob > sbest[tid] || (ob == sbest[tid] && oi < sarg[tid])) {
+      if (better(ob, oi, sbest[tid], sarg[tid])) {
         sbest[tid] = ob;
         sarg[tid] = oi;
       }
@@ -84,7 +92,7 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, in
   }
   if (tid == 0) {
     scale_out[blockIdx.x] = lim / sqrtf(sbest[0]);
-    arg_out[blockIdx.x] = sarg[0];
+    arg_out[blockIdx.x] = min(max(sarg[0], 0), n - 1);
   }
 }
 

@@ -9,7 +9,8 @@ import torch
 
 from . import _cabi
 
-_WS: Dict[Tuple[int, int], torch.Tensor] = {}
+# one workspace per (device, stream, purpose): calls on different streams never share one
+_WS: Dict[Tuple[int, int, int], torch.Tensor] = {}
 
 
 def _dtype_code(t: torch.Tensor) -> int:
@@ -31,10 +32,13 @@ def _check_inputs(*ts: torch.Tensor) -> None:
             raise RuntimeError("fastmax: tensors must share dtype and device")
         if t.dim() != 3:
             raise RuntimeError("fastmax: expected (b*h, n, d) tensors at this level")
+        if t.shape[2] != first.shape[2]:
+            raise RuntimeError(f"fastmax: head dimensions differ ({t.shape[2]} and {first.shape[2]})")
 
 
 def _workspace(dev: torch.device, nbytes: int, slot: int) -> torch.Tensor:
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), slot)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    key = (index, torch.cuda.current_stream(dev).cuda_stream, slot)
     ws = _WS.get(key)
     if ws is None or ws.numel() < nbytes:
         _WS[key] = ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)

@@ -140,7 +140,7 @@ int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* 
 /* In-place q <- lim*q/max||q_n||, k likewise: the side effect the reference's forward has
  * on its inputs (calc_norms/find_max/apply_norm, fastmax_cuda_forward.cu:223-269,368-382,
  * with the PyTorch path's definition of the norm, example.py:105-108).  Only the legacy
- * forwardpass binding uses it.  workspace: >= 16*bh bytes. */
+ * forwardpass binding uses it.  workspace: >= 16*bh + 512 bytes, 256-byte aligned. */
 int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k,
                               void* workspace, size_t workspace_bytes, fastmax_stream_t stream);
 
