@@ -27,6 +27,7 @@ EXPORTS = (
     "fastmax_profile_begin", "fastmax_profile_end",
     "fastmax_state_bytes", "fastmax_decode_workspace_bytes", "fastmax_state_update", "fastmax_decode_step",
     "fastmax_saved_state_bytes", "fastmax_forward_saving", "fastmax_backward_saved", "fastmax_qkv_rope",
+    "fastmax_noalloc_scratch_bytes", "fastmax_forward_noalloc",
 )
 
 KERNEL_NAMES = ("rowstat", "build", "fwd_apply", "bwd_prep", "bwd_dq", "bwd_dk", "bwd_dv", "norm_fix")
@@ -91,6 +92,10 @@ def load() -> C.CDLL:
     lib.fastmax_backward_saved.restype = C.c_int
     lib.fastmax_backward_saved.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, sz, vp,
                                            sz, vp]
+    lib.fastmax_noalloc_scratch_bytes.restype = sz
+    lib.fastmax_noalloc_scratch_bytes.argtypes = []
+    lib.fastmax_forward_noalloc.restype = C.c_int
+    lib.fastmax_forward_noalloc.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp]
     lib.fastmax_qkv_rope.restype = C.c_int
     lib.fastmax_qkv_rope.argtypes = [C.POINTER(RopeDesc), C.c_int, vp, vp, vp, vp, vp, vp, vp]
     lib.fastmax_normalize_inplace.restype = C.c_int

@@ -1,10 +1,13 @@
 // C ABI of the gfx950 Fastmax library: argument checking, workspace carving, head batching
-// and kernel launches.  No torch, no allocation, no global mutable state.
+// and kernel launches.  No torch, no allocation; the only state kept between calls is the
+// per-device address of the built-in scratch array (fastmax_forward_noalloc) and the opt-in
+// per-thread kernel timer.
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
 #include <vector>
 
 #include "fastmax_amd.h"
@@ -15,6 +18,11 @@
 #include "fm_grad.h"
 #include "fm_linear.h"
 #include "fm_rope.h"
+
+// Scratch memory of fastmax_forward_noalloc: lives in every device's copy of the code object from
+// the moment the library is loaded there until the process ends.  In host code the name is only a
+// handle for hipGetSymbolAddress; kernels and copies get the per-device address it returns.
+static __device__ __align__(256) unsigned char scratch[FASTMAX_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -619,6 +627,28 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
   return FASTMAX_OK;
 }
 
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_on_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(FASTMAX_E_NO_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(FASTMAX_E_NO_DEVICE, "device index %d outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(FASTMAX_E_NO_DEVICE, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return FASTMAX_OK;
+}
+
 constexpr int kDecodeSplits = 8;  // blocks per head in a decode step (row slices of the state)
 
 size_t decode_ws_bytes(const fastmax_desc* ds) {
@@ -760,6 +790,27 @@ int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, cons
                     fastmax_stream_t stream) {
   return fastmax_forward_saving(desc, q, k, v, o, ldo, den, den_stride, qk_scale, qk_argmax, workspace,
                                 workspace_bytes, nullptr, 0, stream);
+}
+
+size_t fastmax_noalloc_scratch_bytes(void) { return FASTMAX_NOALLOC_SCRATCH_BYTES; }
+
+int fastmax_forward_noalloc(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
+                            int64_t ldo, float* den, int64_t den_stride, float* qk_scale,
+                            int32_t* qk_argmax, fastmax_stream_t stream) {
+  g_err[0] = 0;
+  FM_TRY(check_desc(desc));
+  const Plan pl = make_plan(desc, FASTMAX_PASS_FORWARD);
+  const size_t need = pl.fixed_bytes + pl.ratio * batch_bytes_per_head(pl, false);
+  if (need > (size_t)FASTMAX_NOALLOC_SCRATCH_BYTES)
+    return fail(FASTMAX_E_WORKSPACE,
+                "this problem needs %zu bytes of scratch memory; the allocation-free entry point holds %zu "
+                "(use fastmax_forward with a workspace of the caller's)", need, (size_t)FASTMAX_NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  FM_TRY(scratch_on_current_device(&ws));
+  // nothing in the forward pass reads scratch memory it has not written in the same call, so the
+  // previous call's contents need no clearing
+  return fastmax_forward_saving(desc, q, k, v, o, ldo, den, den_stride, qk_scale, qk_argmax, ws,
+                                FASTMAX_NOALLOC_SCRATCH_BYTES, nullptr, 0, stream);
 }
 
 int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* k, const void* v,

@@ -5,8 +5,9 @@
  *     o_i = sum_j f(q_i.k_j) v_j / sum_j f(q_i.k_j),   f(s) = a0 + a1 s + a2 s^2  (p=2)
  * (j <= i when mask != 0).  This header is the whole drop-in boundary for that path:
  * plain pointers and sizes, no torch types.  Every entry point is asynchronous on the
- * given stream, allocates nothing on the device, keeps no state between calls (the opt-in
- * kernel timer at the end of this header aside) and returns 0 or a negative FASTMAX_E_* code (text via fastmax_last_error()).
+ * given stream, allocates nothing on the device, keeps no state between calls (the built-in
+ * scratch array of fastmax_forward_noalloc and the opt-in kernel timer at the end of this
+ * header aside) and returns 0 or a negative FASTMAX_E_* code (text via fastmax_last_error()).
  *
  * Layout contract (reference: fastmax_cuda_forward.cu:331-336): q, k, v, grad_output and
  * the gradients are (bh, n, d) row-major with d contiguous; a (b,h,n,d) tensor is the
@@ -136,6 +137,23 @@ int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* 
                            const float* qk_scale, const int32_t* qk_argmax,
                            void* workspace, size_t workspace_bytes,
                            const void* saved_states, size_t saved_bytes, fastmax_stream_t stream);
+
+/* Forward pass for callers that cannot allocate device memory or carry a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose launcher allocates five tensors per call,
+ * fastmax_cuda_forward.cu:347-358).  Same arguments and results as fastmax_forward (bit for bit),
+ * minus the workspace: the head statistics and moment states go to a scratch array of
+ * FASTMAX_NOALLOC_SCRATCH_BYTES that is part of the library's device image (every GPU the library
+ * runs on holds it until the process ends; its address is looked up on the first call per device).
+ * The call allocates and frees nothing.  Problems whose smallest workspace
+ * (fastmax_workspace_min_bytes(desc, FASTMAX_PASS_FORWARD)) exceeds the array are refused with
+ * FASTMAX_E_WORKSPACE.  All calls on one GPU share the array: calls that overlap in time on
+ * one GPU (different streams, or threads) race and must be serialised by the caller. */
+#define FASTMAX_NOALLOC_SCRATCH_BYTES (64u << 20)
+size_t fastmax_noalloc_scratch_bytes(void);
+int fastmax_forward_noalloc(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                            void* o, int64_t ldo, float* den, int64_t den_stride,
+                            float* qk_scale, int32_t* qk_argmax, fastmax_stream_t stream);
 
 /* In-place q <- lim*q/max||q_n||, k likewise: the side effect the reference's forward has
  * on its inputs (calc_norms/find_max/apply_norm, fastmax_cuda_forward.cu:223-269,368-382,
