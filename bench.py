@@ -69,6 +69,63 @@ def algorithmic_flops(d: int, p: int) -> dict:
     }
 
 
+def executed_mfma_flops(cfg: dict, bh: int, chunk: int = 384) -> dict:
+    """Flops of the matrix instructions each kernel class of the chunked p = 2 path issues per head set and
+    pass (2*32*32*K per instruction: 4096 for v_mfma_f32_32x32x2f32, 32768 for v_mfma_f32_32x32x16_bf16),
+    counted the way the kernels launch them: every wave of every block, dummy row-tile slots and ragged
+    tiles included.  The kernels store each unordered channel pair once, so this is about half of the
+    reference-form count of algorithmic_flops().  Keys: build_fwd, build_bwd (one state each), fwd_apply,
+    bwd_dq, bwd_dk, bwd_dv."""
+    d, n, masked, bf = cfg["D"], cfg["N"], cfg["mask"], cfg["dtype"] == "bf16"
+    assert cfg["p"] == 2
+    h2, ns, cb = d // 2, d // 2 + 1, d // 32
+    per = 32768 if bf else 4096                 # flop per matrix instruction
+    ksteps = (lambda k: k // 16) if bf else (lambda k: k // 2)   # instructions for a contraction length k
+    # state build: gsplit blocks x 4 waves x rtw row tiles x cb column tiles, one 32-token step at a time
+    rt_total = ns * cb + cb
+    rtw = 3 if d == 64 else 5
+    gsplit = -(-rt_total // (4 * rtw))
+    per_step = gsplit * 4 * rtw * cb * ksteps(32) * per
+    nc = -(-n // chunk)
+    spc = chunk // 32
+    if masked:
+        steps_f = (nc - 1) * spc
+        steps_r = (-(-(n - (nc - 1) * chunk) // 32) + (nc - 2) * spc) if nc > 1 else 0
+    else:
+        z = min(max(-(-1024 // (gsplit * bh)), 1), -(-n // 256))
+        zlen = -(-(-(-n // z)) // 32) * 32
+        steps_f = steps_r = sum(-(-(min(n, (i + 1) * zlen) - i * zlen) // 32) for i in range(-(-n // zlen)))
+    out = {"build_fwd": bh * steps_f * per_step, "build_bwd": bh * steps_r * per_step}
+    # consumers: blocks of 128 tokens, 4 waves of 32; the state part runs ns + 1 slabs (none in the first chunk
+    # in scan order), then one score tile + one product per streamed 32-token tile of the own chunk
+    den_tile = 1 if bf else 0                    # bf16 forward: a third accumulator tile carries the denominator
+    slab = {"fwd_apply": ksteps(d) * (cb + den_tile), "bwd_dv": ksteps(d) * cb,
+            "bwd_dq": cb * (ksteps(d) + 1), "bwd_dk": cb * (ksteps(d) + 1)}
+    tile = {"fwd_apply": ksteps(d) + ksteps(32) * (cb + den_tile), "bwd_dv": ksteps(d) + ksteps(32) * cb,
+            "bwd_dq": 2 * ksteps(d) + ksteps(32) * cb, "bwd_dk": 2 * ksteps(d) + ksteps(32) * cb}
+    count = {k: 0 for k in slab}
+    for blk in range(-(-n // 128)):
+        tok0 = blk * 128
+        c = tok0 // chunk
+        for name, forward_scan in (("fwd_apply", True), ("bwd_dq", True), ("bwd_dv", False), ("bwd_dk", False)):
+            has_state = not masked or (c > 0 if forward_scan else c < nc - 1)
+            insts = 4 * (ns + 1) * slab[name] if has_state else 0
+            if masked:
+                for w in range(4):
+                    mine = tok0 // 32 + w
+                    if forward_scan:
+                        last = min(tok0 + 127, n - 1) // 32
+                        active = max(0, min(mine, last) - (c * chunk) // 32 + 1)
+                    else:
+                        cend = min((c + 1) * chunk, n)
+                        active = max(0, (cend - 1) // 32 - mine + 1)
+                    insts += active * tile[name]
+            count[name] += insts
+    for name, insts in count.items():
+        out[name] = bh * insts * per
+    return out
+
+
 def cpu_baseline(cfg: dict, seconds_hint: float) -> dict:
     """Reference-form fwd+bwd (oracle/fastmax_oracle.py::fastmax_reference_form, the op sequence of
     the reference's fastmax_function) on one head and a token prefix that fits in memory."""
@@ -98,7 +155,30 @@ def cpu_baseline(cfg: dict, seconds_hint: float) -> dict:
         reps += 1
     t = t_tot / reps
     token_heads_per_s = n_s / t
+
+    # second row: the package's own PyTorch function (fastmax_amd.attention.fastmax_function, what
+    # use_custom_gradient=False runs), which walks the sequence in chunks and so fits one whole head
+    from fastmax_amd.attention import fastmax_function
+    qf, kf, vf, gof = O.seeded_inputs((1, 1, cfg["N"], d), seed=0)
+
+    def chunked_step():
+        qq, kk, vv = (x.clone().requires_grad_(True) for x in (qf, kf, vf))
+        fastmax_function(qq, kk, vv, mask, 0.0, 1, 1.0, COEF["a0"], COEF["a1"], COEF["a2"], COEF["lim"], p).backward(gof)
+
+    chunked_step()
+    creps, ct = 0, 0.0
+    while creps < 2 or (ct < seconds_hint / 2 and creps < 20):
+        t0 = time.perf_counter()
+        chunked_step()
+        ct += time.perf_counter() - t0
+        creps += 1
+    ct /= creps
     return {
+        "chunked": {"value": cfg["N"] / ct / cfg["H"], "unit": "tokens/s", "cores": torch.get_num_threads(),
+                    "kind": "port",
+                    "sample": (f"chunked-scan PyTorch function (128-token chunks, fp32, autograd) on 1 of "
+                               f"{cfg['B'] * cfg['H']} heads, all {cfg['N']} tokens, {creps} reps of {ct:.3f} s; "
+                               "tokens/s = (N/t)/H")},
         "value": token_heads_per_s / cfg["H"],
         "unit": "tokens/s",
         "cores": torch.get_num_threads(),
@@ -121,6 +201,8 @@ def main() -> int:
                     help="also run one plain 1 GiB device copy, so that a counter profile of this command "
                          "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true",
+                    help="skip the error metrics of one sampled head against the CPU oracle")
     ap.add_argument("--recompute-states", action="store_true",
                     help="backward rebuilds the prefix states instead of reading the ones the forward pass "
                          "kept (saves bhkv * chunks * 592 KB of HBM, costs one more state build)")
@@ -167,6 +249,10 @@ def main() -> int:
         # the forward pass leaves its prefix states behind for the backward pass
         o, den, sc, arg, saved = ops.forward(q, k, v, save_states=True, **kw)
         return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, saved_states=saved, **kw)
+
+    def step_outputs():
+        o, den, sc, arg = fwd()
+        return (o,) + tuple(ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw))
 
     for _ in range(args.warmup):
         step()
@@ -241,34 +327,53 @@ def main() -> int:
 
     fl = algorithmic_flops(D, cfg["p"])
     token_heads = bh * N
+    peak = PEAK_TFLOPS[cfg["dtype"]]
     kernels = {}
     for i, name in enumerate(_cabi.KERNEL_NAMES):
         if kt.launches[i]:
             kernels[name] = {"ms_per_step": kt.ms[i] / args.steps, "launches_per_step": kt.launches[i] / args.steps}
-    # algorithmic flops each kernel class executes per step (builds: fwd prefix, bwd suffix, and the bwd prefix
-    # again when the states are not kept)
+    # Flops per step and kernel class, two ways.  "algorithmic": the reference-form count per token-head (every
+    # ordered channel pair).  "executed": what the matrix instructions of this build really issue (each unordered
+    # pair once, plus intra-chunk tiles, dummy tile slots and ragged tiles).  Both count the state builds the timed
+    # step runs: the forward prefix build and the backward suffix build, plus the backward prefix build when the
+    # states are rebuilt instead of kept.
     n_builds = 3 if args.recompute_states else 2
-    per_step_flops = {"build": n_builds * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
-                      "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dk": fl["bwd_dk"] * token_heads,
-                      "bwd_dv": fl["bwd_dv"] * token_heads}
-    dom = max(per_step_flops, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0))
+    algo = {"build": n_builds * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
+            "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dk": fl["bwd_dk"] * token_heads,
+            "bwd_dv": fl["bwd_dv"] * token_heads}
+    executed = None
+    if cfg["p"] == 2:
+        ex = executed_mfma_flops(cfg, bh)
+        executed = {"build": ex["build_fwd"] * (n_builds - 1) + ex["build_bwd"],
+                    **{k: ex[k] for k in ("fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv")}}
+    for name, f in algo.items():
+        if name in kernels:
+            sec = kernels[name]["ms_per_step"] * 1e-3
+            kernels[name]["algorithmic_tflops"] = f / sec / 1e12
+            kernels[name]["algorithmic_frac"] = f / sec / 1e12 / peak
+            if executed:
+                kernels[name]["executed_tflops"] = executed[name] / sec / 1e12
+                kernels[name]["executed_frac"] = executed[name] / sec / 1e12 / peak
+    step_summary = {"algorithmic_tflops": sum(algo.values()) / (ms_step * 1e-3) / 1e12}
+    step_summary["algorithmic_frac"] = step_summary["algorithmic_tflops"] / peak
+    if executed:
+        step_summary["executed_tflops"] = sum(executed.values()) / (ms_step * 1e-3) / 1e12
+        step_summary["executed_frac"] = step_summary["executed_tflops"] / peak
+    dom = max(algo, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0))
     dom_ms = kernels[dom]["ms_per_step"]
     launches = kernels[dom]["launches_per_step"]
-    achieved = per_step_flops[dom] / (dom_ms * 1e-3) / 1e12
-    # fp32 inputs run every contraction on v_mfma_f32_32x32x2f32; bf16 inputs on v_mfma_f32_32x32x8_bf16
-    peak = PEAK_TFLOPS[cfg["dtype"]]
-    roofline = {
-        "bound": "mfma", "kernel": dom, "achieved": achieved, "peak": peak, "unit": "TFLOP/s",
-        "frac": achieved / peak, "traffic": None,
-        "flops_per_launch": per_step_flops[dom] / launches, "avg_launch_ms": dom_ms / launches,
-    }
-    # what the build kernel really executes (the pair symmetry halves the order-2 rows): row-tile
-    # slots per head x 32 rows x d columns MACs per token
-    if dom == "build" and cfg["p"] == 2:
-        slots = {64: 72, 32: 20}[D]  # 6 blocks x 4 waves x 3 tiles; 1 block x 4 waves x 5 tiles
-        executed = 2.0 * slots * 32 * D * token_heads * n_builds / (dom_ms * 1e-3) / 1e12
-        roofline["executed_tflops"] = executed
-        roofline["executed_frac"] = executed / peak
+    # fp32 inputs run every contraction on v_mfma_f32_32x32x2f32, bf16 inputs on v_mfma_f32_32x32x16_bf16.
+    # frac is the executed rate over the peak (at most 1, and what SQ_VALU_MFMA_BUSY_CYCLES over the kernel's
+    # duration shows); algorithmic_frac prices the same time with the reference-form count and can exceed 1.
+    if executed:
+        roofline = {
+            "bound": "mfma", "kernel": dom, "achieved": kernels[dom]["executed_tflops"], "peak": peak,
+            "unit": "TFLOP/s", "frac": kernels[dom]["executed_frac"],
+            "algorithmic_achieved": kernels[dom]["algorithmic_tflops"],
+            "algorithmic_frac": kernels[dom]["algorithmic_frac"], "traffic": None,
+            "flops_per_launch": executed[dom] / launches, "algorithmic_flops_per_launch": algo[dom] / launches,
+            "avg_launch_ms": dom_ms / launches,
+        }
     if cfg["p"] == 1:
         # p = 1 is HBM-bound (about 19 flop per byte): price the slowest kernel against the (bh, n, d)
         # tensors it must move; the per-token scalars and the (d+1) x (d+1) states are negligible.
@@ -279,7 +384,7 @@ def main() -> int:
         #     forward q -> o; dq grad -> dq; dk v -> dk; dv k -> dv: two tensors each
         es = 4 if cfg["dtype"] == "f32" else 2
         tensors = 4 if "build" not in kernels else 2
-        dom = max(per_step_flops, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0)
+        dom = max(algo, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0)
                   / kernels.get(n, {}).get("launches_per_step", 1.0))
         dom_ms = kernels[dom]["ms_per_step"]
         launches = kernels[dom]["launches_per_step"]
@@ -295,9 +400,22 @@ def main() -> int:
         n_states = n_builds if dom == "build" else 1
         roofline["traffic"] = per_th * token_heads * n_states / launches  # bytes per launch (profiled, not live)
         roofline["traffic_source"] = TRAFFIC_SOURCE[args.workload]
-    for name, f in per_step_flops.items():
-        if name in kernels:
-            kernels[name]["algorithmic_tflops"] = f / (kernels[name]["ms_per_step"] * 1e-3) / 1e12
+
+    # parity of this very run: one sampled head of the timed tensors against the fp64 dense form (CPU oracle)
+    parity = None
+    if not args.no_parity:
+        from oracle import fastmax_oracle as O
+        h = bh // 2
+        outs = step_outputs()
+        torch.cuda.synchronize()
+        sl = slice(h, h + 1)
+        ref = O.dense_truth(*(t[sl].float().cpu().double() for t in (q, k, v, go)), mask=cfg["mask"], normalize=True,
+                            a0=COEF["a0"], a1=COEF["a1"], a2=COEF["a2"], lim=COEF["lim"], p=cfg["p"])
+        parity = {"head": h, "reference": "fp64 dense closed form on the same inputs (oracle.dense_truth)",
+                  "tolerance": 1e-4 if cfg["dtype"] == "f32" else 2e-2}
+        for name, got, want in zip(("o", "dq", "dk", "dv"), outs, ref):
+            parity[name] = O.error_metrics(got[sl].float().cpu(), want)
+        del outs, ref
 
     result = {
         "metric": "fwd+bwd tokens/sec and MFMA % of peak at B64 H16 N10000 D64 p2, 1 GPU",
@@ -316,10 +434,10 @@ def main() -> int:
         "module_autograd_ms_per_step": ms_module,
         "hip_graph_replay_ms_per_step": ms_graph,
         "fwd_tflops": fl["fwd"] * token_heads / (ms_fwd * 1e-3) / 1e12,
-        "fwd_bwd_tflops": (fl["fwd"] + fl["bwd"]) * token_heads / (ms_step * 1e-3) / 1e12,
-        "mfma_frac_of_peak_fwd_bwd": (fl["fwd"] + fl["bwd"]) * token_heads / (ms_step * 1e-3) / 1e12 / peak,
+        "step": step_summary,
         "kernels": kernels,
         "roofline": roofline,
+        "parity": parity,
     }
     if not args.no_cpu_baseline:
         del q, k, v, go

@@ -31,18 +31,12 @@ from . import _ext
 SAVE_STATES_MEMORY_FRACTION = 0.25
 
 
-def _states_fit(k3: torch.Tensor, mask: bool) -> bool:
-    """True when the prefix states of this call (one 592 KB state per key/value head per 384
-    tokens at d = 64, p = 2; half of that for causal bf16 passes, whose states are kept packed)
-    take less than SAVE_STATES_MEMORY_FRACTION of the free memory."""
-    heads, n, d = k3.shape
-    rows = (d // 2 + 1) * d + d + 1
-    state_bytes = rows * (d + 4) * 4 + 256
-    if mask and k3.dtype == torch.bfloat16:
-        state_bytes = state_bytes // 2 + 512
-    slots = (n + 127) // 128 if mask else 8  # upper bounds: the chunk is at least 128 tokens
+def _states_fit(q3: torch.Tensor, k3: torch.Tensor, mask: bool, p: int) -> bool:
+    """True when the prefix states of this call (the library's own figure: one state per key/value
+    head per chunk or token split) take less than SAVE_STATES_MEMORY_FRACTION of the free memory."""
+    need = _ext.load().saved_state_bytes(q3, k3, bool(mask), int(p))
     free, _ = torch.cuda.mem_get_info(k3.device)
-    return heads * slots * state_bytes <= SAVE_STATES_MEMORY_FRACTION * free
+    return need <= SAVE_STATES_MEMORY_FRACTION * free
 
 
 class FASTMultiHeadAttention_Function(torch.autograd.Function):
@@ -83,7 +77,7 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
         # keep the prefix states for the backward pass (it then skips rebuilding them) when a
         # backward pass will come and the states fit comfortably in free device memory
         need_grad = any(t.requires_grad for t in (q, k, v))
-        save = need_grad and _states_fit(k3, bool(mask))
+        save = need_grad and _states_fit(q3, k3, bool(mask), int(p))
         o, den, scale, arg, saved = ext.forward_ex(q3, k3, v3, bool(mask), bool(normalize), float(temperature),
                                                    float(a0), float(a1), float(a2), float(lim), int(p), save)
         if lead:

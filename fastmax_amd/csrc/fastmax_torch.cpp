@@ -1,7 +1,9 @@
 // PyTorch-ROCm binding of the Fastmax C ABI.  The module is named `fastmax_cuda` and exports
 // `forwardpass` / `backwardpass` with the positional signatures of the reference extension
-// (fastmax_cuda.cpp:17-37, minus the rpe_matrix argument the live kernels do not take:
-// fastmax_cuda_forward.cu:297-314), so the reference's autograd Function runs on it unchanged.
+// (fastmax_cuda.cpp:17-37).  forwardpass exists in both forms the reference's files call: the
+// 13-argument one of the live kernels (fastmax_cuda_forward.cu:297-314; example.py:36,
+// model.py:37) and the 14-argument one with rpe_matrix after drop_noise (fastmax_cuda.cpp:17,
+// test_fastmax.py:32), so the reference's autograd Functions run on it unchanged.
 // `forward_ex` / `backward_ex` are the non-mutating entry points the package's own autograd
 // Function uses: they differentiate through the normalisation and accept bf16.
 //
@@ -118,6 +120,7 @@ std::vector<torch::Tensor> backward_ex(torch::Tensor q, torch::Tensor k, torch::
   check_same(q, v, "v");
   check_same(q, o, "o");
   check_same(q, go, "grad_output");
+  TORCH_CHECK(k.sizes() == v.sizes(), "k and v must have the same shape");
   TORCH_CHECK(o.sizes() == q.sizes() && go.sizes() == q.sizes(), "o and grad_output must be shaped like q");
   TORCH_CHECK(den.scalar_type() == torch::kFloat32 && den.numel() == q.size(0) * q.size(1), "den must be float32 (bh, n)");
   TORCH_CHECK(scale.scalar_type() == torch::kFloat32 && scale.numel() == 2 * q.size(0), "qk_scale must be float32 (2*bh)");
@@ -165,7 +168,8 @@ torch::Tensor forwardpass(torch::Tensor q, torch::Tensor k, torch::Tensor v, tor
   check_same(q, v, "v");
   TORCH_CHECK(q.scalar_type() == torch::kFloat32, "forwardpass takes float32 tensors (use forward_ex for bfloat16)");
   TORCH_CHECK(q.dim() == 3 && k.dim() == 3, "q, k, v must be (b*h, n, d)");
-  TORCH_CHECK(k.sizes() == v.sizes(), "k and v must have the same shape");
+  TORCH_CHECK(k.sizes() == v.sizes() && k.size(2) == q.size(2),
+              "k and v must have the same shape and q's head dimension");
   const int64_t lead = k.size(1) - q.size(1);
   TORCH_CHECK(lead >= 0, "k, v have ", k.size(1), " tokens but q has ", q.size(1),
               ": fewer keys than queries is not supported");
@@ -215,6 +219,7 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
   TORCH_CHECK(o.dim() == 3 && o.size(0) == q.size(0) && o.size(1) == q.size(1) && o.size(2) == d + 1,
               "o must be the (bh, n, d+1) tensor forwardpass returned");
   TORCH_CHECK(grad_output.sizes() == q.sizes(), "grad_output must be shaped like q");
+  TORCH_CHECK(k.sizes() == v.sizes() && k.size(2) == d, "k and v must have the same shape and q's head dimension");
   const int64_t lead = k.size(1) - q.size(1);
   TORCH_CHECK(lead >= 0, "k, v have ", k.size(1), " tokens but q has ", q.size(1),
               ": fewer keys than queries is not supported");
@@ -241,10 +246,30 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
   return {dq, dk, dv};
 }
 
+// The 14-argument form (fastmax_cuda.cpp:17, called at test_fastmax.py:32): rpe_matrix sits between
+// drop_noise and mask.  The relative positional encoding is switched off in every kernel of the
+// reference (README.md:16), so the matrix is accepted and not read.
+torch::Tensor forwardpass_rpe(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor drop_noise,
+                              torch::Tensor rpe_matrix, bool mask, double dropout, bool normalize,
+                              double temperature, double a0, double a1, double a2, double lim, int64_t p) {
+  (void)rpe_matrix;
+  return forwardpass(q, k, v, drop_noise, mask, dropout, normalize, temperature, a0, a1, a2, lim, p);
+}
+
+// Bytes of the buffer forward_ex(save_states = true) would allocate for these tensors.
+int64_t saved_state_bytes(torch::Tensor q, torch::Tensor k, bool mask, int64_t p) {
+  const fastmax_desc ds = make_desc(q, k, mask, false, 1.0, 1.0, 1.0, 0.5, 1.0, p);
+  const size_t sb = fastmax_saved_state_bytes(&ds);
+  TORCH_CHECK(sb > 0, "fastmax: ", fastmax_last_error());
+  return (int64_t)sb;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("forwardpass", &forwardpass, "forwardpass");
+  m.def("forwardpass", &forwardpass_rpe, "forwardpass with rpe_matrix (accepted, not used)");
+  m.def("saved_state_bytes", &saved_state_bytes, "size of the prefix states forward_ex can keep");
   m.def("backwardpass", &backwardpass, "backwardpass");
   m.def("forward_ex", &forward_ex, "forward returning (o, den, qk_scale, qk_argmax, saved_states)");
   m.def("backward_ex", &backward_ex, "backward through the normalisation, returns [dq, dk, dv]");

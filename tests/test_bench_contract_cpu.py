@@ -26,3 +26,29 @@ def test_algorithmic_flops_closed_forms():
     assert fl1["fwd"] == 16900 and fl1["bwd"] == 41860
     fl32 = bench.algorithmic_flops(32, 2)
     assert fl32["fwd"] == 139524 and fl32["bwd"] == 346564
+
+
+def test_executed_flops_model():
+    """The executed count is pinned where it has a closed form: the d = 64 state build issues 72 row-tile
+    slots x 32 rows x 64 columns MACs per token, an unmasked consumer runs 34 slabs of 64 rows over 64
+    (+1 for the gradients' extra) columns, and everything stays below the reference-form count."""
+    sys.path.insert(0, ROOT)
+    import bench
+
+    cfg = dict(B=1, H=4, N=384 * 5, D=64, mask=False, p=2, dtype="f32")
+    ex = bench.executed_mfma_flops(cfg, 4)
+    th = 4 * cfg["N"]
+    assert ex["build_fwd"] == 2 * 72 * 32 * 64 * th
+    assert ex["fwd_apply"] == ex["bwd_dv"] == 2 * 34 * 64 * 64 * th
+    assert ex["bwd_dq"] == ex["bwd_dk"] == 2 * 34 * 64 * 66 * th
+    al = bench.algorithmic_flops(64, 2)
+    for wl in ("headline", "c4", "c2"):
+        c = bench.WORKLOADS[wl]
+        e = bench.executed_mfma_flops(c, c["B"] * c["H"])
+        tokens = c["B"] * c["H"] * c["N"]
+        f = bench.algorithmic_flops(c["D"], 2)
+        assert e["build_fwd"] < f["build"] * tokens and e["fwd_apply"] < f["fwd_apply"] * tokens
+        assert e["bwd_dq"] < f["bwd_dq"] * tokens and e["bwd_dv"] < f["bwd_dv"] * tokens
+    # bf16 forward carries the denominator in a third accumulator tile
+    cb = dict(cfg, dtype="bf16")
+    assert bench.executed_mfma_flops(cb, 4)["fwd_apply"] == 2 * 34 * 64 * 96 * th

@@ -454,6 +454,12 @@ def test_legacy_extension_entry_points(built):
     _, rdq, rdk, rdv = O.dense_truth(qh[0], kh[0], v, go, mask=True, normalize=False)
     for name, got, ref in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
         assert_close(name, got, ref, 1e-4)
+    # the 14-argument form (fastmax_cuda.cpp:17, test_fastmax.py:32): rpe_matrix after drop_noise, not used
+    from fastmax_amd import rpe_matrix_creator
+    q2, k2, v2 = (t.cuda() for t in (q, k, v))
+    rpe = rpe_matrix_creator(300, 64, q2.device, q2.dtype, structured=True)
+    o14 = ext.forwardpass(q2, k2, v2, torch.zeros_like(q2), rpe, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
+    assert torch.equal(o14, o) and torch.equal(q2, qd) and torch.equal(k2, kd)
     with pytest.raises(RuntimeError, match="contiguous"):
         ext.forwardpass(qd.transpose(0, 1), kd, vd, qd, True, 0.0, True, 1.0, 1.0, 1.0, 0.5, 1.0, 2)
     with pytest.raises(RuntimeError, match="p must be 1 or 2"):
