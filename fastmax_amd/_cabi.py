@@ -28,6 +28,8 @@ EXPORTS = (
     "fastmax_state_bytes", "fastmax_decode_workspace_bytes", "fastmax_state_update", "fastmax_decode_step",
     "fastmax_saved_state_bytes", "fastmax_forward_saving", "fastmax_backward_saved", "fastmax_qkv_rope",
     "fastmax_noalloc_scratch_bytes", "fastmax_forward_noalloc",
+    "fastmax_workspace_bytes_strided", "fastmax_workspace_min_bytes_strided", "fastmax_saved_state_bytes_strided",
+    "fastmax_forward_strided", "fastmax_backward_strided",
 )
 
 KERNEL_NAMES = ("rowstat", "build", "fwd_apply", "bwd_prep", "bwd_dq", "bwd_dk", "bwd_dv", "norm_fix")
@@ -44,6 +46,15 @@ class FastmaxDesc(C.Structure):
         ("p", C.c_int32), ("lim", C.c_float), ("temperature", C.c_float),
         ("a0", C.c_float), ("a1", C.c_float), ("a2", C.c_float),
     ]
+
+
+class FastmaxStrides(C.Structure):
+    _fields_ = [("batch", C.c_int64), ("group", C.c_int64), ("head", C.c_int64), ("token", C.c_int64)]
+
+
+class FastmaxLayout(C.Structure):
+    _fields_ = [("groups", C.c_int32), ("reserved", C.c_int32)] + [
+        (name, FastmaxStrides) for name in ("q", "k", "v", "o", "go", "dq", "dk", "dv")]
 
 
 class RopeDesc(C.Structure):
@@ -92,6 +103,18 @@ def load() -> C.CDLL:
     lib.fastmax_backward_saved.restype = C.c_int
     lib.fastmax_backward_saved.argtypes = [dp, vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, sz, vp,
                                            sz, vp]
+    lp = C.POINTER(FastmaxLayout)
+    lib.fastmax_workspace_bytes_strided.restype = sz
+    lib.fastmax_workspace_bytes_strided.argtypes = [dp, lp, C.c_int]
+    lib.fastmax_workspace_min_bytes_strided.restype = sz
+    lib.fastmax_workspace_min_bytes_strided.argtypes = [dp, lp, C.c_int]
+    lib.fastmax_saved_state_bytes_strided.restype = sz
+    lib.fastmax_saved_state_bytes_strided.argtypes = [dp, lp]
+    lib.fastmax_forward_strided.restype = C.c_int
+    lib.fastmax_forward_strided.argtypes = [dp, lp, vp, vp, vp, vp, vp, i64, vp, vp, vp, sz, vp, sz, vp]
+    lib.fastmax_backward_strided.restype = C.c_int
+    lib.fastmax_backward_strided.argtypes = [dp, lp, vp, vp, vp, vp, vp, i64, vp, vp, vp, vp, vp, vp, vp, sz, vp,
+                                             sz, vp]
     lib.fastmax_noalloc_scratch_bytes.restype = sz
     lib.fastmax_noalloc_scratch_bytes.argtypes = []
     lib.fastmax_forward_noalloc.restype = C.c_int

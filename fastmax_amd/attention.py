@@ -65,14 +65,11 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
         if pad:
             # zero channels change neither q.k nor the row norms, and give zero output columns
             q3, k3, v3 = (torch.nn.functional.pad(t, (0, pad)) for t in (q3, k3, v3))
-        # key prefix: nk - nq zero query rows in front.  They see only prefix keys, take no part in
-        # the row-norm maximum, and with a zero upstream gradient contribute nothing to dk, dv.
-        lead = k3.shape[1] - q3.shape[1]
-        if lead < 0:
+        # a key prefix (k, v longer than q under the mask: the first nk - nq keys are visible to every
+        # query, fastmax_cuda_forward.cu:109-150) goes to the library as it is
+        if mask and k3.shape[1] < q3.shape[1]:
             raise ValueError(f"k, v have {k3.shape[1]} tokens but q has {q3.shape[1]}: fewer keys than "
-                             "queries is not supported")
-        if lead:
-            q3 = torch.cat((q3.new_zeros(q3.shape[0], lead, q3.shape[2]), q3), dim=1)
+                             "queries is not supported under the causal mask")
         q3, k3, v3 = q3.contiguous(), k3.contiguous(), v3.contiguous()
         # keep the prefix states for the backward pass (it then skips rebuilding them) when a
         # backward pass will come and the states fit comfortably in free device memory
@@ -80,24 +77,20 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
         save = need_grad and _states_fit(q3, k3, bool(mask), int(p))
         o, den, scale, arg, saved = ext.forward_ex(q3, k3, v3, bool(mask), bool(normalize), float(temperature),
                                                    float(a0), float(a1), float(a2), float(lim), int(p), save)
-        if lead:
-            # a zero query row has den = a0 * (keys seen); keep its saved o, den harmless whatever a0 is
-            o[:, :lead] = 0
-            den[:, :lead] = 1
         noise = None
-        out = o[:, lead:] if lead else o
+        out = o
         if dropout and dropout > 0.0:
             if drop_noise is None:
                 raise ValueError("dropout > 0 needs drop_noise (a standard-normal tensor shaped like q)")
             # multiplicative Gaussian noise on the output, fastmax_cuda_forward.cu:271-280
-            noise = 1.0 + float(dropout) * drop_noise.reshape(q3.shape[0], q3.shape[1] - lead, -1).to(o.dtype)
+            noise = 1.0 + float(dropout) * drop_noise.reshape(q3.shape[0], q3.shape[1], -1).to(o.dtype)
             if pad:
                 noise = torch.nn.functional.pad(noise, (0, pad), value=1.0)
             out = out * noise
         ctx.save_for_backward(q3, k3, v3, o, den, scale, arg, noise if noise is not None else o.new_empty(0),
                               saved)
         ctx.cfg = (bool(mask), bool(normalize), float(temperature), float(a0), float(a1), float(a2), float(lim), int(p))
-        ctx.kshape, ctx.vshape, ctx.pad, ctx.lead = k.shape, v.shape, pad, lead
+        ctx.kshape, ctx.vshape, ctx.pad = k.shape, v.shape, pad
         if pad:
             out = out[..., :d]
         return out.reshape(shape)
@@ -107,19 +100,14 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
         ext = _ext.load()
         q3, k3, v3, o, den, scale, arg, noise, saved = ctx.saved_tensors
         mask, normalize, temperature, a0, a1, a2, lim, p = ctx.cfg
-        lead = ctx.lead
-        go = grad_output.reshape(q3.shape[0], q3.shape[1] - lead, -1)
+        go = grad_output.reshape(q3.shape[0], q3.shape[1], -1)
         if ctx.pad:
             go = torch.nn.functional.pad(go, (0, ctx.pad))
         if noise.numel():
             go = go * noise
-        if lead:
-            go = torch.cat((go.new_zeros(go.shape[0], lead, go.shape[2]), go), dim=1)
         go = go.contiguous()
         dq, dk, dv = ext.backward_ex(q3, k3, v3, o, den, go, scale, arg, mask, normalize, temperature,
                                      a0, a1, a2, lim, p, saved)
-        if lead:
-            dq = dq[:, lead:]
         if ctx.pad:
             d = grad_output.shape[-1]
             dq, dk, dv = dq[..., :d], dk[..., :d], dv[..., :d]

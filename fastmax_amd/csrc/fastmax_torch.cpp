@@ -146,9 +146,125 @@ std::vector<torch::Tensor> backward_ex(torch::Tensor q, torch::Tensor k, torch::
   return {dq, dk, dv};
 }
 
-// `lead` rows of zeros in front of a (bh, n, w) tensor.
-torch::Tensor lead_rows(const torch::Tensor& t, int64_t lead) {
-  return torch::cat({torch::zeros({t.size(0), lead, t.size(2)}, t.options()), t}, 1);
+// ---- strided tensors -----------------------------------------------------------------------
+// q, o, grad_output, dq: (B, G, R, T, D) views (G key/value groups of R query heads); k, v, dk, dv:
+// (B, G, T, D) views; any strides with unit channel stride, e.g. slices of the fused projection of a
+// GPT block (model.py:474-499) -- no .contiguous() copies (model.py:572-574) and no transpose of the
+// result (model.py:603).
+fastmax_strides strides5(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.dim() == 5 && t.stride(4) == 1, name, " must be a (B, G, R, T, D) view with unit channel stride");
+  return fastmax_strides{t.stride(0), t.stride(1), t.stride(2), t.stride(3)};
+}
+fastmax_strides strides4(const torch::Tensor& t, const char* name) {
+  TORCH_CHECK(t.dim() == 4 && t.stride(3) == 1, name, " must be a (B, G, T, D) view with unit channel stride");
+  return fastmax_strides{t.stride(0), t.stride(1), 0, t.stride(2)};
+}
+fastmax_desc make_desc5(const torch::Tensor& q, const torch::Tensor& k, bool mask, bool normalize,
+                        double temperature, double a0, double a1, double a2, double lim, int64_t p) {
+  TORCH_CHECK(q.dim() == 5 && k.dim() == 4 && k.size(0) == q.size(0) && k.size(1) == q.size(1) && k.size(3) == q.size(4),
+              "q must be (B, G, R, T, D) and k, v (B, G, T, D)");
+  TORCH_CHECK(q.scalar_type() == torch::kFloat32 || q.scalar_type() == torch::kBFloat16, "q must be float32 or bfloat16");
+  fastmax_desc ds;
+  ds.bh = (int32_t)(q.size(0) * q.size(1) * q.size(2));
+  ds.bhkv = (int32_t)(q.size(0) * q.size(1));
+  ds.nq = (int32_t)q.size(3);
+  ds.nk = (int32_t)k.size(2);
+  ds.d = (int32_t)q.size(4);
+  ds.dtype = q.scalar_type() == torch::kFloat32 ? FASTMAX_F32 : FASTMAX_BF16;
+  ds.mask = mask;
+  ds.normalize = normalize;
+  ds.p = (int32_t)p;
+  ds.lim = (float)lim;
+  ds.temperature = (float)temperature;
+  ds.a0 = (float)a0;
+  ds.a1 = (float)a1;
+  ds.a2 = (float)a2;
+  raise_on(fastmax_check_desc(&ds));
+  return ds;
+}
+
+// (o, den, qk_scale, qk_argmax, saved_states); o is the (B, G, R, T, D) view of freshly allocated
+// token-major (B, T, G, R, D) memory.
+std::vector<torch::Tensor> forward_strided(torch::Tensor q, torch::Tensor k, torch::Tensor v, bool mask,
+                                           bool normalize, double temperature, double a0, double a1,
+                                           double a2, double lim, int64_t p, bool save_states) {
+  CHECK_GPU(q);
+  CHECK_GPU(k);
+  CHECK_GPU(v);
+  check_same(q, k, "k");
+  check_same(q, v, "v");
+  TORCH_CHECK(k.sizes() == v.sizes(), "k and v must have the same shape");
+  const fastmax_desc ds = make_desc5(q, k, mask, normalize, temperature, a0, a1, a2, lim, p);
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+  auto o = torch::empty({q.size(0), q.size(3), q.size(1), q.size(2), q.size(4)}, q.options()).permute({0, 2, 3, 1, 4});
+  fastmax_layout lay{};
+  lay.groups = (int32_t)q.size(1);
+  lay.q = strides5(q, "q");
+  lay.k = strides4(k, "k");
+  lay.v = strides4(v, "v");
+  lay.o = strides5(o, "o");
+  auto den = torch::empty({(int64_t)ds.bh, q.size(3)}, q.options().dtype(torch::kFloat32));
+  auto scale = torch::empty({2 * (int64_t)ds.bh}, q.options().dtype(torch::kFloat32));
+  auto arg = torch::empty({2 * (int64_t)ds.bh}, q.options().dtype(torch::kInt32));
+  size_t wsb = 0;
+  torch::Tensor ws, saved;
+  if (save_states) {
+    const size_t sb = fastmax_saved_state_bytes_strided(&ds, &lay);
+    TORCH_CHECK(sb > 0, "fastmax: ", fastmax_last_error());
+    saved = torch::empty({(int64_t)sb}, q.options().dtype(torch::kUInt8));
+    wsb = (size_t)16 * ds.bh + 512;
+  } else {
+    saved = torch::empty({0}, q.options().dtype(torch::kUInt8));
+    wsb = fastmax_workspace_bytes_strided(&ds, &lay, FASTMAX_PASS_FORWARD);
+    TORCH_CHECK(wsb > 0, "fastmax: ", fastmax_last_error());
+  }
+  ws = torch::empty({(int64_t)wsb}, q.options().dtype(torch::kUInt8));
+  raise_on(fastmax_forward_strided(&ds, &lay, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                   den.data_ptr<float>(), 1, scale.data_ptr<float>(), arg.data_ptr<int32_t>(),
+                                   ws.data_ptr(), wsb, save_states ? saved.data_ptr() : nullptr,
+                                   (size_t)saved.numel(), current_stream(q)));
+  return {o, den, scale, arg, saved};
+}
+
+// Writes dq, dk, dv into the views the caller hands in (e.g. slices of the gradient of the fused
+// projection).
+void backward_strided(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor o, torch::Tensor den,
+                      torch::Tensor go, torch::Tensor scale, torch::Tensor arg, torch::Tensor dq, torch::Tensor dk,
+                      torch::Tensor dv, bool mask, bool normalize, double temperature, double a0, double a1,
+                      double a2, double lim, int64_t p, torch::Tensor saved) {
+  for (const torch::Tensor* t : {&q, &k, &v, &o, &go, &dq, &dk, &dv}) {
+    TORCH_CHECK(t->device().is_cuda() && t->device() == q.device() && t->scalar_type() == q.scalar_type(),
+                "all tensors must live on q's device and share its dtype");
+  }
+  CHECK_INPUT(den);
+  CHECK_INPUT(scale);
+  CHECK_INPUT(arg);
+  TORCH_CHECK(o.sizes() == q.sizes() && go.sizes() == q.sizes() && dq.sizes() == q.sizes(), "o, grad_output and dq must be shaped like q");
+  TORCH_CHECK(k.sizes() == v.sizes() && dk.sizes() == k.sizes() && dv.sizes() == k.sizes(), "v, dk and dv must be shaped like k");
+  const fastmax_desc ds = make_desc5(q, k, mask, normalize, temperature, a0, a1, a2, lim, p);
+  TORCH_CHECK(den.scalar_type() == torch::kFloat32 && den.numel() == (int64_t)ds.bh * ds.nq, "den must be float32 (bh, n)");
+  TORCH_CHECK(scale.scalar_type() == torch::kFloat32 && scale.numel() == 2 * (int64_t)ds.bh, "qk_scale must be float32 (2*bh)");
+  TORCH_CHECK(arg.scalar_type() == torch::kInt32 && arg.numel() == 2 * (int64_t)ds.bh, "qk_argmax must be int32 (2*bh)");
+  const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
+  fastmax_layout lay{};
+  lay.groups = (int32_t)q.size(1);
+  lay.q = strides5(q, "q");
+  lay.k = strides4(k, "k");
+  lay.v = strides4(v, "v");
+  lay.o = strides5(o, "o");
+  lay.go = strides5(go, "grad_output");
+  lay.dq = strides5(dq, "dq");
+  lay.dk = strides4(dk, "dk");
+  lay.dv = strides4(dv, "dv");
+  const size_t wsb = fastmax_workspace_bytes_strided(&ds, &lay, FASTMAX_PASS_BACKWARD);
+  TORCH_CHECK(wsb > 0, "fastmax: ", fastmax_last_error());
+  auto ws = torch::empty({(int64_t)wsb}, q.options().dtype(torch::kUInt8));
+  const bool have_saved = saved.defined() && saved.numel() > 0;
+  raise_on(fastmax_backward_strided(&ds, &lay, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
+                                    den.data_ptr<float>(), 1, go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                    scale.data_ptr<float>(), arg.data_ptr<int32_t>(), ws.data_ptr(), wsb,
+                                    have_saved ? saved.data_ptr() : nullptr,
+                                    have_saved ? (size_t)(saved.numel() * saved.element_size()) : 0, current_stream(q)));
 }
 
 // Reference signature and side effects (fastmax_cuda.cpp:17-24, fastmax_cuda_forward.cu:366-399):
@@ -156,8 +272,7 @@ torch::Tensor lead_rows(const torch::Tensor& t, int64_t lead) {
 // q, k are the ones backwardpass expects; the result is (bh, nq, d+1) with the row denominators
 // in column d; dropout > 0 multiplies the output by 1 + dropout * drop_noise.
 // k, v longer than q (fastmax_cuda_forward.cu:109-150: the first nk - nq keys are visible to
-// every query): the pass runs on q with nk - nq zero rows in front, which see only those keys,
-// do not move the row-norm maximum and are cut from the result.
+// every query) go to the library as they are: the descriptor carries nq and nk.
 torch::Tensor forwardpass(torch::Tensor q, torch::Tensor k, torch::Tensor v, torch::Tensor drop_noise,
                           bool mask, double dropout, bool normalize, double temperature, double a0,
                           double a1, double a2, double lim, int64_t p) {
@@ -170,27 +285,21 @@ torch::Tensor forwardpass(torch::Tensor q, torch::Tensor k, torch::Tensor v, tor
   TORCH_CHECK(q.dim() == 3 && k.dim() == 3, "q, k, v must be (b*h, n, d)");
   TORCH_CHECK(k.sizes() == v.sizes() && k.size(2) == q.size(2),
               "k and v must have the same shape and q's head dimension");
-  const int64_t lead = k.size(1) - q.size(1);
-  TORCH_CHECK(lead >= 0, "k, v have ", k.size(1), " tokens but q has ", q.size(1),
-              ": fewer keys than queries is not supported");
   const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
-  torch::Tensor qp = lead ? lead_rows(q, lead) : q;
-  fastmax_desc ds = make_desc(qp, k, mask, normalize, 1.0, a0, a1, a2, lim, p);
+  fastmax_desc ds = make_desc(q, k, mask, normalize, 1.0, a0, a1, a2, lim, p);
   const fastmax_stream_t stream = current_stream(q);
   if (temperature != 1.0) k.div_(temperature);
   if (normalize) {
     auto nws = torch::empty({16 * (int64_t)ds.bh + 1024}, q.options().dtype(torch::kUInt8));
-    raise_on(fastmax_normalize_inplace(&ds, qp.data_ptr(), k.data_ptr(), nws.data_ptr(), (size_t)nws.numel(), stream));
+    raise_on(fastmax_normalize_inplace(&ds, q.data_ptr(), k.data_ptr(), nws.data_ptr(), (size_t)nws.numel(), stream));
     ds.normalize = 0;
-    if (lead) q.copy_(qp.narrow(1, lead, q.size(1)));
   }
   const int64_t d = q.size(2);
-  auto o = torch::empty({qp.size(0), qp.size(1), d + 1}, q.options());
+  auto o = torch::empty({q.size(0), q.size(1), d + 1}, q.options());
   size_t wsb = 0;
   auto ws = workspace(ds, FASTMAX_PASS_FORWARD, q, &wsb);
-  raise_on(fastmax_forward(&ds, qp.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d + 1,
+  raise_on(fastmax_forward(&ds, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), d + 1,
                            o.data_ptr<float>() + d, d + 1, nullptr, nullptr, ws.data_ptr(), wsb, stream));
-  if (lead) o = o.narrow(1, lead, q.size(1)).contiguous();
   if (dropout > 0.0) {
     TORCH_CHECK(drop_noise.defined() && drop_noise.sizes() == q.sizes(), "drop_noise must be shaped like q");
     o.narrow(2, 0, d).mul_(drop_noise * dropout + 1.0);
@@ -220,18 +329,7 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
               "o must be the (bh, n, d+1) tensor forwardpass returned");
   TORCH_CHECK(grad_output.sizes() == q.sizes(), "grad_output must be shaped like q");
   TORCH_CHECK(k.sizes() == v.sizes() && k.size(2) == d, "k and v must have the same shape and q's head dimension");
-  const int64_t lead = k.size(1) - q.size(1);
-  TORCH_CHECK(lead >= 0, "k, v have ", k.size(1), " tokens but q has ", q.size(1),
-              ": fewer keys than queries is not supported");
   const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device());
-  if (lead) {
-    // key prefix: zero query rows in front with a zero upstream gradient add nothing to dk, dv;
-    // their denominator column is set to 1 so that 0 / den stays 0 whatever a0 is
-    q = lead_rows(q, lead);
-    grad_output = lead_rows(grad_output, lead);
-    o = lead_rows(o, lead);
-    o.narrow(1, 0, lead).select(2, d).fill_(1.0);
-  }
   const fastmax_desc ds = make_desc(q, k, mask, false, 1.0, a0, a1, a2, 1.0, p);
   auto dq = torch::empty_like(q);
   auto dk = torch::empty_like(k);
@@ -242,7 +340,6 @@ std::vector<torch::Tensor> backwardpass(torch::Tensor q, torch::Tensor k, torch:
                             o.data_ptr<float>() + d, d + 1, grad_output.data_ptr(), dq.data_ptr(),
                             dk.data_ptr(), dv.data_ptr(), nullptr, nullptr, ws.data_ptr(), wsb,
                             current_stream(q)));
-  if (lead) dq = dq.narrow(1, lead, dq.size(1) - lead).contiguous();
   return {dq, dk, dv};
 }
 
@@ -273,5 +370,7 @@ PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("backwardpass", &backwardpass, "backwardpass");
   m.def("forward_ex", &forward_ex, "forward returning (o, den, qk_scale, qk_argmax, saved_states)");
   m.def("backward_ex", &backward_ex, "backward through the normalisation, returns [dq, dk, dv]");
+  m.def("forward_strided", &forward_strided, "forward on strided (B, G, R, T, D) / (B, G, T, D) views");
+  m.def("backward_strided", &backward_strided, "backward on strided views, writes dq, dk, dv in place");
   m.def("version", []() { return std::string(fastmax_version()); });
 }

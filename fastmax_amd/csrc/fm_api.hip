@@ -78,14 +78,20 @@ constexpr int kChunk = 384;
 constexpr size_t kWorkspaceBudget = 16ull << 30;   // what fastmax_workspace_bytes aims for
 
 struct Plan {
-  int d, p2, masked, n, bh;
+  int d, p2, masked, bh;
+  int nq, nk;          // query rows, key rows per head
+  int n;               // positions the scans and state slots are laid out over: nk under the causal
+                       // mask (queries sit at positions off .. nk-1), max(nq, nk) otherwise
+  int off;             // causal: position of the first query, nk - nq (the key prefix); else 0
+  int nblk_q, nblk_k;  // 128-token blocks launched by the kernels whose own rows are query-side /
+                       // key-side tensors
   int bhkv, ratio;     // key/value heads; query heads per key/value head
   int rtw, gsplit;     // build kernel: row tiles per wave, feature splits per head
   int nslots, zlen;    // state slots per head; tokens per slot when unmasked
   int nparts;          // token splits the unmasked build sums separately (1 when masked); bf16
                        // inputs add one slot that receives their sum in packed form
   int chunk;           // tokens between causal state snapshots
-  int nblk;            // 128-token blocks per head
+  bool plain;          // every tensor is a plain contiguous (heads, tokens, d) array
   bool scan;           // causal p = 1 as one scan per head (fm_linear.h): no states in memory
   bool rowpass;        // unmasked p = 1: states from the build kernel, one pass over the rows per output
   int64_t state_floats;
@@ -112,12 +118,18 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 #endif
 bool use_linear_scan(const fastmax_desc* ds, const Plan& pl);
 
-Plan make_plan(const fastmax_desc* ds, int pass) {
+Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true) {
   Plan pl;
   pl.d = ds->d;
   pl.p2 = ds->p == 2;
   pl.masked = ds->mask != 0;
-  pl.n = ds->nq;
+  pl.plain = plain;
+  pl.nq = ds->nq;
+  pl.nk = ds->nk;
+  pl.n = pl.masked ? ds->nk : (ds->nq > ds->nk ? ds->nq : ds->nk);
+  pl.off = pl.masked ? ds->nk - ds->nq : 0;
+  pl.nblk_k = (ds->nk + 127) / 128;
+  pl.nblk_q = pl.masked ? pl.nblk_k - pl.off / 128 : (ds->nq + 127) / 128;
   pl.bh = ds->bh;
   pl.bhkv = ds->bhkv;
   pl.ratio = ds->bh / ds->bhkv;
@@ -134,7 +146,6 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
     pl.rtw = 5;
   }
   pl.gsplit = splits(pl.rtw);
-  pl.nblk = (pl.n + 127) / 128;
   // p = 1: a state is only (d+1) rows, so a snapshot per 128-token block is cheaper than a longer
   // intra-chunk part
   pl.chunk = pl.p2 ? kChunk : kChunkP1;
@@ -158,25 +169,25 @@ Plan make_plan(const fastmax_desc* ds, int pass) {
   pl.state_floats = slot_floats_for(pl.d, pl.p2, pl.masked && ds->dtype == FASTMAX_BF16);
   size_t fixed = align256((size_t)2 * pl.bh * sizeof(float)) + align256((size_t)2 * pl.bh * sizeof(int));
   if (pass == FASTMAX_PASS_BACKWARD) {
-    fixed += align256((size_t)pl.bh * pl.n * sizeof(float));            // c_i
-    fixed += align256((size_t)2 * pl.bh * pl.nblk * sizeof(float));     // norm partials for q, k
+    fixed += align256((size_t)pl.bh * pl.nq * sizeof(float));                        // c_i
+    fixed += align256((size_t)pl.bh * (pl.nblk_q + pl.nblk_k) * sizeof(float));      // norm partials for q, k
   }
   pl.fixed_bytes = fixed;
   pl.per_head_bytes = (size_t)pl.nslots * pl.state_floats * sizeof(float) *
                       (pass == FASTMAX_PASS_BACKWARD ? 2 : 1);
   // grouped key/value heads, backward: dk and dv are formed per query head and then added up
   if (pass == FASTMAX_PASS_BACKWARD && pl.ratio > 1)
-    pl.per_head_bytes += 2 * (size_t)pl.n * pl.d * (ds->dtype == FASTMAX_BF16 ? 2 : 4);
+    pl.per_head_bytes += 2 * (size_t)pl.nk * pl.d * (ds->dtype == FASTMAX_BF16 ? 2 : 4);
   pl.scan = use_linear_scan(ds, pl);
   if (pl.scan) pl.per_head_bytes = 0;
-  pl.rowpass = !pl.p2 && !pl.masked && pl.d == 64 && pl.ratio == 1 && pl.n >= 32;
+  pl.rowpass = !pl.p2 && !pl.masked && pl.d == 64 && pl.ratio == 1 && pl.n >= 32 && pl.plain && pl.nq == pl.nk;
   return pl;
 }
 
 bool use_linear_scan(const fastmax_desc* ds, const Plan& pl) {
   // (its kernels keep the weights divided by a1, and every tile is a full 32 rows)
   return !pl.p2 && pl.masked && pl.d == 64 && pl.ratio == 1 && pl.n >= 32 && ds->a1 != 0.f &&
-         pl.bh >= FM_LINEAR_MIN_HEADS;
+         pl.bh >= FM_LINEAR_MIN_HEADS && pl.plain && pl.nq == pl.nk;
 }
 
 // Heads per launch that fit the workspace.  When several batches are needed the batch is
@@ -213,8 +224,11 @@ int check_desc(const fastmax_desc* ds) {
   if (ds->bhkv < 1 || ds->bh % ds->bhkv != 0)
     return fail(FASTMAX_E_SHAPE, "bhkv = %d does not divide bh = %d", ds->bhkv, ds->bh);
   if (ds->nq < 1) return fail(FASTMAX_E_SHAPE, "nq = %d < 1", ds->nq);
-  if (ds->nk != ds->nq) return fail(FASTMAX_E_SHAPE, "nk = %d != nq = %d: a key prefix is not supported", ds->nk, ds->nq);
-  if ((int64_t)ds->nq * ds->d * ds->bh >= (int64_t)1 << 40) return fail(FASTMAX_E_SHAPE, "tensor too large");
+  if (ds->nk < 1) return fail(FASTMAX_E_SHAPE, "nk = %d < 1", ds->nk);
+  if (ds->mask && ds->nk < ds->nq)
+    return fail(FASTMAX_E_SHAPE, "nk = %d < nq = %d under the causal mask (the keys are a prefix plus one per query)", ds->nk, ds->nq);
+  if ((int64_t)(ds->nq > ds->nk ? ds->nq : ds->nk) * ds->d * ds->bh >= (int64_t)1 << 40)
+    return fail(FASTMAX_E_SHAPE, "tensor too large");
   if (ds->p != 1 && ds->p != 2) return fail(FASTMAX_E_PARAM, "p must be 1 or 2, got: %d", ds->p);
   if (ds->normalize) {
     if (!(ds->lim > 0.f)) return fail(FASTMAX_E_PARAM, "lim = %g must be positive when normalize is set", (double)ds->lim);
@@ -259,17 +273,78 @@ int launch_status(const char* what) {
     if (rc_ != FASTMAX_OK) return rc_; \
   } while (0)
 
+// Strides of one tensor (elements): head h sits at (h / (ng nh)) sb + ((h / nh) % ng) sg + (h % nh) sh
+struct Str {
+  int64_t sb, sg, sh, pitch;
+  int ng, nh;
+};
+// a plain (heads, rows, pitch) array
+Str plain_str(int64_t rows, int64_t pitch) { return Str{rows * pitch, 0, 0, pitch, 1, 1}; }
+// levels with uniform strides are merged (a contiguous tensor ends up as one level)
+Str make_str(const fastmax_strides& f, int groups, int heads_per_group) {
+  Str t{f.batch, f.group, heads_per_group > 1 ? f.head : 0, f.token, groups, heads_per_group};
+  if (t.nh > 1 && t.sg == t.nh * t.sh) {
+    t.ng *= t.nh;
+    t.sg = t.sh;
+    t.nh = 1;
+    t.sh = 0;
+  }
+  if (t.nh == 1 && t.sb == t.ng * t.sg) {
+    t.sb = t.sg;
+    t.ng = 1;
+    t.sg = 0;
+  }
+  return t;
+}
+struct Layout {
+  Str q, k, v, o, go, dq, dk, dv;
+};
+Layout plain_layout(const fastmax_desc* ds, int64_t ldo) {
+  const Str tq = plain_str(ds->nq, ds->d), tk = plain_str(ds->nk, ds->d);
+  return Layout{tq, tk, tk, plain_str(ds->nq, ldo), tq, tq, tk, tk};
+}
+bool is_plain(const Str& t, int64_t rows, int64_t pitch) { return t.ng == 1 && t.nh == 1 && t.pitch == pitch && t.sb == rows * pitch; }
+bool is_plain(const Layout& L, const fastmax_desc* ds, bool backward) {
+  const int d = ds->d;
+  bool ok = is_plain(L.q, ds->nq, d) && is_plain(L.k, ds->nk, d) && is_plain(L.v, ds->nk, d) &&
+            L.o.ng == 1 && L.o.nh == 1 && L.o.sb == ds->nq * L.o.pitch;
+  if (backward)
+    ok = ok && is_plain(L.go, ds->nq, d) && is_plain(L.dq, ds->nq, d) && is_plain(L.dk, ds->nk, d) &&
+         is_plain(L.dv, ds->nk, d);
+  return ok;
+}
+
+// first head of a batch h0, first position lo (the pointer is moved back by lo rows, so that
+// position t >= lo is row t - lo of the tensor)
+template <class T>
+Rows<T> mk_rows(T* p, const Str& t, int h0 = 0, int lo = 0) {
+  return Rows<T>{p - (int64_t)lo * t.pitch, t.sb, t.sg, t.sh, t.pitch, t.ng, t.nh, h0, lo};
+}
+template <class F>
+RowScalarsT<F> mk_scalars(F* p, int64_t rows, int64_t stride, int h0 = 0, int lo = 0) {
+  if (!p) return RowScalarsT<F>{nullptr, 0, 0};
+  return RowScalarsT<F>{p + ((int64_t)h0 * rows - lo) * stride, rows * stride, stride};
+}
+const RowScalars kNoScalars{nullptr, 0, 0};
+
+// the kernels read and write whole 16-byte pieces of rows
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+bool aligned16(const Str& t, size_t es) {
+  return (t.sb * es) % 16 == 0 && (t.sg * es) % 16 == 0 && (t.sh * es) % 16 == 0 && (t.pitch * es) % 16 == 0;
+}
+
 // scale[0..bh) for q, scale[bh..2bh) for k
 template <class T>
-int compute_scales(const fastmax_desc* ds, const T* q, const T* k, float* scale, int* arg,
+int compute_scales(const fastmax_desc* ds, const Layout& L, const T* q, const T* k, float* scale, int* arg,
                    hipStream_t stream) {
   const int bh = ds->bh, bhkv = ds->bhkv;
   ScopedKernel sk(FASTMAX_K_ROWSTAT, stream);
   if (ds->normalize) {
-    if (bh >= 512) rowstat_kernel<T, 256><<<bh, 256, 0, stream>>>(q, ds->nq, ds->d, ds->lim, scale, arg);
-    else rowstat_kernel<T, 1024><<<bh, 1024, 0, stream>>>(q, ds->nq, ds->d, ds->lim, scale, arg);
-    if (bhkv >= 512) rowstat_kernel<T, 256><<<bhkv, 256, 0, stream>>>(k, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
-    else rowstat_kernel<T, 1024><<<bhkv, 1024, 0, stream>>>(k, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
+    const Rows<const T> qr = mk_rows(q, L.q), kr = mk_rows(k, L.k);
+    if (bh >= 512) rowstat_kernel<T, 256><<<bh, 256, 0, stream>>>(qr, ds->nq, ds->d, ds->lim, scale, arg);
+    else rowstat_kernel<T, 1024><<<bh, 1024, 0, stream>>>(qr, ds->nq, ds->d, ds->lim, scale, arg);
+    if (bhkv >= 512) rowstat_kernel<T, 256><<<bhkv, 256, 0, stream>>>(kr, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
+    else rowstat_kernel<T, 1024><<<bhkv, 1024, 0, stream>>>(kr, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
   } else {
     fill_scale_kernel<<<(bh + 255) / 256, 256, 0, stream>>>(scale, arg, bh, 1.0f);
     fill_scale_kernel<<<(bhkv + 255) / 256, 256, 0, stream>>>(scale + bh, arg + bh, bhkv, 1.0f / ds->temperature);
@@ -283,16 +358,17 @@ constexpr bool kBf16Mfma = false;
 template <>
 constexpr bool kBf16Mfma<bf16_t> = true;
 
+// State of (X, Y, extra) over n positions of `heads` heads (X.h0 is the first of them).
 template <int D, class T>
-int launch_build(const Plan& pl, int heads, const T* X, const T* Y, const float* xscale,
-                 const float* yden, int64_t yden_stride, const float* ew, float* state, int reverse,
+int launch_build(const Plan& pl, int heads, int n, const Rows<const T>& X, const Rows<const T>& Y,
+                 const float* xscale, const RowScalars& yden, const RowScalars& ew, float* state, int reverse,
                  hipStream_t stream, bool finish = true) {
   const dim3 grid(pl.gsplit, heads, pl.nparts);
   if (pl.masked && pl.nslots < 2) return FASTMAX_OK;  // a single chunk never needs a state
   ScopedKernel sk(FASTMAX_K_BUILD, stream);
 #define FM_BUILD(RTW)                                                                            \
-  build_kernel<D, T, RTW, kBf16Mfma<T>><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, yden_stride, ew, state, \
-                                                    pl.n, pl.chunk, pl.nslots, pl.masked, reverse, \
+  build_kernel<D, T, RTW, kBf16Mfma<T>><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, ew, state, \
+                                                    n, pl.chunk, pl.nslots, pl.masked, reverse, \
                                                     pl.p2, pl.zlen)
   if (pl.rtw == 1) {
     FM_BUILD(1);
@@ -327,10 +403,11 @@ inline int finish_state_fp32(const Plan& pl, int heads, float* state, hipStream_
 }
 
 template <int D, class T>
-int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k, const T* v, T* o,
-                 int64_t ldo, float* den, int64_t den_stride, float* scale_out, int32_t* arg_out,
+int forward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v, T* o,
+                 float* den, int64_t den_stride, float* scale_out, int32_t* arg_out,
                  char* ws, size_t ws_bytes, float* saved, hipStream_t stream) {
-  const int bh = pl.bh, n = pl.n;
+  const int bh = pl.bh, nq = pl.nq, nk = pl.nk;
+  const int64_t ldo = L.o.pitch;
   // per-head factors and arg-max rows: straight into the caller's arrays when it wants them
   float* scale = scale_out ? scale_out : reinterpret_cast<float*>(ws);
   int* arg = arg_out ? arg_out : reinterpret_cast<int*>(ws + align256((size_t)2 * bh * sizeof(float)));
@@ -339,10 +416,11 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   const int hb = heads_per_batch(pl, ws_bytes, saved != nullptr);
   const int64_t head_floats = (int64_t)pl.nslots * pl.state_floats;
 
-  FM_TRY(compute_scales<T>(ds, q, k, scale, arg, stream));
+  FM_TRY(compute_scales<T>(ds, L, q, k, scale, arg, stream));
 
   if constexpr (D == 64) {
-    if (pl.scan) {
+    if (pl.scan) {   // (plain tensors, nq == nk)
+      const int n = nq;
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       // (pairs of output columns go out as one store when the row pitch keeps them aligned)
       if (ldo % 2 == 0)
@@ -356,17 +434,19 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   }
 
   const int ratio = pl.ratio;
+  // positions the consumers' own rows run over (the queries sit at off .. nk-1 under the mask)
+  const int nown = pl.masked ? nk : nq;
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
-    const int64_t off = (int64_t)h0 * n * D;             // query-head tensors
     const int kv0 = h0 / ratio;                          // first key/value head of the batch
-    const int64_t koff = (int64_t)kv0 * n * D;
     float* state = saved ? saved + kv0 * head_floats : reinterpret_cast<float*>(ws + pl.fixed_bytes);
-    // (bf16: a saved state is also read by the dq kernel, which needs the column-packed section)
     if constexpr (D == 64) {
-      if (pl.rowpass) {
-        FM_TRY((launch_build<D, T>(pl, heads, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state, 0,
-                                   stream, false)));
+      if (pl.rowpass) {   // (plain tensors, nq == nk)
+        const int n = nq;
+        const int64_t off = (int64_t)h0 * n * D, koff = (int64_t)kv0 * n * D;
+        FM_TRY((launch_build<D, T>(pl, heads, n, mk_rows(k, L.k, kv0), mk_rows(v, L.v, kv0), scale + bh + kv0, kNoScalars,
+                                   kNoScalars, state, 0, stream, false)));
+        (void)koff;
         const int slot = finish_state_fp32(pl, heads, state, stream);
         ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
         const dim3 rgrid((n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE, heads);
@@ -380,20 +460,22 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
         continue;
       }
     }
-    FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr,
-                               state, 0, stream)));
+    const Rows<const T> kr = mk_rows(k, L.k, kv0), vr = mk_rows(v, L.v, kv0);
+    FM_TRY((launch_build<D, T>(pl, heads / ratio, nk, kr, vr, scale + bh + kv0, kNoScalars, kNoScalars, state, 0,
+                               stream)));
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
-      const dim3 agrid(pl.nblk, heads);
+      const dim3 agrid(pl.nblk_q, heads);
+      const Rows<const T> qr = mk_rows(q, L.q, h0, pl.off);
+      const Rows<T> orow = mk_rows(o, L.o, h0, pl.off);
+      const RowScalarsOut dn = mk_scalars(den, nq, den_stride, h0, pl.off);
       if constexpr (kBf16Mfma<T>) {
         apply_kernel_bf<D, 0><<<agrid, 256, 0, stream>>>(
-            q + off, k + koff, v + koff, scale + h0, scale + bh + kv0, nullptr, 0, state, pl.nslots,
-            o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, pl.chunk,
+            qr, kr, vr, scale + h0, scale + bh + kv0, kNoScalars, state, pl.nslots, orow, dn, nown, pl.chunk,
             pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f, 1, ratio);
       } else {
         apply_kernel<D, T, 0><<<agrid, 256, 0, stream>>>(
-            q + off, k + koff, v + koff, scale + h0, scale + bh + kv0, nullptr, 0, state, pl.nslots,
-            o + (int64_t)h0 * n * ldo, ldo, den + (int64_t)h0 * n * den_stride, den_stride, n, pl.chunk,
+            qr, kr, vr, scale + h0, scale + bh + kv0, kNoScalars, state, pl.nslots, orow, dn, nown, pl.chunk,
             pl.masked, pl.p2, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f, 1, ratio);
       }
     }
@@ -402,28 +484,31 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k,
   return FASTMAX_OK;
 }
 
-// c_i = go_i . o_i / den_i for every token: 16-byte accesses when the rows of o allow it
+// c_i = go_i . o_i / den_i for every query row: 16-byte accesses when the rows of o allow it
 template <int D, class T>
-int launch_bwd_prep(const T* go, const T* o, int64_t ldo, const float* den, int64_t den_stride, float* cvec,
-                    int64_t rows, hipStream_t stream) {
+int launch_bwd_prep(const Plan& pl, const Layout& L, const T* go, const T* o, const float* den, int64_t den_stride,
+                    float* cvec, hipStream_t stream) {
   ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
-  const bool vec = (ldo * sizeof(T)) % 16 == 0 && ((uintptr_t)o & 15) == 0 && ((uintptr_t)go & 15) == 0;
+  const bool vec = aligned16(L.o, sizeof(T)) && aligned16(o) && aligned16(L.go, sizeof(T)) && aligned16(go);
+  const Rows<const T> gr = mk_rows(go, L.go), orow = mk_rows(o, L.o);
+  const RowScalars dn = mk_scalars(den, pl.nq, den_stride);
   if (vec) {
     const int rpp = 256 / (D * (int)sizeof(T) / 16);
-    bwd_prep_kernel<T, true><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
+    bwd_prep_kernel<T, true><<<dim3((pl.nq + rpp - 1) / rpp, pl.bh), 256, 0, stream>>>(gr, orow, dn, cvec, pl.nq, D);
   } else {
     const int rpp = 256 / (D / 4);
-    bwd_prep_kernel<T, false><<<(unsigned)((rows + rpp - 1) / rpp), 256, 0, stream>>>(go, o, ldo, den, den_stride, cvec, rows, D);
+    bwd_prep_kernel<T, false><<<dim3((pl.nq + rpp - 1) / rpp, pl.bh), 256, 0, stream>>>(gr, orow, dn, cvec, pl.nq, D);
   }
   return launch_status("bwd_prep_kernel");
 }
 
 template <int D, class T>
-int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k, const T* v,
-                  const T* o, int64_t ldo, const float* den, int64_t den_stride, const T* go, T* dq,
+int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v,
+                  const T* o, const float* den, int64_t den_stride, const T* go, T* dq,
                   T* dk, T* dv, const float* scale_in, const int32_t* arg_in, char* ws,
                   size_t ws_bytes, const float* saved, hipStream_t stream) {
-  const int bh = pl.bh, n = pl.n;
+  const int bh = pl.bh, nq = pl.nq, nk = pl.nk;
+  const int64_t ldo = L.o.pitch;
   char* p = ws;
   const bool given = scale_in && arg_in;  // the forward pass's values: read in place
   const float* scale = given ? scale_in : reinterpret_cast<float*>(p);
@@ -433,14 +518,16 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
   int* arg_ws = reinterpret_cast<int*>(p);
   p += align256((size_t)2 * bh * sizeof(int));
   float* cvec = reinterpret_cast<float*>(p);
-  p += align256((size_t)bh * n * sizeof(float));
-  float* rpart = reinterpret_cast<float*>(p);
+  p += align256((size_t)bh * nq * sizeof(float));
+  float* rpart = reinterpret_cast<float*>(p);           // q: bh x nblk_q, then k: bh x nblk_k
+  float* rpart_k = rpart + (int64_t)bh * pl.nblk_q;
   float* state = reinterpret_cast<float*>(ws + pl.fixed_bytes);
   const int hb = heads_per_batch(pl, ws_bytes, saved != nullptr);
 
-  if (!given) FM_TRY(compute_scales<T>(ds, q, k, scale_ws, arg_ws, stream));
+  if (!given) FM_TRY(compute_scales<T>(ds, L, q, k, scale_ws, arg_ws, stream));
   if constexpr (D == 64) {
-    if (pl.scan) {
+    if (pl.scan) {   // (plain tensors, nq == nk)
+      const int n = nq;
       const float* qs = scale;
       const float* ks = scale + bh;
       // one normalisation partial per head, shared by q and k:
@@ -450,7 +537,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       // separate pass does
       const bool prep_in_dq = ldo == D;
       if (!prep_in_dq) {
-        FM_TRY((launch_bwd_prep<D, T>(go, o, ldo, den, den_stride, cvec, (int64_t)bh * n, stream)));
+        FM_TRY((launch_bwd_prep<D, T>(pl, L, go, o, den, den_stride, cvec, stream)));
       }
       {
         ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
@@ -477,50 +564,46 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
       FM_TRY(launch_status("linear_dv_kernel"));
       if (ds->normalize) {
         ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
-        norm_fix_kernel<T><<<bh, D, 0, stream>>>(dq, q, qs, arg, rq, 1, n, D, ds->lim);
-        norm_fix_kernel<T><<<bh, D, 0, stream>>>(dk, k, ks, arg + bh, rq, 1, n, D, ds->lim);
+        norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), qs, arg, rq, 1, n, D, ds->lim);
+        norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), ks, arg + bh, rq, 1, n, D, ds->lim);
         FM_TRY(launch_status("norm_fix_kernel"));
       }
       return FASTMAX_OK;
     }
   }
   {
-    FM_TRY((launch_bwd_prep<D, T>(go, o, ldo, den, den_stride, cvec, (int64_t)bh * n, stream)));
+    FM_TRY((launch_bwd_prep<D, T>(pl, L, go, o, den, den_stride, cvec, stream)));
   }
   const float a2 = pl.p2 ? ds->a2 : 0.f;
   const int ratio = pl.ratio, bhkv = pl.bhkv;
   const int64_t state_bytes = (int64_t)pl.nslots * pl.state_floats * sizeof(float);
+  // positions the own rows of the query-side / key-side kernels run over, and where the query-side
+  // rows start (the queries sit at positions off .. nk-1 under the mask)
+  const int nown_q = pl.masked ? nk : nq, nown_k = nk, off = pl.off;
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
-    const int64_t off = (int64_t)h0 * n * D;   // query-head tensors
     const int kv0 = h0 / ratio;                // first key/value head of the batch
-    const int64_t koff = (int64_t)kv0 * n * D;
     // prefix states: the ones the forward pass saved, or rebuilt into the workspace
     const float* stS = saved ? saved + (int64_t)kv0 * pl.nslots * pl.state_floats : state;
     float* stR = saved ? state : state + (int64_t)hb * pl.nslots * pl.state_floats;
-    // grouped key/value heads: dk and dv per query head, added up over each group afterwards
-    T* dk_q = dk + off;
-    T* dv_q = dv + off;
-    if (ratio > 1) {
-      char* tmp = reinterpret_cast<char*>(state) + (saved ? 1 : 2) * hb * state_bytes;
-      dk_q = reinterpret_cast<T*>(tmp);
-      dv_q = dk_q + (int64_t)hb * n * D;
-    }
-    const float* denh = den + (int64_t)h0 * n * den_stride;
-    const float* ch = cvec + (int64_t)h0 * n;
     if constexpr (D == 64) {
-      if (pl.rowpass) {
+      if (pl.rowpass) {   // (plain tensors, nq == nk)
+        const int n = nq;
+        const int64_t toff = (int64_t)h0 * n * D, koff = (int64_t)kv0 * n * D;
+        const float* denh = den + (int64_t)h0 * n * den_stride;
+        const float* ch = cvec + (int64_t)h0 * n;
         // states of the whole sequence in fp32 (S as the forward pass left it when it was kept), then one
         // pass over the rows per gradient
         const int64_t ss = pl.state_floats, hf = (int64_t)pl.nslots * ss;
         int slot = pl.nparts > 1 ? pl.nparts : 0;
         if (!saved) {
-          FM_TRY((launch_build<D, T>(pl, heads, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state, 0,
-                                     stream, false)));
+          FM_TRY((launch_build<D, T>(pl, heads, n, mk_rows(k, L.k, kv0), mk_rows(v, L.v, kv0), scale + bh + kv0,
+                                     kNoScalars, kNoScalars, state, 0, stream, false)));
           slot = finish_state_fp32(pl, heads, state, stream);
         }
-        FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, stream,
-                                   false)));
+        FM_TRY((launch_build<D, T>(pl, heads, n, mk_rows(q, L.q, h0), mk_rows(go, L.go, h0), scale + h0,
+                                   mk_scalars(den, n, den_stride, h0), mk_scalars<const float>(cvec, n, 1, h0), stR, 1,
+                                   stream, false)));
         finish_state_fp32(pl, heads, stR, stream);
         const int nrb = (n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE;
         const dim3 rgrid(nrb, heads);
@@ -528,100 +611,114 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const T* q, const T* k
           ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
           if (ds->normalize)
             lin::linear_rowpass_kernel<T, lin::ROWPASS_DQ, true, true><<<rgrid, 64, 0, stream>>>(
-                go + off, stS + slot * ss, hf, scale + h0, denh, den_stride, ch, q + off, dq + off, D, nullptr,
+                go + toff, stS + slot * ss, hf, scale + h0, denh, den_stride, ch, q + toff, dq + toff, D, nullptr,
                 rpart + (int64_t)h0 * nrb, n, ds->a0, ds->a1);
           else
             lin::linear_rowpass_kernel<T, lin::ROWPASS_DQ, false, true><<<rgrid, 64, 0, stream>>>(
-                go + off, stS + slot * ss, hf, scale + h0, denh, den_stride, ch, q + off, dq + off, D, nullptr,
+                go + toff, stS + slot * ss, hf, scale + h0, denh, den_stride, ch, q + toff, dq + toff, D, nullptr,
                 nullptr, n, ds->a0, ds->a1);
         }
         FM_TRY(launch_status("linear_rowpass_kernel (dq)"));
         {
           ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
           lin::linear_rowpass_kernel<T, lin::ROWPASS_DK, false, true><<<rgrid, 64, 0, stream>>>(
-              v + koff, stR + slot * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dk + off, D, nullptr,
+              v + koff, stR + slot * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dk + toff, D, nullptr,
               nullptr, n, ds->a0, ds->a1);
         }
         FM_TRY(launch_status("linear_rowpass_kernel (dk)"));
         {
           ScopedKernel sk(FASTMAX_K_BWD_DV, stream);
           lin::linear_rowpass_kernel<T, lin::ROWPASS_DV, false, true><<<rgrid, 64, 0, stream>>>(
-              k + koff, stR + slot * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dv + off, D, nullptr,
+              k + koff, stR + slot * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dv + toff, D, nullptr,
               nullptr, n, ds->a0, ds->a1);
         }
         FM_TRY(launch_status("linear_rowpass_kernel (dv)"));
         continue;
       }
     }
+    const Rows<const T> kr = mk_rows(k, L.k, kv0), vr = mk_rows(v, L.v, kv0);
+    const Rows<const T> qr = mk_rows(q, L.q, h0, off), gr = mk_rows(go, L.go, h0, off);
+    const RowScalars dn = mk_scalars(den, nq, den_stride, h0, off);
+    const RowScalars cv = mk_scalars<const float>(cvec, nq, 1, h0, off);
+    // grouped key/value heads: dk and dv per query head (plain arrays in the workspace), added up
+    // over each group afterwards
+    Rows<T> dk_q = mk_rows(dk, L.dk, kv0), dv_q = mk_rows(dv, L.dv, kv0);
+    T* dk_tmp = nullptr;
+    T* dv_tmp = nullptr;
+    if (ratio > 1) {
+      char* tmp = reinterpret_cast<char*>(state) + (saved ? 1 : 2) * hb * state_bytes;
+      dk_tmp = reinterpret_cast<T*>(tmp);
+      dv_tmp = dk_tmp + (int64_t)hb * nk * D;
+      dk_q = mk_rows(dk_tmp, plain_str(nk, D));
+      dv_q = mk_rows(dv_tmp, plain_str(nk, D));
+    }
     // prefix state of (kh, v, 1) per key/value head and suffix state of (qh, go/den, c) per query head
     if (!saved)
-      FM_TRY((launch_build<D, T>(pl, heads / ratio, k + koff, v + koff, scale + bh + kv0, nullptr, 0, nullptr, state,
-                                 0, stream)));
-    FM_TRY((launch_build<D, T>(pl, heads, q + off, go + off, scale + h0, denh, den_stride, ch, stR, 1, stream)));
-    const dim3 grid(pl.nblk, heads);
+      FM_TRY((launch_build<D, T>(pl, heads / ratio, nk, kr, vr, scale + bh + kv0, kNoScalars, kNoScalars, state, 0,
+                                 stream)));
+    FM_TRY((launch_build<D, T>(pl, heads, nown_q, qr, gr, scale + h0, dn, cv, stR, 1, stream)));
     {
       ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
+      const dim3 grid(pl.nblk_q, heads);
+      const Rows<T> dqr = mk_rows(dq, L.dq, h0, off);
       if constexpr (kBf16Mfma<T>) {
         grad_kernel_bf<D, 0><<<grid, 256, 0, stream>>>(
-            q + off, go + off, denh, den_stride, ch, k + koff, v + koff, nullptr, 0, scale + h0,
-            scale + bh + kv0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, pl.chunk,
-            pl.masked, pl.p2, ds->a1, a2, 1, ratio);
+            qr, gr, dn, cv, kr, vr, kNoScalars, scale + h0, scale + bh + kv0, stS, pl.nslots, dqr,
+            rpart + (int64_t)h0 * pl.nblk_q, nown_q, pl.chunk, pl.masked, pl.p2, ds->a1, a2, 1, ratio);
       } else {
         grad_kernel<D, T, 0><<<grid, 256, 0, stream>>>(
-            q + off, go + off, denh, den_stride, ch, k + koff, v + koff, nullptr, 0, scale + h0,
-            scale + bh + kv0, stS, pl.nslots, dq + off, rpart + (int64_t)h0 * pl.nblk, n, pl.chunk,
-            pl.masked, pl.p2, ds->a1, a2, 1, ratio);
+            qr, gr, dn, cv, kr, vr, kNoScalars, scale + h0, scale + bh + kv0, stS, pl.nslots, dqr,
+            rpart + (int64_t)h0 * pl.nblk_q, nown_q, pl.chunk, pl.masked, pl.p2, ds->a1, a2, 1, ratio);
       }
     }
     FM_TRY(launch_status("grad_kernel (dq)"));
+    const dim3 kgrid(pl.nblk_k, heads);
     {
       ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
       if constexpr (kBf16Mfma<T>) {
-        grad_kernel_bf<D, 1><<<grid, 256, 0, stream>>>(
-            k + koff, v + koff, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + kv0,
-            scale + h0, stR, pl.nslots, dk_q, rpart + (int64_t)(bh + h0) * pl.nblk, n, pl.chunk,
-            pl.masked, pl.p2, ds->a1, a2, ratio, 1);
+        grad_kernel_bf<D, 1><<<kgrid, 256, 0, stream>>>(
+            kr, vr, kNoScalars, cv, qr, gr, dn, scale + bh + kv0, scale + h0, stR, pl.nslots, dk_q,
+            rpart_k + (int64_t)h0 * pl.nblk_k, nown_k, pl.chunk, pl.masked, pl.p2, ds->a1, a2, ratio, 1);
       } else {
-        grad_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
-            k + koff, v + koff, nullptr, 0, ch, q + off, go + off, denh, den_stride, scale + bh + kv0,
-            scale + h0, stR, pl.nslots, dk_q, rpart + (int64_t)(bh + h0) * pl.nblk, n, pl.chunk,
-            pl.masked, pl.p2, ds->a1, a2, ratio, 1);
+        grad_kernel<D, T, 1><<<kgrid, 256, 0, stream>>>(
+            kr, vr, kNoScalars, cv, qr, gr, dn, scale + bh + kv0, scale + h0, stR, pl.nslots, dk_q,
+            rpart_k + (int64_t)h0 * pl.nblk_k, nown_k, pl.chunk, pl.masked, pl.p2, ds->a1, a2, ratio, 1);
       }
     }
     FM_TRY(launch_status("grad_kernel (dk)"));
     {
       ScopedKernel sk(FASTMAX_K_BWD_DV, stream);
       if constexpr (kBf16Mfma<T>) {
-        apply_kernel_bf<D, 1><<<grid, 256, 0, stream>>>(
-            k + koff, q + off, go + off, scale + bh + kv0, scale + h0, denh, den_stride, stR, pl.nslots,
-            dv_q, D, nullptr, 0, n, pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2, ratio, 1);
+        apply_kernel_bf<D, 1><<<kgrid, 256, 0, stream>>>(
+            kr, qr, gr, scale + bh + kv0, scale + h0, dn, stR, pl.nslots, dv_q, RowScalarsOut{nullptr, 0, 0}, nown_k,
+            pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2, ratio, 1);
       } else {
-        apply_kernel<D, T, 1><<<grid, 256, 0, stream>>>(
-            k + koff, q + off, go + off, scale + bh + kv0, scale + h0, denh, den_stride, stR, pl.nslots,
-            dv_q, D, nullptr, 0, n, pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2, ratio, 1);
+        apply_kernel<D, T, 1><<<kgrid, 256, 0, stream>>>(
+            kr, qr, gr, scale + bh + kv0, scale + h0, dn, stR, pl.nslots, dv_q, RowScalarsOut{nullptr, 0, 0}, nown_k,
+            pl.chunk, pl.masked, pl.p2, ds->a0, ds->a1, a2, ratio, 1);
       }
     }
     FM_TRY(launch_status("apply_kernel (dv)"));
     if (ratio > 1) {
-      const int64_t per_head = (int64_t)n * D;
+      const int64_t per_head = (int64_t)nk * D;
       const dim3 sgrid((unsigned)((per_head / 4 + 255) / 256), heads / ratio);
-      group_sum_kernel<T><<<sgrid, 256, 0, stream>>>(dk_q, dk + koff, per_head, ratio);
-      group_sum_kernel<T><<<sgrid, 256, 0, stream>>>(dv_q, dv + koff, per_head, ratio);
+      group_sum_kernel<T><<<sgrid, 256, 0, stream>>>(dk_tmp, mk_rows(dk, L.dk, kv0), nk, D, ratio);
+      group_sum_kernel<T><<<sgrid, 256, 0, stream>>>(dv_tmp, mk_rows(dv, L.dv, kv0), nk, D, ratio);
       FM_TRY(launch_status("group_sum_kernel"));
     }
   }
   if (ds->normalize && pl.rowpass) {
     // one partial per row block of the dq pass; sum_j dk_hat_j . k_hat_j is the same number
-    const int nrb = (n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE;
+    const int nrb = (nq + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE;
     ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
-    norm_fix_kernel<T><<<bh, D, 0, stream>>>(dq, q, scale, arg, rpart, nrb, n, D, ds->lim);
-    norm_fix_kernel<T><<<bh, D, 0, stream>>>(dk, k, scale + bh, arg + bh, rpart, nrb, n, D, ds->lim);
+    norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, nrb, nq, D, ds->lim);
+    norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh, rpart, nrb, nk, D, ds->lim);
     FM_TRY(launch_status("norm_fix_kernel"));
   } else if (ds->normalize) {
     ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
-    norm_fix_kernel<T><<<bh, D, 0, stream>>>(dq, q, scale, arg, rpart, pl.nblk, n, D, ds->lim);
-    norm_fix_kernel<T><<<bhkv, D, 0, stream>>>(dk, k, scale + bh, arg + bh, rpart + (int64_t)bh * pl.nblk,
-                                               pl.nblk * ratio, n, D, ds->lim);
+    norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, pl.nblk_q, nq, D, ds->lim);
+    norm_fix_kernel<T><<<bhkv, D, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh, rpart_k,
+                                               pl.nblk_k * ratio, nk, D, ds->lim);
     FM_TRY(launch_status("norm_fix_kernel"));
   }
   return FASTMAX_OK;
@@ -655,10 +752,11 @@ size_t decode_ws_bytes(const fastmax_desc* ds) {
   return align256((size_t)ds->bh * kDecodeSplits * (ds->d + 4) * sizeof(float));
 }
 
+// one state per key/value head: the descriptor handed in has bh = bhkv = the key/value heads
 template <int D, class T>
 int state_update_impl(const fastmax_desc* ds, const Plan& pl, const T* k, const T* v, const float* kscale,
                       float* state, int accumulate, char* ws, size_t ws_bytes, hipStream_t stream) {
-  const int bh = pl.bh, n = pl.n;
+  const int bh = pl.bh, n = pl.nk;
   float* scale = reinterpret_cast<float*>(ws);
   int* arg = reinterpret_cast<int*>(ws + align256((size_t)2 * bh * sizeof(float)));
   float* slots = reinterpret_cast<float*>(ws + pl.fixed_bytes);
@@ -668,11 +766,11 @@ int state_update_impl(const fastmax_desc* ds, const Plan& pl, const T* k, const 
     kscale = scale + bh;
   }
   const int64_t ss = pl.state_floats;
+  const Str t = plain_str(n, D);
   for (int h0 = 0; h0 < bh; h0 += hb) {
     const int heads = bh - h0 < hb ? bh - h0 : hb;
-    const int64_t off = (int64_t)h0 * n * D;
-    FM_TRY((launch_build<D, T>(pl, heads, k + off, v + off, kscale + h0, nullptr, 0, nullptr, slots, 0, stream,
-                               false)));
+    FM_TRY((launch_build<D, T>(pl, heads, n, mk_rows(k, t, h0), mk_rows(v, t, h0), kscale + h0, kNoScalars, kNoScalars,
+                               slots, 0, stream, false)));
     state_accumulate_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads), 256, 0, stream>>>(
         state + (int64_t)h0 * ss, ss, slots, pl.nslots, pl.nparts, ss, accumulate);
   }
@@ -684,10 +782,59 @@ int decode_impl(const fastmax_desc* ds, const T* q, const T* k, const T* v, cons
                 const float* kscale, float* state, T* o, int64_t ldo, float* den, int64_t den_stride,
                 float* part, hipStream_t stream) {
   const int p2 = ds->p == 2;
-  decode_update_kernel<D, T><<<dim3(kDecodeSplits, ds->bh), 256, 0, stream>>>(
-      q, k, v, qscale, kscale, 1.0f / ds->temperature, state, part, p2, ds->a0, ds->a1, p2 ? ds->a2 : 0.f);
+  decode_update_kernel<D, T><<<dim3(kDecodeSplits, ds->bhkv), 256, 0, stream>>>(
+      q, k, v, qscale, kscale, 1.0f / ds->temperature, state, part, p2, ds->a0, ds->a1, p2 ? ds->a2 : 0.f,
+      ds->bh / ds->bhkv);
   decode_finish_kernel<D, T><<<ds->bh, D + 4, 0, stream>>>(part, kDecodeSplits, o, ldo, den, den_stride);
   return launch_status("decode kernels");
+}
+
+// The kernels address a row by a 32-bit byte offset from its head's first position.
+int check_spans(const fastmax_desc* ds, const Layout& L, int64_t den_stride, bool backward) {
+  const int64_t es = ds->dtype == FASTMAX_BF16 ? 2 : 4, lim = (int64_t)1 << 32;
+  const int64_t nq = ds->mask ? ds->nk : ds->nq, nk = ds->nk;   // positions (queries sit behind the prefix)
+  bool ok = nq * L.q.pitch * es < lim && nk * L.k.pitch * es < lim && nk * L.v.pitch * es < lim &&
+            nq * L.o.pitch * es < lim && nq * den_stride * 4 < lim;
+  if (backward)
+    ok = ok && nq * L.go.pitch * es < lim && nq * L.dq.pitch * es < lim && nk * L.dk.pitch * es < lim &&
+         nk * L.dv.pitch * es < lim;
+  if (!ok) return fail(FASTMAX_E_SHAPE, "the rows of one head span 4 GiB or more (tokens x token stride)");
+  return FASTMAX_OK;
+}
+
+// checks a caller's layout and turns it into the kernels' strides (layout == NULL: plain arrays)
+int resolve_layout(const fastmax_desc* ds, const fastmax_layout* lay, int64_t ldo, bool backward, Layout* out) {
+  if (!lay) {
+    *out = plain_layout(ds, ldo);
+    return FASTMAX_OK;
+  }
+  const int ratio = ds->bh / ds->bhkv;
+  if (lay->groups < 1 || ds->bhkv % lay->groups != 0)
+    return fail(FASTMAX_E_SHAPE, "layout.groups = %d does not divide bhkv = %d", lay->groups, ds->bhkv);
+  const size_t es = ds->dtype == FASTMAX_BF16 ? 2 : 4;
+  auto one = [&](const fastmax_strides& f, bool kv, bool is_o, const char* name, Str* t) {
+    if (f.token < ds->d) return fail(FASTMAX_E_PARAM, "layout.%s.token = %lld < d = %d", name, (long long)f.token, ds->d);
+    if (f.batch < 0 || f.group < 0 || f.head < 0) return fail(FASTMAX_E_PARAM, "layout.%s has a negative stride", name);
+    *t = make_str(f, lay->groups, kv ? 1 : ratio);
+    if (!is_o && !aligned16(*t, es))
+      return fail(FASTMAX_E_PARAM, "layout.%s: every stride must be a multiple of 16 bytes", name);
+    return (int)FASTMAX_OK;
+  };
+  // (the rows of one head must span less than 4 GiB: the kernels address them with 32-bit offsets)
+  FM_TRY(one(lay->q, false, false, "q", &out->q));
+  FM_TRY(one(lay->k, true, false, "k", &out->k));
+  FM_TRY(one(lay->v, true, false, "v", &out->v));
+  FM_TRY(one(lay->o, false, true, "o", &out->o));
+  if (backward) {
+    FM_TRY(one(lay->go, false, false, "go", &out->go));
+    FM_TRY(one(lay->dq, false, false, "dq", &out->dq));
+    FM_TRY(one(lay->dk, true, false, "dk", &out->dk));
+    FM_TRY(one(lay->dv, true, false, "dv", &out->dv));
+  } else {
+    out->go = out->dq = out->q;
+    out->dk = out->dv = out->k;
+  }
+  return FASTMAX_OK;
 }
 
 }  // namespace
@@ -730,21 +877,30 @@ int fastmax_check_desc(const fastmax_desc* desc) {
   return check_desc(desc);
 }
 
-size_t fastmax_workspace_min_bytes(const fastmax_desc* desc, int pass) {
+// (a layout only matters through "plain or not": plain tensors may take the register-resident
+// p = 1 paths, which need no state memory)
+static bool layout_is_plain(const fastmax_desc* desc, const fastmax_layout* layout, bool backward) {
+  if (!layout) return true;
+  Layout L;
+  if (resolve_layout(desc, layout, desc->d, backward, &L) != FASTMAX_OK) return false;
+  return is_plain(L, desc, backward) && L.o.pitch == desc->d;
+}
+
+size_t fastmax_workspace_min_bytes_strided(const fastmax_desc* desc, const fastmax_layout* layout, int pass) {
   g_err[0] = 0;
   if (check_desc(desc) != FASTMAX_OK) return 0;
   if (pass != FASTMAX_PASS_FORWARD && pass != FASTMAX_PASS_BACKWARD) {
     fail(FASTMAX_E_PARAM, "pass = %d", pass);
     return 0;
   }
-  const Plan pl = make_plan(desc, pass);
+  const Plan pl = make_plan(desc, pass, layout_is_plain(desc, layout, pass == FASTMAX_PASS_BACKWARD));
   return pl.fixed_bytes + pl.ratio * pl.per_head_bytes;  // one whole key/value group
 }
 
-size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass) {
-  const size_t mn = fastmax_workspace_min_bytes(desc, pass);
+size_t fastmax_workspace_bytes_strided(const fastmax_desc* desc, const fastmax_layout* layout, int pass) {
+  const size_t mn = fastmax_workspace_min_bytes_strided(desc, layout, pass);
   if (!mn) return 0;
-  const Plan pl = make_plan(desc, pass);
+  const Plan pl = make_plan(desc, pass, layout_is_plain(desc, layout, pass == FASTMAX_PASS_BACKWARD));
   if (!pl.per_head_bytes) return mn;
   size_t heads = (kWorkspaceBudget - (pl.fixed_bytes < kWorkspaceBudget ? pl.fixed_bytes : 0)) / pl.per_head_bytes;
   if (heads < (size_t)pl.ratio) heads = pl.ratio;
@@ -752,28 +908,40 @@ size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass) {
   return pl.fixed_bytes + heads * pl.per_head_bytes;
 }
 
-size_t fastmax_saved_state_bytes(const fastmax_desc* desc) {
+size_t fastmax_saved_state_bytes_strided(const fastmax_desc* desc, const fastmax_layout* layout) {
   g_err[0] = 0;
   if (check_desc(desc) != FASTMAX_OK) return 0;
-  return saved_bytes_for(make_plan(desc, FASTMAX_PASS_FORWARD));
+  return saved_bytes_for(make_plan(desc, FASTMAX_PASS_FORWARD, layout_is_plain(desc, layout, false)));
 }
 
-int fastmax_forward_saving(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
-                           int64_t ldo, float* den, int64_t den_stride, float* qk_scale,
-                           int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
-                           void* saved_states, size_t saved_bytes, fastmax_stream_t stream) {
+size_t fastmax_workspace_min_bytes(const fastmax_desc* desc, int pass) {
+  return fastmax_workspace_min_bytes_strided(desc, nullptr, pass);
+}
+size_t fastmax_workspace_bytes(const fastmax_desc* desc, int pass) {
+  return fastmax_workspace_bytes_strided(desc, nullptr, pass);
+}
+size_t fastmax_saved_state_bytes(const fastmax_desc* desc) { return fastmax_saved_state_bytes_strided(desc, nullptr); }
+
+static int forward_entry(const fastmax_desc* desc, const fastmax_layout* layout, const void* q, const void* k,
+                         const void* v, void* o, int64_t ldo, float* den, int64_t den_stride, float* qk_scale,
+                         int32_t* qk_argmax, void* workspace, size_t workspace_bytes, void* saved_states,
+                         size_t saved_bytes, fastmax_stream_t stream) {
   g_err[0] = 0;
   FM_TRY(check_desc(desc));
   if (!q || !k || !v || !o || !den) return fail(FASTMAX_E_NULL, "q, k, v, o and den must be non-NULL");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v)) return fail(FASTMAX_E_PARAM, "q, k and v must be 16-byte aligned");
   if (ldo < desc->d) return fail(FASTMAX_E_PARAM, "ldo = %lld < d = %d", (long long)ldo, desc->d);
   if (den_stride < 1) return fail(FASTMAX_E_PARAM, "den_stride = %lld < 1", (long long)den_stride);
-  const Plan pl = make_plan(desc, FASTMAX_PASS_FORWARD);
+  Layout L;
+  FM_TRY(resolve_layout(desc, layout, ldo, false, &L));
+  FM_TRY(check_spans(desc, L, den_stride, false));
+  const Plan pl = make_plan(desc, FASTMAX_PASS_FORWARD, is_plain(L, desc, false));
   FM_TRY(check_ws(pl, workspace, workspace_bytes, saved_states != nullptr));
   FM_TRY(check_saved(pl, saved_states, saved_bytes));
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 #define FM_FWD(DD, TT)                                                                             \
-  return forward_impl<DD, TT>(desc, pl, (const TT*)q, (const TT*)k, (const TT*)v, (TT*)o, ldo, den, \
+  return forward_impl<DD, TT>(desc, pl, L, (const TT*)q, (const TT*)k, (const TT*)v, (TT*)o, den, \
                               den_stride, qk_scale, qk_argmax, ws, workspace_bytes, (float*)saved_states, st)
   if (desc->dtype == FASTMAX_F32) {
     if (desc->d == 64) FM_FWD(64, float);
@@ -782,6 +950,26 @@ int fastmax_forward_saving(const fastmax_desc* desc, const void* q, const void* 
   if (desc->d == 64) FM_FWD(64, bf16_t);
   FM_FWD(32, bf16_t);
 #undef FM_FWD
+}
+
+int fastmax_forward_saving(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
+                           int64_t ldo, float* den, int64_t den_stride, float* qk_scale,
+                           int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                           void* saved_states, size_t saved_bytes, fastmax_stream_t stream) {
+  return forward_entry(desc, nullptr, q, k, v, o, ldo, den, den_stride, qk_scale, qk_argmax, workspace,
+                       workspace_bytes, saved_states, saved_bytes, stream);
+}
+
+int fastmax_forward_strided(const fastmax_desc* desc, const fastmax_layout* layout, const void* q, const void* k,
+                            const void* v, void* o, float* den, int64_t den_stride, float* qk_scale,
+                            int32_t* qk_argmax, void* workspace, size_t workspace_bytes, void* saved_states,
+                            size_t saved_bytes, fastmax_stream_t stream) {
+  if (!layout) {
+    g_err[0] = 0;
+    return fail(FASTMAX_E_NULL, "layout is NULL");
+  }
+  return forward_entry(desc, layout, q, k, v, o, layout->o.token, den, den_stride, qk_scale, qk_argmax, workspace,
+                       workspace_bytes, saved_states, saved_bytes, stream);
 }
 
 int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
@@ -813,24 +1001,29 @@ int fastmax_forward_noalloc(const fastmax_desc* desc, const void* q, const void*
                                 FASTMAX_NOALLOC_SCRATCH_BYTES, nullptr, 0, stream);
 }
 
-int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* k, const void* v,
-                           const void* o, int64_t ldo, const float* den, int64_t den_stride,
-                           const void* go, void* dq, void* dk, void* dv, const float* qk_scale,
-                           const int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
-                           const void* saved_states, size_t saved_bytes, fastmax_stream_t stream) {
+static int backward_entry(const fastmax_desc* desc, const fastmax_layout* layout, const void* q, const void* k,
+                          const void* v, const void* o, int64_t ldo, const float* den, int64_t den_stride,
+                          const void* go, void* dq, void* dk, void* dv, const float* qk_scale,
+                          const int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                          const void* saved_states, size_t saved_bytes, fastmax_stream_t stream) {
   g_err[0] = 0;
   FM_TRY(check_desc(desc));
   if (!q || !k || !v || !o || !den || !go || !dq || !dk || !dv)
     return fail(FASTMAX_E_NULL, "q, k, v, o, den, go, dq, dk and dv must be non-NULL");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(go) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
+    return fail(FASTMAX_E_PARAM, "q, k, v, go, dq, dk and dv must be 16-byte aligned");
   if (ldo < desc->d) return fail(FASTMAX_E_PARAM, "ldo = %lld < d = %d", (long long)ldo, desc->d);
   if (den_stride < 1) return fail(FASTMAX_E_PARAM, "den_stride = %lld < 1", (long long)den_stride);
-  const Plan pl = make_plan(desc, FASTMAX_PASS_BACKWARD);
+  Layout L;
+  FM_TRY(resolve_layout(desc, layout, ldo, true, &L));
+  FM_TRY(check_spans(desc, L, den_stride, true));
+  const Plan pl = make_plan(desc, FASTMAX_PASS_BACKWARD, is_plain(L, desc, true));
   FM_TRY(check_ws(pl, workspace, workspace_bytes, saved_states != nullptr));
   FM_TRY(check_saved(pl, saved_states, saved_bytes));
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 #define FM_BWD(DD, TT)                                                                              \
-  return backward_impl<DD, TT>(desc, pl, (const TT*)q, (const TT*)k, (const TT*)v, (const TT*)o, ldo, \
+  return backward_impl<DD, TT>(desc, pl, L, (const TT*)q, (const TT*)k, (const TT*)v, (const TT*)o, \
                                den, den_stride, (const TT*)go, (TT*)dq, (TT*)dk, (TT*)dv, qk_scale,  \
                                qk_argmax, ws, workspace_bytes, (const float*)saved_states, st)
   if (desc->dtype == FASTMAX_F32) {
@@ -840,6 +1033,28 @@ int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* 
   if (desc->d == 64) FM_BWD(64, bf16_t);
   FM_BWD(32, bf16_t);
 #undef FM_BWD
+}
+
+int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* k, const void* v,
+                           const void* o, int64_t ldo, const float* den, int64_t den_stride,
+                           const void* go, void* dq, void* dk, void* dv, const float* qk_scale,
+                           const int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                           const void* saved_states, size_t saved_bytes, fastmax_stream_t stream) {
+  return backward_entry(desc, nullptr, q, k, v, o, ldo, den, den_stride, go, dq, dk, dv, qk_scale, qk_argmax,
+                        workspace, workspace_bytes, saved_states, saved_bytes, stream);
+}
+
+int fastmax_backward_strided(const fastmax_desc* desc, const fastmax_layout* layout, const void* q, const void* k,
+                             const void* v, const void* o, const float* den, int64_t den_stride, const void* go,
+                             void* dq, void* dk, void* dv, const float* qk_scale, const int32_t* qk_argmax,
+                             void* workspace, size_t workspace_bytes, const void* saved_states, size_t saved_bytes,
+                             fastmax_stream_t stream) {
+  if (!layout) {
+    g_err[0] = 0;
+    return fail(FASTMAX_E_NULL, "layout is NULL");
+  }
+  return backward_entry(desc, layout, q, k, v, o, layout->o.token, den, den_stride, go, dq, dk, dv, qk_scale,
+                        qk_argmax, workspace, workspace_bytes, saved_states, saved_bytes, stream);
 }
 
 int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, const void* v,
@@ -863,17 +1078,18 @@ int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k, void* 
   const int bh = desc->bh;
   float* scale = static_cast<float*>(workspace);
   int* arg = reinterpret_cast<int*>(static_cast<char*>(workspace) + align256((size_t)2 * bh * sizeof(float)));
-  const int64_t per_head = (int64_t)desc->nq * desc->d;
+  const int64_t per_head = (int64_t)desc->nq * desc->d, per_head_k = (int64_t)desc->nk * desc->d;
   const dim3 grid((unsigned)((per_head / 4 + 255) / 256), bh);
-  const dim3 kgrid(grid.x, desc->bhkv);
+  const dim3 kgrid((unsigned)((per_head_k / 4 + 255) / 256), desc->bhkv);
+  const Layout L = plain_layout(desc, desc->d);
   if (desc->dtype == FASTMAX_F32) {
-    FM_TRY(compute_scales<float>(desc, (const float*)q, (const float*)k, scale, arg, st));
+    FM_TRY(compute_scales<float>(desc, L, (const float*)q, (const float*)k, scale, arg, st));
     scale_rows_kernel<float><<<grid, 256, 0, st>>>((float*)q, scale, per_head);
-    scale_rows_kernel<float><<<kgrid, 256, 0, st>>>((float*)k, scale + bh, per_head);
+    scale_rows_kernel<float><<<kgrid, 256, 0, st>>>((float*)k, scale + bh, per_head_k);
   } else {
-    FM_TRY(compute_scales<bf16_t>(desc, (const bf16_t*)q, (const bf16_t*)k, scale, arg, st));
+    FM_TRY(compute_scales<bf16_t>(desc, L, (const bf16_t*)q, (const bf16_t*)k, scale, arg, st));
     scale_rows_kernel<bf16_t><<<grid, 256, 0, st>>>((bf16_t*)q, scale, per_head);
-    scale_rows_kernel<bf16_t><<<kgrid, 256, 0, st>>>((bf16_t*)k, scale + bh, per_head);
+    scale_rows_kernel<bf16_t><<<kgrid, 256, 0, st>>>((bf16_t*)k, scale + bh, per_head_k);
   }
   return launch_status("scale_rows_kernel");
 }
@@ -896,11 +1112,13 @@ int fastmax_state_update(const fastmax_desc* desc, const void* k, const void* v,
   g_err[0] = 0;
   FM_TRY(check_desc(desc));
   if (!k || !v || !state) return fail(FASTMAX_E_NULL, "k, v and state must be non-NULL");
-  if (desc->bhkv != desc->bh) return fail(FASTMAX_E_SHAPE, "the recurrent form needs bhkv == bh (one state per head)");
   if (desc->normalize && !k_scale)
     return fail(FASTMAX_E_NULL, "normalize is set: k_scale (the factor a forward pass reported) is required");
+  // one state per key/value head: the build runs over the bhkv heads of k, v
   fastmax_desc d2 = *desc;
   d2.mask = 0;
+  d2.bh = d2.bhkv;
+  d2.nq = d2.nk;
   const Plan pl = make_plan(&d2, FASTMAX_PASS_FORWARD);
   FM_TRY(check_ws(pl, workspace, workspace_bytes));
   char* ws = static_cast<char*>(workspace);
@@ -924,8 +1142,7 @@ int fastmax_decode_step(const fastmax_desc* desc, const void* q, const void* k, 
   g_err[0] = 0;
   FM_TRY(check_desc(desc));
   if (!q || !k || !v || !state || !o) return fail(FASTMAX_E_NULL, "q, k, v, state and o must be non-NULL");
-  if (desc->bhkv != desc->bh) return fail(FASTMAX_E_SHAPE, "the recurrent form needs bhkv == bh (one state per head)");
-  if (desc->nq != 1) return fail(FASTMAX_E_SHAPE, "a decode step takes one token per head (nq = nk = 1), got nq = %d", desc->nq);
+  if (desc->nq != 1 || desc->nk != 1) return fail(FASTMAX_E_SHAPE, "a decode step takes one token per head (nq = nk = 1), got nq = %d", desc->nq);
   if (desc->normalize && (!q_scale || !k_scale))
     return fail(FASTMAX_E_NULL, "normalize is set: q_scale and k_scale (the factors a forward pass reported) are required");
   if (ldo < desc->d) return fail(FASTMAX_E_PARAM, "ldo = %lld < d = %d", (long long)ldo, desc->d);

@@ -37,10 +37,10 @@
 // ---------------------------------------------------------------------------------------
 template <int D, class T, int MODE>
 __global__ __launch_bounds__(256, 2) void apply_kernel(
-    const T* __restrict__ X, const T* __restrict__ A1, const T* __restrict__ A2,
+    Rows<const T> X, Rows<const T> A1, Rows<const T> A2,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
-    const float* __restrict__ a2den, int64_t a2den_stride, const float* __restrict__ state,
-    int nslots, T* __restrict__ OUT, int64_t ldo, float* __restrict__ den, int64_t den_stride, int n,
+    RowScalars a2den, const float* __restrict__ state,
+    int nslots, Rows<T> OUT, RowScalarsOut den, int n,
     int chunk, int masked, int p2, float a0, float a1, float a2, int xdiv,
     int adiv) {
   using G = Geo<D>;
@@ -54,7 +54,8 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   // logical block = (128-token block fastest, then head): neighbours in a chunk share their state
   const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
-  const int head = lid / gridDim.x, tblk = lid % gridDim.x, tok0 = tblk * 128;
+  // (own positions start at X.lo: the grid covers the 128-token blocks from that one on)
+  const int head = lid / gridDim.x, tblk = (X.lo >> 7) + lid % gridDim.x, tok0 = tblk * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
@@ -62,10 +63,9 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
   // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
   // and the state to head ha = head / adiv (one of the divisors is 1)
   const int hx = head / xdiv, ha = head / adiv;
-  const T* Xh = X + (int64_t)hx * n * D;
-  const T* A1h = A1 + (int64_t)ha * n * D;
-  const T* A2h = A2 + (int64_t)ha * n * D;
-  const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
+  const HeadRows<const T> Xh = X.head(hx), A1h = A1.head(ha), A2h = A2.head(ha);
+  const float* a2dh = a2den.head(ha);
+  const int64_t a2den_stride = a2den.stride;
   const float xs = xscale[hx], a1s = a1scale[ha];
 
   // (the own rows are requested here and staged after the first slab and streamed tile have been
@@ -305,19 +305,19 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
     const int tok = tok0 + xrow;
     if (hh == 0) {
       denl[xrow] = dtot;
-      if (tok < n) den[((int64_t)head * n + tok) * den_stride] = dtot;
+      if (tok < n && tok >= Xh.lo) den.head(head)[(int64_t)tok * den.stride] = dtot;
     }
     __syncthreads();
   }
-  T* Oh = OUT + (int64_t)head * n * ldo;
+  const HeadRows<T> Oh = OUT.head(head);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int row = w * 32 + trow(r, hh);
     const int tk = tok0 + row;
-    if (tk < n) {
+    if (tk < n && tk >= Xh.lo) {
       const float inv = FWD ? 1.0f / denl[row] : 1.0f;
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) Oh[(int64_t)tk * ldo + cb * 32 + i] = from_f32<T>(acc[cb][r] * inv);
+      for (int cb = 0; cb < CB; ++cb) Oh.base[(unsigned)tk * Oh.pitch + (unsigned)(cb * 32 + i)] = from_f32<T>(acc[cb][r] * inv);
     }
   }
 }
@@ -343,10 +343,10 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
 // ---------------------------------------------------------------------------------------
 template <int D, int MODE>
 __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
-    const bf16_t* __restrict__ X, const bf16_t* __restrict__ A1, const bf16_t* __restrict__ A2,
+    Rows<const bf16_t> X, Rows<const bf16_t> A1, Rows<const bf16_t> A2,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
-    const float* __restrict__ a2den, int64_t a2den_stride, const float* state,
-    int nslots, bf16_t* __restrict__ OUT, int64_t ldo, float* __restrict__ den, int64_t den_stride,
+    RowScalars a2den, const float* state,
+    int nslots, Rows<bf16_t> OUT, RowScalarsOut den,
     int n, int chunk, int masked, int p2, float a0, float a1, float a2, int xdiv,
     int adiv) {
   using G = Geo<D>;
@@ -376,7 +376,8 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
-  const int head = lid / gridDim.x, tblk = lid % gridDim.x, tok0 = tblk * 128;
+  // (own positions start at X.lo: the grid covers the 128-token blocks from that one on)
+  const int head = lid / gridDim.x, tblk = (X.lo >> 7) + lid % gridDim.x, tok0 = tblk * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
@@ -384,10 +385,9 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
   // and the state to head ha = head / adiv (one of the divisors is 1)
   const int hx = head / xdiv, ha = head / adiv;
-  const T* Xh = X + (int64_t)hx * n * D;
-  const T* A1h = A1 + (int64_t)ha * n * D;
-  const T* A2h = A2 + (int64_t)ha * n * D;
-  const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
+  const HeadRows<const T> Xh = X.head(hx), A1h = A1.head(ha), A2h = A2.head(ha);
+  const float* a2dh = a2den.head(ha);
+  const int64_t a2den_stride = a2den.stride;
   const float xs = xscale[hx], a1s = a1scale[ha];
 
   // (the own rows are requested here and staged after the first slabs and streamed tiles have been
@@ -672,15 +672,16 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     }
   }
 
-  T* Oh = OUT + (int64_t)head * n * ldo;
+  const HeadRows<T> Oh = OUT.head(head);
+  float* denh = FWD ? den.head(head) : nullptr;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int tk = tok0 + w * 32 + trow(r, hh);
-    if (tk < n) {
+    if (tk < n && tk >= Xh.lo) {
       const float inv = FWD ? 1.0f / accd[r] : 1.0f;
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) Oh[(int64_t)tk * ldo + cb * 32 + i] = from_f32<T>(acc[cb][r] * inv);
-      if (FWD && i == 0) den[((int64_t)head * n + tk) * den_stride] = accd[r];
+      for (int cb = 0; cb < CB; ++cb) Oh.base[(unsigned)tk * Oh.pitch + (unsigned)(cb * 32 + i)] = from_f32<T>(acc[cb][r] * inv);
+      if (FWD && i == 0) denh[(int64_t)tk * den.stride] = accd[r];
     }
   }
 }

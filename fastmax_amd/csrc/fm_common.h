@@ -123,6 +123,47 @@ __device__ __forceinline__ void store4(bf16_t* p, const float (&v)[4]) {
   *reinterpret_cast<uint2*>(p) = t;
 }
 
+// Rows of one tensor the way a kernel addresses them.  The tensor is (batch, group, head within the
+// group, token, channel) with unit channel stride: head h of the tensor, counted over all batch
+// elements, starts at
+//     p + (h / (ng nh)) sb + ((h / nh) % ng) sg + (h % nh) sh
+// and consecutive tokens are `pitch` elements apart.  A contiguous (heads, tokens, D) tensor has
+// ng = nh = 1 and sb = tokens * D.  Token positions below `lo` have no row (a key prefix: query-side
+// tensors start at position nk - nq); the host moves p back by lo * pitch, so position t >= lo is
+// at head(h) + t * pitch like everywhere else, and loads clamp their position to [lo, n).  h0 is
+// added to the head index a kernel derives from its block index (head batches).
+// (the rows of one head span less than 4 GiB -- the host checks it -- so a row's offset from the
+// head's base fits 32 bits: uniform 64-bit base + 32-bit lane offset is the cheapest address form)
+template <class T>
+struct HeadRows {
+  T* base;
+  unsigned pitch;
+  int lo;
+  __device__ __forceinline__ T* row(int tok) const { return base + (unsigned)tok * pitch; }
+};
+template <class T>
+struct Rows {
+  T* p;
+  int64_t sb, sg, sh, pitch;
+  int ng, nh, h0, lo;
+  __device__ __forceinline__ HeadRows<T> head(int h) const {
+    h += h0;
+    if (ng == 1 && nh == 1) return HeadRows<T>{p + (int64_t)h * sb, (unsigned)pitch, lo};   // one level (no divisions)
+    const int gb = h / nh, j = h - gb * nh, b = gb / ng, g = gb - b * ng;
+    return HeadRows<T>{p + ((int64_t)b * sb + (int64_t)g * sg + (int64_t)j * sh), (unsigned)pitch, lo};
+  }
+};
+// One float per (head, token): den, c.  Head h starts at p + h * hs, tokens are `stride` apart;
+// like Rows, p is moved back by lo * stride when positions start at lo.
+template <class F>
+struct RowScalarsT {
+  F* p;
+  int64_t hs, stride;
+  __device__ __forceinline__ F* head(int h) const { return p ? p + (int64_t)h * hs : nullptr; }
+};
+using RowScalars = RowScalarsT<const float>;
+using RowScalarsOut = RowScalarsT<float>;
+
 // Geometry of the symmetric moment state for head dimension D.
 //
 // The order-2 feature of a vector x is stored once per unordered channel pair, indexed by
@@ -190,8 +231,7 @@ struct RowTile {
   static constexpr int NV = (TOTAL + 255) / 256;
   // The pieces stay as loaded (and the divisors unread) until a store converts, masks and scales
   // them: nothing in load() consumes what it fetches, and it has no branch, so the loads of a
-  // tile can stay in flight under whatever work separates load() from the store.  Rows >= n are
-  // fetched from row n-1 (a valid address) and zeroed by the store.
+  // tile can stay in flight under whatever work separates load() from the store.
   using Raw = typename std::conditional<std::is_same<T, float>::value, float4, uint2>::type;
   Raw raw[NV];
   float rdiv[NV];  // per-row divisors fetched by load(), applied by the stores
@@ -215,9 +255,10 @@ struct RowTile {
     for (int e = 0; e < 4; ++e) o[e] = live[u] ? o[e] * sc : 0.f;
   }
 
-  // rows tok0.. of one head (base points at the head's first row); rows >= n read as zero.
+  // rows tok0.. of one head; rows outside [lo, n) read as zero (they are fetched from the nearest
+  // row inside, a valid address, and zeroed by the store).
   // rowdiv, when given, makes the stores divide every row by rowdiv[tok * rowdiv_stride].
-  __device__ __forceinline__ void load(const T* base, int tok0, int n, int tid,
+  __device__ __forceinline__ void load(const HeadRows<const T>& hr, int tok0, int n, int tid,
                                        const float* rowdiv = nullptr, int64_t rowdiv_stride = 0) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
@@ -225,11 +266,11 @@ struct RowTile {
       const bool in = idx < TOTAL;
       const int row = in ? row_of(idx) : 0, c4 = in ? c4_of(idx) : 0;
       const int tok = tok0 + row;
-      live[u] = in && tok < n;
-      const int tk = tok < n ? tok : n - 1;
-      raw[u] = *reinterpret_cast<const Raw*>(base + (int64_t)tk * D + c4 * 4);
+      live[u] = in && tok < n && tok >= hr.lo;
+      const int tk = max(tok < n ? tok : n - 1, hr.lo);
+      raw[u] = *reinterpret_cast<const Raw*>(hr.base + ((unsigned)tk * hr.pitch + (unsigned)(c4 * 4)));
       rdiv[u] = 1.0f;
-      if (rowdiv) rdiv[u] = rowdiv[(int64_t)tk * rowdiv_stride];
+      if (rowdiv) rdiv[u] = rowdiv[(unsigned)tk * (unsigned)rowdiv_stride];
     }
   }
   // dst is [ROWS][ld] floats in LDS, 16-byte aligned, ld a multiple of 4
@@ -316,12 +357,12 @@ struct RawTileBf {
   uint2 raw[NV];
   float rdiv;
 
-  __device__ __forceinline__ void load(const bf16_t* base, int tok0, int n, int tid,
+  __device__ __forceinline__ void load(const HeadRows<const bf16_t>& hr, int tok0, int n, int tid,
                                        const float* rowdiv = nullptr, int64_t rowdiv_stride = 0) {
     const int tok = tok0 + tid % ROWS;
-    const bool live = tok < n;
-    const bf16_t* src = base + (int64_t)(live ? tok : 0) * D + (tid / ROWS) * 4;
-    rdiv = (live && rowdiv) ? rowdiv[(int64_t)tok * rowdiv_stride] : 1.0f;
+    const bool live = tok < n && tok >= hr.lo;
+    const bf16_t* src = hr.base + ((unsigned)(live ? tok : hr.lo) * hr.pitch + (unsigned)((tid / ROWS) * 4));
+    rdiv = (live && rowdiv) ? rowdiv[(unsigned)tok * (unsigned)rowdiv_stride] : 1.0f;
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
       const uint2 t = *reinterpret_cast<const uint2*>(src + u * RG * 4);

@@ -28,13 +28,16 @@ __global__ __launch_bounds__(256) void state_accumulate_kernel(float* __restrict
   *dst = a;
 }
 
-// grid = (rsplit, heads).  Block (split, head) owns state rows [rows*split/rsplit,
-// rows*(split+1)/rsplit); a thread owns one 16-byte piece of a row per sweep.
+// grid = (rsplit, key/value heads).  Block (split, head) owns state rows [rows*split/rsplit,
+// rows*(split+1)/rsplit) of that key/value head's state; a thread owns one 16-byte piece of a row
+// per sweep.  The state takes in (k, v) during the sweep for the group's first query head; the
+// other `ratio - 1` query heads of the group (fastmax_cuda_forward.cu:38) sweep the updated rows
+// again (each thread re-reads what it wrote itself).
 template <int D, class T>
 __global__ __launch_bounds__(256) void decode_update_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
     const float* __restrict__ qscale, const float* __restrict__ kscale, float kdefault,
-    float* __restrict__ state, float* __restrict__ part, int p2, float a0, float a1, float a2) {
+    float* __restrict__ state, float* __restrict__ part, int p2, float a0, float a1, float a2, int ratio) {
   using G = Geo<D>;
   constexpr int LD = G::LD, VPR = LD / 4, RPI = 256 / VPR, H2 = G::H2;
   __shared__ float ql[D], kl[D];
@@ -42,49 +45,55 @@ __global__ __launch_bounds__(256) void decode_update_kernel(
   __shared__ float4 red[RPI][VPR];
   const int tid = threadIdx.x, split = blockIdx.x, rsplit = gridDim.x, head = blockIdx.y;
   if (tid < D) {
-    ql[tid] = to_f32(q[(int64_t)head * D + tid]) * (qscale ? qscale[head] : 1.0f);
     kl[tid] = to_f32(k[(int64_t)head * D + tid]) * (kscale ? kscale[head] : kdefault);
     vl[tid] = to_f32(v[(int64_t)head * D + tid]);
   } else if (tid < LD) {
     vl[tid] = tid == D ? 1.0f : 0.f;  // the extra column counts the token; the padding stays put
   }
-  __syncthreads();
   const int rows = G::rows(p2), rows2 = G::rows2(p2);
   const int r_lo = (int)((int64_t)rows * split / rsplit), r_hi = (int)((int64_t)rows * (split + 1) / rsplit);
   const int c4 = tid % VPR, rr = tid / VPR;
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (rr < RPI) {
-    const float4 vx = *reinterpret_cast<const float4*>(vl + 4 * c4);
-    float* sh = state + (int64_t)head * G::state_floats(p2);
-    for (int row = r_lo + rr; row < r_hi; row += RPI) {
-      float fk, fq;
-      if (row < rows2) {
-        const int s = row / D, a = row % D, b = (a + s) & (D - 1);
-        fk = kl[a] * kl[b];
-        fq = ((s == 0 || s == H2) ? a2 : 2.0f * a2) * ql[a] * ql[b];
-      } else if (row < rows2 + D) {
-        fk = kl[row - rows2];
-        fq = a1 * ql[row - rows2];
-      } else {
-        fk = 1.0f;
-        fq = a0;
+  for (int j = 0; j < ratio; ++j) {
+    const int qh = head * ratio + j;
+    __syncthreads();   // (ql and red of the previous query head are no longer read)
+    if (tid < D) ql[tid] = to_f32(q[(int64_t)qh * D + tid]) * (qscale ? qscale[qh] : 1.0f);
+    __syncthreads();
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (rr < RPI) {
+      const float4 vx = *reinterpret_cast<const float4*>(vl + 4 * c4);
+      float* sh = state + (int64_t)head * G::state_floats(p2);
+      for (int row = r_lo + rr; row < r_hi; row += RPI) {
+        float fk, fq;
+        if (row < rows2) {
+          const int s = row / D, a = row % D, b = (a + s) & (D - 1);
+          fk = kl[a] * kl[b];
+          fq = ((s == 0 || s == H2) ? a2 : 2.0f * a2) * ql[a] * ql[b];
+        } else if (row < rows2 + D) {
+          fk = kl[row - rows2];
+          fq = a1 * ql[row - rows2];
+        } else {
+          fk = 1.0f;
+          fq = a0;
+        }
+        float4* sp = reinterpret_cast<float4*>(sh + (int64_t)row * LD + 4 * c4);
+        float4 s4 = *sp;
+        if (j == 0) {
+          s4.x += fk * vx.x; s4.y += fk * vx.y; s4.z += fk * vx.z; s4.w += fk * vx.w;
+          *sp = s4;
+        }
+        acc.x += fq * s4.x; acc.y += fq * s4.y; acc.z += fq * s4.z; acc.w += fq * s4.w;
       }
-      float4* sp = reinterpret_cast<float4*>(sh + (int64_t)row * LD + 4 * c4);
-      float4 s4 = *sp;
-      s4.x += fk * vx.x; s4.y += fk * vx.y; s4.z += fk * vx.z; s4.w += fk * vx.w;
-      *sp = s4;
-      acc.x += fq * s4.x; acc.y += fq * s4.y; acc.z += fq * s4.z; acc.w += fq * s4.w;
+      red[rr][c4] = acc;
     }
-    red[rr][c4] = acc;
-  }
-  __syncthreads();
-  if (tid < VPR) {
-    float4 t = red[0][tid];
-    for (int r = 1; r < RPI; ++r) {
-      const float4 u = red[r][tid];
-      t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+    __syncthreads();
+    if (tid < VPR) {
+      float4 t = red[0][tid];
+      for (int r = 1; r < RPI; ++r) {
+        const float4 u = red[r][tid];
+        t.x += u.x; t.y += u.y; t.z += u.z; t.w += u.w;
+      }
+      *reinterpret_cast<float4*>(part + ((int64_t)qh * rsplit + split) * LD + 4 * tid) = t;
     }
-    *reinterpret_cast<float4*>(part + ((int64_t)head * rsplit + split) * LD + 4 * tid) = t;
   }
 }
 

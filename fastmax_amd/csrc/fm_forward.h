@@ -35,7 +35,7 @@ struct RowPiece<bf16_t> {
 };
 
 template <class T, int NT>
-__global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, int n, int d,
+__global__ __launch_bounds__(NT) void rowstat_kernel(Rows<const T> x, int n, int d,
                                                      float lim, float* __restrict__ scale_out,
                                                      int* __restrict__ arg_out) {
   __shared__ float sbest[NT];
@@ -44,7 +44,9 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, in
   const int tid = threadIdx.x;
   const int tpr = d / EPT, rpp = NT / tpr;
   const int sub = tid % tpr, rowi = tid / tpr;
-  const T* base = x + (int64_t)blockIdx.x * n * d;
+  const HeadRows<const T> xh = x.head(blockIdx.x);   // rows 0 .. n-1 of the tensor itself (lo is not used)
+  const T* base = xh.base;
+  const unsigned pitch = xh.pitch;
   // A NaN row norm wins over every number (the maximum of the reference's path propagates NaN,
   // example.py:105-108), so the head's scale becomes NaN and the reported row is always a row
   // of the tensor: first NaN row if there is one, else first row of maximal norm.
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(const T* __restrict__ x, in
     for (int u = 0; u < 4; ++u) {
       const int i = i0 + u * rpp + rowi;
       idx[u] = i < n ? i : n - 1;
-      ssq[u] = RowPiece<T>::sumsq(base + (int64_t)idx[u] * d + sub * EPT);
+      ssq[u] = RowPiece<T>::sumsq(base + ((unsigned)idx[u] * pitch + (unsigned)(sub * EPT)));
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -141,10 +143,9 @@ __global__ void scale_rows_kernel(T* x, const float* __restrict__ scale, int64_t
 // ---------------------------------------------------------------------------------------
 template <int D, class T, int RTW, bool BF>
 __global__ __launch_bounds__(256, 2) void build_kernel(
-    const T* __restrict__ X, const T* __restrict__ Y, const float* __restrict__ xscale,
-    const float* __restrict__ yden, int64_t yden_stride, const float* __restrict__ ew,
-    float* __restrict__ state, int n, int chunk, int nslots, int masked, int reverse, int p2,
-    int zlen) {
+    Rows<const T> X, Rows<const T> Y, const float* __restrict__ xscale, RowScalars yden,
+    RowScalars ew, float* __restrict__ state, int n, int chunk, int nslots, int masked, int reverse,
+    int p2, int zlen) {
   using G = Geo<D>;
   constexpr int TS = 32;  // tokens per pipeline step (64 for bf16 halves the barriers but does not fit the
                         // register file next to three row tiles of accumulators)
@@ -217,11 +218,14 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   }
   float s0 = 0.f;  // order-0 sums: threads 0..D-1 of split 0 own a value column, thread D the extra one
 
-  const T* Xh = X + (int64_t)head * n * D;
-  const T* Yh = Y + (int64_t)head * n * D;
-  const float* ydh = yden ? yden + (int64_t)head * n * yden_stride : nullptr;
-  const float* ewh = ew ? ew + (int64_t)head * n : nullptr;
+  const HeadRows<const T> Xh = X.head(head), Yh = Y.head(head);
+  const float* ydh = yden.head(head);
+  const float* ewh = ew.head(head);
+  const int64_t yden_stride = yden.stride;
   const float xs = xscale[head];
+  // positions below lo have no row (query-side tensors behind a key prefix): they read as zero, and
+  // a reverse scan stops at the chunk that holds position lo (the chunks below add nothing)
+  const int lo = Xh.lo;
 
   // a step is staged in halves of 32 tokens (one half when TS == 32), so that only one half's
   // rows are in registers at a time
@@ -234,7 +238,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     vy.load(Yh, t0, tend, tid, ydh, yden_stride);
     if (tid < 32) {
       const int tok = t0 + tid;
-      ereg = (tok < tend) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
+      ereg = (tok < tend && tok >= lo) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
     }
   };
   auto store = [&](int buf, int h, int t0, int tend) {
@@ -243,7 +247,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     else vy.store_t(Vt[buf] + 32 * h, TP, 1.0f, tid);
     if (tid < 32) {
       El[buf][32 * h + tid] = ereg;
-      Kt[buf][D * TP + 32 * h + tid] = (t0 + tid < tend) ? 1.0f : 0.f;
+      Kt[buf][D * TP + 32 * h + tid] = (t0 + tid < tend && t0 + tid >= lo) ? 1.0f : 0.f;
     }
   };
   // operands of one group of 8 tokens (lane half hh takes tokens 8*grp + 4*hh + u, u = 0..3,
@@ -412,14 +416,15 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     const int nc = (n + chunk - 1) / chunk;
     if (reverse) {
       first_len = (n - (nc - 1) * chunk + TS - 1) / TS;  // the last chunk may be short
-      nsteps = nc > 1 ? first_len + (nc - 2) * spc : 0;
+      const int cl = lo / chunk;   // (<= nc - 1)
+      nsteps = nc > 1 ? first_len + (nc - 1 - (cl > 1 ? cl : 1)) * spc : 0;
     } else {
       nsteps = (nc - 1) * spc;
     }
   } else {
     tbase = zsplit * zlen;
     tend = tbase + zlen < n ? tbase + zlen : n;
-    nsteps = (tend - tbase + TS - 1) / TS;
+    nsteps = tend > tbase ? (tend - tbase + TS - 1) / TS : 0;
   }
   // token base of step p and the slot to write after it (-1: none)
   auto step_tok = [&](int p) {
@@ -452,7 +457,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       v_.load(Yh, t0, tend, tid, ydh, yden_stride);
       if (tid < 32) {
         const int tok = t0 + tid;
-        e_ = (tok < tend) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
+        e_ = (tok < tend && tok >= lo) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
       }
     };
     auto store_from = [&](auto& k_, auto& v_, float e_, int buf, int t0) __attribute__((always_inline)) {
@@ -460,7 +465,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       v_.store_t_bf(Vtb[buf], TPB, 1.0f, tid, ydh == nullptr);
       if (tid < 32) {
         El[buf][tid] = e_;
-        Kt[buf][D * TP + tid] = (t0 + tid < tend) ? 1.0f : 0.f;
+        Kt[buf][D * TP + tid] = (t0 + tid < tend && t0 + tid >= lo) ? 1.0f : 0.f;
       }
     };
     auto step = [&](int p, auto& lk, auto& lv, float& le, auto& sk, auto& sv, float se) __attribute__((always_inline)) {
@@ -512,6 +517,10 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     }
   }
   if (!masked && nsteps == 0) emit(zsplit);  // an empty token split still owns its slot
+  if (masked && reverse && nsteps > 0) {
+    // chunks below the one that holds position lo see the same suffix state
+    for (int slot = lo / chunk - 2; slot >= 0; --slot) emit(slot);
+  }
 }
 
 // ---------------------------------------------------------------------------------------

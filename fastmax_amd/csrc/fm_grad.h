@@ -32,11 +32,10 @@
 // ---------------------------------------------------------------------------------------
 template <int D, class T, int MODE>
 __global__ __launch_bounds__(256, 2) void grad_kernel(
-    const T* __restrict__ X, const T* __restrict__ Y, const float* __restrict__ yden,
-    int64_t yden_stride, const float* __restrict__ cvec, const T* __restrict__ A1,
-    const T* __restrict__ A2, const float* __restrict__ a2den, int64_t a2den_stride,
+    Rows<const T> X, Rows<const T> Y, RowScalars yden, RowScalars cvec, Rows<const T> A1,
+    Rows<const T> A2, RowScalars a2den,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
-    const float* __restrict__ state, int nslots, T* __restrict__ OUT, float* __restrict__ rpart,
+    const float* __restrict__ state, int nslots, Rows<T> OUT, float* __restrict__ rpart,
     int n, int chunk, int masked, int p2, float a1, float a2, int xdiv, int adiv) {
   using G = Geo<D>;
   constexpr bool DQ = MODE == 0;
@@ -49,7 +48,8 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   // logical block = (128-token block fastest, then head): neighbours in a chunk share their state
   const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
-  const int head = lid / gridDim.x, tblk = lid % gridDim.x, tok0 = tblk * 128;
+  // (own positions start at X.lo: the grid covers the 128-token blocks from that one on)
+  const int head = lid / gridDim.x, bidx = lid % gridDim.x, tblk = (X.lo >> 7) + bidx, tok0 = tblk * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
@@ -58,13 +58,13 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   // and the state to head ha = head / adiv (one of the divisors is 1; c_i, the output and the
   // normalisation partial are per query head = head)
   const int hx = head / xdiv, ha = head / adiv;
-  const T* Xh = X + (int64_t)hx * n * D;
-  const T* Yh = Y + (int64_t)hx * n * D;
-  const T* A1h = A1 + (int64_t)ha * n * D;
-  const T* A2h = A2 + (int64_t)ha * n * D;
-  const float* ydh = yden ? yden + (int64_t)hx * n * yden_stride : nullptr;
-  const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
-  const float* ch = cvec + (int64_t)head * n;
+  const HeadRows<const T> Xh = X.head(hx), Yh = Y.head(hx), A1h = A1.head(ha), A2h = A2.head(ha);
+  const float* ydh = yden.head(hx);
+  const float* a2dh = a2den.head(ha);
+  const int64_t yden_stride = yden.stride, a2den_stride = a2den.stride;
+  // c belongs to the query side: own tokens for dq, streamed tokens for dk (cvec.stride == 1)
+  const float* ch = cvec.head(head);
+  const int xlo = Xh.lo, alo = A1h.lo;
   const float xs = xscale[hx], a1s = a1scale[ha];
   const int xrow = w * 32 + i, tok = tok0 + xrow;
 
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
     const int r0 = (tile0 + kk) * 32;
     t1.load(A1h, r0, n, tid);
     t2.load(A2h, r0, n, tid, a2dh, a2den_stride);
-    if (!DQ && tid < 32) creg = (r0 + tid < n) ? ch[r0 + tid] : 0.f;
+    if (!DQ && tid < 32) creg = (r0 + tid < n && r0 + tid >= alo) ? ch[r0 + tid] : 0.f;
   };
   auto tiles_store = [&](int buf) {
     t1.store(Sl + buf * SLABF, LD, a1s, tid);
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   // token, the own rows.
   if (n_tile > 0) tiles_load(0);
   if (n_state > 0) slab_load(0);
-  const float c_ld = DQ ? ch[tok < n ? tok : n - 1] : 0.f;
+  const float c_ld = DQ ? ch[max(tok < n ? tok : n - 1, xlo)] : 0.f;
   {
     RowTile<D, T, 128> t, u;
     t.load(Xh, tok0, n, tid);
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
     const float4 y4 = *reinterpret_cast<const float4*>(Sl + xrow * LD + hh * H2 + t);
     Yr[t] = y4.x; Yr[t + 1] = y4.y; Yr[t + 2] = y4.z; Yr[t + 3] = y4.w;
   }
-  const float c_own = (DQ && tok < n) ? c_ld : 0.f;
+  const float c_own = (DQ && tok < n && tok >= xlo) ? c_ld : 0.f;
   const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f;
   __syncthreads();
   if (n_state > 0) {
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 
   // rows of out are tokens, lanes are channels: store directly, scaled by the normaliser
   float rs = 0.f;
-  T* Oh = OUT + (int64_t)head * n * D;
+  const HeadRows<T> Oh = OUT.head(head);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int tk = tok0 + w * 32 + trow(r, hh);
@@ -292,11 +292,11 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
     for (int ab = 0; ab < AB; ++ab) {
       const float g = out[ab][r];
       rs += g * xown[ab][r];
-      if (tk < n) Oh[(int64_t)tk * D + ab * 32 + i] = from_f32<T>(g * xs);
+      if (tk < n && tk >= xlo) Oh.base[(unsigned)tk * Oh.pitch + (unsigned)(ab * 32 + i)] = from_f32<T>(g * xs);
     }
   }
   rs = block_sum_256(rs, red, tid);
-  if (tid == 0) rpart[(int64_t)head * gridDim.x + tblk] = rs;
+  if (tid == 0) rpart[(int64_t)head * gridDim.x + bidx] = rs;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -313,11 +313,10 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 // ---------------------------------------------------------------------------------------
 template <int D, int MODE>
 __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
-    const bf16_t* __restrict__ X, const bf16_t* __restrict__ Y, const float* __restrict__ yden,
-    int64_t yden_stride, const float* __restrict__ cvec, const bf16_t* __restrict__ A1,
-    const bf16_t* __restrict__ A2, const float* __restrict__ a2den, int64_t a2den_stride,
+    Rows<const bf16_t> X, Rows<const bf16_t> Y, RowScalars yden, RowScalars cvec, Rows<const bf16_t> A1,
+    Rows<const bf16_t> A2, RowScalars a2den,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
-    const float* state, int nslots, bf16_t* __restrict__ OUT, float* __restrict__ rpart,
+    const float* state, int nslots, Rows<bf16_t> OUT, float* __restrict__ rpart,
     int n, int chunk, int masked, int p2, float a1, float a2, int xdiv, int adiv) {
   using G = Geo<D>;
   using T = bf16_t;
@@ -334,7 +333,8 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int lid = xcd_logical_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
-  const int head = lid / gridDim.x, tblk = lid % gridDim.x, tok0 = tblk * 128;
+  // (own positions start at X.lo: the grid covers the 128-token blocks from that one on)
+  const int head = lid / gridDim.x, bidx = lid % gridDim.x, tblk = (X.lo >> 7) + bidx, tok0 = tblk * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
   const int rows2 = G::rows2(p2);
@@ -343,13 +343,13 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   // and the state to head ha = head / adiv (one of the divisors is 1; c_i, the output and the
   // normalisation partial are per query head = head)
   const int hx = head / xdiv, ha = head / adiv;
-  const T* Xh = X + (int64_t)hx * n * D;
-  const T* Yh = Y + (int64_t)hx * n * D;
-  const T* A1h = A1 + (int64_t)ha * n * D;
-  const T* A2h = A2 + (int64_t)ha * n * D;
-  const float* ydh = yden ? yden + (int64_t)hx * n * yden_stride : nullptr;
-  const float* a2dh = a2den ? a2den + (int64_t)ha * n * a2den_stride : nullptr;
-  const float* ch = cvec + (int64_t)head * n;
+  const HeadRows<const T> Xh = X.head(hx), Yh = Y.head(hx), A1h = A1.head(ha), A2h = A2.head(ha);
+  const float* ydh = yden.head(hx);
+  const float* a2dh = a2den.head(ha);
+  const int64_t yden_stride = yden.stride, a2den_stride = a2den.stride;
+  // c belongs to the query side: own tokens for dq, streamed tokens for dk (cvec.stride == 1)
+  const float* ch = cvec.head(head);
+  const int xlo = Xh.lo, alo = A1h.lo;
   const float xs = xscale[hx], a1s = a1scale[ha];
   const int xrow = w * 32 + i, tok = tok0 + xrow;
 
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     const int r0 = (tile0 + kk) * 32;
     t1.load(A1h, r0, n, tid);
     t2.load(A2h, r0, n, tid, a2dh, a2den_stride);
-    if (!DQ && tid < 32) creg = (r0 + tid < n) ? ch[r0 + tid] : 0.f;
+    if (!DQ && tid < 32) creg = (r0 + tid < n && r0 + tid >= alo) ? ch[r0 + tid] : 0.f;
   };
   auto tiles_store = [&](int buf) {
     t1.store_bf(Sb[buf], LB, a1s, tid);
@@ -418,7 +418,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   // token, the own rows.
   if (n_tile > 0) tiles_load(0);
   if (n_state > 0) slab_load(0);
-  const float c_ld = DQ ? ch[tok < n ? tok : n - 1] : 0.f;
+  const float c_ld = DQ ? ch[max(tok < n ? tok : n - 1, xlo)] : 0.f;
   {
     RowTile<D, T, 128> t, u;
     t.load(Xh, tok0, n, tid);
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
 #pragma unroll
   for (int g4 = 0; g4 < H2 / 4; ++g4)
     Yp[g4] = *reinterpret_cast<const uint2*>(&Sb[0][0] + xrow * LB + hh * H2 + 4 * g4);
-  const float c_own = (DQ && tok < n) ? c_ld : 0.f;
+  const float c_own = (DQ && tok < n && tok >= xlo) ? c_ld : 0.f;
   const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
   // pairs with (e_hi, e_hi, e_lo, e_lo); the upper four k slots of that MFMA are empty
   const bf8v yxp = as_bf8(pack_bf4u(yxhi, yx - yxhi, yxhi, yx - yxhi), make_uint2(0u, 0u));
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   }
 
   float rs = 0.f;
-  T* Oh = OUT + (int64_t)head * n * D;
+  const HeadRows<T> Oh = OUT.head(head);
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int tk = tok0 + w * 32 + trow(r, hh);
@@ -603,9 +603,9 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     for (int ab = 0; ab < AB; ++ab) {
       const float g = out[ab][r];
       rs += g * xown[ab][r];
-      if (tk < n) Oh[(int64_t)tk * D + ab * 32 + i] = from_f32<T>(g * xs);
+      if (tk < n && tk >= xlo) Oh.base[(unsigned)tk * Oh.pitch + (unsigned)(ab * 32 + i)] = from_f32<T>(g * xs);
     }
   }
   rs = block_sum_256(rs, red, tid);
-  if (tid == 0) rpart[(int64_t)head * gridDim.x + tblk] = rs;
+  if (tid == 0) rpart[(int64_t)head * gridDim.x + bidx] = rs;
 }

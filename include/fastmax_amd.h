@@ -14,6 +14,15 @@
  * same memory.  The output may carry a row pitch ldo >= d so that the reference's
  * (bh, n, d+1) "o with the denominator in column d" (fastmax_cuda_forward.cu:353,
  * example.py:47) is written in place: pass ldo = d+1, den = o + d, den_stride = d+1.
+ * q, k, v, grad_output and the gradients must be 16-byte aligned.  The *_strided entry points
+ * take the same tensors with explicit batch / group / head / token strides (fastmax_layout), e.g.
+ * views into a fused (b, t, groups*(q_per_kv+2)*hs) projection and a token-major (b, t, h*hs)
+ * output, which is how the reference's GPT block holds them before its permute / .contiguous()
+ * copies (model.py:474-499, 572-574, 603).
+ *
+ * Key prefix (fastmax_cuda_forward.cu:109-150): with mask != 0 and nk > nq, query i sits at
+ * key position i + (nk - nq), i.e. the first nk - nq keys are visible to every query.  With
+ * mask == 0 any nq, nk are allowed (every query sees every key).
  */
 #ifndef FASTMAX_AMD_H
 #define FASTMAX_AMD_H
@@ -30,7 +39,7 @@ typedef struct ihipStream_t* fastmax_stream_t; /* == hipStream_t */
 enum {
   FASTMAX_OK = 0,
   FASTMAX_E_NULL = -1,        /* a required pointer is NULL                         */
-  FASTMAX_E_SHAPE = -2,       /* unsupported bh / n / d, bhkv not dividing bh, nq != nk */
+  FASTMAX_E_SHAPE = -2,       /* unsupported bh / n / d, bhkv not dividing bh, nk < nq under mask */
   FASTMAX_E_DTYPE = -3,       /* dtype not FASTMAX_F32 / FASTMAX_BF16               */
   FASTMAX_E_PARAM = -4,       /* p not in {1,2}, bad lim / temperature / pitch      */
   FASTMAX_E_WORKSPACE = -5,   /* workspace NULL, misaligned or too small            */
@@ -51,8 +60,13 @@ typedef struct fastmax_desc {
                           i / (bh / bhkv)  (fastmax_cuda_forward.cu:38); k, v, dk, dv are
                           then (bhkv, n, d)                                              */
   int32_t nq;          /* query tokens                                                   */
-  int32_t nk;          /* key tokens; must equal nq                                      */
-  int32_t d;           /* head dimension: 32 or 64                                        */
+  int32_t nk;          /* key tokens; mask != 0: nk >= nq, the first nk - nq keys are a
+                          prefix every query sees (fastmax_cuda_forward.cu:109-150)      */
+  int32_t d;           /* head dimension: 32 or 64 (the reference's kernels take d at run
+                          time, fastmax_cuda_forward.cu:331-338; this library's kernels keep
+                          a head's state tiles in registers and exist for these two sizes
+                          only -- d = 128 is deliberately not built, other d <= 64 are
+                          zero-padded by the Python module)                              */
   int32_t dtype;       /* FASTMAX_F32 or FASTMAX_BF16 (bf16 in/out, fp32 accumulation)    */
   int32_t mask;        /* 0: every key visible, 1: causal (j <= i)                       */
   int32_t normalize;   /* 1: x <- lim * x / max_n ||x_n||_2 per head for q and k,
@@ -112,6 +126,43 @@ int fastmax_backward(const fastmax_desc* desc, const void* q, const void* k, con
                      const float* qk_scale, const int32_t* qk_argmax,
                      void* workspace, size_t workspace_bytes, fastmax_stream_t stream);
 
+/* Strided tensors.  A tensor is addressed as (batch b, key/value group g, query head j within
+ * the group, token t, channel c) at  b*batch + g*group + j*head + t*token + c  elements from its
+ * pointer; key/value tensors (k, v, dk, dv) have no j.  Head index h of the plain entry points is
+ * (b*groups + g)*q_per_kv + j for query-side tensors, b*groups + g for key/value tensors, with
+ * q_per_kv = bh / bhkv; groups must divide bhkv.  Every stride must keep rows 16-byte aligned
+ * (o: any token stride >= d).  No counterpart in the reference's kernels, which require the
+ * contiguous (b, h, n, d) copies its callers make (model.py:572-574); this replaces those copies
+ * and the transpose of the result (model.py:603).
+ * Causal p = 1 at d = 64 with many heads runs as a register-resident scan only for plain
+ * contiguous tensors with nq == nk; strided or prefixed calls of that shape use the chunked
+ * kernels, so their workspace sizes come from the *_strided queries below (layout == NULL there
+ * means contiguous).  den stays (bh, nq) with den_stride between tokens. */
+typedef struct fastmax_strides {
+  int64_t batch, group, head, token;
+} fastmax_strides;
+typedef struct fastmax_layout {
+  int32_t groups;       /* key/value heads per batch element                              */
+  int32_t reserved;     /* 0                                                              */
+  fastmax_strides q, k, v, o, go, dq, dk, dv;
+} fastmax_layout;
+size_t fastmax_workspace_bytes_strided(const fastmax_desc* desc, const fastmax_layout* layout, int pass);
+size_t fastmax_workspace_min_bytes_strided(const fastmax_desc* desc, const fastmax_layout* layout, int pass);
+size_t fastmax_saved_state_bytes_strided(const fastmax_desc* desc, const fastmax_layout* layout);
+/* As fastmax_forward_saving / fastmax_backward_saved (saved_states may be NULL); layout->o.token
+ * takes the place of ldo.  The forward pass reads layout->q, k, v, o; the backward pass reads
+ * all eight members. */
+int fastmax_forward_strided(const fastmax_desc* desc, const fastmax_layout* layout, const void* q,
+                            const void* k, const void* v, void* o, float* den, int64_t den_stride,
+                            float* qk_scale, int32_t* qk_argmax, void* workspace, size_t workspace_bytes,
+                            void* saved_states, size_t saved_bytes, fastmax_stream_t stream);
+int fastmax_backward_strided(const fastmax_desc* desc, const fastmax_layout* layout, const void* q,
+                             const void* k, const void* v, const void* o, const float* den,
+                             int64_t den_stride, const void* go, void* dq, void* dk, void* dv,
+                             const float* qk_scale, const int32_t* qk_argmax, void* workspace,
+                             size_t workspace_bytes, const void* saved_states, size_t saved_bytes,
+                             fastmax_stream_t stream);
+
 /* Keeping the prefix states for the backward pass (no counterpart in the reference, whose
  * backward re-walks the sequence, fastmax_cuda_backward.cu:26-882).  The backward pass needs
  * the same prefix states S of (k, v) the forward pass built; fastmax_backward rebuilds them
@@ -167,17 +218,19 @@ int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k,
  * which caches k and v because its attention is recomputed from them).  The reference has
  * no such kernel; the arithmetic is the running state of its causal loop
  * (fastmax_cuda_forward.cu:102-197).  A state is fastmax_state_bytes(desc) bytes of fp32 per
- * head, heads contiguous; its layout is private to the library.  The normalisation by the
+ * key/value head (bhkv of them), heads contiguous; its layout is private to the library.  The normalisation by the
  * maximum row norm is not causal, so with normalize != 0 the caller passes the per-head
  * factors (bh floats each, device memory) that a forward pass over the prompt reported in
  * qk_scale (q factors first, then k factors); with normalize == 0 they may be NULL (q: 1,
  * k: 1/temperature).  mask is ignored by these calls.
  *
- * fastmax_state_update: state (+)= the sum over desc->nk tokens of k, v (bh, nk, d); with
+ * fastmax_state_update: state (+)= the sum over desc->nk tokens of k, v (bhkv, nk, d); with
  *   accumulate == 0 the state is overwritten.  workspace: as fastmax_forward for the same
  *   descriptor with mask = 0.
- * fastmax_decode_step: one new token per head (desc->nq = desc->nk = 1; q, k, v are (bh, 1, d)):
- *   the state takes in (k, v), then o = phi(q).S / den -- the causal output row of that token.
+ * fastmax_decode_step: one new token per head (desc->nq = desc->nk = 1; q is (bh, 1, d), k and v
+ *   are (bhkv, 1, d)): the state of a key/value head takes in (k, v), then every query head of its
+ *   group gets o = phi(q).S / den -- the causal output row of that token
+ *   (fastmax_cuda_forward.cu:38).
  *   den may be NULL.  workspace: fastmax_decode_workspace_bytes(desc), 256-byte aligned. */
 size_t fastmax_state_bytes(const fastmax_desc* desc);
 size_t fastmax_decode_workspace_bytes(const fastmax_desc* desc);

@@ -75,3 +75,32 @@ def test_decode_argument_errors(built):
     with pytest.raises(_cabi.FastmaxError, match="k_scale"):
         ops.state_update(state, torch.zeros(2, 8, 64, device="cuda"), torch.zeros(2, 8, 64, device="cuda"),
                          normalize=True)
+
+
+@pytest.mark.parametrize("d,p,dtype,tol", [(64, 2, torch.float32, 1e-4), (32, 1, torch.float32, 1e-4),
+                                           (64, 2, torch.bfloat16, 2e-2)])
+def test_grouped_heads_in_the_recurrent_form(built, d, p, dtype, tol):
+    """bhkv < bh: one state per key/value head, read by every query head of its group
+    (fastmax_cuda_forward.cu:38)."""
+    from fastmax_amd import ops
+
+    bh, bhkv, n, n_prompt = 6, 2, 150, 130
+    ratio = bh // bhkv
+    q, _, _, _ = O.seeded_inputs((bh, n, d), seed=33, dtype=dtype)
+    _, k, v, _ = O.seeded_inputs((bhkv, n, d), seed=34, dtype=dtype)
+    ke, ve = k.repeat_interleave(ratio, dim=0), v.repeat_interleave(ratio, dim=0)
+    ref, rden = O.dense_truth(q.float(), ke.float(), ve.float(), None, mask=True, normalize=True, p=p)
+    qs, ks = _scales(q.float(), k.float())
+    qd, kd, vd, qsd, ksd = (t.cuda() for t in (q, k, v, qs, ks))
+    state = ops.new_state(bhkv, d, p=p, dtype=dtype)
+    ops.state_update(state, kd[:, :n_prompt].contiguous(), vd[:, :n_prompt].contiguous(), k_scale=ksd,
+                     accumulate=False, normalize=True, p=p)
+    outs, dens = [], []
+    for t in range(n_prompt, n):
+        o, den = ops.decode_step(state, qd[:, t:t + 1].contiguous(), kd[:, t:t + 1].contiguous(),
+                                 vd[:, t:t + 1].contiguous(), q_scale=qsd, k_scale=ksd, normalize=True, p=p)
+        assert o.shape == (bh, 1, d)
+        outs.append(o)
+        dens.append(den)
+    assert_close("decode rows", torch.cat(outs, dim=1), ref[:, n_prompt:], tol)
+    assert_close("decode den", torch.cat(dens, dim=1), rden[:, n_prompt:], tol)
