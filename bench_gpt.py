@@ -42,9 +42,9 @@ def apply_rope(x, cos, sin):
 
 
 class Block(nn.Module):
-    def __init__(self, d_model, n_head, d_mlp, attn, p, fused_rope):
+    def __init__(self, d_model, n_head, d_mlp, attn, p, layout):
         super().__init__()
-        self.n_head, self.hs, self.p, self.fused_rope = n_head, d_model // n_head, p, fused_rope
+        self.n_head, self.hs, self.p, self.layout = n_head, d_model // n_head, p, layout
         self.ln1 = nn.LayerNorm(d_model)
         self.qkv = nn.Linear(d_model, 3 * d_model)
         self.proj = nn.Linear(d_model, d_model)
@@ -56,7 +56,15 @@ class Block(nn.Module):
     def forward(self, x, cos, sin):
         B, T, C = x.shape
         qkv = self.qkv(self.ln1(x))
-        if self.fused_rope:
+        if self.layout == "packed":
+            # no layout copies at all: RoPE in place in the projection (packed per head as [q, k, v], the
+            # reference's group-major layout with one query per group, model.py:474-497), q, k, v read as
+            # strided views of it, the output written token-major, and in backward dq, dk, dv written
+            # straight into the projection's gradient
+            y = self.attn(qkv, cos, sin, self.n_head, 1, self.hs, self.hs, True, True, 1.0, 1.0, 1.0, 0.5, 1.0, self.p)
+            x = x + self.proj(y)
+            return x + self.out(F.gelu(self.fc(self.ln2(x))))
+        if self.layout == "split":
             # one HBM pass: split of the projection (packed per head as [q, k, v], the reference's
             # group-major layout with one query per group, model.py:474-497), RoPE on q and k,
             # contiguous (B, H, T, hs) outputs
@@ -73,10 +81,10 @@ class Block(nn.Module):
 
 
 class MiniGPT(nn.Module):
-    def __init__(self, vocab, d_model, n_layer, n_head, d_mlp, seq, attn, p, fused_rope):
+    def __init__(self, vocab, d_model, n_layer, n_head, d_mlp, seq, attn, p, layout):
         super().__init__()
         self.wte = nn.Embedding(vocab, d_model)
-        self.blocks = nn.ModuleList(Block(d_model, n_head, d_mlp, attn, p, fused_rope) for _ in range(n_layer))
+        self.blocks = nn.ModuleList(Block(d_model, n_head, d_mlp, attn, p, layout) for _ in range(n_layer))
         self.ln_f = nn.LayerNorm(d_model)
         self.lm_head = nn.Linear(d_model, vocab, bias=False)
         self.seq, self.hs = seq, d_model // n_head
@@ -95,6 +103,14 @@ class MiniGPT(nn.Module):
         for b in self.blocks:
             x = b(x, cos, sin)
         return self.lm_head(self.ln_f(x))
+
+
+class PackedAttention(nn.Module):
+    """The attention of a block on its packed projection (layout "packed")."""
+
+    def forward(self, *args):
+        from fastmax_amd import qkv_attention
+        return qkv_attention(*args)
 
 
 class TimedAttention(nn.Module):
@@ -140,6 +156,10 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--seq", type=int, default=2048)
     ap.add_argument("--pytorch-attention", action="store_true", help="use_custom_gradient=False path")
+    ap.add_argument("--split-rope", action="store_true",
+                    help="split the projection into contiguous (B, H, T, hs) q, k, v with RoPE in one fused kernel and "
+                         "transpose the attention output back (two extra passes over q, k, v, o per direction) "
+                         "instead of running the attention on strided views of the packed projection")
     ap.add_argument("--unfused-rope", action="store_true",
                     help="split the projection, apply RoPE and make q, k, v contiguous with PyTorch ops "
                          "(the reference's chain, model.py:474-497, 812-825, 572-574) instead of the fused kernel")
@@ -151,8 +171,12 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-    attn = TimedAttention(FASTMultiHeadAttention(use_custom_gradient=not args.pytorch_attention))
-    model = MiniGPT(50304, 768, args.layers, 12, 3072, args.seq, attn, args.p, not args.unfused_rope).to(dev)
+    layout = "pytorch" if args.unfused_rope else ("split" if (args.split_rope or args.pytorch_attention) else "packed")
+    if layout == "packed":
+        attn = TimedAttention(PackedAttention())
+    else:
+        attn = TimedAttention(FASTMultiHeadAttention(use_custom_gradient=not args.pytorch_attention))
+    model = MiniGPT(50304, 768, args.layers, 12, 3072, args.seq, attn, args.p, layout).to(dev)
     opt = torch.optim.AdamW(model.parameters(), lr=3e-4, weight_decay=0.1)
     gen = torch.Generator(device=dev).manual_seed(0)
     idx = torch.randint(0, 50304, (args.batch, args.seq + 1), device=dev, generator=gen)
@@ -186,7 +210,9 @@ def main() -> int:
         "config": {"workload": f"{args.layers} layers, d_model 768, 12 heads x 64, MLP 3072 GELU, RoPE, vocab 50304, "
                                f"seq {args.seq}, batch {args.batch}, p={args.p}, AdamW",
                    "attention": "pytorch function" if args.pytorch_attention else "hip kernels",
-                   "qkv split + rope": "pytorch ops" if args.unfused_rope else "fused hip kernel"},
+                   "qkv split + rope": {"pytorch": "pytorch ops", "split": "fused hip kernel, contiguous q/k/v",
+                                        "packed": "rope in place, attention on strided views of the projection, "
+                                                  "token-major output (includes the rope pass in the attention time)"}[layout]},
         "loss_first_last": [losses[0], losses[-1]], "steps": args.steps, "warmup": args.warmup,
     }))
     return 0 if all(math.isfinite(v) for v in losses) else 1

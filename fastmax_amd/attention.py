@@ -39,6 +39,13 @@ def _states_fit(q3: torch.Tensor, k3: torch.Tensor, mask: bool, p: int) -> bool:
     return need <= SAVE_STATES_MEMORY_FRACTION * free
 
 
+def _states_fit_bytes(ext, q5: torch.Tensor, k4: torch.Tensor, mask: bool, p: int) -> bool:
+    """The same test for strided (B, G, R, T, D) / (B, G, T, D) views."""
+    need = ext.saved_state_bytes_strided(q5, k4, bool(mask), int(p))
+    free, _ = torch.cuda.mem_get_info(k4.device)
+    return need <= SAVE_STATES_MEMORY_FRACTION * free
+
+
 class FASTMultiHeadAttention_Function(torch.autograd.Function):
     """Same call signature as example.py:8 / model.py:22."""
 

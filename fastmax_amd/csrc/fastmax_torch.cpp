@@ -361,6 +361,17 @@ int64_t saved_state_bytes(torch::Tensor q, torch::Tensor k, bool mask, int64_t p
   return (int64_t)sb;
 }
 
+int64_t saved_state_bytes_strided(torch::Tensor q, torch::Tensor k, bool mask, int64_t p) {
+  const fastmax_desc ds = make_desc5(q, k, mask, false, 1.0, 1.0, 1.0, 0.5, 1.0, p);
+  fastmax_layout lay{};
+  lay.groups = (int32_t)q.size(1);
+  lay.q = lay.o = strides5(q, "q");
+  lay.k = lay.v = strides4(k, "k");
+  const size_t sb = fastmax_saved_state_bytes_strided(&ds, &lay);
+  TORCH_CHECK(sb > 0, "fastmax: ", fastmax_last_error());
+  return (int64_t)sb;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(fastmax_cuda, m) {
@@ -370,6 +381,7 @@ PYBIND11_MODULE(fastmax_cuda, m) {
   m.def("backwardpass", &backwardpass, "backwardpass");
   m.def("forward_ex", &forward_ex, "forward returning (o, den, qk_scale, qk_argmax, saved_states)");
   m.def("backward_ex", &backward_ex, "backward through the normalisation, returns [dq, dk, dv]");
+  m.def("saved_state_bytes_strided", &saved_state_bytes_strided, "the same for strided (B, G, R, T, D) / (B, G, T, D) views");
   m.def("forward_strided", &forward_strided, "forward on strided (B, G, R, T, D) / (B, G, T, D) views");
   m.def("backward_strided", &backward_strided, "backward on strided views, writes dq, dk, dv in place");
   m.def("version", []() { return std::string(fastmax_version()); });

@@ -1166,7 +1166,9 @@ int fastmax_qkv_rope(const fastmax_rope_desc* desc, int grad, void* qkv, const f
                      void* q, void* k, void* v, fastmax_stream_t stream) {
   g_err[0] = 0;
   if (!desc) return fail(FASTMAX_E_NULL, "desc is NULL");
-  if (!qkv || !q || !k || !v) return fail(FASTMAX_E_NULL, "qkv, q, k and v must be non-NULL");
+  if (!qkv) return fail(FASTMAX_E_NULL, "qkv must be non-NULL");
+  if ((k || v) && (!q || !k || !v))
+    return fail(FASTMAX_E_NULL, "q, k and v must be all non-NULL (split), q alone (rotated q, k rows packed), or all NULL (in place)");
   if (desc->dtype != FASTMAX_F32 && desc->dtype != FASTMAX_BF16)
     return fail(FASTMAX_E_DTYPE, "dtype %d is neither FASTMAX_F32 nor FASTMAX_BF16", desc->dtype);
   if (desc->b < 1 || desc->t < 1 || desc->groups < 1 || desc->q_per_kv < 1 || desc->hs < 4 || desc->hs % 4)

@@ -6,6 +6,11 @@
 // once and written once.
 //   out = x * cos + rot(x) * sin,  rot(x) = (-x2, x1) with x1, x2 the halves of x[:rope_n]
 // The gradient kernel is the adjoint: dx = dy * cos + rotT(dy * sin), rotT(z) = (z2, -z1).
+// With q == nullptr the rotation (or its adjoint) is applied IN PLACE to the q and k rows of the
+// packed tensor and nothing is copied (a thread reads and writes both halves of its channels, so in
+// place is safe).  With q != nullptr and k == nullptr, q is a second packed tensor
+// (b, t, groups, q_per_kv + 1, hs) that receives the rotated q and k rows (v is not touched).  Either
+// way the attention kernels then read q, k, v as strided views of the packed tensors.
 #pragma once
 #include "fm_common.h"
 
@@ -35,7 +40,10 @@ __global__ __launch_bounds__(256) void qkv_rope_kernel(RopeShape s, T* __restric
   const int b = (int)(r / s.t);
   T* src = qkv + ((((int64_t)b * s.t + t) * s.groups + g) * (s.qpk + 2) + slot) * s.hs;
   T* dst;
-  if (slot < s.qpk) dst = q + (((int64_t)b * s.groups * s.qpk + g * s.qpk + slot) * s.t + t) * s.hs;
+  const bool inplace = q == nullptr, packed = k == nullptr;   // (packed: no split, no copy units)
+  if (inplace) dst = src;
+  else if (packed) dst = q + ((((int64_t)b * s.t + t) * s.groups + g) * (s.qpk + 1) + (slot <= s.qpk ? slot : 0)) * s.hs;
+  else if (slot < s.qpk) dst = q + (((int64_t)b * s.groups * s.qpk + g * s.qpk + slot) * s.t + t) * s.hs;
   else if (slot == s.qpk) dst = k + (((int64_t)b * s.groups + g) * s.t + t) * s.hs;
   else dst = v + (((int64_t)b * s.groups + g) * s.t + t) * s.hs;
   // forward reads the packed row and writes the split tensor; the gradient goes the other way
@@ -66,7 +74,7 @@ __global__ __launch_bounds__(256) void qkv_rope_kernel(RopeShape s, T* __restric
     }
     store4(to + c, y1);
     store4(to + c + h, y2);
-  } else {
+  } else if (!packed || (!inplace && slot <= s.qpk)) {
     const int c = rn + 4 * (u - nrot);
     if (c < s.hs) {
       float x[4];
@@ -116,7 +124,10 @@ __global__ __launch_bounds__(256) void qkv_rope16_kernel(RopeShape s, T* __restr
   const int b = (int)(r / s.t);
   T* src = qkv + ((((int64_t)b * s.t + t) * s.groups + g) * (s.qpk + 2) + slot) * s.hs;
   T* dst;
-  if (slot < s.qpk) dst = q + (((int64_t)b * s.groups * s.qpk + g * s.qpk + slot) * s.t + t) * s.hs;
+  const bool inplace = q == nullptr, packed = k == nullptr;   // (packed: no split, no copy units)
+  if (inplace) dst = src;
+  else if (packed) dst = q + ((((int64_t)b * s.t + t) * s.groups + g) * (s.qpk + 1) + (slot <= s.qpk ? slot : 0)) * s.hs;
+  else if (slot < s.qpk) dst = q + (((int64_t)b * s.groups * s.qpk + g * s.qpk + slot) * s.t + t) * s.hs;
   else if (slot == s.qpk) dst = k + (((int64_t)b * s.groups + g) * s.t + t) * s.hs;
   else dst = v + (((int64_t)b * s.groups + g) * s.t + t) * s.hs;
   T* from = GRAD ? dst : src;
@@ -144,7 +155,7 @@ __global__ __launch_bounds__(256) void qkv_rope16_kernel(RopeShape s, T* __restr
     }
     store8(to + c, y1);
     store8(to + c + h, y2);
-  } else {
+  } else if (!packed || (!inplace && slot <= s.qpk)) {
     const int c = rn + 16 * (u - nrot);
     float x[8], y[8];
     load8(from + c, x);

@@ -251,7 +251,13 @@ int fastmax_decode_step(const fastmax_desc* desc, const void* q, const void* k, 
  *              y = x*cos + (-x2, x1)*sin on channels [0, rope_n), x1/x2 = its halves
  *   grad != 0: the adjoint: q, k, v hold the gradients of the three outputs (in), qkv receives
  *              the gradient of the projection (out)
- * cos, sin: (t, rope_n) fp32, rope_n a multiple of 8 (0: no rotation, they may be NULL). */
+ * cos, sin: (t, rope_n) fp32, rope_n a multiple of 8 (0: no rotation, they may be NULL).
+ * No split, for callers that hand strided views to the *_strided attention entry points:
+ *   q == k == v == NULL: the rotation (grad == 0) or its adjoint (grad != 0) is applied in place to
+ *              the q and k rows of qkv (e.g. to the gradient of the projection after the backward pass
+ *              has written dq, dk, dv into it);
+ *   k == v == NULL, q != NULL: q is (b, t, groups, q_per_kv + 1, hs) and receives the rotated q and k rows
+ *              of qkv (grad == 0; v is read by the attention from qkv itself). */
 typedef struct fastmax_rope_desc {
   int32_t b, t, groups, q_per_kv, hs, rope_n;
   int32_t dtype;       /* FASTMAX_F32 or FASTMAX_BF16 */

@@ -8,15 +8,25 @@ import torch.nn.functional as F
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("p", [1, 2])
-def test_small_gpt_gradients_match_pytorch_path(built, p):
+def _hip_attention(layout):
+    import bench_gpt
+    from fastmax_amd import FASTMultiHeadAttention
+
+    return bench_gpt.PackedAttention() if layout == "packed" else FASTMultiHeadAttention(use_custom_gradient=True)
+
+
+@pytest.mark.parametrize("p,layout", [(1, "split"), (2, "split"), (1, "packed"), (2, "packed")])
+def test_small_gpt_gradients_match_pytorch_path(built, p, layout):
+    """layout "split": contiguous q, k, v from the fused split + RoPE kernel; "packed": RoPE in place and
+    the attention on strided views of the packed projection, token-major output, gradients written
+    straight into the projection's gradient."""
     import bench_gpt
     from fastmax_amd import FASTMultiHeadAttention
 
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-    ref_model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 300, FASTMultiHeadAttention(use_custom_gradient=False), p, False).to(dev)
-    hip_model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 300, FASTMultiHeadAttention(use_custom_gradient=True), p, True).to(dev)
+    ref_model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 300, FASTMultiHeadAttention(use_custom_gradient=False), p, "pytorch").to(dev)
+    hip_model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 300, _hip_attention(layout), p, layout).to(dev)
     hip_model.load_state_dict(ref_model.state_dict())
     idx = torch.randint(0, 512, (2, 301), device=dev, generator=torch.Generator(device=dev).manual_seed(1))
     x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
@@ -45,8 +55,8 @@ class _Fp32PyTorchAttention(torch.nn.Module):
         return o.to(q.dtype)
 
 
-@pytest.mark.parametrize("p", [2, 1])
-def test_gpt_at_config5_widths_bf16_gradients(built, p):
+@pytest.mark.parametrize("p,layout", [(2, "split"), (1, "split"), (2, "packed"), (1, "packed")])
+def test_gpt_at_config5_widths_bf16_gradients(built, p, layout):
     """d_model 768, 12 heads x 64, MLP 3072, T = 2048, bf16 autocast, fused projection split + RoPE
     (two layers, batch 2, a small vocabulary): loss and every parameter gradient of the model on the
     HIP kernels against the same model with the PyTorch attention function, at the bf16 tolerance."""
@@ -56,8 +66,8 @@ def test_gpt_at_config5_widths_bf16_gradients(built, p):
     dev = torch.device("cuda:0")
     vocab, T = 1024, 2048
     torch.manual_seed(0)
-    ref_model = bench_gpt.MiniGPT(vocab, 768, 2, 12, 3072, T, _Fp32PyTorchAttention(), p, False).to(dev)
-    hip_model = bench_gpt.MiniGPT(vocab, 768, 2, 12, 3072, T, FASTMultiHeadAttention(), p, True).to(dev)
+    ref_model = bench_gpt.MiniGPT(vocab, 768, 2, 12, 3072, T, _Fp32PyTorchAttention(), p, "pytorch").to(dev)
+    hip_model = bench_gpt.MiniGPT(vocab, 768, 2, 12, 3072, T, _hip_attention(layout), p, layout).to(dev)
     hip_model.load_state_dict(ref_model.state_dict())
     idx = torch.randint(0, vocab, (2, T + 1), device=dev, generator=torch.Generator(device=dev).manual_seed(3))
     x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
@@ -85,7 +95,7 @@ def test_bf16_autocast_step_runs_and_learns(built):
 
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-    model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 256, FASTMultiHeadAttention(), 2, True).to(dev)
+    model = bench_gpt.MiniGPT(512, 128, 2, 2, 256, 256, bench_gpt.PackedAttention(), 2, "packed").to(dev)
     opt = torch.optim.AdamW(model.parameters(), lr=1e-3)
     idx = torch.randint(0, 512, (4, 257), device=dev, generator=torch.Generator(device=dev).manual_seed(2))
     x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
