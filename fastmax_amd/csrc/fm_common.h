@@ -11,6 +11,7 @@
 // score tiles into value/gradient tiles without going through memory.
 #pragma once
 #include <type_traits>
+#include <utility>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -49,6 +50,17 @@ __device__ __forceinline__ uint2 pack_bf4u(float a, float b, float c, float d) {
 __device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
+// The value lane l ^ 32 holds (hh = l / 32): v_permlane32_swap exchanges lanes 32..63 of its first
+// operand with lanes 0..31 of its second, so with the same value in both, the first result carries
+// the lower half's values in the upper lanes and the second the upper half's in the lower lanes.
+// (A ds_bpermute with the address (l ^ 32) * 4 does the same, but a loop of them over the elements of
+// a register vector was seen compiled into ONE permute whose result went to every element.)
+__device__ __forceinline__ float other_half(float v, int hh) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, hh ? r[0] : r[1]);
+}
+
 // row of a 32x32 accumulator tile held by register r in lane half hh
 __device__ __forceinline__ int trow(int r, int hh) { return 8 * (r >> 2) + 4 * hh + (r & 3); }
 
@@ -66,6 +78,17 @@ __device__ __forceinline__ int xcd_logical_id(int linear, int total) {
 struct bf16_t {
   uint16_t x;
 };
+
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N-1>): a loop whose index is a
+// compile-time constant in every iteration
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v.x) << 16); }
@@ -201,7 +224,11 @@ struct Geo {
 // i.e. 8-byte words of four consecutive rows, which is the B operand layout of the bf16 matrix
 // instruction for a contraction over features (apply kernels: plain 64-bit LDS reads); for a
 // contraction over columns (grad kernels) the same words are read through the transposing LDS
-// load (lds_read_tr16).  Consumers stage a slab with plain 16-byte copies.  Columns D..D+3 hold
+// load (lds_read_tr16).  The D/4 row groups of a slab are stored interleaved, group g at position
+// rgpos(g) = 2 (g mod D/8) + g div D/8, i.e. a group of the first half of the channels is followed
+// by the same group of the second half: the grad kernels read one of each per 16 lanes, and next
+// to each other they fall in different LDS banks.  Consumers stage a slab with plain 16-byte
+// copies.  Columns D..D+3 hold
 // the extra (denominator) column split into hi + lo bf16 parts as (hi, hi, lo, lo), because in the
 // grad kernels that term nearly cancels the value columns' sum.  The slabs are followed by the
 // order-0 row as D+1 floats.
@@ -210,6 +237,7 @@ struct PackedGeo {
   using G = Geo<D>;
   static constexpr int NCF = D + 4;
   static constexpr int FSL = (D / 4) * NCF * 4;  // bf16 elements of a slab (a multiple of 128)
+  __host__ __device__ static constexpr int rgpos(int g) { return 2 * (g % (D / 8)) + g / (D / 8); }
   __host__ __device__ static constexpr int nslab(int p2) { return (p2 ? G::NS : 0) + 1; }
   __host__ __device__ static constexpr int64_t z_off(int p2) { return ((int64_t)nslab(p2) * FSL * 2 + 255) / 256 * 256; }
   __host__ __device__ static constexpr int64_t bytes(int p2) { return z_off(p2) + (D + 1) * 4; }

@@ -301,15 +301,26 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 
 // ---------------------------------------------------------------------------------------
 // bf16 variant of grad_kernel (bf16 inputs and outputs): every contraction runs on
-// v_mfma_f32_32x32x16_bf16 with fp32 accumulation.  The state arrives in the packed bf16 form
-// (PackedGeo): a feature-packed slab ([row / 4][column][row % 4], rows carrying their pair weights,
-// extra column split into hi + lo parts) is copied to LDS as it is and read through the
-// transposing LDS load, which hands every lane = row four consecutive columns per 64-bit piece;
-// the two slabs of pair weight 1 are doubled after their contraction, a2 multiplies the
-// accumulated order-2 credits and a1 the order-1 tile.  The token's extended value vector is
-// packed once, so a 32-row tile costs D/8 + 1 MFMAs; the credits are the fp32 register/LDS work
-// of the fp32 kernel.  Streamed tiles are staged as bf16, the first one in both orientations
-// (rows for the scores, transposed for the product with W).
+// v_mfma_f32_32x32x16_bf16 with fp32 accumulation, and the result tiles are TRANSPOSED with
+// respect to the fp32 kernel: rows = channels, lanes = own tokens.  A lane (token, half hh)
+// then holds, for its token, the H2 = D/2 channels [hh H2, (hh+1) H2) of a slab's tile T in
+// registers, next to the token's whole x row and the output accumulators, so both credits of a
+// pair are register FMAs with compile-time register numbers (the shift loop is fully unrolled):
+//     out[jj]     += T[jj] x[jj + s]        out[jj + s] += T[jj] x[jj]
+// Channels jj + s >= H2 belong to the lane of the other half: their x comes from the lane's copy
+// of the other half of the row, and what is owed to them is collected in a second accumulator
+// bank that the two halves exchange once at the end (one v_permlane32_swap per channel).
+//
+// The state arrives in the packed bf16 form (PackedGeo): a slab goes global -> LDS directly, two
+// slabs ahead, into four buffers, one barrier per two slabs.  The state rows are the A operand,
+// read through the transposing LDS load (four consecutive columns of a row per 64-bit piece);
+// the row -> lane assignment of a tile is chosen so that accumulator register r of tile ab is
+// channel hh H2 + 16 ab + r.  The token's extended value vector [y, yx] is the B operand, packed
+// once; a 32-row tile costs D/16 + 1 MFMAs.  The matrix instructions of one tile run while the
+// credits of the tile before are formed and the operands of the next are read.  The two slabs of
+// pair weight 1 are doubled, a2 multiplies the accumulated order-2 credits and a1 the order-1 tile.
+// Streamed tiles of the intra-chunk part have buffers of their own (staged as bf16 in both
+// orientations: rows for the scores, transposed for the product with W).
 // ---------------------------------------------------------------------------------------
 template <int D, int MODE>
 __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
@@ -320,14 +331,25 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     int n, int chunk, int masked, int p2, float a1, float a2, int xdiv, int adiv) {
   using G = Geo<D>;
   using T = bf16_t;
+  using PG = PackedGeo<D>;
   constexpr bool DQ = MODE == 0;
-  constexpr int LD = G::LD, AB = G::AB, H2 = G::H2, NS = G::NS;
+  constexpr int AB = G::AB, H2 = G::H2, NS = G::NS;
   constexpr int LB = D + 4;   // bf16 row pitch (elements)
   constexpr int TPB = 36;     // pitch of the transposed 32-token tile
-  constexpr int SLB0 = D * LB, SLB1 = 2 * 32 * LB + D * TPB;
-  constexpr int SLB = ((SLB0 > SLB1 ? SLB0 : SLB1) + 7) / 8 * 8;
-  __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
-  __shared__ __attribute__((aligned(16))) uint16_t Sb[2][SLB];
+  constexpr int NCF = PG::NCF, FSL = PG::FSL;
+  constexpr int NPC = FSL / 8;                       // 16-byte pieces of a slab
+  constexpr int NPCR = (NPC + 63) / 64 * 64;
+  constexpr int NVS = (NPC + 255) / 256;             // transfers per wave and slab
+  constexpr int SLB = NPCR * 8;
+  constexpr int TILE = (2 * 32 * LB + D * TPB + 7) / 8 * 8;
+  // four slab buffers as four arrays (the compiler tracks outstanding global -> LDS transfers per
+  // LDS object), a dump for transfers nobody needs, two buffers for the streamed tiles
+  __shared__ __attribute__((aligned(16))) uint16_t Sb0[SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb1[SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb2[SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sb3[SLB];
+  __shared__ __attribute__((aligned(16))) uint16_t Sjunk[512];
+  __shared__ __attribute__((aligned(16))) uint16_t Tl[2][TILE];
   __shared__ float Cl[2][32];
   __shared__ float red[4];
 
@@ -337,8 +359,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   const int head = lid / gridDim.x, bidx = lid % gridDim.x, tblk = (X.lo >> 7) + bidx, tok0 = tblk * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
-  const int rows2 = G::rows2(p2);
-  const int64_t SS = masked ? PackedGeo<D>::slot_floats(p2) : G::state_floats(p2);   // slot pitch
+  const int64_t SS = masked ? PG::slot_floats(p2) : G::state_floats(p2);   // slot pitch
   // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
   // and the state to head ha = head / adiv (one of the divisors is 1; c_i, the output and the
   // normalisation partial are per query head = head)
@@ -351,7 +372,9 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   const float* ch = cvec.head(head);
   const int xlo = Xh.lo, alo = A1h.lo;
   const float xs = xscale[hx], a1s = a1scale[ha];
-  const int xrow = w * 32 + i, tok = tok0 + xrow;
+  const int tok = tok0 + w * 32 + i;   // the lane's own token
+  const bool live = tok < n && tok >= xlo;
+  const int tokc = max(tok < n ? tok : n - 1, xlo);
 
   const bool no_state = masked && (DQ ? c == 0 : c == nc - 1);
   const int n_state = no_state ? 0 : (p2 ? NS : 0) + 1;
@@ -368,194 +391,252 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     }
   }
   // packed state of this block's chunk (masked) or the head's summed state (last slot)
-  using PG = PackedGeo<D>;
-  constexpr int NCF = PG::NCF;
-  static_assert(PG::FSL <= SLB, "a feature-packed slab must fit a stage buffer");
   const char* sbase = reinterpret_cast<const char*>(state + ((int64_t)ha * nslots + (masked ? c : nslots - 1)) * SS);
   const uint16_t* fsec = reinterpret_cast<const uint16_t*>(sbase);
 
-  // a C slab is copied as it is: 16-byte pieces global -> registers -> LDS
-  // (no branches: threads past the end wrap round and copy an early piece a second time, so that
-  // every load is issued up front and stays in flight under the MFMAs)
-  constexpr int NPC = PG::FSL / 8, NVS = (NPC + 255) / 256;
-  static_assert(NVS <= 3, "three named pieces per thread (an indexed array would live in scratch)");
-  uint4 sv0, sv1, sv2;
+  // Transfers of slab st into `buf` (wave-uniform).  No branches: pieces past the slab's end wrap
+  // round at the source, and a wave transfer that lies wholly past the end, or a slab past the
+  // last one, is sent to Sjunk.
+  auto slab_dma = [&](int st, uint16_t* buf) __attribute__((always_inline)) {
+    const bool on = st < n_state;
+    const uint16_t* src = fsec + (on ? st : 0) * FSL;
+#pragma unroll
+    for (int r = 0; r < NVS; ++r) {
+      const int first = r * 256 + w * 64;
+      uint16_t* dst = (on && first < NPCR) ? buf + first * 8 : Sjunk;
+      __builtin_amdgcn_global_load_lds(src + ((first + l) % NPC) * 8,
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
+  };
   RowTile<D, T, 32> t1, t2;
   float creg = 0.f;
-  auto slab_load = [&](int st) {
-    const uint4* src = reinterpret_cast<const uint4*>(fsec + st * PG::FSL);
-    sv0 = src[tid % NPC];
-    if constexpr (NVS > 1) sv1 = src[(tid + 256) % NPC];
-    if constexpr (NVS > 2) sv2 = src[(tid + 512) % NPC];
-  };
-  auto slab_store = [&](int st) {
-    uint4* dst = reinterpret_cast<uint4*>(Sb[st & 1]);
-    dst[tid % NPC] = sv0;
-    if constexpr (NVS > 1) dst[(tid + 256) % NPC] = sv1;
-    if constexpr (NVS > 2) dst[(tid + 512) % NPC] = sv2;
-  };
-  auto tiles_load = [&](int kk) {
+  auto tiles_load = [&](int kk) __attribute__((always_inline)) {
     const int r0 = (tile0 + kk) * 32;
     t1.load(A1h, r0, n, tid);
     t2.load(A2h, r0, n, tid, a2dh, a2den_stride);
     if (!DQ && tid < 32) creg = (r0 + tid < n && r0 + tid >= alo) ? ch[r0 + tid] : 0.f;
   };
-  auto tiles_store = [&](int buf) {
-    t1.store_bf(Sb[buf], LB, a1s, tid);
-    t2.store_bf(Sb[buf] + 32 * LB, LB, 1.0f, tid);
-    t1.store_t_bf(Sb[buf] + 2 * 32 * LB, TPB, a1s, tid);
+  auto tiles_store = [&](int buf) __attribute__((always_inline)) {
+    t1.store_bf(Tl[buf], LB, a1s, tid);
+    t2.store_bf(Tl[buf] + 32 * LB, LB, 1.0f, tid);
+    t1.store_t_bf(Tl[buf] + 2 * 32 * LB, TPB, a1s, tid);
     if (!DQ && tid < 32) Cl[buf][tid] = creg;
   };
 
-  f16v out[AB];
+  // Everything the block needs first is requested before anything is waited for: the first two
+  // slabs, the first streamed tile, the own rows, c of the own token.
+  if (n_state > 0) {
+    slab_dma(0, Sb0);
+    slab_dma(1, Sb1);
+  }
+  if (n_tile > 0) tiles_load(0);
+  const float c_ld = DQ ? ch[tokc] : 0.f;
+  // the lane's own token: its whole x row (own half of the channels in xo, the other half in xp),
+  // scaled, and its half of y packed (B operand of the state contraction and of g.v)
+  float xo[H2], xp[H2];
+  uint2 Yp[H2 / 4];
+  {
+    const uint4* xr = reinterpret_cast<const uint4*>(Xh.row(tokc));
+    const uint4* yr = reinterpret_cast<const uint4*>(Yh.row(tokc) + hh * H2);
+    uint4 xa[H2 / 8], xb[H2 / 8], ya[H2 / 8];
+#pragma unroll
+    for (int u = 0; u < H2 / 8; ++u) {
+      xa[u] = xr[hh * (H2 / 8) + u];
+      xb[u] = xr[(1 - hh) * (H2 / 8) + u];
+      ya[u] = yr[u];
+    }
+    const float ydiv = ydh ? ydh[(unsigned)tokc * (unsigned)yden_stride] : 1.0f;
+    const float xsc = live ? xs : 0.f;
+    auto unpack8 = [](const uint4& t, float* o, float sc) {
+      o[0] = bf_lo(t.x) * sc; o[1] = bf_hi(t.x) * sc; o[2] = bf_lo(t.y) * sc; o[3] = bf_hi(t.y) * sc;
+      o[4] = bf_lo(t.z) * sc; o[5] = bf_hi(t.z) * sc; o[6] = bf_lo(t.w) * sc; o[7] = bf_hi(t.w) * sc;
+    };
+#pragma unroll
+    for (int u = 0; u < H2 / 8; ++u) {
+      unpack8(xa[u], xo + 8 * u, xsc);
+      unpack8(xb[u], xp + 8 * u, xsc);
+      uint4 t = ya[u];
+      if (ydh) {   // y = grad_out / den, rounded once
+        float f[8];
+        unpack8(t, f, 1.0f / ydiv);
+        t = make_uint4(pack_bf2(f[0], f[1]), pack_bf2(f[2], f[3]), pack_bf2(f[4], f[5]), pack_bf2(f[6], f[7]));
+      }
+      if (!live) t = make_uint4(0u, 0u, 0u, 0u);
+      Yp[2 * u] = make_uint2(t.x, t.y);
+      Yp[2 * u + 1] = make_uint2(t.z, t.w);
+    }
+  }
+  const float c_own = (DQ && live) ? c_ld : 0.f;
+  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
+  // pairs with the state's extra column stored as (e_hi, e_hi, e_lo, e_lo); the upper four k slots
+  // of that MFMA are empty
+  const bf8v yxp = as_bf8(pack_bf4u(yxhi, yx - yxhi, yxhi, yx - yxhi), make_uint2(0u, 0u));
+  if (n_tile > 0) tiles_store(0);
+
+  // out[ab][r]: channel hh*H2 + 16*ab + r of the lane's token; outx: what the lane collects for
+  // channel (1-hh)*H2 + 16*ab + r of the same token, which the lane of the other half holds
+  f16v out[AB], outx[AB];
 #pragma unroll
   for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) out[ab][r] = 0.f;
+    for (int r = 0; r < 16; ++r) out[ab][r] = outx[ab][r] = 0.f;
 
-  // Everything the block needs first is requested before anything is waited for (one memory
-  // latency instead of three in a row): the first slab, the first streamed tile, c of the own
-  // token, the own rows.
-  if (n_tile > 0) tiles_load(0);
-  if (n_state > 0) slab_load(0);
-  const float c_ld = DQ ? ch[max(tok < n ? tok : n - 1, xlo)] : 0.f;
+  // A operand of tile ab: tile row m = lane i holds channel H2*((m>>2)&1) + 16*ab + 4*(m>>3) + (m&3),
+  // so that accumulator register r of lane half hh (tile row 8*(r>>2) + 4*hh + (r&3)) is channel
+  // hh*H2 + 16*ab + r.  The transposing read hands the lanes 4g..4g+3 of a group of 16 the four rows
+  // of the row group that the lanes J with J % 4 == g addressed, column slot J / 4.
+  int tro[AB];
   {
-    RowTile<D, T, 128> t, u;
-    t.load(Xh, tok0, n, tid);
-    u.load(Yh, tok0, n, tid, ydh, yden_stride);
-    t.store(Xl, LD, xs, tid);
-    // the own y rows only pass through LDS to reach their lanes: [128][LB] bf16 fits one stage pair
-    static_assert(128 * LB <= 2 * SLB, "own-row staging must fit the stage buffers");
-    u.store_bf(&Sb[0][0], LB, 1.0f, tid);
-  }
-  __syncthreads();
-  // own token of this lane = row xrow: its half of y, packed (A operand of the state
-  // contraction, B operand of g.v)
-  uint2 Yp[H2 / 4];
+    const int trj = l & 15;
+    const int mg = 4 * (i >> 4) + (trj & 3);   // row group of the tile
 #pragma unroll
-  for (int g4 = 0; g4 < H2 / 4; ++g4)
-    Yp[g4] = *reinterpret_cast<const uint2*>(&Sb[0][0] + xrow * LB + hh * H2 + 4 * g4);
-  const float c_own = (DQ && tok < n && tok >= xlo) ? c_ld : 0.f;
-  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
-  // pairs with (e_hi, e_hi, e_lo, e_lo); the upper four k slots of that MFMA are empty
-  const bf8v yxp = as_bf8(pack_bf4u(yxhi, yx - yxhi, yxhi, yx - yxhi), make_uint2(0u, 0u));
-  __syncthreads();
-  if (n_state > 0) {
-    slab_store(0);
-  } else if (n_tile > 0) {
-    tiles_store(0);
+    for (int ab = 0; ab < AB; ++ab) {
+      const int cg = (H2 / 4) * (mg & 1) + 4 * ab + (mg >> 1);   // row group of the slab
+      tro[ab] = (PG::rgpos(cg) * NCF + (trj >> 2)) * 4;
+    }
   }
-  __syncthreads();
-
-  // The slab is feature-packed, [row / 4][column][row % 4]; the B operand of the contraction over
-  // columns wants, per lane = row, four consecutive columns per 64-bit piece: the transposing LDS
-  // read delivers exactly that when, in every group of 16 lanes (16 consecutive rows), lane J
-  // addresses the word of row group J % 4 and column J / 4 of the piece.
-  const int trj = l & 15;
-  const int troff = (((i >> 4) * 4 + (trj & 3)) * NCF + (trj >> 2)) * 4;   // + (ab * 8 * NCF + column) * 4
-  auto chain = [&](const uint16_t* sl, int ab) {
-    const uint16_t* ar = sl + ab * 8 * NCF * 4 + troff;
-    uint2 b[H2 / 4 + 1];
+  constexpr int NB = H2 / 4 + 1;
+  struct BOps {
+    uint2 b[NB];
+  };
+  auto fetch = [&](const uint16_t* sl, int ab, BOps& o) __attribute__((always_inline)) {
+    const uint16_t* ar = sl + tro[ab];
 #pragma unroll
-    for (int g4 = 0; g4 < H2 / 4; ++g4) b[g4] = lds_read_tr16(ar + (hh * H2 + 4 * g4) * 4);
-    b[H2 / 4] = lds_read_tr16(ar + D * 4);  // extra column as (hi, hi, lo, lo)
+    for (int g4 = 0; g4 < H2 / 4; ++g4) o.b[g4] = lds_read_tr16(ar + (hh * H2 + 4 * g4) * 4);
+    o.b[H2 / 4] = lds_read_tr16(ar + D * 4);  // extra column as (hi, hi, lo, lo)
+  };
+  auto chain = [&](const BOps& o) __attribute__((always_inline)) {
     f16v t;
 #pragma unroll
     for (int r = 0; r < 16; ++r) t[r] = 0.f;
 #pragma unroll
-    for (int m = 0; m < H2 / 8; ++m) t = FM_MFMA_BF16(as_bf8(Yp[2 * m], Yp[2 * m + 1]), as_bf8(b[2 * m], b[2 * m + 1]), t);
-    return FM_MFMA_BF16(yxp, as_bf8(b[H2 / 4], make_uint2(0u, 0u)), t);
+    for (int m = 0; m < H2 / 8; ++m)
+      t = FM_MFMA_BF16(as_bf8(o.b[2 * m], o.b[2 * m + 1]), as_bf8(Yp[2 * m], Yp[2 * m + 1]), t);
+    return FM_MFMA_BF16(as_bf8(o.b[H2 / 4], make_uint2(0u, 0u)), yxp, t);
   };
-  const float* xtok = Xl + (w * 32 + 4 * hh) * LD;
-  auto xat = [&](int r, int col) { return xtok[((r >> 2) * 8 + (r & 3)) * LD + col]; };
-  // x of the lane's own channels for the 16 token rows of its accumulator registers (the factor
-  // of the mirrored credit and of the normalisation partial), read once
-  float xown[AB][16];
+  // both credits of tile ab of shift S (a compile-time constant; S == NS: the order-1 slab)
+  auto credit = [&](const f16v& t, auto stag, auto abtag) __attribute__((always_inline)) {
+    constexpr int S = decltype(stag)::value, ABI = decltype(abtag)::value;
 #pragma unroll
-  for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) xown[ab][r] = xat(r, ab * 32 + i);
-
-  auto slab_step = [&](int st) {
-    const uint16_t* sl = Sb[st & 1];
-    f16v tt[AB];
-#pragma unroll
-    for (int ab = 0; ab < AB; ++ab) tt[ab] = chain(sl, ab);
-    if (p2 && st < NS) {
-      const int s = st;
-      // the order-2 slabs carry their pair weights (2, except shifts 0 and D/2): bring those two up
-      // to the others, the common factor goes into the final scale
-      if (s == 0 || s == H2) {
-#pragma unroll
-        for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) tt[ab][r] *= 2.0f;
+    for (int r = 0; r < 16; ++r) {
+      const int jj = 16 * ABI + r;
+      const float v = t[r];
+      if constexpr (S == NS) {           // the order-1 slab (its coefficient is applied here)
+        out[ABI][r] += a1 * v;
+      } else if constexpr (S == 0) {     // the diagonal: one member, weight 1 stored, 2 owed
+        out[ABI][r] += (v + v) * xo[jj];
+      } else if constexpr (S == H2) {    // listed from both sides, weight 1 stored, 2 owed
+        out[ABI][r] += (v + v) * xp[jj];
+      } else {
+        const int p = jj + S;
+        if (p < H2) {
+          out[ABI][r] += v * xo[p];
+          out[p >> 4][p & 15] += v * xo[jj];
+        } else {
+          out[ABI][r] += v * xp[p - H2];
+          outx[(p - H2) >> 4][(p - H2) & 15] += v * xo[jj];
+        }
       }
-#pragma unroll
-      for (int ab = 0; ab < AB; ++ab) {
-        const int rc = (ab * 32 + i + s) & (D - 1);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) out[ab][r] += tt[ab][r] * xat(r, rc);
-      }
-      if (s > 0 && s < H2) {
-#pragma unroll
-        for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) tt[ab][r] *= xown[ab][r];
-        const bool keep = i < 32 - s;
-        const int src = (((i - s) & 31) + 32 * hh) << 2;
-#pragma unroll
-        for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float v = keep ? tt[ab][r] : tt[(ab + 1) % AB][r];
-            out[ab][r] += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, v)));
-          }
-      }
-      if (st == NS - 1) {  // f'(s) contributes 2*a2 to the order-2 sum, the pair weight 2 is already in
-#pragma unroll
-        for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) out[ab][r] *= a2;
-      }
-    } else {
-#pragma unroll
-      for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) out[ab][r] += a1 * tt[ab][r];
     }
   };
-  // the last slab is peeled off so that load and store of the next slab are unconditional in
-  // the loop (a load whose only use sits in a branch is moved there and waited for at once)
-  for (int st = 0; st + 1 < n_state; ++st) {
-    slab_load(st + 1);
-    slab_step(st);
-    slab_store(st + 1);
-    __syncthreads();
-  }
+
+
   if (n_state > 0) {
-    slab_step(n_state - 1);
-    if (n_tile > 0) tiles_store(n_state & 1);
+    FM_WAIT_VM(0);
     __syncthreads();
   }
+  if (n_state > 1) {
+    // p = 2.  Tile units u = slab * AB + ab over slabs 0 .. NS (slab NS is the order-1 slab).  Slabs
+    // 2k, 2k+1 sit in buffers (Sb0, Sb1) for even k and (Sb2, Sb3) for odd k.  Per unit: read the
+    // operands of the next unit, run this unit's matrix instructions, form the credits of the unit
+    // before (whose results are complete by now).
+    static_assert(NS % 2 == 1, "the order-2 slabs and the order-1 slab make whole steps of two");
+    constexpr int NU = (NS + 1) * AB;
+    BOps bc, bn;
+    f16v tp, tn;
+    fetch(Sb0, 0, bc);
+    static_for<(NS + 1) / 2>([&](auto ktag) __attribute__((always_inline)) {
+      constexpr int K = decltype(ktag)::value;
+      uint16_t* cur0 = (K & 1) ? Sb2 : Sb0;
+      uint16_t* cur1 = (K & 1) ? Sb3 : Sb1;
+      uint16_t* nxt0 = (K & 1) ? Sb0 : Sb2;
+      uint16_t* nxt1 = (K & 1) ? Sb1 : Sb3;
+      __builtin_amdgcn_sched_barrier(0);
+      // (every wave is past the buffers of the step before: it has passed the barrier)
+      slab_dma(2 * K + 2, nxt0);
+      slab_dma(2 * K + 3, nxt1);
+      static_for<2 * AB>([&](auto vtag) __attribute__((always_inline)) {
+        constexpr int V = decltype(vtag)::value, U = 2 * K * AB + V;
+        // operands of the next unit of this step (the first unit of the next step is read after the barrier)
+        if constexpr (V + 1 < 2 * AB) fetch(((V + 1) / AB) ? cur1 : cur0, (V + 1) % AB, bn);
+        tn = chain(bc);
+        if constexpr (U > 0) {
+          constexpr int PS = (U - 1) / AB, PAB = (U - 1) % AB;
+          if constexpr (PS == NS && PAB == 0) {
+            // order 2 is complete: its coefficient (the pair weight 2 of f' is in the stored rows)
+#pragma unroll
+            for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                out[ab][r] *= a2;
+                outx[ab][r] *= a2;
+              }
+          }
+          credit(tp, std::integral_constant<int, PS>{}, std::integral_constant<int, PAB>{});
+        }
+        tp = tn;
+        if constexpr (V + 1 < 2 * AB) bc = bn;
+      });
+      if constexpr (2 * K + 2 <= NS) {
+        FM_WAIT_VM(0);
+        __builtin_amdgcn_s_barrier();
+        fetch(nxt0, 0, bc);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if constexpr (AB == 1) {   // the order-1 slab is a single unit: order 2 ends with the unit before
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        out[0][r] *= a2;
+        outx[0][r] *= a2;
+      }
+    }
+    credit(tp, std::integral_constant<int, (NU - 1) / AB>{}, std::integral_constant<int, (NU - 1) % AB>{});
+    // hand over what was collected for the channels of the other half
+#pragma unroll
+    for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) out[ab][r] += other_half(outx[ab][r], hh);
+  } else if (n_state == 1) {
+    // p = 1: the order-1 slab is the only one
+    static_for<AB>([&](auto abtag) __attribute__((always_inline)) {
+      BOps b1;
+      fetch(Sb0, decltype(abtag)::value, b1);
+      const f16v t = chain(b1);
+      credit(t, std::integral_constant<int, NS>{}, abtag);
+    });
+  }
+  if (n_tile > 0) __syncthreads();   // the first streamed tile is staged
 
   if (n_tile > 0) {
     uint2 Xp[H2 / 4];
 #pragma unroll
-    for (int g4 = 0; g4 < H2 / 4; ++g4) {
-      const float4 x4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + hh * H2 + 4 * g4);
-      Xp[g4] = pack_bf4u(x4.x, x4.y, x4.z, x4.w);
-    }
+    for (int g4 = 0; g4 < H2 / 4; ++g4) Xp[g4] = pack_bf4u(xo[4 * g4], xo[4 * g4 + 1], xo[4 * g4 + 2], xo[4 * g4 + 3]);
     const int mine = (tok0 >> 5) + w;
     const float twoa2 = 2.0f * a2;
+    // tile row m = lane i of the product with W is channel chrow[ab] (same assignment as the state tiles)
+    int chrow[AB];
+#pragma unroll
+    for (int ab = 0; ab < AB; ++ab) chrow[ab] = H2 * ((i >> 2) & 1) + 16 * ab + 4 * (i >> 3) + (i & 3);
     for (int kk = 0; kk < n_tile; ++kk) {
-      const int buf = (n_state + kk) & 1;
+      const int buf = kk & 1;
       tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
       const int tl = tile0 + kk;
       if (DQ ? tl <= mine : tl >= mine) {
-        const uint16_t* l1 = Sb[buf];
+        const uint16_t* l1 = Tl[buf];
         const uint16_t* l2 = l1 + 32 * LB;
         const uint16_t* l1t = l1 + 2 * 32 * LB;
+        // scores and g.v: rows = streamed tokens trow(r,hh), lanes = own tokens
         f16v sc, gv;
 #pragma unroll
         for (int r = 0; r < 16; ++r) sc[r] = gv[r] = 0.f;
@@ -576,16 +657,17 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
           if (diag && (DQ ? trow(r, hh) > i : trow(r, hh) < i)) wv = 0.f;
           sc[r] = wv;
         }
+        // out (channels x own) += A1^T (channels x streamed) . W (streamed x own)
 #pragma unroll
         for (int m = 0; m < 2; ++m) {
-          // accumulator rows 8m..8m+7 of this lane half = tokens 16m + 4hh + {0..3} and + 8
+          // accumulator rows 8m..8m+7 of this lane half = streamed tokens 16m + 4hh + {0..3} and + 8
           const bf8v wp = as_bf8(pack_bf4u(sc[8 * m], sc[8 * m + 1], sc[8 * m + 2], sc[8 * m + 3]),
                                  pack_bf4u(sc[8 * m + 4], sc[8 * m + 5], sc[8 * m + 6], sc[8 * m + 7]));
 #pragma unroll
           for (int ab = 0; ab < AB; ++ab) {
-            const uint16_t* trw = l1t + (ab * 32 + i) * TPB + 16 * m + 4 * hh;
-            out[ab] = FM_MFMA_BF16(wp, as_bf8(*reinterpret_cast<const uint2*>(trw), *reinterpret_cast<const uint2*>(trw + 8)),
-                                   out[ab]);
+            const uint16_t* trw = l1t + chrow[ab] * TPB + 16 * m + 4 * hh;
+            out[ab] = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(trw), *reinterpret_cast<const uint2*>(trw + 8)),
+                                   wp, out[ab]);
           }
         }
       }
@@ -594,16 +676,20 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     }
   }
 
+  // the lane holds H2 consecutive channels of its token: 16-byte stores, scaled by the normaliser
   float rs = 0.f;
-  const HeadRows<T> Oh = OUT.head(head);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int tk = tok0 + w * 32 + trow(r, hh);
+  for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
-    for (int ab = 0; ab < AB; ++ab) {
-      const float g = out[ab][r];
-      rs += g * xown[ab][r];
-      if (tk < n && tk >= xlo) Oh.base[(unsigned)tk * Oh.pitch + (unsigned)(ab * 32 + i)] = from_f32<T>(g * xs);
+    for (int r = 0; r < 16; ++r) rs += out[ab][r] * xo[16 * ab + r];
+  if (live) {
+    uint4* orow = reinterpret_cast<uint4*>(OUT.head(head).row(tok) + hh * H2);
+#pragma unroll
+    for (int u = 0; u < H2 / 8; ++u) {
+      const f16v& o = out[u >> 1];
+      const int r0 = 8 * (u & 1);
+      orow[u] = make_uint4(pack_bf2(o[r0] * xs, o[r0 + 1] * xs), pack_bf2(o[r0 + 2] * xs, o[r0 + 3] * xs),
+                           pack_bf2(o[r0 + 4] * xs, o[r0 + 5] * xs), pack_bf2(o[r0 + 6] * xs, o[r0 + 7] * xs));
     }
   }
   rs = block_sum_256(rs, red, tid);
