@@ -61,6 +61,14 @@ __device__ __forceinline__ float other_half(float v, int hh) {
   return __builtin_bit_cast(float, hh ? r[0] : r[1]);
 }
 
+// For a lane of the lower half: the value `from_upper` holds in lane l + 32; for a lane of the upper
+// half: the value `from_lower` holds in lane l - 32 (one v_permlane32_swap serves both directions).
+__device__ __forceinline__ float swap_halves(float from_upper, float from_lower, int hh) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, from_upper),
+                                                  __builtin_bit_cast(unsigned, from_lower), false, false);
+  return __builtin_bit_cast(float, hh ? r[0] : r[1]);
+}
+
 // row of a 32x32 accumulator tile held by register r in lane half hh
 __device__ __forceinline__ int trow(int r, int hh) { return 8 * (r >> 2) + 4 * hh + (r & 3); }
 

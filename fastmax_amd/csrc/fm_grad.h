@@ -10,19 +10,29 @@
 #include "fm_common.h"
 
 // ---------------------------------------------------------------------------------------
-// One block = 128 own tokens of one head, one wave = 32 of them.  Per shift slab s of the state
-// the kernel contracts the token's extended value vector y_ext = [y, yx] (A operand straight
-// from registers, one extra MFMA for the extra column) with 32 state rows at a time (B operand,
-// 128-bit LDS reads along the columns).  The result tile T (tokens x channels a) holds entry
-// (a, a+s) of every token's symmetric matrix; the state stores each unordered pair once, so
-// both members are credited from the same T:
-//     out[tok][a]         += T[tok][a] * x[tok][(a+s)%D]        (one LDS read, lanes = channels)
-//     out[tok][(a+s)%D]   += T[tok][a] * x[tok][a]              (0 < s < D/2 only)
-// The second credit moves along the channel ring, which is the lane dimension here: the two
-// 32-channel blocks are merged by a lane select and rotated by s with one ds_bpermute.
+// One block = 128 own tokens of one head, one wave = 32 of them, one lane pair (i, hh = 0/1) per
+// token.  Per shift slab s of the state the kernel contracts 32 state rows at a time (A operand,
+// 128-bit LDS reads along the columns) with the token's extended value vector y_ext = [y, yx]
+// (B operand straight from registers, one extra MFMA for the extra column).  The result tile T
+// (channels a x tokens) holds entry (a, a+s) of every token's symmetric matrix; rows = channels,
+// lanes = tokens, so a lane holds, for ITS token, the channels 32 ab + 8 j + 4 hh + e (j, e = 0..3)
+// of tile ab in its 16 accumulator registers: the lane halves own alternating groups of four
+// channels.  The state stores each unordered pair once, so both members are credited from the
+// same T, and with the token's whole x row in registers both credits are register FMAs with
+// compile-time register numbers (the shift loop is fully unrolled):
+//     out[a]         += T[a] * x[(a+s)%D]
+//     out[(a+s)%D]   += T[a] * x[a]                 (0 < s < D/2 only)
+// Whether channel a+s lies in the lane's own half depends only on (a mod 4) + (s mod 8), not on hh;
+// when it does not, it is one of "the four channels just above an own group", for both halves:
+// those x values sit in a second register bank (xp), and what is owed to them is collected in a
+// second accumulator bank (outx) that the two lanes of a token exchange once at the end.
+// Slabs go global -> LDS directly (no staging registers), two slabs ahead into four buffers, one
+// barrier per two slabs; the coefficients multiply the accumulated sums (2 a2 after the order-2
+// slabs, a1 on the order-1 tile).  The matrix instructions of one tile run while the credits of
+// the tile before are formed and the operands of the next are read.
 // Causal intra-chunk part: for every streamed 32-token tile the transposed score and g.v tiles
-// are formed (streamed x own), W is built in registers and fed back as the A operand of
-// out += W^T-as-rows . A1.
+// are formed (streamed x own), W is built in registers and fed back as the B operand of
+// out (channels x own) += A1^T (channels x streamed) . W (streamed x own).
 //
 //   MODE 0 (dq): X = q, Y = grad_out/den, yx = -c_i, state S, streamed A1 = k, A2 = v over tiles
 //                at or before the own tile, W = f'(s)(g.v - c_own)
@@ -35,13 +45,27 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
     Rows<const T> X, Rows<const T> Y, RowScalars yden, RowScalars cvec, Rows<const T> A1,
     Rows<const T> A2, RowScalars a2den,
     const float* __restrict__ xscale, const float* __restrict__ a1scale,
-    const float* __restrict__ state, int nslots, Rows<T> OUT, float* __restrict__ rpart,
+    const float* state, int nslots, Rows<T> OUT, float* __restrict__ rpart,
     int n, int chunk, int masked, int p2, float a1, float a2, int xdiv, int adiv) {
+  static_assert(std::is_same<T, float>::value, "fp32 rows (bf16 rows run grad_kernel_bf)");
   using G = Geo<D>;
   constexpr bool DQ = MODE == 0;
-  constexpr int LD = G::LD, AB = G::AB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
-  __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
-  __shared__ __attribute__((aligned(16))) float Sl[2 * SLABF];
+  constexpr int LD = G::LD, AB = G::AB, H2 = G::H2, NS = G::NS;
+  constexpr int NG = D / 8;                          // groups of eight channels
+  constexpr int SLF = D * LD;                        // floats of a slab (D rows)
+  constexpr int NPC = SLF / 4;                       // 16-byte pieces of a slab
+  constexpr int NPCR = (NPC + 63) / 64 * 64;
+  constexpr int NVS = (NPC + 255) / 256;             // transfers per wave and slab
+  constexpr int TILEF = 2 * 32 * LD;                 // both 32-token tiles of a streamed step
+  constexpr int SLB = NPCR * 4 > TILEF ? NPCR * 4 : TILEF;
+  // four slab buffers as four arrays (the compiler tracks outstanding global -> LDS transfers per
+  // LDS object) and a dump for transfers nobody needs; the streamed tiles of the intra-chunk part
+  // go through Sb2 and Sb3, which the last step of the state part leaves alone
+  __shared__ __attribute__((aligned(16))) float Sb0[SLB];
+  __shared__ __attribute__((aligned(16))) float Sb1[SLB];
+  __shared__ __attribute__((aligned(16))) float Sb2[SLB];
+  __shared__ __attribute__((aligned(16))) float Sb3[SLB];
+  __shared__ __attribute__((aligned(16))) float Sjunk[256];
   __shared__ float Cl[2][32];
   __shared__ float red[4];
 
@@ -52,7 +76,6 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   const int head = lid / gridDim.x, bidx = lid % gridDim.x, tblk = (X.lo >> 7) + bidx, tok0 = tblk * 128;
   const int c = tok0 / chunk;
   const int nc = (n + chunk - 1) / chunk;
-  const int rows2 = G::rows2(p2);
   const int64_t SS = G::state_floats(p2);
   // grouped key/value heads: the own rows belong to head hx = head / xdiv, the streamed rows
   // and the state to head ha = head / adiv (one of the divisors is 1; c_i, the output and the
@@ -66,7 +89,9 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   const float* ch = cvec.head(head);
   const int xlo = Xh.lo, alo = A1h.lo;
   const float xs = xscale[hx], a1s = a1scale[ha];
-  const int xrow = w * 32 + i, tok = tok0 + xrow;
+  const int tok = tok0 + w * 32 + i;   // the lane's own token
+  const bool live = tok < n && tok >= xlo;
+  const int tokc = max(tok < n ? tok : n - 1, xlo);
 
   const bool no_state = masked && (DQ ? c == 0 : c == nc - 1);
   const int n_state = no_state ? 0 : (p2 ? NS : 0) + 1;
@@ -82,181 +107,261 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
       n_tile = ((cend - 1) >> 5) - tile0 + 1;
     }
   }
-  // this block's chunk snapshot (masked) or the head's summed state (last slot)
+  // this block's chunk snapshot (masked) or the head's summed state (last slot); the order-2 slabs
+  // and the order-1 slab are consecutive runs of D rows
   const float* sbase = state + ((int64_t)ha * nslots + (masked ? c : nslots - 1)) * SS;
 
-  StateSlab<D * LD> slab;
+  // Transfers of slab st into `buf` (wave-uniform).  No branches: pieces past the slab's end wrap
+  // round at the source, and a wave transfer that lies wholly past the end, or a slab past the
+  // last one, is sent to Sjunk.
+  auto slab_dma = [&](int st, float* buf) __attribute__((always_inline)) {
+    const bool on = st < n_state;
+    const float* src = sbase + (on ? st : 0) * SLF;
+#pragma unroll
+    for (int r = 0; r < NVS; ++r) {
+      const int first = r * 256 + w * 64;
+      float* dst = (on && first < NPCR) ? buf + first * 4 : Sjunk;
+      __builtin_amdgcn_global_load_lds(src + ((first + l) % NPC) * 4,
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
+  };
   RowTile<D, T, 32> t1, t2;
   float creg = 0.f;
-  auto slab_load = [&](int st) {
-    slab.load(sbase + ((p2 && st < NS) ? st * D * LD : rows2 * LD), D * LD, tid);
-  };
-  auto slab_store = [&](int st) {
-    const float cf = (p2 && st < NS) ? 2.0f * a2 : a1;
-    slab.store(Sl + (st & 1) * SLABF, D * LD, D * LD, cf, cf, tid);
-  };
-  auto tiles_load = [&](int kk) {
+  auto tiles_load = [&](int kk) __attribute__((always_inline)) {
     const int r0 = (tile0 + kk) * 32;
     t1.load(A1h, r0, n, tid);
     t2.load(A2h, r0, n, tid, a2dh, a2den_stride);
     if (!DQ && tid < 32) creg = (r0 + tid < n && r0 + tid >= alo) ? ch[r0 + tid] : 0.f;
   };
-  auto tiles_store = [&](int buf) {
-    t1.store(Sl + buf * SLABF, LD, a1s, tid);
-    t2.store(Sl + buf * SLABF + 32 * LD, LD, 1.0f, tid);
-    if (!DQ && tid < 32) Cl[buf][tid] = creg;
+  auto tiles_store = [&](int kk) __attribute__((always_inline)) {
+    float* tb = (kk & 1) ? Sb3 : Sb2;
+    t1.store(tb, LD, a1s, tid);
+    t2.store(tb + 32 * LD, LD, 1.0f, tid);
+    if (!DQ && tid < 32) Cl[kk & 1][tid] = creg;
   };
 
-  // out[ab][r]: token w*32 + trow(r,hh), channel ab*32 + i
-  f16v out[AB];
+  // Everything the block needs first is requested before anything is waited for: the first two
+  // slabs, the first streamed tile, the own rows, c of the own token.
+  if (n_state > 0) {
+    slab_dma(0, Sb0);
+    slab_dma(1, Sb1);
+  }
+  if (n_tile > 0) tiles_load(0);
+  const float c_ld = DQ ? ch[tokc] : 0.f;
+  // the lane's own token: x of its own channels (xo[4g + e] = channel 8g + 4hh + e) and of the four
+  // channels just above each own group (xp[4g + e] = channel 8g + 4hh + 4 + e, round the ring),
+  // scaled; its half of y (channels hh H2 ..), the B operand of the state contraction and of g.v
+  float xo[H2], xp[H2], Yr[H2];
+  {
+    const float4* xr = reinterpret_cast<const float4*>(Xh.row(tokc));
+    const float4* yr = reinterpret_cast<const float4*>(Yh.row(tokc) + hh * H2);
+    float4 xa[NG], xb[NG], ya[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      xa[g] = xr[2 * g + hh];
+      xb[g] = xr[(2 * g + hh + 1) % (2 * NG)];
+      ya[g] = yr[g];
+    }
+    const float ysc = live ? (ydh ? 1.0f / ydh[(unsigned)tokc * (unsigned)yden_stride] : 1.0f) : 0.f;
+    const float xsc = live ? xs : 0.f;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      xo[4 * g] = xa[g].x * xsc; xo[4 * g + 1] = xa[g].y * xsc; xo[4 * g + 2] = xa[g].z * xsc; xo[4 * g + 3] = xa[g].w * xsc;
+      xp[4 * g] = xb[g].x * xsc; xp[4 * g + 1] = xb[g].y * xsc; xp[4 * g + 2] = xb[g].z * xsc; xp[4 * g + 3] = xb[g].w * xsc;
+      Yr[4 * g] = ya[g].x * ysc; Yr[4 * g + 1] = ya[g].y * ysc; Yr[4 * g + 2] = ya[g].z * ysc; Yr[4 * g + 3] = ya[g].w * ysc;
+    }
+  }
+  const float c_own = (DQ && live) ? c_ld : 0.f;
+  const float yx = hh == 0 ? (DQ ? -c_own : (live ? -1.0f : 0.f)) : 0.f;
+
+  // out[ab][r]: channel 32 ab + 8 (r / 4) + 4 hh + r % 4 of the lane's token, i.e. own index
+  // 16 ab + r; outx[.]: what the lane collects for the channel four above that one
+  f16v out[AB], outx[AB];
 #pragma unroll
   for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) out[ab][r] = 0.f;
+    for (int r = 0; r < 16; ++r) out[ab][r] = outx[ab][r] = 0.f;
 
-  // Everything the block needs first is requested before anything is waited for (one memory
-  // latency instead of three in a row): the first slab, the first streamed tile, c of the own
-  // token, the own rows.
-  if (n_tile > 0) tiles_load(0);
-  if (n_state > 0) slab_load(0);
-  const float c_ld = DQ ? ch[max(tok < n ? tok : n - 1, xlo)] : 0.f;
-  {
-    RowTile<D, T, 128> t, u;
-    t.load(Xh, tok0, n, tid);
-    u.load(Yh, tok0, n, tid, ydh, yden_stride);
-    t.store(Xl, LD, xs, tid);
-    u.store(Sl, LD, 1.0f, tid);
-  }
-  __syncthreads();
-  // own token of this lane = row xrow: its half of y (A operand of the state contraction, B of g.v)
-  float Yr[H2];
-#pragma unroll
-  for (int t = 0; t < H2; t += 4) {
-    const float4 y4 = *reinterpret_cast<const float4*>(Sl + xrow * LD + hh * H2 + t);
-    Yr[t] = y4.x; Yr[t + 1] = y4.y; Yr[t + 2] = y4.z; Yr[t + 3] = y4.w;
-  }
-  const float c_own = (DQ && tok < n && tok >= xlo) ? c_ld : 0.f;
-  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f;
-  __syncthreads();
-  if (n_state > 0) {
-    slab_store(0);
-  } else if (n_tile > 0) {
-    tiles_store(0);
-  }
-  __syncthreads();
-
-  // B operands of one 32-row tile of a slab: the row's D value columns and its extra column
-  struct BOps {
+  // A operands of one 32-row tile of a slab: the row's D value columns (this lane half's part) and
+  // its extra column
+  struct AOps {
     float4 b4[H2 / 4];
     float bx;
   };
-  auto fetch = [&](const float* sl, int ab, BOps& o) {
+  auto fetch = [&](const float* sl, int ab, AOps& o) __attribute__((always_inline)) {
     const float* ar = sl + (ab * 32 + i) * LD;
 #pragma unroll
     for (int k = 0; k < H2 / 4; ++k) o.b4[k] = *reinterpret_cast<const float4*>(ar + hh * H2 + 4 * k);
     o.bx = ar[D];
   };
-  auto chain = [&](const BOps& o) {
+  auto chain = [&](const AOps& o) __attribute__((always_inline)) {
     f16v t;
 #pragma unroll
     for (int r = 0; r < 16; ++r) t[r] = 0.f;
 #pragma unroll
     for (int k = 0; k < H2 / 4; ++k) {
-      t = FM_MFMA(Yr[4 * k], o.b4[k].x, t);
-      t = FM_MFMA(Yr[4 * k + 1], o.b4[k].y, t);
-      t = FM_MFMA(Yr[4 * k + 2], o.b4[k].z, t);
-      t = FM_MFMA(Yr[4 * k + 3], o.b4[k].w, t);
+      t = FM_MFMA(o.b4[k].x, Yr[4 * k], t);
+      t = FM_MFMA(o.b4[k].y, Yr[4 * k + 1], t);
+      t = FM_MFMA(o.b4[k].z, Yr[4 * k + 2], t);
+      t = FM_MFMA(o.b4[k].w, Yr[4 * k + 3], t);
     }
-    return FM_MFMA(yx, o.bx, t);
+    return FM_MFMA(o.bx, yx, t);
   };
-  // x rows of the 16 tokens this lane holds results for: row w*32 + trow(r,hh), r = 4j+e
-  const float* xtok = Xl + (w * 32 + 4 * hh) * LD;
-  auto xat = [&](int r, int col) { return xtok[((r >> 2) * 8 + (r & 3)) * LD + col]; };
-  // x of the lane's own channels for the 16 token rows of its accumulator registers (the factor
-  // of the mirrored credit and of the normalisation partial), read once
-  float xown[AB][16];
+  // both credits of tile ab of shift S (compile-time; S == NS: the order-1 slab).  With s = 8 sg + tau
+  // and u = r % 4 + tau: u <= 3 and u >= 8 keep the partner in the lane's own half (group + sg, or
+  // + sg + 1), 4 <= u <= 7 puts it four above own index 4 (group + sg) + u - 4.
+  auto credit = [&](const f16v& t, auto stag, auto abtag) __attribute__((always_inline)) {
+    constexpr int S = decltype(stag)::value, ABI = decltype(abtag)::value;
 #pragma unroll
-  for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) xown[ab][r] = xat(r, ab * 32 + i);
-
-  for (int st = 0; st < n_state; ++st) {
-    slab_load(st + 1 < n_state ? st + 1 : st);
-    const float* sl = Sl + (st & 1) * SLABF;
-    BOps ops[AB];
-#pragma unroll
-    for (int ab = 0; ab < AB; ++ab) fetch(sl, ab, ops[ab]);
-    f16v tt[AB];
-#pragma unroll
-    for (int ab = 0; ab < AB; ++ab) tt[ab] = chain(ops[ab]);
-    if (p2 && st < NS) {
-      const int s = st;
-#pragma unroll
-      for (int ab = 0; ab < AB; ++ab) {
-        const int rc = (ab * 32 + i + s) & (D - 1);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) out[ab][r] += tt[ab][r] * xat(r, rc);
+    for (int r = 0; r < 16; ++r) {
+      const int e = r & 3, grp = 4 * ABI + (r >> 2), own = 16 * ABI + r;
+      const float v = t[r];
+      if constexpr (S == NS) {           // the order-1 slab (its coefficient is applied here)
+        out[ABI][r] += a1 * v;
+      } else if constexpr (S == 0) {     // the diagonal: one member
+        out[ABI][r] += v * xo[own];
+      } else {
+        constexpr int TAU = S % 8, SG = S / 8;
+        const int u = e + TAU;
+        const int g2 = (grp + SG + (u >= 8 ? 1 : 0)) % NG;
+        const int idx = 4 * g2 + (u & 3);
+        if (u <= 3 || u >= 8) {
+          out[ABI][r] += v * xo[idx];
+          if constexpr (S != H2) out[idx >> 4][idx & 15] += v * xo[own];   // (s = D/2 lists every pair from both sides)
+        } else {
+          out[ABI][r] += v * xp[idx];
+          outx[idx >> 4][idx & 15] += v * xo[own];
+        }
       }
-      if (s > 0 && s < H2) {
-        // credit the other member of each pair: channel (a+s)%D gets T[a]*x[a]
-#pragma unroll
-        for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) tt[ab][r] *= xown[ab][r];
-        const bool keep = i < 32 - s;                    // source lanes that stay in their block
-        const int src = (((i - s) & 31) + 32 * hh) << 2;  // byte index of the source lane
-#pragma unroll
-        for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            // lanes i >= s of block ab take U[ab][i-s]; lanes i < s take U[ab-1][i-s+32]
-            const float v = keep ? tt[ab][r] : tt[(ab + 1) % AB][r];
-            out[ab][r] += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src, __builtin_bit_cast(int, v)));
-          }
-      }
-    } else {
-#pragma unroll
-      for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) out[ab][r] += tt[ab][r];
     }
-    if (st + 1 < n_state) slab_store(st + 1);
-    else if (n_tile > 0) tiles_store((st + 1) & 1);
+  };
+
+  // The credits are pure arithmetic, which instruction selection may order freely between the
+  // matrix instructions' results and the end of the kernel (it was seen to postpone them all, keeping
+  // every tile in scratch memory): an empty volatile statement that takes the accumulators in and out
+  // keeps each unit's credits in that unit.
+  auto pin_accumulators = [&]() __attribute__((always_inline)) {
+    if constexpr (AB == 2) asm volatile("" : "+v"(out[0]), "+v"(out[1]), "+v"(outx[0]), "+v"(outx[1]));
+    else asm volatile("" : "+v"(out[0]), "+v"(outx[0]));
+  };
+
+  if (n_state > 0) {
+    FM_WAIT_VM(0);
     __syncthreads();
   }
+  if (n_state > 1) {
+    // p = 2.  Tile units u = slab * AB + ab over slabs 0 .. NS (slab NS is the order-1 slab).  Slabs
+    // 2k, 2k+1 sit in buffers (Sb0, Sb1) for even k and (Sb2, Sb3) for odd k.  Per unit: read the
+    // operands of the next unit, run this unit's matrix instructions, form the credits of the unit
+    // before (whose results are complete by now).
+    static_assert(NS % 2 == 1 && ((NS + 1) / 2) % 2 == 1, "whole steps of two slabs, the last one in Sb0 and Sb1");
+    constexpr int NU = (NS + 1) * AB;
+    AOps bc;
+    f16v tp, tn;
+    fetch(Sb0, 0, bc);
+    static_for<(NS + 1) / 2>([&](auto ktag) __attribute__((always_inline)) {
+      constexpr int K = decltype(ktag)::value;
+      float* cur0 = (K & 1) ? Sb2 : Sb0;
+      float* cur1 = (K & 1) ? Sb3 : Sb1;
+      float* nxt0 = (K & 1) ? Sb0 : Sb2;
+      float* nxt1 = (K & 1) ? Sb1 : Sb3;
+      __builtin_amdgcn_sched_barrier(0);
+      // (every wave is past the buffers of the step before: it has passed the barrier)
+      slab_dma(2 * K + 2, nxt0);
+      slab_dma(2 * K + 3, nxt1);
+      static_for<2 * AB>([&](auto vtag) __attribute__((always_inline)) {
+        constexpr int V = decltype(vtag)::value, U = 2 * K * AB + V;
+        tn = chain(bc);
+        __builtin_amdgcn_sched_barrier(0);
+        // the operands of the next unit of this step go into the registers the matrix instructions
+        // have just read (the first unit of the next step is read after the barrier); they travel
+        // while the credits of the unit before are formed
+        if constexpr (V + 1 < 2 * AB) fetch(((V + 1) / AB) ? cur1 : cur0, (V + 1) % AB, bc);
+        if constexpr (U > 0) {
+          constexpr int PS = (U - 1) / AB, PAB = (U - 1) % AB;
+          if constexpr (PS == NS && PAB == 0) {
+            // order 2 is complete: f'(s) contributes 2 a2
+#pragma unroll
+            for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                out[ab][r] *= 2.0f * a2;
+                outx[ab][r] *= 2.0f * a2;
+              }
+          }
+          credit(tp, std::integral_constant<int, PS>{}, std::integral_constant<int, PAB>{});
+          pin_accumulators();
+        }
+        tp = tn;
+        __builtin_amdgcn_sched_barrier(0);   // (keeps the units apart: register pressure)
+      });
+      if constexpr (2 * K + 2 <= NS) {
+        FM_WAIT_VM(0);
+        __builtin_amdgcn_s_barrier();
+        fetch(nxt0, 0, bc);
+      } else {
+        // the last step: the first streamed tile can be staged (Sb2 was last read a step ago)
+        if (n_tile > 0) tiles_store(0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if constexpr (AB == 1) {   // the order-1 slab is a single unit: order 2 ends with the unit before
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        out[0][r] *= 2.0f * a2;
+        outx[0][r] *= 2.0f * a2;
+      }
+    }
+    credit(tp, std::integral_constant<int, (NU - 1) / AB>{}, std::integral_constant<int, (NU - 1) % AB>{});
+    // hand over what was collected for the channels four above: the lane of half 1 holds those of
+    // the same own index, the lane of half 0 those of the own index four higher (round the ring)
+#pragma unroll
+    for (int ab = 0; ab < AB; ++ab)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int idx = 16 * ab + r, below = (idx + H2 - 4) % H2;
+        out[ab][r] += swap_halves(outx[below >> 4][below & 15], outx[ab][r], hh);
+      }
+  } else {
+    if (n_state == 1) {
+      // p = 1: the order-1 slab is the only one
+      static_for<AB>([&](auto abtag) __attribute__((always_inline)) {
+        AOps b1;
+        fetch(Sb0, decltype(abtag)::value, b1);
+        const f16v t = chain(b1);
+        credit(t, std::integral_constant<int, NS>{}, abtag);
+      });
+    }
+    if (n_tile > 0) tiles_store(0);
+  }
+  if (n_tile > 0) __syncthreads();   // the first streamed tile is staged
 
   if (n_tile > 0) {
-    float Xr[H2];
-#pragma unroll
-    for (int t = 0; t < H2; t += 4) {
-      const float4 x4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + hh * H2 + t);
-      Xr[t] = x4.x; Xr[t + 1] = x4.y; Xr[t + 2] = x4.z; Xr[t + 3] = x4.w;
-    }
     const int mine = (tok0 >> 5) + w;
     const float twoa2 = 2.0f * a2;
     for (int kk = 0; kk < n_tile; ++kk) {
-      const int buf = (n_state + kk) & 1;
       tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
       const int tl = tile0 + kk;
       if (DQ ? tl <= mine : tl >= mine) {
-        const float* l1 = Sl + buf * SLABF;
+        const float* l1 = (kk & 1) ? Sb3 : Sb2;
         const float* l2 = l1 + 32 * LD;
-        // rows = streamed tokens trow(r,hh), lanes = own tokens
+        // scores and g.v: rows = streamed tokens trow(r,hh), lanes = own tokens (the scores pair the
+        // channels in the order of xo)
         f16v sc, gv;
 #pragma unroll
         for (int r = 0; r < 16; ++r) sc[r] = gv[r] = 0.f;
 #pragma unroll
-        for (int t = 0; t < H2; t += 4) {
-          const float4 p4 = *reinterpret_cast<const float4*>(l1 + i * LD + hh * H2 + t);
-          const float4 v4 = *reinterpret_cast<const float4*>(l2 + i * LD + hh * H2 + t);
-          sc = FM_MFMA(p4.x, Xr[t], sc);
-          gv = FM_MFMA(v4.x, Yr[t], gv);
-          sc = FM_MFMA(p4.y, Xr[t + 1], sc);
-          gv = FM_MFMA(v4.y, Yr[t + 1], gv);
-          sc = FM_MFMA(p4.z, Xr[t + 2], sc);
-          gv = FM_MFMA(v4.z, Yr[t + 2], gv);
-          sc = FM_MFMA(p4.w, Xr[t + 3], sc);
-          gv = FM_MFMA(v4.w, Yr[t + 3], gv);
+        for (int g = 0; g < NG; ++g) {
+          const float4 p4 = *reinterpret_cast<const float4*>(l1 + i * LD + 8 * g + 4 * hh);
+          const float4 v4 = *reinterpret_cast<const float4*>(l2 + i * LD + hh * H2 + 4 * g);
+          sc = FM_MFMA(p4.x, xo[4 * g], sc);
+          gv = FM_MFMA(v4.x, Yr[4 * g], gv);
+          sc = FM_MFMA(p4.y, xo[4 * g + 1], sc);
+          gv = FM_MFMA(v4.y, Yr[4 * g + 1], gv);
+          sc = FM_MFMA(p4.z, xo[4 * g + 2], sc);
+          gv = FM_MFMA(v4.z, Yr[4 * g + 2], gv);
+          sc = FM_MFMA(p4.w, xo[4 * g + 3], sc);
+          gv = FM_MFMA(v4.w, Yr[4 * g + 3], gv);
         }
         float pa[16][AB];
 #pragma unroll
@@ -266,33 +371,36 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
         const bool diag = tl == mine;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float cc = DQ ? c_own : Cl[buf][trow(r, hh)];
+          const float cc = DQ ? c_own : Cl[kk & 1][trow(r, hh)];
           float wv = (a1 + twoa2 * sc[r]) * (gv[r] - cc);
           if (diag && (DQ ? trow(r, hh) > i : trow(r, hh) < i)) wv = 0.f;
           sc[r] = wv;
         }
-        // out (own x channels) += W (own x streamed) . A1 (streamed x channels)
+        // out (channels x own) += A1^T (channels x streamed) . W (streamed x own)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
 #pragma unroll
-          for (int ab = 0; ab < AB; ++ab) out[ab] = FM_MFMA(sc[r], pa[r][ab], out[ab]);
+          for (int ab = 0; ab < AB; ++ab) out[ab] = FM_MFMA(pa[r][ab], sc[r], out[ab]);
       }
-      if (kk + 1 < n_tile) tiles_store(buf ^ 1);
+      if (kk + 1 < n_tile) tiles_store(kk + 1);
       __syncthreads();
     }
   }
 
-  // rows of out are tokens, lanes are channels: store directly, scaled by the normaliser
+  // the lane holds groups of four consecutive channels of its token: 16-byte stores, scaled by the
+  // normaliser
   float rs = 0.f;
-  const HeadRows<T> Oh = OUT.head(head);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int tk = tok0 + w * 32 + trow(r, hh);
+  for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
-    for (int ab = 0; ab < AB; ++ab) {
-      const float g = out[ab][r];
-      rs += g * xown[ab][r];
-      if (tk < n && tk >= xlo) Oh.base[(unsigned)tk * Oh.pitch + (unsigned)(ab * 32 + i)] = from_f32<T>(g * xs);
+    for (int r = 0; r < 16; ++r) rs += out[ab][r] * xo[16 * ab + r];
+  if (live) {
+    T* orow = OUT.head(head).row(tok) + 4 * hh;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      const f16v& o = out[g >> 2];
+      const int r0 = 4 * (g & 3);
+      *reinterpret_cast<float4*>(orow + 8 * g) = make_float4(o[r0] * xs, o[r0 + 1] * xs, o[r0 + 2] * xs, o[r0 + 3] * xs);
     }
   }
   rs = block_sum_256(rs, red, tid);
