@@ -69,7 +69,17 @@ def algorithmic_flops(d: int, p: int) -> dict:
     }
 
 
-def executed_mfma_flops(cfg: dict, bh: int, chunk: int = 384) -> dict:
+def chunk_tokens(cfg: dict) -> int:
+    """Tokens between the causal state snapshots of the chunked kernels (the library's choice: p = 2
+    bf16 384, fp32 d = 64 256, fp32 d = 32 128; p = 1 128)."""
+    if cfg["p"] != 2:
+        return 128
+    if cfg["dtype"] == "bf16":
+        return 384
+    return 256 if cfg["D"] == 64 else 128
+
+
+def executed_mfma_flops(cfg: dict, bh: int, chunk: int = 0) -> dict:
     """Flops of the matrix instructions each kernel class of the chunked p = 2 path issues per head set and
     pass (2*32*32*K per instruction: 4096 for v_mfma_f32_32x32x2f32, 32768 for v_mfma_f32_32x32x16_bf16),
     counted the way the kernels launch them: every wave of every block, dummy row-tile slots and ragged
@@ -78,6 +88,7 @@ def executed_mfma_flops(cfg: dict, bh: int, chunk: int = 384) -> dict:
     bwd_dq, bwd_dk, bwd_dv."""
     d, n, masked, bf = cfg["D"], cfg["N"], cfg["mask"], cfg["dtype"] == "bf16"
     assert cfg["p"] == 2
+    chunk = chunk or chunk_tokens(cfg)
     h2, ns, cb = d // 2, d // 2 + 1, d // 32
     per = 32768 if bf else 4096                 # flop per matrix instruction
     ksteps = (lambda k: k // 16) if bf else (lambda k: k // 2)   # instructions for a contraction length k

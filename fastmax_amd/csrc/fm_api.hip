@@ -71,10 +71,16 @@ struct ScopedKernel {
 };
 
 // Tokens between causal state snapshots (a multiple of the 128-token block of the consumers).
-// Longer chunks mean fewer snapshots to write and read but more intra-chunk score tiles; measured
-// at the headline shapes, 384 beats 256 and 512 for p = 2 (fp32 and bf16 alike).
+// Longer chunks mean fewer snapshots to write and read but more intra-chunk score tiles (at 384 tokens
+// they are more than a quarter of a consumer's matrix instructions).  Measured at the headline shapes,
+// p = 2: fp32 d = 64 is fastest at 256 (384: +2.4 %, 128: +0.8 %), fp32 d = 32 at 128, bf16 d = 64 at 384
+// (256: +2 %: its build kernel pays more per snapshot).
 constexpr int kChunkP1 = 128;  // p = 1: a state is only d+1 rows, a snapshot per block is cheapest
-constexpr int kChunk = 384;
+inline int chunk_for(int d, int p2, int dtype) {
+  if (!p2) return kChunkP1;
+  if (dtype == FASTMAX_BF16) return 384;
+  return d == 64 ? 256 : 128;
+}
 constexpr size_t kWorkspaceBudget = 16ull << 30;   // what fastmax_workspace_bytes aims for
 
 struct Plan {
@@ -148,7 +154,7 @@ Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true) {
   pl.gsplit = splits(pl.rtw);
   // p = 1: a state is only (d+1) rows, so a snapshot per 128-token block is cheaper than a longer
   // intra-chunk part
-  pl.chunk = pl.p2 ? kChunk : kChunkP1;
+  pl.chunk = chunk_for(pl.d, pl.p2, ds->dtype);
   if (pl.masked) {
     pl.nslots = (pl.n + pl.chunk - 1) / pl.chunk;
     pl.nparts = 1;

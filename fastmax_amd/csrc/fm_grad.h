@@ -28,8 +28,8 @@
 // second accumulator bank (outx) that the two lanes of a token exchange once at the end.
 // Slabs go global -> LDS directly (no staging registers), two slabs ahead into four buffers, one
 // barrier per two slabs; the coefficients multiply the accumulated sums (2 a2 after the order-2
-// slabs, a1 on the order-1 tile).  The matrix instructions of one tile run while the credits of
-// the tile before are formed and the operands of the next are read.
+// slabs, a1 on the order-1 tile).  Two tiles are contracted at a time, their matrix instructions
+// taking turns (back-to-back instructions on one accumulator wait for each other).
 // Causal intra-chunk part: for every streamed 32-token tile the transposed score and g.v tiles
 // are formed (streamed x own), W is built in registers and fed back as the B operand of
 // out (channels x own) += A1^T (channels x streamed) . W (streamed x own).
@@ -182,30 +182,40 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 #pragma unroll
     for (int r = 0; r < 16; ++r) out[ab][r] = outx[ab][r] = 0.f;
 
-  // A operands of one 32-row tile of a slab: the row's D value columns (this lane half's part) and
-  // its extra column
-  struct AOps {
-    float4 b4[H2 / 4];
-    float bx;
-  };
-  auto fetch = [&](const float* sl, int ab, AOps& o) __attribute__((always_inline)) {
-    const float* ar = sl + (ab * 32 + i) * LD;
+  // Two 32-row tiles at a time (tile ab0 of slab sl0 and tile ab1 of slab sl1), their matrix
+  // instructions interleaved: consecutive instructions on the same accumulator wait for each other's
+  // result, two accumulators that take turns do not.  A operands: a row's D value columns (this lane
+  // half's part) in 128-bit LDS reads, one read ahead of their use, and its extra column.
+  auto tile_pair = [&](const float* sl0, int ab0, const float* sl1, int ab1, f16v& t0, f16v& t1) __attribute__((always_inline)) {
+    constexpr int NK = H2 / 4;
+    const float* r0 = sl0 + (ab0 * 32 + i) * LD;
+    const float* r1 = sl1 + (ab1 * 32 + i) * LD;
 #pragma unroll
-    for (int k = 0; k < H2 / 4; ++k) o.b4[k] = *reinterpret_cast<const float4*>(ar + hh * H2 + 4 * k);
-    o.bx = ar[D];
-  };
-  auto chain = [&](const AOps& o) __attribute__((always_inline)) {
-    f16v t;
+    for (int r = 0; r < 16; ++r) t0[r] = t1[r] = 0.f;
+    float4 c0 = *reinterpret_cast<const float4*>(r0 + hh * H2), c1 = *reinterpret_cast<const float4*>(r1 + hh * H2);
+    const float x0 = r0[D], x1 = r1[D];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) t[r] = 0.f;
-#pragma unroll
-    for (int k = 0; k < H2 / 4; ++k) {
-      t = FM_MFMA(o.b4[k].x, Yr[4 * k], t);
-      t = FM_MFMA(o.b4[k].y, Yr[4 * k + 1], t);
-      t = FM_MFMA(o.b4[k].z, Yr[4 * k + 2], t);
-      t = FM_MFMA(o.b4[k].w, Yr[4 * k + 3], t);
+    for (int k = 0; k < NK; ++k) {
+      float4 n0 = c0, n1 = c1;
+      if (k + 1 < NK) {
+        n0 = *reinterpret_cast<const float4*>(r0 + hh * H2 + 4 * (k + 1));
+        n1 = *reinterpret_cast<const float4*>(r1 + hh * H2 + 4 * (k + 1));
+      }
+      t0 = FM_MFMA(c0.x, Yr[4 * k], t0);
+      t1 = FM_MFMA(c1.x, Yr[4 * k], t1);
+      t0 = FM_MFMA(c0.y, Yr[4 * k + 1], t0);
+      t1 = FM_MFMA(c1.y, Yr[4 * k + 1], t1);
+      t0 = FM_MFMA(c0.z, Yr[4 * k + 2], t0);
+      t1 = FM_MFMA(c1.z, Yr[4 * k + 2], t1);
+      t0 = FM_MFMA(c0.w, Yr[4 * k + 3], t0);
+      t1 = FM_MFMA(c1.w, Yr[4 * k + 3], t1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // the two reads ahead ...
+      __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);   // ... then this step's eight matrix instructions
+      c0 = n0;
+      c1 = n1;
     }
-    return FM_MFMA(o.bx, yx, t);
+    t0 = FM_MFMA(x0, yx, t0);
+    t1 = FM_MFMA(x1, yx, t1);
   };
   // both credits of tile ab of shift S (compile-time; S == NS: the order-1 slab).  With s = 8 sg + tau
   // and u = r % 4 + tau: u <= 3 and u >= 8 keep the partner in the lane's own half (group + sg, or
@@ -250,15 +260,10 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
     __syncthreads();
   }
   if (n_state > 1) {
-    // p = 2.  Tile units u = slab * AB + ab over slabs 0 .. NS (slab NS is the order-1 slab).  Slabs
-    // 2k, 2k+1 sit in buffers (Sb0, Sb1) for even k and (Sb2, Sb3) for odd k.  Per unit: read the
-    // operands of the next unit, run this unit's matrix instructions, form the credits of the unit
-    // before (whose results are complete by now).
+    // p = 2.  Slabs 0 .. NS (slab NS is the order-1 slab); slabs 2k, 2k+1 sit in buffers (Sb0, Sb1) for
+    // even k and (Sb2, Sb3) for odd k.
     static_assert(NS % 2 == 1 && ((NS + 1) / 2) % 2 == 1, "whole steps of two slabs, the last one in Sb0 and Sb1");
-    constexpr int NU = (NS + 1) * AB;
-    AOps bc;
-    f16v tp, tn;
-    fetch(Sb0, 0, bc);
+    f16v t0, t1;
     static_for<(NS + 1) / 2>([&](auto ktag) __attribute__((always_inline)) {
       constexpr int K = decltype(ktag)::value;
       float* cur0 = (K & 1) ? Sb2 : Sb0;
@@ -269,17 +274,15 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
       // (every wave is past the buffers of the step before: it has passed the barrier)
       slab_dma(2 * K + 2, nxt0);
       slab_dma(2 * K + 3, nxt1);
-      static_for<2 * AB>([&](auto vtag) __attribute__((always_inline)) {
-        constexpr int V = decltype(vtag)::value, U = 2 * K * AB + V;
-        tn = chain(bc);
+      // the 2 AB tile units of the step, two at a time: units v and v + 1 (unit v = tile v % AB of
+      // slab 2K + v / AB)
+      static_for<AB>([&](auto vtag) __attribute__((always_inline)) {
+        constexpr int V0 = 2 * decltype(vtag)::value, V1 = V0 + 1;
+        constexpr int S0 = 2 * K + V0 / AB, S1 = 2 * K + V1 / AB;
+        tile_pair((V0 / AB) ? cur1 : cur0, V0 % AB, (V1 / AB) ? cur1 : cur0, V1 % AB, t0, t1);
         __builtin_amdgcn_sched_barrier(0);
-        // the operands of the next unit of this step go into the registers the matrix instructions
-        // have just read (the first unit of the next step is read after the barrier); they travel
-        // while the credits of the unit before are formed
-        if constexpr (V + 1 < 2 * AB) fetch(((V + 1) / AB) ? cur1 : cur0, (V + 1) % AB, bc);
-        if constexpr (U > 0) {
-          constexpr int PS = (U - 1) / AB, PAB = (U - 1) % AB;
-          if constexpr (PS == NS && PAB == 0) {
+        auto scale_if_order2_done = [&](auto stag, auto abtag) __attribute__((always_inline)) {
+          if constexpr (decltype(stag)::value == NS && decltype(abtag)::value == 0) {
             // order 2 is complete: f'(s) contributes 2 a2
 #pragma unroll
             for (int ab = 0; ab < AB; ++ab)
@@ -289,30 +292,23 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
                 outx[ab][r] *= 2.0f * a2;
               }
           }
-          credit(tp, std::integral_constant<int, PS>{}, std::integral_constant<int, PAB>{});
-          pin_accumulators();
-        }
-        tp = tn;
+        };
+        scale_if_order2_done(std::integral_constant<int, S0>{}, std::integral_constant<int, V0 % AB>{});
+        credit(t0, std::integral_constant<int, S0>{}, std::integral_constant<int, V0 % AB>{});
+        scale_if_order2_done(std::integral_constant<int, S1>{}, std::integral_constant<int, V1 % AB>{});
+        credit(t1, std::integral_constant<int, S1>{}, std::integral_constant<int, V1 % AB>{});
+        pin_accumulators();
         __builtin_amdgcn_sched_barrier(0);   // (keeps the units apart: register pressure)
       });
       if constexpr (2 * K + 2 <= NS) {
         FM_WAIT_VM(0);
         __builtin_amdgcn_s_barrier();
-        fetch(nxt0, 0, bc);
       } else {
         // the last step: the first streamed tile can be staged (Sb2 was last read a step ago)
         if (n_tile > 0) tiles_store(0);
       }
       __builtin_amdgcn_sched_barrier(0);
     });
-    if constexpr (AB == 1) {   // the order-1 slab is a single unit: order 2 ends with the unit before
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        out[0][r] *= 2.0f * a2;
-        outx[0][r] *= 2.0f * a2;
-      }
-    }
-    credit(tp, std::integral_constant<int, (NU - 1) / AB>{}, std::integral_constant<int, (NU - 1) % AB>{});
     // hand over what was collected for the channels four above: the lane of half 1 holds those of
     // the same own index, the lane of half 0 those of the own index four higher (round the ring)
 #pragma unroll
@@ -325,12 +321,10 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
   } else {
     if (n_state == 1) {
       // p = 1: the order-1 slab is the only one
-      static_for<AB>([&](auto abtag) __attribute__((always_inline)) {
-        AOps b1;
-        fetch(Sb0, decltype(abtag)::value, b1);
-        const f16v t = chain(b1);
-        credit(t, std::integral_constant<int, NS>{}, abtag);
-      });
+      f16v t0, t1;
+      tile_pair(Sb0, 0, Sb0, AB - 1, t0, t1);
+      credit(t0, std::integral_constant<int, NS>{}, std::integral_constant<int, 0>{});
+      if constexpr (AB == 2) credit(t1, std::integral_constant<int, NS>{}, std::integral_constant<int, 1>{});
     }
     if (n_tile > 0) tiles_store(0);
   }

@@ -72,10 +72,10 @@ def test_workspace_sizes(built):
             hi = built.fastmax_workspace_bytes(C.byref(ds), pas)
             assert 0 < lo <= hi
             assert hi <= (16 << 30) + lo
-    # causal d=64 p=2: one state is (33*64 + 64 + 1) rows of 68 floats, one per 384-token chunk
+    # causal d=64 p=2 fp32: one state is (33*64 + 64 + 1) rows of 68 floats, one per 256-token chunk
     ds = desc(bh=1, n=1000, mask=True)
     state = ((33 * 64 + 65) * 68 + 63) // 64 * 64 * 4
-    assert built.fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_FORWARD) == 512 + 3 * state
+    assert built.fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_FORWARD) == 512 + 4 * state
     assert built.fastmax_workspace_bytes(C.byref(ds), 9) == 0  # unknown pass
 
 

@@ -59,8 +59,8 @@ def test_golden_vectors(ops, name):
 @pytest.mark.parametrize("d", [32, 64])
 @pytest.mark.parametrize("mask", [False, True])
 @pytest.mark.parametrize("p", [1, 2])
-@pytest.mark.parametrize("n", [1, 31, 128, 257, 383, 384, 385, 700, 769])  # around the 128-token block and
-def test_shapes_fp32(ops, d, mask, p, n):                                  # the 384-token chunk
+@pytest.mark.parametrize("n", [1, 31, 128, 255, 256, 257, 383, 384, 385, 700, 769])  # around the 128-token block
+def test_shapes_fp32(ops, d, mask, p, n):                       # and the 128-, 256- and 384-token chunks
     run_case(ops, (3, n, d), seed=n + d, mask=mask, normalize=True, p=p)
 
 
