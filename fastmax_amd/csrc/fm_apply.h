@@ -487,10 +487,8 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     constexpr int WO = decltype(wo)::value;   // Wn[WO + t] is the partner of channel t for this shift
     constexpr int NB = FWD ? CB + 1 : CB;
     constexpr int NM = H2 / 8;  // MFMA steps per column tile
-    // feature group 2m + u of lane half hh is row group hh * H2/4 + 2m + u, stored at position
-    // PG::rgpos(.) = 2 (2m + u) + hh
-    const uint16_t* brow = sl + (hh * NCF + i) * 4;
-    const uint16_t* erow = sl + (hh * NCF + D) * 4;
+    const uint16_t* brow = sl + (hh * (H2 / 4) * NCF + i) * 4;
+    const uint16_t* erow = sl + (hh * (H2 / 4) * NCF + D) * 4;
     // (the two halves of an operand are read next to each other, so that they pair into one
     // two-address LDS read whose four destination registers are the operand)
     auto fetch = [&](int m, uint2 (&b)[2 * NB]) {
@@ -498,12 +496,12 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
       for (int cb = 0; cb < CB; ++cb) {
 #pragma unroll
         for (int u = 0; u < 2; ++u)
-          b[2 * cb + u] = *reinterpret_cast<const uint2*>(brow + (2 * (2 * m + u) * NCF + cb * 32) * 4);
+          b[2 * cb + u] = *reinterpret_cast<const uint2*>(brow + ((2 * m + u) * NCF + cb * 32) * 4);
       }
       if (FWD) {
 #pragma unroll
         for (int u = 0; u < 2; ++u)
-          b[2 * (NB - 1) + u] = *reinterpret_cast<const uint2*>(erow + 2 * (2 * m + u) * NCF * 4);
+          b[2 * (NB - 1) + u] = *reinterpret_cast<const uint2*>(erow + (2 * m + u) * NCF * 4);
       }
     };
     auto feat = [&](int g4) {

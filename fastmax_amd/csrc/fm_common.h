@@ -232,11 +232,7 @@ struct Geo {
 // i.e. 8-byte words of four consecutive rows, which is the B operand layout of the bf16 matrix
 // instruction for a contraction over features (apply kernels: plain 64-bit LDS reads); for a
 // contraction over columns (grad kernels) the same words are read through the transposing LDS
-// load (lds_read_tr16).  The D/4 row groups of a slab are stored interleaved, group g at position
-// rgpos(g) = 2 (g mod D/8) + g div D/8, i.e. a group of the first half of the channels is followed
-// by the same group of the second half: the grad kernels read one of each per 16 lanes, and next
-// to each other they fall in different LDS banks.  Consumers stage a slab with plain 16-byte
-// copies.  Columns D..D+3 hold
+// load (lds_read_tr16).  Consumers stage a slab with plain 16-byte copies.  Columns D..D+3 hold
 // the extra (denominator) column split into hi + lo bf16 parts as (hi, hi, lo, lo), because in the
 // grad kernels that term nearly cancels the value columns' sum.  The slabs are followed by the
 // order-0 row as D+1 floats.
@@ -245,7 +241,6 @@ struct PackedGeo {
   using G = Geo<D>;
   static constexpr int NCF = D + 4;
   static constexpr int FSL = (D / 4) * NCF * 4;  // bf16 elements of a slab (a multiple of 128)
-  __host__ __device__ static constexpr int rgpos(int g) { return 2 * (g % (D / 8)) + g / (D / 8); }
   __host__ __device__ static constexpr int nslab(int p2) { return (p2 ? G::NS : 0) + 1; }
   __host__ __device__ static constexpr int64_t z_off(int p2) { return ((int64_t)nslab(p2) * FSL * 2 + 255) / 256 * 256; }
   __host__ __device__ static constexpr int64_t bytes(int p2) { return z_off(p2) + (D + 1) * 4; }

@@ -373,24 +373,21 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
         const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
         {
           const float wgt = dbl ? 2.0f : 1.0f;
-          // accumulator registers 4j..4j+3 are the four rows of row group g = (arow / 4) + 2j + hh,
-          // stored at position rgpos(g) = 2 (2j mod Q) + 2 hh + (arow / 4) / Q + 2j / Q with Q = D / 8
-          // (arow / 4 is a multiple of Q and 2j mod Q + hh < Q): a lane part plus a compile-time part
-          constexpr int Q = D / 8;
-          uint16_t* fx = fsec + (unsigned)(slab * PG::FSL);
-          const unsigned lo = (unsigned)(((2 * hh + (arow >> 2) / Q) * PG::NCF + cbase * 32 + i) * 4);
+          // accumulator registers 4j..4j+3 are the four rows of row group (arow / 4) + 2j + hh
+          uint16_t* fx = fsec + (unsigned)(slab * PG::FSL + (arow >> 2) * PG::NCF * 4);
+          const unsigned lo = (unsigned)((hh * PG::NCF + cbase * 32 + i) * 4);
 #pragma unroll
           for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
               const f16v& a = acc[x][cb];
-              *reinterpret_cast<uint2*>(fx + lo + (unsigned)(((2 * ((2 * j) % Q) + (2 * j) / Q) * PG::NCF + cb * 32) * 4)) =
+              *reinterpret_cast<uint2*>(fx + lo + (unsigned)((2 * j * PG::NCF + cb * 32) * 4)) =
                   make_uint2(pack_bf2(a[4 * j] * wgt, a[4 * j + 1] * wgt), pack_bf2(a[4 * j + 2] * wgt, a[4 * j + 3] * wgt));
             }
           if (hh == 0 && cbase == 0) {   // the extra column, split into hi + lo parts: columns D..D+3 = (hi, hi, lo, lo)
             const float ew = ds * wgt, ehi = bf_lo(pack_bf2(ew, 0.f));
             const uint16_t h16 = (uint16_t)pack_bf2(ehi, 0.f), l16 = (uint16_t)pack_bf2(ew - ehi, 0.f);
-            uint16_t* ex = fx + (unsigned)((PG::rgpos((arow >> 2) + (i >> 2)) * PG::NCF + D) * 4 + (i & 3));
+            uint16_t* ex = fx + (unsigned)(((i >> 2) * PG::NCF + D) * 4 + (i & 3));
             ex[0] = h16; ex[4] = h16; ex[8] = l16; ex[12] = l16;
           }
         }
@@ -559,7 +556,7 @@ __global__ __launch_bounds__(256) void state_pack_kernel(float* __restrict__ sta
     const int tg = idx / (D + 1), col = idx % (D + 1);
     const float* f = Sl + 4 * tg * LD + col;
     const float f0 = f[0] * wgt, f1 = f[LD] * wgt, f2 = f[2 * LD] * wgt, f3 = f[3 * LD] * wgt;
-    uint2* dst = reinterpret_cast<uint2*>(fsec + (PG::rgpos(tg) * PG::NCF + col) * 4);
+    uint2* dst = reinterpret_cast<uint2*>(fsec + (tg * PG::NCF + col) * 4);
     if (col < D) {
       *dst = make_uint2(pack_bf2(f0, f1), pack_bf2(f2, f3));
     } else {   // the extra column, split into hi + lo parts: columns D..D+3 = (hi, hi, lo, lo)

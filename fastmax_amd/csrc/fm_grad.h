@@ -10,6 +10,61 @@
 #include "fm_common.h"
 
 // ---------------------------------------------------------------------------------------
+// Shared by the fp32 and the bf16 kernel.  A result tile T of slab s has rows = channels and lanes
+// = own tokens: lane (i, hh) holds, for its token, channel 32 ab + 8 (r / 4) + 4 hh + r % 4 of tile ab
+// in accumulator register r, i.e. the lane halves own alternating groups of four channels, and
+// own index 16 ab + r counts a half's channels.  xo[own index] is x of that channel, xp[own index]
+// x of the channel four above it (round the ring), out / outx the sums owed to those channels.
+//
+// credit_tile: both credits of tile ABI of shift S (compile-time; S == NS: the order-1 slab, added
+// with coefficient a1).  With S = 8 sg + tau and u = r % 4 + tau: u <= 3 and u >= 8 keep the partner
+// in the lane's own half (group + sg, or + sg + 1), 4 <= u <= 7 puts it four above own index
+// 4 (group + sg) + u - 4 -- for both halves alike.  WEIGHTED: the rows carry their pair weights
+// (1 for shifts 0 and D/2, 2 otherwise), so those two tiles are doubled.
+// ---------------------------------------------------------------------------------------
+template <int D, int S, int ABI, bool WEIGHTED>
+__device__ __forceinline__ void credit_tile(const f16v& t, f16v (&out)[D / 32], f16v (&outx)[D / 32],
+                                            const float (&xo)[D / 2], const float (&xp)[D / 2], float a1) {
+  constexpr int H2 = D / 2, NS = D / 2 + 1, NG = D / 8;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int e = r & 3, grp = 4 * ABI + (r >> 2), own = 16 * ABI + r;
+    const float v = (WEIGHTED && (S == 0 || S == H2)) ? t[r] + t[r] : t[r];
+    if constexpr (S == NS) {           // the order-1 slab
+      out[ABI][r] += a1 * t[r];
+    } else if constexpr (S == 0) {     // the diagonal: one member
+      out[ABI][r] += v * xo[own];
+    } else {
+      constexpr int TAU = S % 8, SG = S / 8;
+      const int u = e + TAU;
+      const int g2 = (grp + SG + (u >= 8 ? 1 : 0)) % NG;
+      const int idx = 4 * g2 + (u & 3);
+      if (u <= 3 || u >= 8) {
+        out[ABI][r] += v * xo[idx];
+        if constexpr (S != H2) out[idx >> 4][idx & 15] += v * xo[own];   // (s = D/2 lists every pair from both sides)
+      } else {
+        out[ABI][r] += v * xp[idx];
+        outx[idx >> 4][idx & 15] += v * xo[own];
+      }
+    }
+  }
+}
+
+// out += what the token's other lane collected for this lane's channels: the lane of half 1 holds
+// those of the same own index, the lane of half 0 those of the own index four higher (round the ring).
+template <int D>
+__device__ __forceinline__ void exchange_halves(f16v (&out)[D / 32], const f16v (&outx)[D / 32], int hh) {
+  constexpr int H2 = D / 2;
+#pragma unroll
+  for (int ab = 0; ab < D / 32; ++ab)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int idx = 16 * ab + r, below = (idx + H2 - 4) % H2;
+      out[ab][r] += swap_halves(outx[below >> 4][below & 15], outx[ab][r], hh);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // One block = 128 own tokens of one head, one wave = 32 of them, one lane pair (i, hh = 0/1) per
 // token.  Per shift slab s of the state the kernel contracts 32 state rows at a time (A operand,
 // 128-bit LDS reads along the columns) with the token's extended value vector y_ext = [y, yx]
@@ -217,33 +272,8 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
     t0 = FM_MFMA(x0, yx, t0);
     t1 = FM_MFMA(x1, yx, t1);
   };
-  // both credits of tile ab of shift S (compile-time; S == NS: the order-1 slab).  With s = 8 sg + tau
-  // and u = r % 4 + tau: u <= 3 and u >= 8 keep the partner in the lane's own half (group + sg, or
-  // + sg + 1), 4 <= u <= 7 puts it four above own index 4 (group + sg) + u - 4.
   auto credit = [&](const f16v& t, auto stag, auto abtag) __attribute__((always_inline)) {
-    constexpr int S = decltype(stag)::value, ABI = decltype(abtag)::value;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int e = r & 3, grp = 4 * ABI + (r >> 2), own = 16 * ABI + r;
-      const float v = t[r];
-      if constexpr (S == NS) {           // the order-1 slab (its coefficient is applied here)
-        out[ABI][r] += a1 * v;
-      } else if constexpr (S == 0) {     // the diagonal: one member
-        out[ABI][r] += v * xo[own];
-      } else {
-        constexpr int TAU = S % 8, SG = S / 8;
-        const int u = e + TAU;
-        const int g2 = (grp + SG + (u >= 8 ? 1 : 0)) % NG;
-        const int idx = 4 * g2 + (u & 3);
-        if (u <= 3 || u >= 8) {
-          out[ABI][r] += v * xo[idx];
-          if constexpr (S != H2) out[idx >> 4][idx & 15] += v * xo[own];   // (s = D/2 lists every pair from both sides)
-        } else {
-          out[ABI][r] += v * xp[idx];
-          outx[idx >> 4][idx & 15] += v * xo[own];
-        }
-      }
-    }
+    credit_tile<D, decltype(stag)::value, decltype(abtag)::value, false>(t, out, outx, xo, xp, a1);
   };
 
   // The credits are pure arithmetic, which instruction selection may order freely between the
@@ -309,15 +339,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
       }
       __builtin_amdgcn_sched_barrier(0);
     });
-    // hand over what was collected for the channels four above: the lane of half 1 holds those of
-    // the same own index, the lane of half 0 those of the own index four higher (round the ring)
-#pragma unroll
-    for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int idx = 16 * ab + r, below = (idx + H2 - 4) % H2;
-        out[ab][r] += swap_halves(outx[below >> 4][below & 15], outx[ab][r], hh);
-      }
+    exchange_halves<D>(out, outx, hh);
   } else {
     if (n_state == 1) {
       // p = 1: the order-1 slab is the only one
@@ -402,26 +424,20 @@ __global__ __launch_bounds__(256, 2) void grad_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// bf16 variant of grad_kernel (bf16 inputs and outputs): every contraction runs on
-// v_mfma_f32_32x32x16_bf16 with fp32 accumulation, and the result tiles are TRANSPOSED with
-// respect to the fp32 kernel: rows = channels, lanes = own tokens.  A lane (token, half hh)
-// then holds, for its token, the H2 = D/2 channels [hh H2, (hh+1) H2) of a slab's tile T in
-// registers, next to the token's whole x row and the output accumulators, so both credits of a
-// pair are register FMAs with compile-time register numbers (the shift loop is fully unrolled):
-//     out[jj]     += T[jj] x[jj + s]        out[jj + s] += T[jj] x[jj]
-// Channels jj + s >= H2 belong to the lane of the other half: their x comes from the lane's copy
-// of the other half of the row, and what is owed to them is collected in a second accumulator
-// bank that the two halves exchange once at the end (one v_permlane32_swap per channel).
+// bf16 variant of grad_kernel (bf16 inputs and outputs): the same decomposition -- result tiles with
+// rows = channels and lanes = own tokens, the lane halves owning alternating groups of four
+// channels, both credits of a pair as register FMAs (credit_tile), one exchange between the two
+// lanes of a token at the end -- with every contraction on v_mfma_f32_32x32x16_bf16 and fp32
+// accumulation.
 //
 // The state arrives in the packed bf16 form (PackedGeo): a slab goes global -> LDS directly, two
 // slabs ahead, into four buffers, one barrier per two slabs.  The state rows are the A operand,
-// read through the transposing LDS load (four consecutive columns of a row per 64-bit piece);
-// the row -> lane assignment of a tile is chosen so that accumulator register r of tile ab is
-// channel hh H2 + 16 ab + r.  The token's extended value vector [y, yx] is the B operand, packed
-// once; a 32-row tile costs D/16 + 1 MFMAs.  The matrix instructions of one tile run while the
-// credits of the tile before are formed and the operands of the next are read.  The two slabs of
-// pair weight 1 are doubled, a2 multiplies the accumulated order-2 credits and a1 the order-1 tile.
-// Streamed tiles of the intra-chunk part have buffers of their own (staged as bf16 in both
+// read through the transposing LDS load (four consecutive columns of a row per 64-bit piece, 16
+// consecutive rows per 16 lanes).  The token's extended value vector [y, yx] is the B operand,
+// packed once; a 32-row tile costs D/16 + 1 MFMAs.  The matrix instructions of one tile run while
+// the credits of the tile before are formed and the operands of the next are read.  The two slabs
+// of pair weight 1 are doubled, a2 multiplies the accumulated order-2 credits and a1 the order-1
+// tile.  Streamed tiles of the intra-chunk part have buffers of their own (staged as bf16 in both
 // orientations: rows for the scores, transposed for the product with W).
 // ---------------------------------------------------------------------------------------
 template <int D, int MODE>
@@ -435,7 +451,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   using T = bf16_t;
   using PG = PackedGeo<D>;
   constexpr bool DQ = MODE == 0;
-  constexpr int AB = G::AB, H2 = G::H2, NS = G::NS;
+  constexpr int AB = G::AB, H2 = G::H2, NS = G::NS, NG = D / 8;
   constexpr int LB = D + 4;   // bf16 row pitch (elements)
   constexpr int TPB = 36;     // pitch of the transposed 32-token tile
   constexpr int NCF = PG::NCF, FSL = PG::FSL;
@@ -533,30 +549,39 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   }
   if (n_tile > 0) tiles_load(0);
   const float c_ld = DQ ? ch[tokc] : 0.f;
-  // the lane's own token: its whole x row (own half of the channels in xo, the other half in xp),
-  // scaled, and its half of y packed (B operand of the state contraction and of g.v)
+  // the lane's own token: x of its own channels (xo[4g + e] = channel 8g + 4hh + e) and of the four
+  // channels just above each own group (xp[4g + e] = channel 8g + 4hh + 4 + e, round the ring),
+  // scaled; its half of y (channels hh H2 ..) packed, the B operand of the state contraction and of g.v
   float xo[H2], xp[H2];
   uint2 Yp[H2 / 4];
   {
     const uint4* xr = reinterpret_cast<const uint4*>(Xh.row(tokc));
     const uint4* yr = reinterpret_cast<const uint4*>(Yh.row(tokc) + hh * H2);
-    uint4 xa[H2 / 8], xb[H2 / 8], ya[H2 / 8];
+    uint4 xa[NG], ya[H2 / 8];
 #pragma unroll
-    for (int u = 0; u < H2 / 8; ++u) {
-      xa[u] = xr[hh * (H2 / 8) + u];
-      xb[u] = xr[(1 - hh) * (H2 / 8) + u];
-      ya[u] = yr[u];
-    }
+    for (int g = 0; g < NG; ++g) xa[g] = xr[g];   // piece g = channels 8g .. 8g+7
+#pragma unroll
+    for (int u = 0; u < H2 / 8; ++u) ya[u] = yr[u];
     const float ydiv = ydh ? ydh[(unsigned)tokc * (unsigned)yden_stride] : 1.0f;
     const float xsc = live ? xs : 0.f;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      const uint4 nx = xa[(g + 1) % NG];
+      // own four: the lower or the upper half of piece g; the four above: its upper half, or the
+      // lower half of the next piece
+      const uint2 own = hh ? make_uint2(xa[g].z, xa[g].w) : make_uint2(xa[g].x, xa[g].y);
+      const uint2 abv = hh ? make_uint2(nx.x, nx.y) : make_uint2(xa[g].z, xa[g].w);
+      xo[4 * g] = bf_lo(own.x) * xsc; xo[4 * g + 1] = bf_hi(own.x) * xsc;
+      xo[4 * g + 2] = bf_lo(own.y) * xsc; xo[4 * g + 3] = bf_hi(own.y) * xsc;
+      xp[4 * g] = bf_lo(abv.x) * xsc; xp[4 * g + 1] = bf_hi(abv.x) * xsc;
+      xp[4 * g + 2] = bf_lo(abv.y) * xsc; xp[4 * g + 3] = bf_hi(abv.y) * xsc;
+    }
     auto unpack8 = [](const uint4& t, float* o, float sc) {
       o[0] = bf_lo(t.x) * sc; o[1] = bf_hi(t.x) * sc; o[2] = bf_lo(t.y) * sc; o[3] = bf_hi(t.y) * sc;
       o[4] = bf_lo(t.z) * sc; o[5] = bf_hi(t.z) * sc; o[6] = bf_lo(t.w) * sc; o[7] = bf_hi(t.w) * sc;
     };
 #pragma unroll
     for (int u = 0; u < H2 / 8; ++u) {
-      unpack8(xa[u], xo + 8 * u, xsc);
-      unpack8(xb[u], xp + 8 * u, xsc);
       uint4 t = ya[u];
       if (ydh) {   // y = grad_out / den, rounded once
         float f[8];
@@ -569,34 +594,29 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     }
   }
   const float c_own = (DQ && live) ? c_ld : 0.f;
-  const float yx = hh == 0 ? (DQ ? -c_own : -1.0f) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
+  const float yx = hh == 0 ? (DQ ? -c_own : (live ? -1.0f : 0.f)) : 0.f, yxhi = bf_lo(pack_bf2(yx, 0.f));
   // pairs with the state's extra column stored as (e_hi, e_hi, e_lo, e_lo); the upper four k slots
   // of that MFMA are empty
   const bf8v yxp = as_bf8(pack_bf4u(yxhi, yx - yxhi, yxhi, yx - yxhi), make_uint2(0u, 0u));
   if (n_tile > 0) tiles_store(0);
 
-  // out[ab][r]: channel hh*H2 + 16*ab + r of the lane's token; outx: what the lane collects for
-  // channel (1-hh)*H2 + 16*ab + r of the same token, which the lane of the other half holds
+  // out[ab][r]: channel 32 ab + 8 (r / 4) + 4 hh + r % 4 of the lane's token, i.e. own index
+  // 16 ab + r; outx[.]: what the lane collects for the channel four above that one
   f16v out[AB], outx[AB];
 #pragma unroll
   for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
     for (int r = 0; r < 16; ++r) out[ab][r] = outx[ab][r] = 0.f;
 
-  // A operand of tile ab: tile row m = lane i holds channel H2*((m>>2)&1) + 16*ab + 4*(m>>3) + (m&3),
-  // so that accumulator register r of lane half hh (tile row 8*(r>>2) + 4*hh + (r&3)) is channel
-  // hh*H2 + 16*ab + r.  The transposing read hands the lanes 4g..4g+3 of a group of 16 the four rows
-  // of the row group that the lanes J with J % 4 == g addressed, column slot J / 4.
+  // A operand of tile ab: tile row m = lane i is state row 32 ab + i.  The slab is feature-packed,
+  // [row / 4][column][row % 4]; the transposing read hands every lane = row four consecutive columns
+  // per 64-bit piece when, in every group of 16 lanes (16 consecutive rows), lane J addresses the
+  // word of row group J % 4 and column J / 4 of the piece.
+  const int trj = l & 15;
+  const int troff = (((i >> 4) * 4 + (trj & 3)) * NCF + (trj >> 2)) * 4;
   int tro[AB];
-  {
-    const int trj = l & 15;
-    const int mg = 4 * (i >> 4) + (trj & 3);   // row group of the tile
 #pragma unroll
-    for (int ab = 0; ab < AB; ++ab) {
-      const int cg = (H2 / 4) * (mg & 1) + 4 * ab + (mg >> 1);   // row group of the slab
-      tro[ab] = (PG::rgpos(cg) * NCF + (trj >> 2)) * 4;
-    }
-  }
+  for (int ab = 0; ab < AB; ++ab) tro[ab] = troff + ab * 8 * NCF * 4;
   constexpr int NB = H2 / 4 + 1;
   struct BOps {
     uint2 b[NB];
@@ -616,32 +636,15 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
       t = FM_MFMA_BF16(as_bf8(o.b[2 * m], o.b[2 * m + 1]), as_bf8(Yp[2 * m], Yp[2 * m + 1]), t);
     return FM_MFMA_BF16(as_bf8(o.b[H2 / 4], make_uint2(0u, 0u)), yxp, t);
   };
-  // both credits of tile ab of shift S (a compile-time constant; S == NS: the order-1 slab)
   auto credit = [&](const f16v& t, auto stag, auto abtag) __attribute__((always_inline)) {
-    constexpr int S = decltype(stag)::value, ABI = decltype(abtag)::value;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int jj = 16 * ABI + r;
-      const float v = t[r];
-      if constexpr (S == NS) {           // the order-1 slab (its coefficient is applied here)
-        out[ABI][r] += a1 * v;
-      } else if constexpr (S == 0) {     // the diagonal: one member, weight 1 stored, 2 owed
-        out[ABI][r] += (v + v) * xo[jj];
-      } else if constexpr (S == H2) {    // listed from both sides, weight 1 stored, 2 owed
-        out[ABI][r] += (v + v) * xp[jj];
-      } else {
-        const int p = jj + S;
-        if (p < H2) {
-          out[ABI][r] += v * xo[p];
-          out[p >> 4][p & 15] += v * xo[jj];
-        } else {
-          out[ABI][r] += v * xp[p - H2];
-          outx[(p - H2) >> 4][(p - H2) & 15] += v * xo[jj];
-        }
-      }
-    }
+    credit_tile<D, decltype(stag)::value, decltype(abtag)::value, true>(t, out, outx, xo, xp, a1);
   };
-
+  // (an empty volatile statement that takes the accumulators in and out keeps each unit's credits in
+  // that unit: see grad_kernel)
+  auto pin_accumulators = [&]() __attribute__((always_inline)) {
+    if constexpr (AB == 2) asm volatile("" : "+v"(out[0]), "+v"(out[1]), "+v"(outx[0]), "+v"(outx[1]));
+    else asm volatile("" : "+v"(out[0]), "+v"(outx[0]));
+  };
 
   if (n_state > 0) {
     FM_WAIT_VM(0);
@@ -685,6 +688,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
               }
           }
           credit(tp, std::integral_constant<int, PS>{}, std::integral_constant<int, PAB>{});
+          pin_accumulators();
         }
         tp = tn;
         if constexpr (V + 1 < 2 * AB) bc = bn;
@@ -704,11 +708,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
       }
     }
     credit(tp, std::integral_constant<int, (NU - 1) / AB>{}, std::integral_constant<int, (NU - 1) % AB>{});
-    // hand over what was collected for the channels of the other half
-#pragma unroll
-    for (int ab = 0; ab < AB; ++ab)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) out[ab][r] += other_half(outx[ab][r], hh);
+    exchange_halves<D>(out, outx, hh);
   } else if (n_state == 1) {
     // p = 1: the order-1 slab is the only one
     static_for<AB>([&](auto abtag) __attribute__((always_inline)) {
@@ -726,10 +726,6 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     for (int g4 = 0; g4 < H2 / 4; ++g4) Xp[g4] = pack_bf4u(xo[4 * g4], xo[4 * g4 + 1], xo[4 * g4 + 2], xo[4 * g4 + 3]);
     const int mine = (tok0 >> 5) + w;
     const float twoa2 = 2.0f * a2;
-    // tile row m = lane i of the product with W is channel chrow[ab] (same assignment as the state tiles)
-    int chrow[AB];
-#pragma unroll
-    for (int ab = 0; ab < AB; ++ab) chrow[ab] = H2 * ((i >> 2) & 1) + 16 * ab + 4 * (i >> 3) + (i & 3);
     for (int kk = 0; kk < n_tile; ++kk) {
       const int buf = kk & 1;
       tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
@@ -744,9 +740,10 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
         for (int r = 0; r < 16; ++r) sc[r] = gv[r] = 0.f;
 #pragma unroll
         for (int m = 0; m < H2 / 8; ++m) {
-          const uint16_t* r1 = l1 + i * LB + hh * H2 + 8 * m;
+          // (the scores pair the channels in the order of xo: groups 2m and 2m+1 of this lane half)
+          const uint16_t* r1 = l1 + i * LB + 16 * m + 4 * hh;
           const uint16_t* r2 = l2 + i * LB + hh * H2 + 8 * m;
-          sc = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(r1), *reinterpret_cast<const uint2*>(r1 + 4)),
+          sc = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(r1), *reinterpret_cast<const uint2*>(r1 + 8)),
                             as_bf8(Xp[2 * m], Xp[2 * m + 1]), sc);
           gv = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(r2), *reinterpret_cast<const uint2*>(r2 + 4)),
                             as_bf8(Yp[2 * m], Yp[2 * m + 1]), gv);
@@ -767,7 +764,7 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
                                  pack_bf4u(sc[8 * m + 4], sc[8 * m + 5], sc[8 * m + 6], sc[8 * m + 7]));
 #pragma unroll
           for (int ab = 0; ab < AB; ++ab) {
-            const uint16_t* trw = l1t + chrow[ab] * TPB + 16 * m + 4 * hh;
+            const uint16_t* trw = l1t + (ab * 32 + i) * TPB + 16 * m + 4 * hh;
             out[ab] = FM_MFMA_BF16(as_bf8(*reinterpret_cast<const uint2*>(trw), *reinterpret_cast<const uint2*>(trw + 8)),
                                    wp, out[ab]);
           }
@@ -778,20 +775,20 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     }
   }
 
-  // the lane holds H2 consecutive channels of its token: 16-byte stores, scaled by the normaliser
+  // the lane holds groups of four consecutive channels of its token: 8-byte stores, scaled by the
+  // normaliser
   float rs = 0.f;
 #pragma unroll
   for (int ab = 0; ab < AB; ++ab)
 #pragma unroll
     for (int r = 0; r < 16; ++r) rs += out[ab][r] * xo[16 * ab + r];
   if (live) {
-    uint4* orow = reinterpret_cast<uint4*>(OUT.head(head).row(tok) + hh * H2);
+    bf16_t* orow = OUT.head(head).row(tok) + 4 * hh;
 #pragma unroll
-    for (int u = 0; u < H2 / 8; ++u) {
-      const f16v& o = out[u >> 1];
-      const int r0 = 8 * (u & 1);
-      orow[u] = make_uint4(pack_bf2(o[r0] * xs, o[r0 + 1] * xs), pack_bf2(o[r0 + 2] * xs, o[r0 + 3] * xs),
-                           pack_bf2(o[r0 + 4] * xs, o[r0 + 5] * xs), pack_bf2(o[r0 + 6] * xs, o[r0 + 7] * xs));
+    for (int g = 0; g < NG; ++g) {
+      const f16v& o = out[g >> 2];
+      const int r0 = 4 * (g & 3);
+      *reinterpret_cast<uint2*>(orow + 8 * g) = make_uint2(pack_bf2(o[r0] * xs, o[r0 + 1] * xs), pack_bf2(o[r0 + 2] * xs, o[r0 + 3] * xs));
     }
   }
   rs = block_sum_256(rs, red, tid);
