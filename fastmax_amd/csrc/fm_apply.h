@@ -487,22 +487,14 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     constexpr int WO = decltype(wo)::value;   // Wn[WO + t] is the partner of channel t for this shift
     constexpr int NB = FWD ? CB + 1 : CB;
     constexpr int NM = H2 / 8;  // MFMA steps per column tile
-    const uint16_t* brow = sl + (hh * (H2 / 4) * NCF + i) * 4;
-    const uint16_t* erow = sl + (hh * (H2 / 4) * NCF + D) * 4;
-    // (the two halves of an operand are read next to each other, so that they pair into one
-    // two-address LDS read whose four destination registers are the operand)
-    auto fetch = [&](int m, uint2 (&b)[2 * NB]) {
+    // the eight features of MFMA step m of lane half hh are row octet hh H2/8 + m: one 16-byte word
+    // per column
+    const uint16_t* brow = sl + (hh * (H2 / 8) * NCF + i) * 8;
+    const uint16_t* erow = sl + (hh * (H2 / 8) * NCF + D) * 8;
+    auto fetch = [&](int m, fm_u4 (&b)[NB]) {
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-          b[2 * cb + u] = *reinterpret_cast<const uint2*>(brow + ((2 * m + u) * NCF + cb * 32) * 4);
-      }
-      if (FWD) {
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-          b[2 * (NB - 1) + u] = *reinterpret_cast<const uint2*>(erow + (2 * m + u) * NCF * 4);
-      }
+      for (int cb = 0; cb < CB; ++cb) b[cb] = *reinterpret_cast<const fm_u4*>(brow + (m * NCF + cb * 32) * 8);
+      if (FWD) b[NB - 1] = *reinterpret_cast<const fm_u4*>(erow + m * NCF * 8);
     };
     auto feat = [&](int g4) {
       const int t = 4 * g4;
@@ -512,7 +504,8 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     };
     // all B operands of the slab are requested first, the features are formed while they are on
     // their way, then the matrix instructions run back to back
-    uint2 b[NM][2 * NB], a[NM][2];
+    fm_u4 b[NM][NB];
+    uint2 a[NM][2];
 #pragma unroll
     for (int m = 0; m < NM; ++m) fetch(m, b[m]);
     __builtin_amdgcn_sched_barrier(0);
@@ -526,8 +519,8 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
     for (int m = 0; m < NM; ++m) {
       const bf8v ap = as_bf8(a[m][0], a[m][1]);
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA_BF16(ap, as_bf8(b[m][2 * cb], b[m][2 * cb + 1]), acc[cb]);
-      if (FWD) accd = FM_MFMA_BF16(ap, as_bf8(b[m][2 * (NB - 1)], b[m][2 * (NB - 1) + 1]), accd);
+      for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA_BF16(ap, __builtin_bit_cast(bf8v, b[m][cb]), acc[cb]);
+      if (FWD) accd = FM_MFMA_BF16(ap, __builtin_bit_cast(bf8v, b[m][NB - 1]), accd);
     }
   };
 

@@ -30,6 +30,7 @@ typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
 // B may be permuted together, two k = 8 operand pairs (each the four k-slots of a lane) are
 // simply concatenated: slots 0..3 from the first pair, 4..7 from the second.
 typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
+typedef uint32_t fm_u4 __attribute__((ext_vector_type(4)));   // the same 16 bytes as four dwords
 #define FM_MFMA_BF16(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16((a), (b), (c), 0, 0, 0)
 // wait until at most n vector-memory operations of this wave are outstanding (they complete in
 // order), leaving the other counters alone: s_waitcnt simm16 = vmcnt[3:0] | expcnt << 4 |
@@ -228,19 +229,19 @@ struct Geo {
 // state_floats slot as the fp32 form).  A "slab" is the D feature rows of one shift s (order 2;
 // rows carry their pair weight: x2 for 0 < s < D/2) or the D order-1 rows (slab NS, or slab 0
 // when p == 1), stored feature-packed,
-//   [a/4][column 0..D+3][a%4]
-// i.e. 8-byte words of four consecutive rows, which is the B operand layout of the bf16 matrix
-// instruction for a contraction over features (apply kernels: plain 64-bit LDS reads); for a
-// contraction over columns (grad kernels) the same words are read through the transposing LDS
-// load (lds_read_tr16).  Consumers stage a slab with plain 16-byte copies.  Columns D..D+3 hold
-// the extra (denominator) column split into hi + lo bf16 parts as (hi, hi, lo, lo), because in the
-// grad kernels that term nearly cancels the value columns' sum.  The slabs are followed by the
-// order-0 row as D+1 floats.
+//   [a/8][column 0..D+3][a%8]
+// i.e. 16-byte words of eight consecutive rows, which is the B operand of the bf16 matrix
+// instruction for a contraction over features (apply kernels: one 128-bit LDS read per operand);
+// for a contraction over columns (grad kernels) the two 8-byte halves of the words are read through
+// the transposing LDS load (lds_read_tr16).  Consumers stage a slab with plain 16-byte copies.
+// Columns D..D+3 hold the extra (denominator) column split into hi + lo bf16 parts as
+// (hi, hi, lo, lo), because in the grad kernels that term nearly cancels the value columns' sum.
+// The slabs are followed by the order-0 row as D+1 floats.
 template <int D>
 struct PackedGeo {
   using G = Geo<D>;
   static constexpr int NCF = D + 4;
-  static constexpr int FSL = (D / 4) * NCF * 4;  // bf16 elements of a slab (a multiple of 128)
+  static constexpr int FSL = (D / 8) * NCF * 8;  // bf16 elements of a slab (a multiple of 128)
   __host__ __device__ static constexpr int nslab(int p2) { return (p2 ? G::NS : 0) + 1; }
   __host__ __device__ static constexpr int64_t z_off(int p2) { return ((int64_t)nslab(p2) * FSL * 2 + 255) / 256 * 256; }
   __host__ __device__ static constexpr int64_t bytes(int p2) { return z_off(p2) + (D + 1) * 4; }

@@ -373,22 +373,23 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
         const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
         {
           const float wgt = dbl ? 2.0f : 1.0f;
-          // accumulator registers 4j..4j+3 are the four rows of row group (arow / 4) + 2j + hh
-          uint16_t* fx = fsec + (unsigned)(slab * PG::FSL + (arow >> 2) * PG::NCF * 4);
-          const unsigned lo = (unsigned)((hh * PG::NCF + cbase * 32 + i) * 4);
+          // accumulator registers 4j..4j+3 are rows 8j + 4hh .. + 3 of the tile: half hh of the
+          // 16-byte word of row octet (arow / 8) + j
+          uint16_t* fx = fsec + (unsigned)(slab * PG::FSL + (arow >> 3) * PG::NCF * 8);
+          const unsigned lo = (unsigned)((cbase * 32 + i) * 8 + 4 * hh);
 #pragma unroll
           for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
               const f16v& a = acc[x][cb];
-              *reinterpret_cast<uint2*>(fx + lo + (unsigned)((2 * j * PG::NCF + cb * 32) * 4)) =
+              *reinterpret_cast<uint2*>(fx + lo + (unsigned)((j * PG::NCF + cb * 32) * 8)) =
                   make_uint2(pack_bf2(a[4 * j] * wgt, a[4 * j + 1] * wgt), pack_bf2(a[4 * j + 2] * wgt, a[4 * j + 3] * wgt));
             }
           if (hh == 0 && cbase == 0) {   // the extra column, split into hi + lo parts: columns D..D+3 = (hi, hi, lo, lo)
             const float ew = ds * wgt, ehi = bf_lo(pack_bf2(ew, 0.f));
             const uint16_t h16 = (uint16_t)pack_bf2(ehi, 0.f), l16 = (uint16_t)pack_bf2(ew - ehi, 0.f);
-            uint16_t* ex = fx + (unsigned)(((i >> 2) * PG::NCF + D) * 4 + (i & 3));
-            ex[0] = h16; ex[4] = h16; ex[8] = l16; ex[12] = l16;
+            uint16_t* ex = fx + (unsigned)(((i >> 3) * PG::NCF + D) * 8 + (i & 7));
+            ex[0] = h16; ex[8] = h16; ex[16] = l16; ex[24] = l16;
           }
         }
       }
@@ -556,7 +557,9 @@ __global__ __launch_bounds__(256) void state_pack_kernel(float* __restrict__ sta
     const int tg = idx / (D + 1), col = idx % (D + 1);
     const float* f = Sl + 4 * tg * LD + col;
     const float f0 = f[0] * wgt, f1 = f[LD] * wgt, f2 = f[2 * LD] * wgt, f3 = f[3 * LD] * wgt;
-    uint2* dst = reinterpret_cast<uint2*>(fsec + (tg * PG::NCF + col) * 4);
+    // rows 4 tg .. 4 tg + 3: half tg % 2 of the 16-byte word of row octet tg / 2 (a column further is
+    // two 8-byte pieces further)
+    uint2* dst = reinterpret_cast<uint2*>(fsec + ((tg >> 1) * PG::NCF + col) * 8 + (tg & 1) * 4);
     if (col < D) {
       *dst = make_uint2(pack_bf2(f0, f1), pack_bf2(f2, f3));
     } else {   // the extra column, split into hi + lo parts: columns D..D+3 = (hi, hi, lo, lo)
@@ -564,7 +567,7 @@ __global__ __launch_bounds__(256) void state_pack_kernel(float* __restrict__ sta
       const float h2 = bf_lo(pack_bf2(f2, 0.f)), h3 = bf_lo(pack_bf2(f3, 0.f));
       const uint2 hi = make_uint2(pack_bf2(h0, h1), pack_bf2(h2, h3));
       const uint2 lo = make_uint2(pack_bf2(f0 - h0, f1 - h1), pack_bf2(f2 - h2, f3 - h3));
-      dst[0] = hi; dst[1] = hi; dst[2] = lo; dst[3] = lo;
+      dst[0] = hi; dst[2] = hi; dst[4] = lo; dst[6] = lo;
     }
   }
   if (ord1 && tid <= D) reinterpret_cast<float*>(sb + PG::z_off(p2))[tid] = Sl[D * LD + tid];

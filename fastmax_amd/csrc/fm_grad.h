@@ -609,14 +609,14 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
     for (int r = 0; r < 16; ++r) out[ab][r] = outx[ab][r] = 0.f;
 
   // A operand of tile ab: tile row m = lane i is state row 32 ab + i.  The slab is feature-packed,
-  // [row / 4][column][row % 4]; the transposing read hands every lane = row four consecutive columns
+  // [row / 8][column][row % 8]; the transposing read hands every lane = row four consecutive columns
   // per 64-bit piece when, in every group of 16 lanes (16 consecutive rows), lane J addresses the
-  // word of row group J % 4 and column J / 4 of the piece.
+  // 8-byte half (J % 4) % 2 of the word of row octet (J % 4) / 2 and column J / 4 of the piece.
   const int trj = l & 15;
-  const int troff = (((i >> 4) * 4 + (trj & 3)) * NCF + (trj >> 2)) * 4;
+  const int troff = (((i >> 4) * 2 + ((trj & 3) >> 1)) * NCF + (trj >> 2)) * 8 + (trj & 1) * 4;
   int tro[AB];
 #pragma unroll
-  for (int ab = 0; ab < AB; ++ab) tro[ab] = troff + ab * 8 * NCF * 4;
+  for (int ab = 0; ab < AB; ++ab) tro[ab] = troff + ab * 4 * NCF * 8;
   constexpr int NB = H2 / 4 + 1;
   struct BOps {
     uint2 b[NB];
@@ -624,8 +624,8 @@ __global__ __launch_bounds__(256, 2) void grad_kernel_bf(
   auto fetch = [&](const uint16_t* sl, int ab, BOps& o) __attribute__((always_inline)) {
     const uint16_t* ar = sl + tro[ab];
 #pragma unroll
-    for (int g4 = 0; g4 < H2 / 4; ++g4) o.b[g4] = lds_read_tr16(ar + (hh * H2 + 4 * g4) * 4);
-    o.b[H2 / 4] = lds_read_tr16(ar + D * 4);  // extra column as (hi, hi, lo, lo)
+    for (int g4 = 0; g4 < H2 / 4; ++g4) o.b[g4] = lds_read_tr16(ar + (hh * H2 + 4 * g4) * 8);
+    o.b[H2 / 4] = lds_read_tr16(ar + D * 8);  // extra column as (hi, hi, lo, lo)
   };
   auto chain = [&](const BOps& o) __attribute__((always_inline)) {
     f16v t;
