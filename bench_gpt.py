@@ -211,7 +211,7 @@ def main() -> int:
                                f"seq {args.seq}, batch {args.batch}, p={args.p}, AdamW",
                    "attention": "pytorch function" if args.pytorch_attention else "hip kernels",
                    "qkv split + rope": {"pytorch": "pytorch ops", "split": "fused hip kernel, contiguous q/k/v",
-                                        "packed": "rope in place, attention on strided views of the projection, "
+                                        "packed": "rotated q, k to a packed tensor, attention on strided views of it and of the projection, "
                                                   "token-major output (includes the rope pass in the attention time)"}[layout]},
         "loss_first_last": [losses[0], losses[-1]], "steps": args.steps, "warmup": args.warmup,
     }))

@@ -167,7 +167,7 @@ int fastmax_backward_strided(const fastmax_desc* desc, const fastmax_layout* lay
  * backward re-walks the sequence, fastmax_cuda_backward.cu:26-882).  The backward pass needs
  * the same prefix states S of (k, v) the forward pass built; fastmax_backward rebuilds them
  * (one of its three state builds).  A caller with memory to spare passes a buffer of
- * fastmax_saved_state_bytes(desc) bytes (256-byte aligned; bhkv * slots * state bytes, 16 GB
+ * fastmax_saved_state_bytes(desc) bytes (256-byte aligned; bhkv * slots * state bytes, 24 GB
  * at bh = 1024, n = 10000, d = 64, p = 2) to fastmax_forward_saving, keeps it untouched, and
  * hands it to fastmax_backward_saved, which then skips that build.  With saved_states == NULL
  * the two calls are fastmax_forward / fastmax_backward.  When a buffer is given the workspace
