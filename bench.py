@@ -95,20 +95,21 @@ def executed_mfma_flops(cfg: dict, bh: int, chunk: int = 0) -> dict:
     h2, ns, cb = d // 2, d // 2 + 1, d // 32
     per = 32768 if bf else 4096                 # flop per matrix instruction
     ksteps = (lambda k: k // 16) if bf else (lambda k: k // 2)   # instructions for a contraction length k
-    # state build: gsplit blocks x 4 waves x rtw row tiles x cb column tiles, one 32-token step at a time
+    # state build: gsplit blocks x 4 waves x rtw row tiles x cb column tiles, one step of ts tokens at a time
     rt_total = ns * cb + cb
     rtw = 3 if d == 64 else 5
     gsplit = -(-rt_total // (4 * rtw))
-    per_step = gsplit * 4 * rtw * cb * ksteps(32) * per
+    ts = 64 if d == 64 else 32                  # tokens per step of the p = 2 build kernel
+    per_step = gsplit * 4 * rtw * cb * ksteps(ts) * per
     nc = -(-n // chunk)
-    spc = chunk // 32
+    spc = chunk // ts
     if masked:
         steps_f = (nc - 1) * spc
-        steps_r = (-(-(n - (nc - 1) * chunk) // 32) + (nc - 2) * spc) if nc > 1 else 0
+        steps_r = (-(-(n - (nc - 1) * chunk) // ts) + (nc - 2) * spc) if nc > 1 else 0
     else:
         z = min(max(-(-1024 // (gsplit * bh)), 1), -(-n // 256))
         zlen = -(-(-(-n // z)) // 32) * 32
-        steps_f = steps_r = sum(-(-(min(n, (i + 1) * zlen) - i * zlen) // 32) for i in range(-(-n // zlen)))
+        steps_f = steps_r = sum(-(-(min(n, (i + 1) * zlen) - i * zlen) // ts) for i in range(-(-n // zlen)))
     out = {"build_fwd": bh * steps_f * per_step, "build_bwd": bh * steps_r * per_step}
     # consumers: blocks of 128 tokens, 4 waves of 32; the state part runs ns + 1 slabs (none in the first chunk
     # in scan order), then one score tile + one product per streamed 32-token tile of the own chunk

@@ -45,6 +45,11 @@ __device__ __forceinline__ bf8v as_bf8(uint2 lo, uint2 hi) {
   const uint4 u = make_uint4(lo.x, lo.y, hi.x, hi.y);
   return __builtin_bit_cast(bf8v, u);
 }
+// acc + a.lo * b.lo + a.hi * b.hi of two bf16 pairs (v_dot2c_f32_bf16)
+typedef __bf16 fm_bf2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float fm_dot2_bf16(uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(fm_bf2, a), __builtin_bit_cast(fm_bf2, b), acc, false);
+}
 __device__ __forceinline__ uint2 pack_bf4u(float a, float b, float c, float d) {
   return make_uint2(pack_bf2(a, b), pack_bf2(c, d));
 }

@@ -147,8 +147,12 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     RowScalars ew, float* __restrict__ state, int n, int chunk, int nslots, int masked, int reverse,
     int p2, int zlen) {
   using G = Geo<D>;
-  constexpr int TS = 32;  // tokens per pipeline step (64 for bf16 halves the barriers but does not fit the
-                        // register file next to three row tiles of accumulators)
+  // tokens per pipeline step (= per barrier).  The p = 2 kernels at D = 64 take 64 tokens, staged as two halves of 32:
+  // the step's fixed costs (barrier, staging round trip, step bookkeeping) are paid half as often
+  // (bf16 build 7 % faster than with 32-token steps, fp32 1 %); the D = 32 kernels, with five row
+  // tiles of accumulators per wave, have no registers for it, and the p = 1 kernels (RTW == 1) keep
+  // the smaller tiles for their occupancy.  chunk is a multiple of TS.
+  constexpr int TS = (D == 64 && RTW > 1) ? 64 : 32;
   constexpr int TP = TS + 4;    // pitch of the transposed tiles: 16-byte aligned rows, and the
                                 // 8 lanes of a 128-bit LDS access phase fall in distinct banks
   constexpr int LD = G::LD;
@@ -289,6 +293,10 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
         const float a2 = cur.own[x].z * cur.rot[x].z, a3 = cur.own[x].w * cur.rot[x].w;
         if constexpr (BF) {
           const uint2 ap = pack_bf4u(a0, a1, a2, a3);
+          // the extra column sums the features as rounded for the matrix instruction (two 2-term
+          // bf16 dot products instead of four fp32 FMAs), so it is consistent with the value columns
+          dacc[x] = fm_dot2_bf16(ap.x, pack_bf2(cur.e4.x, cur.e4.y), dacc[x]);
+          dacc[x] = fm_dot2_bf16(ap.y, pack_bf2(cur.e4.z, cur.e4.w), dacc[x]);
           if ((gq & 1) == 0) {
             ap_even[x] = ap;
           } else {
@@ -305,7 +313,9 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
             acc[x][cb] = FM_MFMA(a3, cur.vv[cb].w, acc[x][cb]);
           }
         }
-        dacc[x] += a0 * cur.e4.x + a1 * cur.e4.y + a2 * cur.e4.z + a3 * cur.e4.w;
+        if constexpr (!BF) {
+          dacc[x] += a0 * cur.e4.x + a1 * cur.e4.y + a2 * cur.e4.z + a3 * cur.e4.w;
+        }
       }
       if constexpr (BF) {
         if ((gq & 1) == 0) {
@@ -451,30 +461,47 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     // take turns; the requests are unconditional, the last ones repeat the last step and are not
     // used), so that a step's global latency and the drain of a snapshot's stores -- which the
     // same in-order counter makes later loads wait for -- are spread over two steps of work.
-    static_assert(NH == 1, "one 32-token half per step");
-    std::conditional_t<BF, RawTileBf<D, 32>, RowTile<D, T, 32, true>> kx2, vy2;
-    float ereg2 = 0.f;
-    auto load_into = [&](auto& k_, auto& v_, float& e_, int t0) __attribute__((always_inline)) {
-      k_.load(Xh, t0, tend, tid);
-      v_.load(Yh, t0, tend, tid, ydh, yden_stride);
-      if (tid < 32) {
-        const int tok = t0 + tid;
-        e_ = (tok < tend && tok >= lo) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
+    using Tile = RawTileBf<D, 32>;
+    Tile kxa[NH], vya[NH], kxb[NH], vyb[NH];
+    float era[NH], erb[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) era[h] = erb[h] = 0.f;
+    auto load_into = [&](Tile (&k_)[NH], Tile (&v_)[NH], float (&e_)[NH], int t0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        k_[h].load(Xh, t0 + 32 * h, tend, tid);
+        v_[h].load(Yh, t0 + 32 * h, tend, tid, ydh, yden_stride);
+        if (tid < 32) {
+          const int tok = t0 + 32 * h + tid;
+          e_[h] = (tok < tend && tok >= lo) ? (ewh ? ewh[tok] : 1.0f) : 0.f;
+        }
       }
     };
-    auto store_from = [&](auto& k_, auto& v_, float e_, int buf, int t0) __attribute__((always_inline)) {
-      k_.store_t(Kt[buf], TP, xs, tid);
-      v_.store_t_bf(Vtb[buf], TPB, 1.0f, tid, ydh == nullptr);
-      if (tid < 32) {
-        El[buf][tid] = e_;
-        Kt[buf][D * TP + tid] = (t0 + tid < tend && t0 + tid >= lo) ? 1.0f : 0.f;
+    auto store_from = [&](const Tile (&k_)[NH], const Tile (&v_)[NH], const float (&e_)[NH], int buf, int t0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        k_[h].store_t(Kt[buf] + 32 * h, TP, xs, tid);
+        v_[h].store_t_bf(Vtb[buf] + 32 * h, TPB, 1.0f, tid, ydh == nullptr);
+        if (tid < 32) {
+          const int tok = t0 + 32 * h + tid;
+          El[buf][32 * h + tid] = e_[h];
+          Kt[buf][D * TP + 32 * h + tid] = (tok < tend && tok >= lo) ? 1.0f : 0.f;
+        }
       }
     };
-    auto step = [&](int p, auto& lk, auto& lv, float& le, auto& sk, auto& sv, float se) __attribute__((always_inline)) {
+    // AHEAD = steps between a tile's request and its staging: two 32-token steps or one 64-token step
+    // (the same time; with one step a single set of registers does)
+    constexpr int AHEAD = NH == 1 ? 2 : 1;
+    auto step = [&](int p, Tile (&lk)[NH], Tile (&lv)[NH], float (&le)[NH], const Tile (&sk)[NH],
+                    const Tile (&sv)[NH], const float (&se)[NH]) __attribute__((always_inline)) {
       __builtin_amdgcn_sched_barrier(0);
-      const int pl2 = p + 2 < nsteps ? p + 2 : nsteps - 1;
-      load_into(lk, lv, le, step_tok(pl2));
-      compute(p & 1, 0);
+      const int pl = p + AHEAD < nsteps ? p + AHEAD : nsteps - 1;
+      load_into(lk, lv, le, step_tok(pl));
+#pragma unroll
+      for (int h = 0; h < NH; ++h) {
+        compute(p & 1, h);
+        __builtin_amdgcn_sched_barrier(0);   // (keeps the halves apart: register pressure)
+      }
       sum0(p & 1);
       if (p + 1 < nsteps) store_from(sk, sv, se, (p + 1) & 1, step_tok(p + 1));
       const int slot = step_slot(p);
@@ -483,14 +510,19 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       __builtin_amdgcn_sched_barrier(0);
     };
     if (nsteps > 0) {
-      load_into(kx, vy, ereg, step_tok(0));
-      store_from(kx, vy, ereg, 0, step_tok(0));
-      load_into(kx2, vy2, ereg2, step_tok(nsteps > 1 ? 1 : 0));
+      load_into(kxa, vya, era, step_tok(0));
+      store_from(kxa, vya, era, 0, step_tok(0));
+      if constexpr (AHEAD == 2) load_into(kxb, vyb, erb, step_tok(nsteps > 1 ? 1 : 0));
     }
     __syncthreads();
-    for (int p = 0; p < nsteps; p += 2) {
-      step(p, kx, vy, ereg, kx2, vy2, ereg2);
-      if (p + 1 < nsteps) step(p + 1, kx2, vy2, ereg2, kx, vy, ereg);
+    if constexpr (AHEAD == 2) {
+      for (int p = 0; p < nsteps; p += 2) {
+        step(p, kxa, vya, era, kxb, vyb, erb);
+        if (p + 1 < nsteps) step(p + 1, kxb, vyb, erb, kxa, vya, era);
+      }
+    } else {
+      // (the set is requested at the start of a step and staged at its end)
+      for (int p = 0; p < nsteps; ++p) step(p, kxa, vya, era, kxa, vya, era);
     }
   } else {
     if (nsteps > 0) {
@@ -504,12 +536,13 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     for (int p = 0; p < nsteps; ++p) {
       const bool more = p + 1 < nsteps;
       const int tnext = step_tok(more ? p + 1 : p);
-  #pragma unroll
+  #pragma unroll 1
       for (int h = 0; h < NH; ++h) {
         if (more) load(tnext + 32 * h, tend);
         compute(p & 1, h);
         if (h == NH - 1) sum0(p & 1);
         if (more) store((p + 1) & 1, h, tnext + 32 * h, tend);
+        if constexpr (NH > 1) __builtin_amdgcn_sched_barrier(0);   // (keeps the halves apart: register pressure)
       }
       // after the staged tile has been consumed: waiting for loads while stores are pending
       // would wait for the stores too (one in-order counter covers both)
