@@ -16,9 +16,9 @@
 
 // ---------------------------------------------------------------------------------------
 // One block = 128 tokens of one head, one wave = 32 of them.  Lane (i = l%32, hh = l/32) keeps
-// its own half of x_i in registers (channels t + hh*D/2) and a sliding window of the rotated
-// partners x_i[(a+s)%D] (reloaded from LDS every fourth shift, slid by one register in
-// between), so an order-2 feature costs one multiply of two registers.  The state streams
+// its own half of x_i in registers (channels t + hh*D/2) and a window of the rotated
+// partners x_i[(a+s)%D] (reloaded from LDS every fourth shift and read at a compile-time position
+// in between), so an order-2 feature costs one multiply of two registers.  The state streams
 // through a double-buffered LDS slab (one shift = D rows at a time), coefficients a2*w_s / a1 /
 // a0 applied while staging; its rows are the B operands (two column tiles per feature) and, in
 // the forward pass, its extra column gives the denominator.
@@ -183,6 +183,10 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
         if (FWD) dn += a * cur.dd[e];
       }
       FM_SCHED_MFMA_DS_VALU(KB * CB)
+      // (an empty volatile statement that takes the denominator sum in and out keeps its FMAs in their
+      // batch; without it the scheduler collects them behind the slab's matrix instructions with every
+      // feature still alive, and the unrolled shifts spill)
+      if (FWD) asm volatile("" : "+v"(dn));
       if (t0 + KB < H2) cur = nxt;
     }
   };
@@ -209,36 +213,7 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  if constexpr (FWD) {
-    // (the forward pass also carries the denominator sums; with them the unrolled form below does not
-    // fit the register file, so its window is slid by one register per shift instead)
-    for (int st = 0; st < n_state; ++st) {
-      slab_load(st + 1 < n_state ? st + 1 : st);
-      const float* sl = Sl[st & 1];
-      if (p2 && st < NS) {
-        if ((st & 3) == 0) {
-          window_load(st);
-        } else {
-#pragma unroll
-          for (int x = 0; x < H2 + 3; ++x) Wn[x] = Wn[x + 1];
-        }
-        slab_compute(sl, std::true_type{}, std::integral_constant<int, 0>{});
-      } else {
-        slab_compute(sl, std::false_type{}, std::integral_constant<int, 0>{});
-        const float* s0 = sl + D * LD;  // order 0 rides at the end of the order-1 slab
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-          const float z = s0[cb * 32 + i];
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[cb][r] += z;
-        }
-        if (hh == 0) dn += s0[D];
-      }
-      if (st + 1 < n_state) slab_store(st + 1);
-      else if (n_tile > 0) tiles_store((st + 1) & 1);
-      __syncthreads();
-    }
-  } else if (n_state > 1) {
+  if (n_state > 1) {
     // p = 2: shifts 0 .. NS-1, then the order-1 slab.  The window of rotated partners is loaded
     // every fourth shift and read at a compile-time position in between (no register moves).
     static_assert((NS - 1) % 4 == 0, "shifts come in groups of four plus the last one");
