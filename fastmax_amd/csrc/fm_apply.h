@@ -19,9 +19,9 @@
 // its own half of x_i in registers (channels t + hh*D/2) and a window of the rotated
 // partners x_i[(a+s)%D] (reloaded from LDS every fourth shift and read at a compile-time position
 // in between), so an order-2 feature costs one multiply of two registers.  The state streams
-// through a double-buffered LDS slab (one shift = D rows at a time), coefficients a2*w_s / a1 /
-// a0 applied while staging; its rows are the B operands (two column tiles per feature) and, in
-// the forward pass, its extra column gives the denominator.
+// through a double-buffered LDS slab (one shift = D rows at a time, global -> LDS directly, one slab
+// ahead); the coefficients a2*w_s / a1 / a0 ride on the features; the slab's rows are the B operands
+// (two column tiles per feature) and, in the forward pass, its extra column gives the denominator.
 // For causal attention 32-token tiles of the block's own chunk follow through the same
 // buffers: scores are formed transposed (streamed tokens x own tokens) so that the polynomial
 // of the score tile, still in accumulator registers, is directly the A operand of the product
@@ -45,10 +45,22 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
     int adiv) {
   using G = Geo<D>;
   constexpr bool FWD = MODE == 0;
-  constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS, SLABF = G::SLABF;
+  constexpr int LD = G::LD, CB = G::CB, H2 = G::H2, NS = G::NS;
   constexpr int KB = 8;  // k-steps per operand batch
+  // A slab (the D rows of one shift, or the order-1 rows) travels global -> LDS without passing through
+  // registers (global_load_lds_dwordx4: lane l of a wave delivers its 16 bytes at a wave-uniform LDS
+  // base + 16 l), one slab ahead of its use, into the buffer the slab before was read from.  Two
+  // separate arrays: the compiler's bookkeeping of outstanding transfers is per LDS object.
+  constexpr int SLF = D * LD;                        // floats of a slab
+  constexpr int NPC = SLF / 4;                       // 16-byte pieces of a slab
+  constexpr int NPCR = (NPC + 63) / 64 * 64;
+  constexpr int NVS = (NPC + 255) / 256;             // transfers per wave and slab
+  constexpr int TILEF = 2 * 32 * LD;                 // both 32-token tiles of a streamed step
+  constexpr int SLB = NPCR * 4 > TILEF ? NPCR * 4 : TILEF;
   __shared__ __attribute__((aligned(16))) float Xl[128 * LD];
-  __shared__ __attribute__((aligned(16))) float Sl[2][SLABF];
+  __shared__ __attribute__((aligned(16))) float Sl0[SLB];
+  __shared__ __attribute__((aligned(16))) float Sl1[SLB];
+  __shared__ __attribute__((aligned(16))) float Sjunk[256];   // where transfers nobody needs end up
   __shared__ float denl[128];
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
@@ -93,37 +105,41 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
   // this block's chunk snapshot (masked) or the head's summed state (last slot)
   const float* sbase = state + ((int64_t)ha * nslots + (masked ? c : nslots - 1)) * SS;
 
-  StateSlab<(D + 1) * LD> slab;
-  RowTile<D, T, 32> t1, t2;
-  auto slab_load = [&](int st) {
-    const bool ord2 = p2 && st < NS;
-    slab.load(sbase + (ord2 ? st * D * LD : rows2 * LD), ord2 ? D * LD : (D + 1) * LD, tid);
-  };
-  auto slab_store = [&](int st) {
-    if (p2 && st < NS) {
-      const float cf = (st == 0 || st == H2) ? a2 : 2.0f * a2;
-      slab.store(Sl[st & 1], D * LD, D * LD, cf, cf, tid);
-    } else {
-      slab.store(Sl[st & 1], (D + 1) * LD, D * LD, a1, a0, tid);
+  // Transfers of slab st into `buf` (wave-uniform; the order-2 slabs and the order-1 slab are
+  // consecutive runs of D rows).  No branches: pieces past the slab's end wrap round at the source, and
+  // a wave transfer that lies wholly past the end, or a slab past the last one, is sent to Sjunk.
+  auto slab_dma = [&](int st, float* buf) __attribute__((always_inline)) {
+    const bool on = st < n_state;
+    const float* src = sbase + (on ? st : 0) * SLF;
+#pragma unroll
+    for (int r = 0; r < NVS; ++r) {
+      const int first = r * 256 + w * 64;
+      float* dst = (on && first < NPCR) ? buf + first * 4 : Sjunk;
+      __builtin_amdgcn_global_load_lds(src + ((first + l) % NPC) * 4,
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
     }
   };
+  RowTile<D, T, 32> t1, t2;
   auto tiles_load = [&](int kk) {
     t1.load(A1h, (tile0 + kk) * 32, n, tid);
     t2.load(A2h, (tile0 + kk) * 32, n, tid, a2dh, a2den_stride);
   };
   auto tiles_store = [&](int buf) {
-    t1.store(Sl[buf], LD, a1s, tid);
-    t2.store(Sl[buf] + 32 * LD, LD, 1.0f, tid);
+    float* tb = buf ? Sl1 : Sl0;
+    t1.store(tb, LD, a1s, tid);
+    t2.store(tb + 32 * LD, LD, 1.0f, tid);
   };
 
   if (n_tile > 0) tiles_load(0);
-  if (n_state > 0) slab_load(0);
+  if (n_state > 0) slab_dma(0, Sl0);
+  // the order-0 row of the state: value columns i and 32 + i, and the extra column
+  float z0[CB], zd = 0.f;
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) z0[cb] = n_state > 0 ? a0 * sbase[(rows2 + D) * LD + cb * 32 + i] : 0.f;
+  if (FWD && n_state > 0 && hh == 0) zd = a0 * sbase[(rows2 + D) * LD + D];
   xt.store(Xl, LD, xs, tid);
-  if (n_state > 0) {
-    slab_store(0);
-  } else if (n_tile > 0) {
-    tiles_store(0);
-  }
+  if (n_state == 0 && n_tile > 0) tiles_store(0);
+  FM_WAIT_VM(0);
   __syncthreads();
 
   const int xrow = w * 32 + i;
@@ -141,14 +157,16 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
     for (int r = 0; r < 16; ++r) acc[cb][r] = 0.f;
   float dn = 0.f;
 
-  // rotated partners: after window_load(s0) (s0 % 4 == 0), Wn[x] = x_i[(hh*H2 + s0 + x) % D]
+  // rotated partners: after window_load(s0, cf) (s0 % 4 == 0), Wn[x] = cf * x_i[(hh*H2 + s0 + x) % D].
+  // The state is stored raw and each unordered pair once: cf carries a2 and the pair weight (2 for the
+  // shifts 0 < s < D/2; the window of shifts 0..3 takes 2 a2 as well and the sums are halved after shift 0).
   float Wn[H2 + 4];
-  auto window_load = [&](int s0) {
+  auto window_load = [&](int s0, float cf) {
 #pragma unroll
     for (int j = 0; j < H2 / 4 + 1; ++j) {
       const int c0 = (hh * H2 + s0 + 4 * j) & (D - 1);
       const float4 q4 = *reinterpret_cast<const float4*>(Xl + xrow * LD + c0);
-      Wn[4 * j] = q4.x; Wn[4 * j + 1] = q4.y; Wn[4 * j + 2] = q4.z; Wn[4 * j + 3] = q4.w;
+      Wn[4 * j] = q4.x * cf; Wn[4 * j + 1] = q4.y * cf; Wn[4 * j + 2] = q4.z * cf; Wn[4 * j + 3] = q4.w * cf;
     }
   };
 
@@ -177,7 +195,7 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
       if (t0 + KB < H2) batch_fetch(sl, t0 + KB, nxt);
 #pragma unroll
       for (int e = 0; e < KB; ++e) {
-        const float a = ORD2 ? Xr[t0 + e] * Wn[WO + t0 + e] : Xr[t0 + e];
+        const float a = ORD2 ? Xr[t0 + e] * Wn[WO + t0 + e] : Xr[t0 + e] * a1;
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) acc[cb] = FM_MFMA(a, cur.b[e][cb], acc[cb]);
         if (FWD) dn += a * cur.dd[e];
@@ -190,45 +208,54 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
       if (t0 + KB < H2) cur = nxt;
     }
   };
-  // one pipeline step: fetch slab st+1, work on slab st, stage slab st+1 (or the first streamed tile)
-  auto slab_iter = [&](int st, auto tag, auto wo) __attribute__((always_inline)) {
+  // one pipeline step: start the transfer of slab st+1 into the other buffer (every wave is past it: it
+  // has passed the barrier), work on slab st, wait for the wave's own transfers, barrier (which covers
+  // the other waves').  After the last slab the first streamed tile is staged instead.  PAR = st % 2.
+  auto slab_iter = [&](int st, auto par, auto tag, auto wo) __attribute__((always_inline)) {
     constexpr bool ORD2 = decltype(tag)::value;
+    constexpr int PAR = decltype(par)::value;
     __builtin_amdgcn_sched_barrier(0);   // (keeps the unrolled steps from being interleaved: register pressure)
-    slab_load(st + 1 < n_state ? st + 1 : st);
-    const float* sl = Sl[st & 1];
-    slab_compute(sl, tag, wo);
+    slab_dma(st + 1, PAR ? Sl0 : Sl1);
+    slab_compute(PAR ? Sl1 : Sl0, tag, wo);
     if (!ORD2) {
-      const float* s0 = sl + D * LD;  // order 0 rides at the end of the order-1 slab
+      // order 0
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) {
-        const float z = s0[cb * 32 + i];
+      for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[cb][r] += z;
-      }
-      if (FWD && hh == 0) dn += s0[D];
+        for (int r = 0; r < 16; ++r) acc[cb][r] += z0[cb];
+      if (FWD) dn += zd;
     }
-    if (st + 1 < n_state) slab_store(st + 1);
-    else if (n_tile > 0) tiles_store((st + 1) & 1);
+    if (st + 1 >= n_state && n_tile > 0) tiles_store(PAR ^ 1);
+    FM_WAIT_VM(0);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
   };
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
 
   if (n_state > 1) {
     // p = 2: shifts 0 .. NS-1, then the order-1 slab.  The window of rotated partners is loaded
     // every fourth shift and read at a compile-time position in between (no register moves).
     static_assert((NS - 1) % 4 == 0, "shifts come in groups of four plus the last one");
     for (int st = 0; st < NS - 1; st += 4) {
-      window_load(st);
-      slab_iter(st, std::true_type{}, std::integral_constant<int, 0>{});
-      slab_iter(st + 1, std::true_type{}, std::integral_constant<int, 1>{});
-      slab_iter(st + 2, std::true_type{}, std::integral_constant<int, 2>{});
-      slab_iter(st + 3, std::true_type{}, std::integral_constant<int, 3>{});
+      window_load(st, 2.0f * a2);
+      slab_iter(st, P0{}, std::true_type{}, std::integral_constant<int, 0>{});
+      if (st == 0) {   // shift 0 lists every pair once
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[cb][r] *= 0.5f;
+        dn *= 0.5f;
+      }
+      slab_iter(st + 1, P1{}, std::true_type{}, std::integral_constant<int, 1>{});
+      slab_iter(st + 2, P0{}, std::true_type{}, std::integral_constant<int, 2>{});
+      slab_iter(st + 3, P1{}, std::true_type{}, std::integral_constant<int, 3>{});
     }
-    window_load(NS - 1);
-    slab_iter(NS - 1, std::true_type{}, std::integral_constant<int, 0>{});
-    slab_iter(NS, std::false_type{}, std::integral_constant<int, 0>{});
+    window_load(NS - 1, a2);   // shift D/2 lists every pair once, too
+    slab_iter(NS - 1, P0{}, std::true_type{}, std::integral_constant<int, 0>{});
+    slab_iter(NS, P1{}, std::false_type{}, std::integral_constant<int, 0>{});
   } else if (n_state == 1) {
-    slab_iter(0, std::false_type{}, std::integral_constant<int, 0>{});
+    slab_iter(0, P0{}, std::false_type{}, std::integral_constant<int, 0>{});
   }
 
   const int mine = (tok0 >> 5) + w;
@@ -237,8 +264,8 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
     tiles_load(kk + 1 < n_tile ? kk + 1 : kk);
     const int tl = tile0 + kk;
     if (FWD ? tl <= mine : tl >= mine) {
-      const float* l1 = Sl[buf];
-      const float* l2 = Sl[buf] + 32 * LD;
+      const float* l1 = buf ? Sl1 : Sl0;
+      const float* l2 = l1 + 32 * LD;
       // scores, transposed: rows = streamed tokens trow(r,hh), lanes = own tokens
       f16v sc;
 #pragma unroll
