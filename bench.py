@@ -46,9 +46,9 @@ COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 # runs summarised under profiles/ (one file per workload, TRAFFIC_SOURCE)
 # (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch x2.0, write x1.0).
 MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD = {
-    "headline": {"build": 3920.0, "fwd_apply": 3426.0, "bwd_dq": 4448.0, "bwd_dk": 4553.0, "bwd_dv": 3675.0},
+    "headline": {"build": 3708.0, "fwd_apply": 3597.0, "bwd_dq": 4440.0, "bwd_dk": 4569.0, "bwd_dv": 3877.0},
     # profiles/config4_causal_bf16_all_kernels.txt
-    "c4": {"build": 1290.0, "fwd_apply": 1298.0, "bwd_dq": 1429.0, "bwd_dk": 1481.0, "bwd_dv": 1383.0},
+    "c4": {"build": 1415.0, "fwd_apply": 1298.0, "bwd_dq": 1429.0, "bwd_dk": 1481.0, "bwd_dv": 1383.0},
     # profiles/headline_p1_causal_fp32_scan_kernels.txt (algorithmic: 1024 B per token-head and kernel,
     # 1280 B for dq, which also reads the forward output)
     "headline-p1": {"fwd_apply": 1164.0, "bwd_dq": 1504.0, "bwd_dk": 1186.0, "bwd_dv": 1178.0},
