@@ -100,6 +100,12 @@ struct Plan {
   bool plain;          // every tensor is a plain contiguous (heads, tokens, d) array
   bool scan;           // causal p = 1 as one scan per head (fm_linear.h): no states in memory
   bool rowpass;        // unmasked p = 1: states from the build kernel, one pass over the rows per output
+  bool split;          // causal p = 1 with few heads: the chunks of a head are built side by side as partial
+                       // states and a prefix pass over the chunks makes the causal states of them
+  size_t scratch_bytes;   // per head: where the fp32 partial states of a split build go when the
+                          // states themselves are packed bf16 (last part of per_head_bytes; a forward
+                          // pass that keeps its states has it behind the states in the caller's buffer)
+  int pass;
   int64_t state_floats;
   size_t fixed_bytes;     // scale/argmax/cvec/rpart
   size_t per_head_bytes;  // states of one head
@@ -126,6 +132,7 @@ bool use_linear_scan(const fastmax_desc* ds, const Plan& pl);
 
 Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true) {
   Plan pl;
+  pl.pass = pass;
   pl.d = ds->d;
   pl.p2 = ds->p == 2;
   pl.masked = ds->mask != 0;
@@ -186,6 +193,12 @@ Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true) {
     pl.per_head_bytes += 2 * (size_t)pl.nk * pl.d * (ds->dtype == FASTMAX_BF16 ? 2 : 4);
   pl.scan = use_linear_scan(ds, pl);
   if (pl.scan) pl.per_head_bytes = 0;
+  // One sequential walk per head leaves most of the chip idle when there are few heads; a p = 1 state
+  // is small (d + 1 rows), so the chunks are built side by side and a cheap pass adds them up.
+  pl.split = pl.masked && !pl.p2 && !pl.scan && pl.nslots >= 3 && (int64_t)pl.bh * pl.gsplit < 1024;
+  pl.scratch_bytes = (pl.split && ds->dtype == FASTMAX_BF16)
+                         ? (size_t)pl.nslots * state_floats_for(pl.d, pl.p2) * sizeof(float) : 0;
+  pl.per_head_bytes += pl.scratch_bytes;
   pl.rowpass = !pl.p2 && !pl.masked && pl.d == 64 && pl.ratio == 1 && pl.n >= 32 && pl.plain && pl.nq == pl.nk;
   return pl;
 }
@@ -202,7 +215,9 @@ bool use_linear_scan(const fastmax_desc* ds, const Plan& pl) {
 // (with_saved: the prefix states live in the caller's saved-state buffer, not in the workspace)
 size_t batch_bytes_per_head(const Plan& pl, bool with_saved) {
   if (pl.scan) return 0;
-  return pl.per_head_bytes - (with_saved ? (size_t)pl.nslots * pl.state_floats * sizeof(float) : 0);
+  if (!with_saved) return pl.per_head_bytes;
+  return pl.per_head_bytes - (size_t)pl.nslots * pl.state_floats * sizeof(float) -
+         (pl.pass == FASTMAX_PASS_FORWARD ? pl.scratch_bytes : 0);
 }
 
 int heads_per_batch(const Plan& pl, size_t ws_bytes, bool with_saved = false) {
@@ -255,7 +270,8 @@ int check_ws(const Plan& pl, void* ws, size_t ws_bytes, bool with_saved = false)
 
 size_t saved_bytes_for(const Plan& pl) {
   if (pl.scan) return 256;   // nothing to keep; a token size, so that 0 still means "bad descriptor"
-  return (size_t)pl.bhkv * pl.nslots * pl.state_floats * sizeof(float);
+  // (a split build of packed states sums fp32 partial states: room for them behind the states)
+  return (size_t)pl.bhkv * (pl.nslots * pl.state_floats * sizeof(float) + pl.scratch_bytes);
 }
 
 int check_saved(const Plan& pl, const void* saved, size_t saved_bytes) {
@@ -368,10 +384,24 @@ constexpr bool kBf16Mfma<bf16_t> = true;
 template <int D, class T>
 int launch_build(const Plan& pl, int heads, int n, const Rows<const T>& X, const Rows<const T>& Y,
                  const float* xscale, const RowScalars& yden, const RowScalars& ew, float* state, int reverse,
-                 hipStream_t stream, bool finish = true) {
-  const dim3 grid(pl.gsplit, heads, pl.nparts);
+                 hipStream_t stream, bool finish = true, float* scratch = nullptr) {
   if (pl.masked && pl.nslots < 2) return FASTMAX_OK;  // a single chunk never needs a state
   ScopedKernel sk(FASTMAX_K_BUILD, stream);
+  if (pl.split) {
+    // every chunk as a token split of its own (the unmasked form of the kernel: fp32 partial states,
+    // slot c = chunk c), then the sums over the chunks before (after, for a reverse scan) each chunk
+    float* part = kBf16Mfma<T> ? scratch : state;
+    const dim3 sgrid(pl.gsplit, heads, pl.nslots);
+    build_kernel<D, T, 1, kBf16Mfma<T>><<<sgrid, 256, 0, stream>>>(X, Y, xscale, yden, ew, part, n, pl.chunk, pl.nslots,
+                                                                   0, 0, pl.p2, pl.chunk);
+    const int64_t ss = state_floats_for(pl.d, pl.p2);
+    state_prefix_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads), 256, 0, stream>>>(part, pl.nslots, ss, reverse);
+    if constexpr (kBf16Mfma<T>)
+      state_pack_slots_kernel<D><<<dim3(PackedGeo<D>::nslab(pl.p2), heads, pl.nslots), 256, 0, stream>>>(part, state,
+                                                                                                      pl.nslots, pl.p2);
+    return launch_status("build_kernel (chunks side by side)");
+  }
+  const dim3 grid(pl.gsplit, heads, pl.nparts);
 #define FM_BUILD(RTW)                                                                            \
   build_kernel<D, T, RTW, kBf16Mfma<T>><<<grid, 256, 0, stream>>>(X, Y, xscale, yden, ew, state, \
                                                     n, pl.chunk, pl.nslots, pl.masked, reverse, \
@@ -467,8 +497,13 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const 
       }
     }
     const Rows<const T> kr = mk_rows(k, L.k, kv0), vr = mk_rows(v, L.v, kv0);
+    // (scratch of a split build: behind the batch's states in the workspace, or behind all states in
+    // the caller's buffer)
+    float* scratch = saved ? reinterpret_cast<float*>(reinterpret_cast<char*>(saved + (int64_t)pl.bhkv * head_floats) +
+                                                      (size_t)kv0 * pl.scratch_bytes)
+                           : reinterpret_cast<float*>(ws + pl.fixed_bytes + (size_t)hb * (pl.per_head_bytes - pl.scratch_bytes));
     FM_TRY((launch_build<D, T>(pl, heads / ratio, nk, kr, vr, scale + bh + kv0, kNoScalars, kNoScalars, state, 0,
-                               stream)));
+                               stream, true, scratch)));
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       const dim3 agrid(pl.nblk_q, heads);
@@ -659,10 +694,12 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
       dv_q = mk_rows(dv_tmp, plain_str(nk, D));
     }
     // prefix state of (kh, v, 1) per key/value head and suffix state of (qh, go/den, c) per query head
+    // (scratch of a split build: behind everything else of the batch in the workspace)
+    float* scratch = reinterpret_cast<float*>(ws + pl.fixed_bytes + (size_t)hb * (batch_bytes_per_head(pl, saved != nullptr) - pl.scratch_bytes));
     if (!saved)
       FM_TRY((launch_build<D, T>(pl, heads / ratio, nk, kr, vr, scale + bh + kv0, kNoScalars, kNoScalars, state, 0,
-                                 stream)));
-    FM_TRY((launch_build<D, T>(pl, heads, nown_q, qr, gr, scale + h0, dn, cv, stR, 1, stream)));
+                                 stream, true, scratch)));
+    FM_TRY((launch_build<D, T>(pl, heads, nown_q, qr, gr, scale + h0, dn, cv, stR, 1, stream, true, scratch)));
     {
       ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
       const dim3 grid(pl.nblk_q, heads);

@@ -438,40 +438,6 @@ struct RawTileBf {
   }
 };
 
-// A run of `count` floats of a moment state staged global -> registers -> LDS.
-template <int MAXF>
-struct StateSlab {
-  static constexpr int NV = ((MAXF + 3) / 4 + 255) / 256;
-  float4 v[NV];
-
-  __device__ __forceinline__ void load(const float* src, int count, int tid) {
-    const int nvec = (count + 3) >> 2;
-#pragma unroll
-    for (int u = 0; u < NV; ++u) {
-      const int idx = tid + u * 256;
-      v[u] = idx < nvec ? *reinterpret_cast<const float4*>(src + idx * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-  }
-  // elements [0, split) are scaled by c_lo, the rest by c_hi
-  __device__ __forceinline__ void store(float* dst, int count, int split, float c_lo, float c_hi,
-                                        int tid) const {
-    const int nvec = (count + 3) >> 2;
-#pragma unroll
-    for (int u = 0; u < NV; ++u) {
-      const int idx = tid + u * 256;
-      if (idx < nvec) {
-        const int e0 = idx * 4;
-        float4 a = v[u];
-        a.x *= (e0 + 0 < split) ? c_lo : c_hi;
-        a.y *= (e0 + 1 < split) ? c_lo : c_hi;
-        a.z *= (e0 + 2 < split) ? c_lo : c_hi;
-        a.w *= (e0 + 3 < split) ? c_lo : c_hi;
-        *reinterpret_cast<float4*>(dst + e0) = a;
-      }
-    }
-  }
-};
-
 // sum over the 256 threads of a block; red is 4 floats of LDS; result valid in every thread
 __device__ __forceinline__ float block_sum_256(float v, float* red, int tid) {
 #pragma unroll

@@ -559,6 +559,37 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
+// Packs one slab of an fp32 state held in LDS (Sl: the D rows of a shift, or the order-1 rows
+// followed by the order-0 row) into the packed bf16 form (PackedGeo) at sb.  256 threads.
+// ---------------------------------------------------------------------------------------
+template <int D>
+__device__ __forceinline__ void pack_slab_from_lds(const float* Sl, char* sb, int slab, bool ord1, int p2, int tid) {
+  using G = Geo<D>;
+  using PG = PackedGeo<D>;
+  constexpr int LD = G::LD;
+  uint16_t* fsec = reinterpret_cast<uint16_t*>(sb) + slab * PG::FSL;
+  const float wgt = (!ord1 && slab != 0 && slab != G::H2) ? 2.0f : 1.0f;
+  for (int idx = tid; idx < (D / 4) * (D + 1); idx += 256) {
+    const int tg = idx / (D + 1), col = idx % (D + 1);
+    const float* f = Sl + 4 * tg * LD + col;
+    const float f0 = f[0] * wgt, f1 = f[LD] * wgt, f2 = f[2 * LD] * wgt, f3 = f[3 * LD] * wgt;
+    // rows 4 tg .. 4 tg + 3: half tg % 2 of the 16-byte word of row octet tg / 2 (a column further is
+    // two 8-byte pieces further)
+    uint2* dst = reinterpret_cast<uint2*>(fsec + ((tg >> 1) * PG::NCF + col) * 8 + (tg & 1) * 4);
+    if (col < D) {
+      *dst = make_uint2(pack_bf2(f0, f1), pack_bf2(f2, f3));
+    } else {   // the extra column, split into hi + lo parts: columns D..D+3 = (hi, hi, lo, lo)
+      const float h0 = bf_lo(pack_bf2(f0, 0.f)), h1 = bf_lo(pack_bf2(f1, 0.f));
+      const float h2 = bf_lo(pack_bf2(f2, 0.f)), h3 = bf_lo(pack_bf2(f3, 0.f));
+      const uint2 hi = make_uint2(pack_bf2(h0, h1), pack_bf2(h2, h3));
+      const uint2 lo = make_uint2(pack_bf2(f0 - h0, f1 - h1), pack_bf2(f2 - h2, f3 - h3));
+      dst[0] = hi; dst[2] = hi; dst[4] = lo; dst[6] = lo;
+    }
+  }
+  if (ord1 && tid <= D) reinterpret_cast<float*>(sb + PG::z_off(p2))[tid] = Sl[D * LD + tid];
+}
+
+// ---------------------------------------------------------------------------------------
 // bf16 inputs, unmasked: sums the nparts fp32 partial states of a head (slots 0..nparts-1)
 // and writes the packed bf16 form (PackedGeo) into the head's last slot, nslots-1.
 // grid = (slabs, heads), 256 threads.
@@ -584,24 +615,47 @@ __global__ __launch_bounds__(256) void state_pack_kernel(float* __restrict__ sta
   }
   __syncthreads();
   char* sb = reinterpret_cast<char*>(state + ((int64_t)head * nslots + nslots - 1) * SS);
-  uint16_t* fsec = reinterpret_cast<uint16_t*>(sb) + slab * PG::FSL;
-  const float wgt = (!ord1 && slab != 0 && slab != G::H2) ? 2.0f : 1.0f;
-  for (int idx = tid; idx < (D / 4) * (D + 1); idx += 256) {
-    const int tg = idx / (D + 1), col = idx % (D + 1);
-    const float* f = Sl + 4 * tg * LD + col;
-    const float f0 = f[0] * wgt, f1 = f[LD] * wgt, f2 = f[2 * LD] * wgt, f3 = f[3 * LD] * wgt;
-    // rows 4 tg .. 4 tg + 3: half tg % 2 of the 16-byte word of row octet tg / 2 (a column further is
-    // two 8-byte pieces further)
-    uint2* dst = reinterpret_cast<uint2*>(fsec + ((tg >> 1) * PG::NCF + col) * 8 + (tg & 1) * 4);
-    if (col < D) {
-      *dst = make_uint2(pack_bf2(f0, f1), pack_bf2(f2, f3));
-    } else {   // the extra column, split into hi + lo parts: columns D..D+3 = (hi, hi, lo, lo)
-      const float h0 = bf_lo(pack_bf2(f0, 0.f)), h1 = bf_lo(pack_bf2(f1, 0.f));
-      const float h2 = bf_lo(pack_bf2(f2, 0.f)), h3 = bf_lo(pack_bf2(f3, 0.f));
-      const uint2 hi = make_uint2(pack_bf2(h0, h1), pack_bf2(h2, h3));
-      const uint2 lo = make_uint2(pack_bf2(f0 - h0, f1 - h1), pack_bf2(f2 - h2, f3 - h3));
-      dst[0] = hi; dst[2] = hi; dst[4] = lo; dst[6] = lo;
-    }
+  pack_slab_from_lds<D>(Sl, sb, slab, ord1, p2, tid);
+}
+
+// ---------------------------------------------------------------------------------------
+// Causal states from per-chunk partial states (a head's chunks built side by side, for cases
+// with too few heads for one sequential walk per head to fill the chip).  part holds, per head,
+// nslots fp32 partial states (slot c = the state of chunk c alone).
+//   forward: slot c of the result = sum of the partial states of chunks < c
+//   reverse: slot c of the result = sum of the partial states of chunks > c
+// state_prefix_kernel works in place on fp32 slots (grid = (ceil(ss / 1024), heads), one
+// float4 per thread); state_pack_slots_kernel then writes every slot in the packed bf16 form
+// into `state` (grid = (slabs, heads, slots)).
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void state_prefix_kernel(float* __restrict__ state, int nslots, int64_t ss, int reverse) {
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= ss) return;
+  float* base = state + (int64_t)blockIdx.y * nslots * ss + idx;
+  float4 run = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int step = 0; step < nslots; ++step) {
+    const int c = reverse ? nslots - 1 - step : step;
+    float4* p = reinterpret_cast<float4*>(base + c * ss);
+    const float4 t = *p;
+    *p = run;
+    run.x += t.x; run.y += t.y; run.z += t.z; run.w += t.w;
   }
-  if (ord1 && tid <= D) reinterpret_cast<float*>(sb + PG::z_off(p2))[tid] = Sl[D * LD + tid];
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void state_pack_slots_kernel(const float* __restrict__ src_states, float* __restrict__ state,
+                                                               int nslots, int p2) {
+  using G = Geo<D>;
+  using PG = PackedGeo<D>;
+  constexpr int LD = G::LD;
+  __shared__ __attribute__((aligned(16))) float Sl[(D + 1) * LD];
+  const int slab = blockIdx.x, head = blockIdx.y, c = blockIdx.z, tid = threadIdx.x;
+  const int64_t SS = G::state_floats(p2), PS = PG::slot_floats(p2);
+  const bool ord1 = slab == PG::nslab(p2) - 1;  // the order-1 rows, followed by the order-0 row
+  const float* src = src_states + ((int64_t)head * nslots + c) * SS + (int64_t)slab * D * LD;
+  const int nf = (ord1 ? D + 1 : D) * LD;
+  for (int idx = tid * 4; idx < nf; idx += 1024)
+    *reinterpret_cast<float4*>(Sl + idx) = *reinterpret_cast<const float4*>(src + idx);
+  __syncthreads();
+  pack_slab_from_lds<D>(Sl, reinterpret_cast<char*>(state + ((int64_t)head * nslots + c) * PS), slab, ord1, p2, tid);
 }

@@ -172,7 +172,9 @@ int fastmax_backward_strided(const fastmax_desc* desc, const fastmax_layout* lay
  * hands it to fastmax_backward_saved, which then skips that build.  With saved_states == NULL
  * the two calls are fastmax_forward / fastmax_backward.  When a buffer is given the workspace
  * need not hold the prefix states: 16*bh + 512 bytes suffice for fastmax_forward_saving, and
- * fastmax_backward_saved needs one state per head less.  (Causal p = 1 at d = 64 with at
+ * fastmax_backward_saved needs one state per head less.  (The size query is the contract: for
+ * causal p = 1 with few heads and bf16 tensors the buffer also holds, behind the states, the
+ * fp32 per-chunk partial states the forward pass adds up.)  (Causal p = 1 at d = 64 with at
  * least 512 heads runs as one register-resident scan per head that keeps no state in memory:
  * there the size is a token 256 bytes, the buffer is left untouched and the workspace only
  * holds per-head and per-token scalars.) */
