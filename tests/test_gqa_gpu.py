@@ -67,3 +67,34 @@ def test_grouped_heads_module_4d(built):
     assert kd.grad.shape == k.shape
     assert_close("dk", kd.grad.reshape(b * hkv, n, d), rdk, 1e-4)
     assert_close("dv", vd.grad.reshape(b * hkv, n, d), rdv, 1e-4)
+
+
+@pytest.mark.parametrize("bh,bhkv,n,dtype,tol", [
+    (1024, 512, 700, torch.float32, 1e-4),    # >= 1024 build blocks: one sequential walk per head
+    (1024, 512, 700, torch.bfloat16, 2e-2),
+    (12, 6, 1500, torch.float32, 1e-4),       # few heads: the chunks of a head built side by side
+    (12, 6, 1500, torch.bfloat16, 2e-2),
+])
+def test_causal_p1_outside_the_scan_kernels(built, bh, bhkv, n, dtype, tol):
+    """Causal p = 1 with grouped heads never takes the scan kernels: the chunked kernels serve it, with
+    the states built by one walk per head (many heads) or from per-chunk partial states (few heads);
+    sampled groups against the oracle, and kept states give the same bits as rebuilt ones."""
+    from fastmax_amd import ops
+
+    d, ratio = 64, bh // bhkv
+    g = torch.Generator(device="cuda").manual_seed(7)
+    qd, god = (torch.randn((bh, n, d), device="cuda", generator=g).to(dtype) for _ in range(2))
+    kd, vd = (torch.randn((bhkv, n, d), device="cuda", generator=g).to(dtype) for _ in range(2))
+    kw = dict(mask=True, normalize=True, p=1)
+    o, den, sc, arg = ops.forward(qd, kd, vd, **kw)
+    dq, dk, dv = ops.backward(qd, kd, vd, o, den, god, qk_scale=sc, qk_argmax=arg, **kw)
+    o2, den2, sc2, arg2, saved = ops.forward(qd, kd, vd, save_states=True, **kw)
+    dq2, dk2, dv2 = ops.backward(qd, kd, vd, o2, den2, god, qk_scale=sc2, qk_argmax=arg2, saved_states=saved, **kw)
+    for a, b in ((o, o2), (dq, dq2), (dk, dk2), (dv, dv2)):
+        assert torch.equal(a, b)
+    for kv in sorted({0, bhkv // 2, bhkv - 1}):
+        hs = slice(kv * ratio, (kv + 1) * ratio)
+        ks = slice(kv, kv + 1)
+        ro, rdq, rdk, rdv = _truth(qd[hs].cpu(), kd[ks].cpu(), vd[ks].cpu(), god[hs].cpu(), ratio, **kw)
+        for name, got, ref in (("o", o[hs], ro), ("dq", dq[hs], rdq), ("dk", dk[ks], rdk), ("dv", dv[ks], rdv)):
+            assert_close(f"group{kv}/{name}", got, ref, tol)
