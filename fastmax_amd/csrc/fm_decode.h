@@ -62,26 +62,40 @@ __global__ __launch_bounds__(256) void decode_update_kernel(
     if (rr < RPI) {
       const float4 vx = *reinterpret_cast<const float4*>(vl + 4 * c4);
       float* sh = state + (int64_t)head * G::state_floats(p2);
-      for (int row = r_lo + rr; row < r_hi; row += RPI) {
-        float fk, fq;
-        if (row < rows2) {
-          const int s = row / D, a = row % D, b = (a + s) & (D - 1);
-          fk = kl[a] * kl[b];
-          fq = ((s == 0 || s == H2) ? a2 : 2.0f * a2) * ql[a] * ql[b];
-        } else if (row < rows2 + D) {
-          fk = kl[row - rows2];
-          fq = a1 * ql[row - rows2];
-        } else {
-          fk = 1.0f;
-          fq = a0;
+      // four rows per sweep: their loads are issued together (the kernel is bound by HBM latency x
+      // bytes in flight, and the compiler cannot move a load above the store of the row before)
+      constexpr int UB = 4;
+      for (int row0 = r_lo + rr; row0 < r_hi; row0 += UB * RPI) {
+        float4 s4[UB];
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+          const int row = row0 + u * RPI;
+          s4[u] = row < r_hi ? *reinterpret_cast<const float4*>(sh + (int64_t)row * LD + 4 * c4)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-        float4* sp = reinterpret_cast<float4*>(sh + (int64_t)row * LD + 4 * c4);
-        float4 s4 = *sp;
-        if (j == 0) {
-          s4.x += fk * vx.x; s4.y += fk * vx.y; s4.z += fk * vx.z; s4.w += fk * vx.w;
-          *sp = s4;
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+          const int row = row0 + u * RPI;
+          if (row >= r_hi) break;
+          float fk, fq;
+          if (row < rows2) {
+            const int s = row / D, a = row % D, b = (a + s) & (D - 1);
+            fk = kl[a] * kl[b];
+            fq = ((s == 0 || s == H2) ? a2 : 2.0f * a2) * ql[a] * ql[b];
+          } else if (row < rows2 + D) {
+            fk = kl[row - rows2];
+            fq = a1 * ql[row - rows2];
+          } else {
+            fk = 1.0f;
+            fq = a0;
+          }
+          float4 t = s4[u];
+          if (j == 0) {
+            t.x += fk * vx.x; t.y += fk * vx.y; t.z += fk * vx.z; t.w += fk * vx.w;
+            *reinterpret_cast<float4*>(sh + (int64_t)row * LD + 4 * c4) = t;
+          }
+          acc.x += fq * t.x; acc.y += fq * t.y; acc.z += fq * t.z; acc.w += fq * t.w;
         }
-        acc.x += fq * s4.x; acc.y += fq * s4.y; acc.z += fq * s4.z; acc.w += fq * s4.w;
       }
       red[rr][c4] = acc;
     }
