@@ -16,6 +16,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -42,20 +43,42 @@ WORKLOADS = {
 }
 COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 
-# HBM bytes per token-head moved by each kernel class, from the FETCH_SIZE / WRITE_SIZE counter
-# runs summarised under profiles/ (one file per workload, TRAFFIC_SOURCE)
-# (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch x2.0, write x1.0).
-MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD = {
-    "headline": {"build": 3708.0, "fwd_apply": 3597.0, "bwd_dq": 4440.0, "bwd_dk": 4569.0, "bwd_dv": 3877.0},
-    # profiles/config4_causal_bf16_all_kernels.txt
-    "c4": {"build": 1415.0, "fwd_apply": 1298.0, "bwd_dq": 1429.0, "bwd_dk": 1481.0, "bwd_dv": 1383.0},
-    # profiles/headline_p1_causal_fp32_scan_kernels.txt (algorithmic: 1024 B per token-head and kernel,
-    # 1280 B for dq, which also reads the forward output)
-    "headline-p1": {"fwd_apply": 1164.0, "bwd_dq": 1504.0, "bwd_dk": 1186.0, "bwd_dv": 1178.0},
-}
+# HBM bytes per token-head moved by each kernel class, from the FETCH_SIZE / WRITE_SIZE counter runs
+# summarised under profiles/ (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch
+# x2.0, write x1.0).  The summaries of the chunked kernels list the figure per kernel ("... B per
+# token-head"); it is read from the committed file at run time, so it changes with the profile and not
+# with an edit here.  The scan-kernel summary lists GiB per launch only: its figures are kept here
+# (algorithmic: 1024 B per token-head and kernel, 1280 B for dq, which also reads the forward output).
 TRAFFIC_SOURCE = {"headline": "profiles/headline_causal_fp32_all_kernels.txt",
                   "c4": "profiles/config4_causal_bf16_all_kernels.txt",
                   "headline-p1": "profiles/headline_p1_causal_fp32_scan_kernels.txt"}
+SCAN_TRAFFIC_BYTES_PER_TOKEN_HEAD = {"fwd_apply": 1164.0, "bwd_dq": 1504.0, "bwd_dk": 1186.0, "bwd_dv": 1178.0}
+_PROFILE_KERNEL_CLASS = (("build_kernel", None, "build"), ("apply_kernel", 0, "fwd_apply"), ("apply_kernel", 1, "bwd_dv"),
+                         ("grad_kernel", 0, "bwd_dq"), ("grad_kernel", 1, "bwd_dk"))
+
+
+def measured_traffic_bytes_per_token_head(workload: str) -> dict:
+    """{kernel class: HBM bytes per token-head (and state, for the build)} of a workload, or {}."""
+    if workload == "headline-p1":
+        return dict(SCAN_TRAFFIC_BYTES_PER_TOKEN_HEAD)
+    path = TRAFFIC_SOURCE.get(workload)
+    if path is None:
+        return {}
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), path)
+    if not os.path.exists(path):
+        return {}
+    out = {}
+    for line in open(path):
+        m = re.match(r"\s+(\w+)<(.*)>\s+\d+ launches\s+[\d.]+ GB\s+([\d.]+) B per token-head", line)
+        if not m:
+            continue
+        name, targs, val = m.group(1).replace("_bf", ""), m.group(2), float(m.group(3))
+        last = targs.split(",")[-1].strip()
+        mode = int(last) if name in ("apply_kernel", "grad_kernel") and last.isdigit() else None
+        for kname, kmode, cls in _PROFILE_KERNEL_CLASS:
+            if name == kname and mode == kmode:
+                out[cls] = val
+    return out
 
 
 def algorithmic_flops(d: int, p: int) -> dict:
@@ -410,7 +433,7 @@ def main() -> int:
         roofline = {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": gbs / PEAK_HBM_GBS, "traffic": None, "bytes_per_launch": bytes_per_launch,
                     "avg_launch_ms": dom_ms / launches}
-    per_th = MEASURED_TRAFFIC_BYTES_PER_TOKEN_HEAD.get(args.workload if not args.batch else "", {}).get(dom)
+    per_th = measured_traffic_bytes_per_token_head(args.workload if not args.batch else "").get(dom)
     if per_th is not None:
         n_states = n_builds if dom == "build" else 1
         roofline["traffic"] = per_th * token_heads * n_states / launches  # bytes per launch (profiled, not live)

@@ -52,3 +52,15 @@ def test_executed_flops_model():
     # bf16 forward carries the denominator in a third accumulator tile
     cb = dict(cfg, dtype="bf16")
     assert bench.executed_mfma_flops(cb, 4)["fwd_apply"] == 2 * 34 * 64 * 96 * th
+
+
+def test_traffic_figures_are_read_from_the_committed_profiles():
+    """roofline.traffic is priced with the HBM bytes per token-head that the rocprofv3 summaries under
+    profiles/ list for each kernel class; the summaries of both chunked workloads parse."""
+    import bench
+
+    for workload in ("headline", "c4"):
+        t = bench.measured_traffic_bytes_per_token_head(workload)
+        assert set(t) == {"build", "fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv"}, (workload, t)
+        assert all(500.0 < v < 20000.0 for v in t.values()), (workload, t)
+    assert bench.measured_traffic_bytes_per_token_head("c2") == {}
