@@ -363,10 +363,11 @@ int compute_scales(const fastmax_desc* ds, const Layout& L, const T* q, const T*
   ScopedKernel sk(FASTMAX_K_ROWSTAT, stream);
   if (ds->normalize) {
     const Rows<const T> qr = mk_rows(q, L.q), kr = mk_rows(k, L.k);
-    if (bh >= 512) rowstat_kernel<T, 256><<<bh, 256, 0, stream>>>(qr, ds->nq, ds->d, ds->lim, scale, arg);
-    else rowstat_kernel<T, 1024><<<bh, 1024, 0, stream>>>(qr, ds->nq, ds->d, ds->lim, scale, arg);
-    if (bhkv >= 512) rowstat_kernel<T, 256><<<bhkv, 256, 0, stream>>>(kr, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
-    else rowstat_kernel<T, 1024><<<bhkv, 1024, 0, stream>>>(kr, ds->nk, ds->d, ds->lim, scale + bh, arg + bh);
+    // (q and k in one launch; with few heads a block is 1024 threads so that the chip still fills)
+    if (bh + bhkv >= 1024)
+      rowstat_kernel<T, 256><<<bh + bhkv, 256, 0, stream>>>(qr, ds->nq, bh, kr, ds->nk, ds->d, ds->lim, scale, arg);
+    else
+      rowstat_kernel<T, 1024><<<bh + bhkv, 1024, 0, stream>>>(qr, ds->nq, bh, kr, ds->nk, ds->d, ds->lim, scale, arg);
   } else {
     fill_scale_kernel<<<(bh + 255) / 256, 256, 0, stream>>>(scale, arg, bh, 1.0f);
     fill_scale_kernel<<<(bhkv + 255) / 256, 256, 0, stream>>>(scale + bh, arg + bh, bhkv, 1.0f / ds->temperature);

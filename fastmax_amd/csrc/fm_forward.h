@@ -34,9 +34,11 @@ struct RowPiece<bf16_t> {
   }
 };
 
+// One launch serves two tensors (q and k): blocks 0 .. nh1-1 take the heads of x1 (n1 rows each),
+// the blocks after them the heads of x2 (n2 rows each); results go to index blockIdx.x.
 template <class T, int NT>
-__global__ __launch_bounds__(NT) void rowstat_kernel(Rows<const T> x, int n, int d,
-                                                     float lim, float* __restrict__ scale_out,
+__global__ __launch_bounds__(NT) void rowstat_kernel(Rows<const T> x1, int n1, int nh1, Rows<const T> x2, int n2,
+                                                     int d, float lim, float* __restrict__ scale_out,
                                                      int* __restrict__ arg_out) {
   __shared__ float sbest[NT];
   __shared__ int sarg[NT];
@@ -44,7 +46,10 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(Rows<const T> x, int n, int
   const int tid = threadIdx.x;
   const int tpr = d / EPT, rpp = NT / tpr;
   const int sub = tid % tpr, rowi = tid / tpr;
-  const HeadRows<const T> xh = x.head(blockIdx.x);   // rows 0 .. n-1 of the tensor itself (lo is not used)
+  const bool second = (int)blockIdx.x >= nh1;
+  const int n = second ? n2 : n1;
+  // rows 0 .. n-1 of the tensor itself (lo is not used)
+  const HeadRows<const T> xh = second ? x2.head(blockIdx.x - nh1) : x1.head(blockIdx.x);
   const T* base = xh.base;
   const unsigned pitch = xh.pitch;
   // A NaN row norm wins over every number (the maximum of the reference's path propagates NaN,
