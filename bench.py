@@ -123,7 +123,10 @@ def executed_mfma_flops(cfg: dict, bh: int, chunk: int = 0) -> dict:
     rtw = 3 if d == 64 else 5
     gsplit = -(-rt_total // (4 * rtw))
     ts = 64 if d == 64 else 32                  # tokens per step of the p = 2 build kernel
-    per_step = gsplit * 4 * rtw * cb * ksteps(ts) * per
+    slots = gsplit * 4 * rtw                     # row-tile slots of a head's blocks (rt_total of them hold a tile)
+    if d == 64 and not bf:
+        slots -= 1.5                            # the idle wave of the last block forms the Gram tiles: 3 instead of 6
+    per_step = slots * cb * ksteps(ts) * per
     nc = -(-n // chunk)
     spc = chunk // ts
     if masked:

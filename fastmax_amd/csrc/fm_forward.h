@@ -210,6 +210,14 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       }
     }
   }
+  // fp32, D = 64, p = 2: the feature list ends inside the last block of a head and leaves one wave
+  // of it without a row tile.  That wave forms the state's extra column for the whole head instead:
+  // the extra column of row (s, a) is sum_t e_t x_a x_(a+s) = G[a][(a+s) % D] with the Gram matrix
+  // G = sum_t e_t x_t x_t^T (three 32 x 32 tiles by symmetry, 12 matrix instructions per 8 tokens),
+  // and that of the order-1 row a is K1[a] = sum_t e_t x_a.  The other waves then spend no VALU
+  // work on the extra column (it was four FMAs per row tile and four tokens).
+  constexpr bool GT = D == 64 && RTW == 3 && !BF;
+  const bool gwave = GT && nx == 0;   // (RTW == 3 is the p = 2 configuration)
   const int cbase = CSPLIT ? w >> 1 : 0;  // first column tile of this wave
   int voff[CB];
 #pragma unroll
@@ -318,7 +326,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
             acc[x][cb] = FM_MFMA(a3, cur.vv[cb].w, acc[x][cb]);
           }
         }
-        if constexpr (!BF) {
+        if constexpr (!BF && !GT) {
           dacc[x] += a0 * cur.e4.x + a1 * cur.e4.y + a2 * cur.e4.z + a3 * cur.e4.w;
         }
       }
@@ -329,6 +337,38 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
         }
       }
       if (gq + 1 < 4) cur = nxt;
+    }
+  };
+  // the Gram wave's share of a half step: G tiles (0,0), (0,1), (1,1) in acc[0][0], acc[0][1],
+  // acc[1][0] (rows = channel a, columns = channel b), K1 of channel blocks 0, 1 in dacc[0], dacc[1]
+  auto compute_gram = [&](int buf, int h) __attribute__((always_inline)) {
+    if constexpr (GT) {
+      const float* kb = Kt[buf];
+      const float* eb = El[buf];
+      const int r0 = i * TP + 4 * hh, r1 = (32 + i) * TP + 4 * hh;
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        const int go8 = 8 * (4 * h + gq);
+        const float4 x0 = *reinterpret_cast<const float4*>(kb + r0 + go8);
+        const float4 x1 = *reinterpret_cast<const float4*>(kb + r1 + go8);
+        const float4 e4 = *reinterpret_cast<const float4*>(eb + go8 + 4 * hh);
+        const float4 y0 = make_float4(x0.x * e4.x, x0.y * e4.y, x0.z * e4.z, x0.w * e4.w);
+        const float4 y1 = make_float4(x1.x * e4.x, x1.y * e4.y, x1.z * e4.z, x1.w * e4.w);
+        acc[0][0] = FM_MFMA(x0.x, y0.x, acc[0][0]);
+        acc[0][1] = FM_MFMA(x0.x, y1.x, acc[0][1]);
+        acc[1][0] = FM_MFMA(x1.x, y1.x, acc[1][0]);
+        acc[0][0] = FM_MFMA(x0.y, y0.y, acc[0][0]);
+        acc[0][1] = FM_MFMA(x0.y, y1.y, acc[0][1]);
+        acc[1][0] = FM_MFMA(x1.y, y1.y, acc[1][0]);
+        acc[0][0] = FM_MFMA(x0.z, y0.z, acc[0][0]);
+        acc[0][1] = FM_MFMA(x0.z, y1.z, acc[0][1]);
+        acc[1][0] = FM_MFMA(x1.z, y1.z, acc[1][0]);
+        acc[0][0] = FM_MFMA(x0.w, y0.w, acc[0][0]);
+        acc[0][1] = FM_MFMA(x0.w, y1.w, acc[0][1]);
+        acc[1][0] = FM_MFMA(x1.w, y1.w, acc[1][0]);
+        dacc[0] += (y0.x + y0.y) + (y0.z + y0.w);
+        dacc[1] += (y1.x + y1.y) + (y1.z + y1.w);
+      }
     }
   };
   // order-0 sums of the staged step
@@ -354,7 +394,8 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   };
   // lane part of a snapshot address: row 4*hh (+ 8j + e per register), column i (+ 32*cb)
   const unsigned lane_off = (unsigned)(4 * hh * LD + cbase * 32 + i);
-  auto snapshot = [&](int slot) __attribute__((always_inline)) {
+  auto snapshot = [&](int slot, auto gtag) __attribute__((always_inline)) {
+    constexpr bool GW = decltype(gtag)::value;   // the Gram wave's own copy of the scan (see below)
     float* st = state + ((int64_t)head * nslots + slot) * SS;  // uniform: scalar base + 32-bit lane offsets
 #pragma unroll
     for (int x = 0; x < RTW; ++x) {
@@ -368,8 +409,43 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) sx[oj + (unsigned)(e * LD + cb * 32)] = acc[x][cb][4 * j + e];
         }
-        const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
-        if (hh == 0 && cbase == 0) sx[(unsigned)(i * LD + D)] = ds;
+        if constexpr (!GT) {
+          const float ds = dacc[x] + __shfl_xor(dacc[x], 32, 64);
+          if (hh == 0 && cbase == 0) sx[(unsigned)(i * LD + D)] = ds;
+        }
+      }
+    }
+    if constexpr (GW) {
+      {
+        // the extra column of the whole head from the Gram tiles: element (a, b) belongs to row
+        // (s, a) with s = (b - a) mod D when s <= D/2, else to row (D - s, b); a diagonal tile holds
+        // every pair twice (the copies with s > D/2 are dropped), and s = D/2 lists every pair from
+        // both sides (rows (D/2, a) and (D/2, b))
+        // (the lane's coordinates pass through an empty volatile statement: the 64 store offsets are
+        // then formed here, not once before the scan loop, where they would occupy 64 registers)
+        int li = i, lh = hh;
+        asm volatile("" : "+v"(li), "+v"(lh));
+        auto put = [&](const f16v& gacc, int ra, int cb) __attribute__((always_inline)) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int a = ra * 32 + trow(r, lh), b = cb * 32 + li, sft = (b - a) & (D - 1);
+            if (sft <= G::H2) {
+              st[(unsigned)((sft * D + a) * LD + D)] = gacc[r];
+              if (sft == G::H2) st[(unsigned)((sft * D + b) * LD + D)] = gacc[r];
+            } else if (ra != cb) {
+              st[(unsigned)(((D - sft) * D + b) * LD + D)] = gacc[r];
+            }
+            if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);   // (a few stores at a time: register pressure)
+          }
+        };
+        put(acc[0][0], 0, 0);
+        put(acc[0][1], 0, 1);
+        put(acc[1][0], 1, 1);
+        const float k0 = dacc[0] + __shfl_xor(dacc[0], 32, 64), k1 = dacc[1] + __shfl_xor(dacc[1], 32, 64);
+        if (lh == 0) {
+          st[(unsigned)((rows2 + li) * LD + D)] = k0;
+          st[(unsigned)((rows2 + 32 + li) * LD + D)] = k1;
+        }
       }
     }
     if (g == 0 && tid <= D) st[(unsigned)((rows2 + D) * LD + tid)] = s0;
@@ -411,14 +487,14 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
     }
     if (g == 0 && tid <= D) reinterpret_cast<float*>(sb + PG::z_off(p2))[tid] = s0;
   };
-  auto emit = [&](int slot) __attribute__((always_inline)) {
+  auto emit = [&](int slot, auto gtag) __attribute__((always_inline)) {
     if constexpr (BF) {
       if (masked) {
         snapshot_packed(slot);
         return;
       }
     }
-    snapshot(slot);
+    snapshot(slot, gtag);
   };
 
   // The walk is one software pipeline over all 32-token steps: the loads of step p+1 are issued
@@ -510,7 +586,7 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       sum0(p & 1);
       if (p + 1 < nsteps) store_from(sk, sv, se, (p + 1) & 1, step_tok(p + 1));
       const int slot = step_slot(p);
-      if (slot >= 0) emit(slot);
+      if (slot >= 0) emit(slot, std::false_type{});
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -529,7 +605,19 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       // (the set is requested at the start of a step and staged at its end)
       for (int p = 0; p < nsteps; ++p) step(p, kxa, vya, era, kxa, vya, era);
     }
-  } else {
+  }
+  // The scan itself, in two copies where a head has a Gram wave (GW: that wave's copy; the copies
+  // differ in the compute and snapshot calls only, and as separate loops they do not add their
+  // register needs).  Every wave of the block stages tiles and meets the barriers alike.
+  auto tail = [&](auto gtag) __attribute__((always_inline)) {
+    if (!masked && nsteps == 0) emit(zsplit, gtag);  // an empty token split still owns its slot
+    if (masked && reverse && nsteps > 0) {
+      // chunks below the one that holds position lo see the same suffix state
+      for (int slot = lo / chunk - 2; slot >= 0; --slot) emit(slot, gtag);
+    }
+  };
+  auto scan = [&](auto gtag) __attribute__((always_inline)) {
+    constexpr bool GW = decltype(gtag)::value;
     if (nsteps > 0) {
   #pragma unroll
       for (int h = 0; h < NH; ++h) {
@@ -544,7 +632,8 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
   #pragma unroll 1
       for (int h = 0; h < NH; ++h) {
         if (more) load(tnext + 32 * h, tend);
-        compute(p & 1, h);
+        if constexpr (GW) compute_gram(p & 1, h);
+        else compute(p & 1, h);
         if (h == NH - 1) sum0(p & 1);
         if (more) store((p + 1) & 1, h, tnext + 32 * h, tend);
         if constexpr (NH > 1) __builtin_amdgcn_sched_barrier(0);   // (keeps the halves apart: register pressure)
@@ -552,14 +641,18 @@ __global__ __launch_bounds__(256, 2) void build_kernel(
       // after the staged tile has been consumed: waiting for loads while stores are pending
       // would wait for the stores too (one in-order counter covers both)
       const int slot = step_slot(p);
-      if (slot >= 0) emit(slot);
+      if (slot >= 0) emit(slot, gtag);
       __syncthreads();
     }
-  }
-  if (!masked && nsteps == 0) emit(zsplit);  // an empty token split still owns its slot
-  if (masked && reverse && nsteps > 0) {
-    // chunks below the one that holds position lo see the same suffix state
-    for (int slot = lo / chunk - 2; slot >= 0; --slot) emit(slot);
+    tail(gtag);
+  };
+  if constexpr (BF) {
+    tail(std::false_type{});
+  } else if constexpr (GT) {
+    if (gwave) scan(std::true_type{});
+    else scan(std::false_type{});
+  } else {
+    scan(std::false_type{});
   }
 }
 
