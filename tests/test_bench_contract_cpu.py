@@ -29,16 +29,19 @@ def test_algorithmic_flops_closed_forms():
 
 
 def test_executed_flops_model():
-    """The executed count is pinned where it has a closed form: the d = 64 state build issues 72 row-tile
-    slots x 32 rows x 64 columns MACs per token, an unmasked consumer runs 34 slabs of 64 rows over 64
-    (+1 for the gradients' extra) columns, and everything stays below the reference-form count."""
+    """The executed count is pinned where it has a closed form: the d = 64 fp32 state build issues 70.5
+    row-tile slots x 32 rows x 64 columns MACs per token (69 tile slots of its 23 tile waves, and the
+    three Gram tiles of the remaining wave, half a slot's worth each; bf16: 72 slots), an unmasked
+    consumer runs 34 slabs of 64 rows over 64 (+1 for the gradients' extra) columns, and everything
+    stays below the reference-form count."""
     sys.path.insert(0, ROOT)
     import bench
 
     cfg = dict(B=1, H=4, N=384 * 5, D=64, mask=False, p=2, dtype="f32")
     ex = bench.executed_mfma_flops(cfg, 4)
     th = 4 * cfg["N"]
-    assert ex["build_fwd"] == 2 * 72 * 32 * 64 * th
+    assert ex["build_fwd"] == 2 * 70.5 * 32 * 64 * th
+    assert bench.executed_mfma_flops(dict(cfg, dtype="bf16"), 4)["build_fwd"] == 2 * 72 * 32 * 64 * th
     assert ex["fwd_apply"] == ex["bwd_dv"] == 2 * 34 * 64 * 64 * th
     assert ex["bwd_dq"] == ex["bwd_dk"] == 2 * 34 * 64 * 66 * th
     al = bench.algorithmic_flops(64, 2)
