@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <mutex>
@@ -14,6 +15,7 @@
 #include "fm_apply.h"
 #include "fm_backward.h"
 #include "fm_decode.h"
+#include "fm_dense.h"
 #include "fm_forward.h"
 #include "fm_grad.h"
 #include "fm_linear.h"
@@ -100,6 +102,8 @@ struct Plan {
   bool plain;          // every tensor is a plain contiguous (heads, tokens, d) array
   bool scan;           // causal p = 1 as one scan per head (fm_linear.h): no states in memory
   bool rowpass;        // unmasked p = 1: states from the build kernel, one pass over the rows per output
+  bool dense;          // dense score tiles, no moment states (fm_dense.h): short sequences, and every head
+                       // dimension other than 32 and 64
   bool split;          // causal p = 1 with few heads: the chunks of a head are built side by side as partial
                        // states and a prefix pass over the chunks makes the causal states of them
   size_t scratch_bytes;   // per head: where the fp32 partial states of a split build go when the
@@ -130,9 +134,29 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 #endif
 bool use_linear_scan(const fastmax_desc* ds, const Plan& pl);
 
-Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true) {
+// Dense score tiles cost 2 n d flop per token under the mask (4 n d without it), the moment form about
+// 2.1 d^3 (p = 2) whatever n is: below these key counts the dense kernels are the faster ones (measured,
+// forward + backward).  Head dimensions without moment kernels always take them.
+bool use_dense(const fastmax_desc* ds) {
+  if (ds->d != 32 && ds->d != 64) return true;
+  // FASTMAX_PATH = moments | dense overrides the choice where both kernel families exist
+  if (const char* e = getenv("FASTMAX_PATH")) {
+    if (!strcmp(e, "moments")) return false;
+    if (!strcmp(e, "dense")) return true;
+  }
+  if (ds->p != 2) return false;
+  const bool bf = ds->dtype == FASTMAX_BF16;
+  int limit;
+  if (ds->d == 64) limit = bf ? 4096 : 2048;
+  else limit = bf ? 1024 : 512;
+  if (!ds->mask) limit /= 2;
+  return ds->nk <= limit;
+}
+
+Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true, bool allow_dense = true) {
   Plan pl;
   pl.pass = pass;
+  pl.dense = allow_dense && use_dense(ds);
   pl.d = ds->d;
   pl.p2 = ds->p == 2;
   pl.masked = ds->mask != 0;
@@ -146,6 +170,21 @@ Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true) {
   pl.bh = ds->bh;
   pl.bhkv = ds->bhkv;
   pl.ratio = ds->bh / ds->bhkv;
+  if (pl.dense) {
+    // no states: the workspace holds the per-head scalars only (and c_i, normalisation partials)
+    pl.rtw = pl.gsplit = pl.nslots = pl.nparts = 1;
+    pl.zlen = pl.chunk = 0;
+    pl.scan = pl.rowpass = pl.split = false;
+    pl.scratch_bytes = pl.per_head_bytes = 0;
+    pl.state_floats = 0;
+    size_t fx = align256((size_t)2 * pl.bh * sizeof(float)) + align256((size_t)2 * pl.bh * sizeof(int));
+    if (pass == FASTMAX_PASS_BACKWARD) {
+      fx += align256((size_t)pl.bh * pl.nq * sizeof(float));
+      fx += align256((size_t)pl.bh * (pl.nblk_q + pl.nblk_k) * sizeof(float));
+    }
+    pl.fixed_bytes = fx;
+    return pl;
+  }
   const int rt_total = (pl.p2 ? (pl.d / 2 + 1) * (pl.d / 32) : 0) + pl.d / 32;
   // (p = 1, d = 64: the four waves of a block share its two row tiles, one column tile each)
   auto splits = [&](int rtw) { return !pl.p2 && pl.d == 64 ? 1 : (rt_total + 4 * rtw - 1) / (4 * rtw); };
@@ -240,7 +279,13 @@ int check_desc(const fastmax_desc* ds) {
   if (!ds) return fail(FASTMAX_E_NULL, "desc is NULL");
   if (ds->dtype != FASTMAX_F32 && ds->dtype != FASTMAX_BF16)
     return fail(FASTMAX_E_DTYPE, "dtype %d is neither FASTMAX_F32 nor FASTMAX_BF16", ds->dtype);
-  if (ds->d != 32 && ds->d != 64) return fail(FASTMAX_E_SHAPE, "d = %d; supported head dims are 32 and 64", ds->d);
+  {
+    // rows are read in 16-byte pieces; the dense kernels hold a head dimension of up to 128 in registers
+    const int step = ds->dtype == FASTMAX_BF16 ? 8 : 4;
+    if (ds->d < step || ds->d > 128 || ds->d % step)
+      return fail(FASTMAX_E_SHAPE, "d = %d; the head dimension must be a multiple of %d (16 bytes of %s) in [%d, 128]",
+                  ds->d, step, ds->dtype == FASTMAX_BF16 ? "bf16" : "fp32", step);
+  }
   if (ds->bh < 1 || ds->bh > 65535) return fail(FASTMAX_E_SHAPE, "bh = %d outside [1, 65535]", ds->bh);
   if (ds->bhkv < 1 || ds->bh % ds->bhkv != 0)
     return fail(FASTMAX_E_SHAPE, "bhkv = %d does not divide bh = %d", ds->bhkv, ds->bh);
@@ -269,7 +314,7 @@ int check_ws(const Plan& pl, void* ws, size_t ws_bytes, bool with_saved = false)
 }
 
 size_t saved_bytes_for(const Plan& pl) {
-  if (pl.scan) return 256;   // nothing to keep; a token size, so that 0 still means "bad descriptor"
+  if (pl.scan || pl.dense) return 256;   // nothing to keep; a token size, so that 0 still means "bad descriptor"
   // (a split build of packed states sums fp32 partial states: room for them behind the states)
   return (size_t)pl.bhkv * (pl.nslots * pl.state_floats * sizeof(float) + pl.scratch_bytes);
 }
@@ -527,19 +572,20 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const 
 }
 
 // c_i = go_i . o_i / den_i for every query row: 16-byte accesses when the rows of o allow it
-template <int D, class T>
+template <class T>
 int launch_bwd_prep(const Plan& pl, const Layout& L, const T* go, const T* o, const float* den, int64_t den_stride,
                     float* cvec, hipStream_t stream) {
   ScopedKernel sk(FASTMAX_K_BWD_PREP, stream);
   const bool vec = aligned16(L.o, sizeof(T)) && aligned16(o) && aligned16(L.go, sizeof(T)) && aligned16(go);
   const Rows<const T> gr = mk_rows(go, L.go), orow = mk_rows(o, L.o);
   const RowScalars dn = mk_scalars(den, pl.nq, den_stride);
+  auto pow2 = [](int x) { int t = 1; while (t < x) t *= 2; return t; };
   if (vec) {
-    const int rpp = 256 / (D * (int)sizeof(T) / 16);
-    bwd_prep_kernel<T, true><<<dim3((pl.nq + rpp - 1) / rpp, pl.bh), 256, 0, stream>>>(gr, orow, dn, cvec, pl.nq, D);
+    const int rpp = 256 / pow2(pl.d * (int)sizeof(T) / 16);
+    bwd_prep_kernel<T, true><<<dim3((pl.nq + rpp - 1) / rpp, pl.bh), 256, 0, stream>>>(gr, orow, dn, cvec, pl.nq, pl.d);
   } else {
-    const int rpp = 256 / (D / 4);
-    bwd_prep_kernel<T, false><<<dim3((pl.nq + rpp - 1) / rpp, pl.bh), 256, 0, stream>>>(gr, orow, dn, cvec, pl.nq, D);
+    const int rpp = 256 / pow2(pl.d / 4);
+    bwd_prep_kernel<T, false><<<dim3((pl.nq + rpp - 1) / rpp, pl.bh), 256, 0, stream>>>(gr, orow, dn, cvec, pl.nq, pl.d);
   }
   return launch_status("bwd_prep_kernel");
 }
@@ -579,7 +625,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
       // separate pass does
       const bool prep_in_dq = ldo == D;
       if (!prep_in_dq) {
-        FM_TRY((launch_bwd_prep<D, T>(pl, L, go, o, den, den_stride, cvec, stream)));
+        FM_TRY((launch_bwd_prep<T>(pl, L, go, o, den, den_stride, cvec, stream)));
       }
       {
         ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
@@ -614,7 +660,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
     }
   }
   {
-    FM_TRY((launch_bwd_prep<D, T>(pl, L, go, o, den, den_stride, cvec, stream)));
+    FM_TRY((launch_bwd_prep<T>(pl, L, go, o, den, den_stride, cvec, stream)));
   }
   const float a2 = pl.p2 ? ds->a2 : 0.f;
   const int ratio = pl.ratio, bhkv = pl.bhkv;
@@ -763,6 +809,126 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
     norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, pl.nblk_q, nq, D, ds->lim);
     norm_fix_kernel<T><<<bhkv, D, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh, rpart_k,
                                                pl.nblk_k * ratio, nk, D, ds->lim);
+    FM_TRY(launch_status("norm_fix_kernel"));
+  }
+  return FASTMAX_OK;
+}
+
+// ---- dense score-tile path (fm_dense.h) ---------------------------------------------------------
+// Blocks that need more than the 64 KB of LDS a kernel gets by default ask for it by attribute.
+int allow_lds(const void* kernel, size_t bytes) {
+  if (bytes <= (size_t)64 * 1024) return FASTMAX_OK;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) return fail(FASTMAX_E_LAUNCH, "hipFuncSetAttribute(%zu bytes of LDS): %s", bytes, hipGetErrorString(e));
+  return FASTMAX_OK;
+}
+
+template <int DP, class T>
+int dense_forward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v, T* o,
+                     float* den, int64_t den_stride, const float* scale, hipStream_t stream) {
+  using S = dense::Shape<DP, T>;
+  constexpr int RT = S::RT_FWD, BN = S::BN, BM = 128 * RT;
+  const size_t smem = dense::Lds<DP, T, BN>::bytes(1, 1, BM);
+  auto kern = dense::dense_fwd_kernel<DP, T, RT, BN>;
+  FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
+  const int npos = pl.masked ? pl.nk : pl.nq;
+  const int nb = (npos + BM - 1) / BM - pl.off / BM;
+  ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
+  kern<<<dim3(pl.bh, nb), 256, smem, stream>>>(mk_rows(q, L.q, 0, pl.off), mk_rows(k, L.k), mk_rows(v, L.v), scale,
+                                               scale + pl.bh, mk_rows(o, L.o, 0, pl.off),
+                                               mk_scalars(den, pl.nq, den_stride, 0, pl.off), npos, pl.nk, ds->d,
+                                               pl.masked, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f, pl.ratio);
+  return launch_status("dense_fwd_kernel");
+}
+
+template <class T>
+int dense_forward(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v, T* o,
+                  float* den, int64_t den_stride, float* scale_out, int32_t* arg_out, char* ws, hipStream_t stream) {
+  float* scale = scale_out ? scale_out : reinterpret_cast<float*>(ws);
+  int* arg = arg_out ? arg_out : reinterpret_cast<int*>(ws + align256((size_t)2 * pl.bh * sizeof(float)));
+  FM_TRY(compute_scales<T>(ds, L, q, k, scale, arg, stream));
+#define FM_DENSE_FWD(DP) return dense_forward_dp<DP, T>(ds, pl, L, q, k, v, o, den, den_stride, scale, stream)
+  if (ds->d <= 32) FM_DENSE_FWD(32);
+  if (ds->d <= 64) FM_DENSE_FWD(64);
+  if (ds->d <= 96) FM_DENSE_FWD(96);
+  FM_DENSE_FWD(128);
+#undef FM_DENSE_FWD
+}
+
+template <int DP, class T>
+int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v,
+                      const float* den, int64_t den_stride, const T* go, T* dq, T* dk, T* dv, const float* scale,
+                      const float* cvec, float* rpart, int* nbq_out, int* nbk_out, hipStream_t stream) {
+  using S = dense::Shape<DP, T>;
+  constexpr int BN = S::BN;
+  const int npos = pl.masked ? pl.nk : pl.nq;
+  const float a2 = pl.p2 ? ds->a2 : 0.f;
+  float* rq = ds->normalize ? rpart : nullptr;
+  const RowScalars dn = mk_scalars(den, pl.nq, den_stride, 0, pl.off);
+  const RowScalars cv = mk_scalars<const float>(cvec, pl.nq, 1, 0, pl.off);
+  const Rows<const T> qr = mk_rows(q, L.q, 0, pl.off), gr = mk_rows(go, L.go, 0, pl.off);
+  const Rows<const T> kr = mk_rows(k, L.k), vr = mk_rows(v, L.v);
+  {
+    constexpr int RT = S::RT_DQ, BM = 128 * RT;
+    const size_t smem = dense::Lds<DP, T, BN>::bytes(2, 1, 4);
+    auto kern = dense::dense_dq_kernel<DP, T, RT, BN>;
+    FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
+    const int nb = (npos + BM - 1) / BM - pl.off / BM;
+    *nbq_out = nb;
+    ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
+    kern<<<dim3(pl.bh, nb), 256, smem, stream>>>(qr, gr, dn, cv, kr, vr, scale, scale + pl.bh, mk_rows(dq, L.dq, 0, pl.off), rq,
+                                                 npos, pl.nk, ds->d, pl.masked, pl.p2 && a2 != 0.f, ds->a1, a2, pl.ratio);
+    FM_TRY(launch_status("dense_dq_kernel"));
+  }
+  {
+    constexpr int RT = S::RT_KV, BM = 128 * RT;
+    const size_t smem = dense::Lds<DP, T, BN>::bytes(2, 2, 2 * BN + 4);
+    auto kern = dense::dense_dkdv_kernel<DP, T, RT, BN>;
+    FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
+    const int nb = (pl.nk + BM - 1) / BM;
+    *nbk_out = nb;
+    float* rk = ds->normalize ? rpart + (int64_t)pl.bh * (*nbq_out) : nullptr;
+    ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
+    kern<<<dim3(pl.bhkv, nb), 256, smem, stream>>>(kr, vr, qr, gr, dn, cv, scale, scale + pl.bh, mk_rows(dk, L.dk),
+                                                   mk_rows(dv, L.dv), rk, npos, pl.nk, ds->d, pl.masked, ds->a0, ds->a1,
+                                                   a2, pl.ratio);
+    FM_TRY(launch_status("dense_dkdv_kernel"));
+  }
+  return FASTMAX_OK;
+}
+
+template <class T>
+int dense_backward(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v,
+                   const T* o, const float* den, int64_t den_stride, const T* go, T* dq, T* dk, T* dv,
+                   const float* scale_in, const int32_t* arg_in, char* ws, hipStream_t stream) {
+  const int bh = pl.bh;
+  char* p = ws;
+  const bool given = scale_in && arg_in;
+  const float* scale = given ? scale_in : reinterpret_cast<float*>(p);
+  float* scale_ws = reinterpret_cast<float*>(p);
+  p += align256((size_t)2 * bh * sizeof(float));
+  const int* arg = given ? arg_in : reinterpret_cast<int*>(p);
+  int* arg_ws = reinterpret_cast<int*>(p);
+  p += align256((size_t)2 * bh * sizeof(int));
+  float* cvec = reinterpret_cast<float*>(p);
+  p += align256((size_t)bh * pl.nq * sizeof(float));
+  float* rpart = reinterpret_cast<float*>(p);
+  if (!given) FM_TRY(compute_scales<T>(ds, L, q, k, scale_ws, arg_ws, stream));
+  FM_TRY((launch_bwd_prep<T>(pl, L, go, o, den, den_stride, cvec, stream)));
+  int nbq = 0, nbk = 0;
+#define FM_DENSE_BWD(DP)                                                                                          \
+  FM_TRY((dense_backward_dp<DP, T>(ds, pl, L, q, k, v, den, den_stride, go, dq, dk, dv, scale, cvec, rpart, &nbq, \
+                                   &nbk, stream)))
+  if (ds->d <= 32) FM_DENSE_BWD(32);
+  else if (ds->d <= 64) FM_DENSE_BWD(64);
+  else if (ds->d <= 96) FM_DENSE_BWD(96);
+  else FM_DENSE_BWD(128);
+#undef FM_DENSE_BWD
+  if (ds->normalize) {
+    ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
+    norm_fix_kernel<T><<<bh, ds->d, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, nbq, pl.nq, ds->d, ds->lim);
+    norm_fix_kernel<T><<<pl.bhkv, ds->d, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh,
+                                                      rpart + (int64_t)bh * nbq, nbk, pl.nk, ds->d, ds->lim);
     FM_TRY(launch_status("norm_fix_kernel"));
   }
   return FASTMAX_OK;
@@ -984,6 +1150,13 @@ static int forward_entry(const fastmax_desc* desc, const fastmax_layout* layout,
   FM_TRY(check_saved(pl, saved_states, saved_bytes));
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (pl.dense) {
+    if (desc->dtype == FASTMAX_F32)
+      return dense_forward<float>(desc, pl, L, (const float*)q, (const float*)k, (const float*)v, (float*)o, den,
+                                  den_stride, qk_scale, qk_argmax, ws, st);
+    return dense_forward<bf16_t>(desc, pl, L, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (bf16_t*)o, den,
+                                 den_stride, qk_scale, qk_argmax, ws, st);
+  }
 #define FM_FWD(DD, TT)                                                                             \
   return forward_impl<DD, TT>(desc, pl, L, (const TT*)q, (const TT*)k, (const TT*)v, (TT*)o, den, \
                               den_stride, qk_scale, qk_argmax, ws, workspace_bytes, (float*)saved_states, st)
@@ -1066,6 +1239,15 @@ static int backward_entry(const fastmax_desc* desc, const fastmax_layout* layout
   FM_TRY(check_saved(pl, saved_states, saved_bytes));
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (pl.dense) {
+    if (desc->dtype == FASTMAX_F32)
+      return dense_backward<float>(desc, pl, L, (const float*)q, (const float*)k, (const float*)v, (const float*)o,
+                                   den, den_stride, (const float*)go, (float*)dq, (float*)dk, (float*)dv, qk_scale,
+                                   qk_argmax, ws, st);
+    return dense_backward<bf16_t>(desc, pl, L, (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)o,
+                                  den, den_stride, (const bf16_t*)go, (bf16_t*)dq, (bf16_t*)dk, (bf16_t*)dv, qk_scale,
+                                  qk_argmax, ws, st);
+  }
 #define FM_BWD(DD, TT)                                                                              \
   return backward_impl<DD, TT>(desc, pl, L, (const TT*)q, (const TT*)k, (const TT*)v, (const TT*)o, \
                                den, den_stride, (const TT*)go, (TT*)dq, (TT*)dk, (TT*)dv, qk_scale,  \
@@ -1138,15 +1320,24 @@ int fastmax_normalize_inplace(const fastmax_desc* desc, void* q, void* k, void* 
   return launch_status("scale_rows_kernel");
 }
 
+// The recurrent form keeps a moment state per head: it exists for the head dimensions the moment
+// kernels are built for.
+static int check_recurrent(const fastmax_desc* desc) {
+  FM_TRY(check_desc(desc));
+  if (desc->d != 32 && desc->d != 64)
+    return fail(FASTMAX_E_SHAPE, "d = %d: the recurrent entry points keep moment states, which exist for d = 32 and 64", desc->d);
+  return FASTMAX_OK;
+}
+
 size_t fastmax_state_bytes(const fastmax_desc* desc) {
   g_err[0] = 0;
-  if (check_desc(desc) != FASTMAX_OK) return 0;
+  if (check_recurrent(desc) != FASTMAX_OK) return 0;
   return (size_t)state_floats_for(desc->d, desc->p == 2) * sizeof(float);
 }
 
 size_t fastmax_decode_workspace_bytes(const fastmax_desc* desc) {
   g_err[0] = 0;
-  if (check_desc(desc) != FASTMAX_OK) return 0;
+  if (check_recurrent(desc) != FASTMAX_OK) return 0;
   return decode_ws_bytes(desc);
 }
 
@@ -1154,7 +1345,7 @@ int fastmax_state_update(const fastmax_desc* desc, const void* k, const void* v,
                          void* state, int accumulate, void* workspace, size_t workspace_bytes,
                          fastmax_stream_t stream) {
   g_err[0] = 0;
-  FM_TRY(check_desc(desc));
+  FM_TRY(check_recurrent(desc));
   if (!k || !v || !state) return fail(FASTMAX_E_NULL, "k, v and state must be non-NULL");
   if (desc->normalize && !k_scale)
     return fail(FASTMAX_E_NULL, "normalize is set: k_scale (the factor a forward pass reported) is required");
@@ -1163,7 +1354,7 @@ int fastmax_state_update(const fastmax_desc* desc, const void* k, const void* v,
   d2.mask = 0;
   d2.bh = d2.bhkv;
   d2.nq = d2.nk;
-  const Plan pl = make_plan(&d2, FASTMAX_PASS_FORWARD);
+  const Plan pl = make_plan(&d2, FASTMAX_PASS_FORWARD, true, false);   // (the moment state itself is wanted)
   FM_TRY(check_ws(pl, workspace, workspace_bytes));
   char* ws = static_cast<char*>(workspace);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -1184,7 +1375,7 @@ int fastmax_decode_step(const fastmax_desc* desc, const void* q, const void* k, 
                         float* den, int64_t den_stride, void* workspace, size_t workspace_bytes,
                         fastmax_stream_t stream) {
   g_err[0] = 0;
-  FM_TRY(check_desc(desc));
+  FM_TRY(check_recurrent(desc));
   if (!q || !k || !v || !state || !o) return fail(FASTMAX_E_NULL, "q, k, v, state and o must be non-NULL");
   if (desc->nq != 1 || desc->nk != 1) return fail(FASTMAX_E_SHAPE, "a decode step takes one token per head (nq = nk = 1), got nq = %d", desc->nq);
   if (desc->normalize && (!q_scale || !k_scale))

@@ -12,12 +12,16 @@ template <class T, bool VEC>
 __global__ __launch_bounds__(256) void bwd_prep_kernel(Rows<const T> go, Rows<const T> o, RowScalars den,
                                                        float* __restrict__ cvec, int rows, int d) {
   constexpr int EPT = VEC ? (std::is_same<T, float>::value ? 4 : 8) : 4;
-  const int tpr = d / EPT, rpp = 256 / tpr;
+  // threads per row: the pieces of a row rounded up to a power of two (shuffle reduction)
+  const int npc = d / EPT;
+  int tpr = 1;
+  while (tpr < npc) tpr *= 2;
+  const int rpp = 256 / tpr;
   const int sub = threadIdx.x % tpr;
   const int head = blockIdx.y;
   const int row = blockIdx.x * rpp + threadIdx.x / tpr;
   float s = 0.f;
-  if (row < rows) {
+  if (row < rows && sub < npc) {
     const HeadRows<const T> gh = go.head(head), oh = o.head(head);
     const T* grow = gh.row(row) + sub * EPT;
     const T* orow = oh.row(row) + sub * EPT;

@@ -1,0 +1,749 @@
+// Dense-tile form of Fastmax attention: every (query, key) score tile is formed and the polynomial
+// applied to it, with no moment states at all.
+//
+// The moment form costs about 2.1 d^3 flop per token and pass whatever the sequence length (p = 2, each
+// unordered channel pair once), the dense form 2 n d per token under the causal mask.  Below n ~ d^2
+// (and for every head dimension the moment kernels are not built for) the dense form is the cheaper
+// one, it needs no workspace, and all of its work is plain matrix tiles.  It is the chunked scan of the
+// other kernels with a single chunk: the intra-chunk masked score tile is all there is.
+//
+//   forward   o_i  = sum_j f(s_ij) v_j / sum_j f(s_ij)                 s_ij = qh_i . kh_j
+//   dq        dqh_i = sum_j W_ij kh_j      W_ij = f'(s_ij) (g_i . v_j - c_i),  g = grad_out / den,  c_i = g_i . o_i
+//   dk, dv    dkh_j = sum_i W_ij qh_i      dv_j = sum_i f(s_ij) g_i
+// (reference: example.py:199-212 is this dense form; fastmax_cuda_forward.cu:102-197 and
+// fastmax_cuda_backward.cu:26-882 are the token loops it replaces).
+//
+// One block = 4 waves; a wave owns RT tiles of 32 "own" rows (queries in forward / dq, keys in dk/dv)
+// whose operands stay in registers, and walks the "streamed" rows (keys, resp. queries) in stages of
+// BN rows that all four waves share through LDS (double buffered, one barrier per stage).  Score tiles
+// are formed with the streamed rows as the A operand (rows of the tile) and the own rows as the B
+// operand (columns = lanes), so that f(score), still in the accumulator registers, is directly the A
+// operand of the second contraction (rows = own... of the transposed tile), whose B operand is the
+// streamed tile stored transposed.  Head dimensions are handled as DP = d rounded up to a multiple of
+// 32: channels past d are zero on load and skipped on store.
+#pragma once
+#include <type_traits>
+
+#include "fm_common.h"
+
+namespace dense {
+
+// Matrix-instruction policy.  A "fragment" is the 16 bytes one lane feeds into one step of a
+// contraction: 8 bf16 (one v_mfma_f32_32x32x16_bf16, lane half hh supplies k = 8 hh .. 8 hh + 7 of the
+// step's 16) or 4 floats (four v_mfma_f32_32x32x2f32, lane half hh supplies k = 4 hh + u to instruction u
+// of the step's 8).  Both operands of a contraction use the same mapping, so any such assignment of k
+// indices is valid.
+template <class T>
+struct Mma;
+
+template <>
+struct Mma<bf16_t> {
+  using Elt = uint16_t;
+  using Frag = fm_u4;
+  static constexpr int EPL = 8;    // elements per lane and fragment
+  static constexpr int KF = 16;    // contraction length of a fragment step
+  static constexpr int PAD = 8;    // row padding of LDS tiles (elements): 16 bytes, conflict-free 128-bit rows
+  static __device__ __forceinline__ Frag zero() { return Frag{0u, 0u, 0u, 0u}; }
+  static __device__ __forceinline__ f16v mma(const Frag& a, const Frag& b, const f16v& c) {
+    return FM_MFMA_BF16(__builtin_bit_cast(bf8v, a), __builtin_bit_cast(bf8v, b), c);
+  }
+  // Fragment f of an accumulator tile used as an operand whose k index is the tile's row: registers
+  // 8 f .. 8 f + 7 of lane half hh are rows 16 f + 8 (e / 4) + 4 hh + e % 4.
+  template <int F>
+  static __device__ __forceinline__ Frag from_acc(const f16v& a) {
+    return Frag{pack_bf2(a[8 * F], a[8 * F + 1]), pack_bf2(a[8 * F + 2], a[8 * F + 3]),
+                pack_bf2(a[8 * F + 4], a[8 * F + 5]), pack_bf2(a[8 * F + 6], a[8 * F + 7])};
+  }
+  // where row x of a transposed tile is stored, so that the eight rows of such a fragment are
+  // contiguous: one 128-bit read at 16 f + 8 hh
+  static __device__ __forceinline__ int tpos(int x) {
+    return (x & ~15) | (((x >> 2) & 1) << 3) | (((x >> 3) & 1) << 2) | (x & 3);
+  }
+  // acc + the sum of the fragment's elements, as rounded
+  static __device__ __forceinline__ float fsum(const Frag& w, float acc) {
+    acc = fm_dot2_bf16(w.x, 0x3f803f80u, acc);
+    acc = fm_dot2_bf16(w.y, 0x3f803f80u, acc);
+    acc = fm_dot2_bf16(w.z, 0x3f803f80u, acc);
+    return fm_dot2_bf16(w.w, 0x3f803f80u, acc);
+  }
+  static __device__ __forceinline__ void unpack(const uint4& r, float (&o)[8]) {
+    o[0] = bf_lo(r.x); o[1] = bf_hi(r.x); o[2] = bf_lo(r.y); o[3] = bf_hi(r.y);
+    o[4] = bf_lo(r.z); o[5] = bf_hi(r.z); o[6] = bf_lo(r.w); o[7] = bf_hi(r.w);
+  }
+  static __device__ __forceinline__ uint4 pack(const float (&o)[8]) {
+    return make_uint4(pack_bf2(o[0], o[1]), pack_bf2(o[2], o[3]), pack_bf2(o[4], o[5]), pack_bf2(o[6], o[7]));
+  }
+  static __device__ __forceinline__ Elt elt(const uint4& r, int e) {
+    const uint32_t w = e < 2 ? r.x : e < 4 ? r.y : e < 6 ? r.z : r.w;
+    return (Elt)((e & 1) ? (w >> 16) : w);
+  }
+};
+
+template <>
+struct Mma<float> {
+  using Elt = float;
+  using Frag = float4;
+  static constexpr int EPL = 4;
+  static constexpr int KF = 8;
+  static constexpr int PAD = 4;
+  static __device__ __forceinline__ Frag zero() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+  static __device__ __forceinline__ f16v mma(const Frag& a, const Frag& b, f16v c) {
+    c = FM_MFMA(a.x, b.x, c);
+    c = FM_MFMA(a.y, b.y, c);
+    c = FM_MFMA(a.z, b.z, c);
+    return FM_MFMA(a.w, b.w, c);
+  }
+  // registers 4 f .. 4 f + 3 of lane half hh are rows 8 f + 4 hh + u
+  template <int F>
+  static __device__ __forceinline__ Frag from_acc(const f16v& a) {
+    return make_float4(a[4 * F], a[4 * F + 1], a[4 * F + 2], a[4 * F + 3]);
+  }
+  static __device__ __forceinline__ int tpos(int x) { return x; }
+  static __device__ __forceinline__ float fsum(const Frag& w, float acc) { return acc + ((w.x + w.y) + (w.z + w.w)); }
+  static __device__ __forceinline__ void unpack(const uint4& r, float (&o)[4]) {
+    o[0] = __uint_as_float(r.x); o[1] = __uint_as_float(r.y); o[2] = __uint_as_float(r.z); o[3] = __uint_as_float(r.w);
+  }
+  static __device__ __forceinline__ uint4 pack(const float (&o)[4]) {
+    return make_uint4(__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3]));
+  }
+  static __device__ __forceinline__ Elt elt(const uint4& r, int e) {
+    return __uint_as_float(e == 0 ? r.x : e == 1 ? r.y : e == 2 ? r.z : r.w);
+  }
+};
+
+// an all-zero accumulator tile (the C operand of a contraction's first step)
+constexpr f16v kZero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+template <class T>
+__device__ __forceinline__ typename Mma<T>::Frag lds_frag(const typename Mma<T>::Elt* p) {
+  return *reinterpret_cast<const typename Mma<T>::Frag*>(p);
+}
+
+// R rows x DP channels of one head on their way global -> registers -> LDS, by 256 threads.
+// Consecutive threads take consecutive rows (16 bytes of a row each), which makes both the row-major
+// and the transposed LDS writes conflict-free.  Rows outside [lo, pend) and channels past d are zero.
+template <int DP, class T, int R>
+struct TileRegs {
+  using M = Mma<T>;
+  using Elt = typename M::Elt;
+  static constexpr int EPP = 16 / (int)sizeof(T);   // elements per 16-byte piece
+  static constexpr int PPR = DP / EPP;
+  static constexpr int TOTAL = R * PPR;
+  static constexpr int NV = (TOTAL + 255) / 256;
+  uint4 raw[NV];
+  float rf[NV];   // row factor of scaled tiles: 1 / rowdiv[row], 0 for a row that does not exist
+
+  __device__ __forceinline__ void load(const HeadRows<const T>& hr, int pos0, int pend, int d, int tid,
+                                       const float* rowdiv = nullptr, int64_t rdstride = 0) {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      const bool in = idx < TOTAL;
+      const int row = in ? idx % R : 0, pc = in ? idx / R : 0;
+      const int pos = pos0 + row;
+      const bool live = in && pos >= hr.lo && pos < pend && pc * EPP < d;
+      const int ps = max(pos < pend ? pos : pend - 1, hr.lo);
+      const uint4 t = *reinterpret_cast<const uint4*>(hr.base + ((unsigned)ps * hr.pitch + (unsigned)(live ? pc * EPP : 0)));
+      raw[u] = live ? t : make_uint4(0u, 0u, 0u, 0u);
+      rf[u] = 0.f;
+      if (rowdiv) rf[u] = live ? 1.0f / rowdiv[(unsigned)ps * (unsigned)rdstride] : 0.f;
+    }
+  }
+  // as loaded: row-major [R][pr] and / or transposed [DP][pt] (row x at column tpos(x))
+  __device__ __forceinline__ void store(Elt* rm, int pr, Elt* tr, int pt, int tid) const {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      if (idx < TOTAL) {
+        const int row = idx % R, pc = idx / R;
+        if (rm) *reinterpret_cast<uint4*>(rm + row * pr + pc * EPP) = raw[u];
+        if (tr) {
+          Elt* t0 = tr + pc * EPP * pt + M::tpos(row);
+#pragma unroll
+          for (int e = 0; e < EPP; ++e) t0[e * pt] = M::elt(raw[u], e);
+        }
+      }
+    }
+  }
+  // times the row factor and a constant each: srm for the row-major copy, str for the transposed one
+  __device__ __forceinline__ void store_scaled(Elt* rm, int pr, float srm, Elt* tr, int pt, float str, int tid) const {
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int idx = tid + u * 256;
+      if (idx < TOTAL) {
+        const int row = idx % R, pc = idx / R;
+        float x[EPP], y[EPP];
+        M::unpack(raw[u], x);
+        const float f1 = rf[u] * srm, f2 = rf[u] * str;
+#pragma unroll
+        for (int e = 0; e < EPP; ++e) {
+          y[e] = x[e] * f2;
+          x[e] *= f1;
+        }
+        *reinterpret_cast<uint4*>(rm + row * pr + pc * EPP) = M::pack(x);
+        const uint4 yt = M::pack(y);
+        Elt* t0 = tr + pc * EPP * pt + M::tpos(row);
+#pragma unroll
+        for (int e = 0; e < EPP; ++e) t0[e * pt] = M::elt(yt, e);
+      }
+    }
+  }
+};
+
+// The fragments of one own row (position pos of the head), times `scale`: fragment m holds channels
+// KF m + EPL hh .. + EPL - 1.  A row outside [lo, pend) gives zeros, and so do channels past d.
+template <int DP, class T>
+__device__ __forceinline__ void load_own_frags(const HeadRows<const T>& hr, int pos, int pend, int d, int hh, float scale,
+                                               typename Mma<T>::Frag (&f)[DP / Mma<T>::KF]) {
+  using M = Mma<T>;
+  const bool live = pos >= hr.lo && pos < pend;
+  const int ps = max(pos < pend ? pos : pend - 1, hr.lo);
+  const T* row = hr.base + (unsigned)ps * hr.pitch;
+#pragma unroll
+  for (int m = 0; m < DP / M::KF; ++m) {
+    const int ch = M::KF * m + M::EPL * hh;
+    const bool ok = live && ch < d;
+    const uint4 t = *reinterpret_cast<const uint4*>(row + (ok ? ch : 0));
+    float x[M::EPL];
+    M::unpack(t, x);
+#pragma unroll
+    for (int e = 0; e < M::EPL; ++e) x[e] = ok ? x[e] * scale : 0.f;
+    f[m] = __builtin_bit_cast(typename M::Frag, M::pack(x));
+  }
+}
+
+// LDS layout shared by the three kernels: NA row-major and NT transposed streamed tiles per buffer, two
+// buffers, then `tail` floats.
+template <int DP, class T, int BN>
+struct Lds {
+  using M = Mma<T>;
+  static constexpr int PR = DP + M::PAD;   // pitch of row-major tiles (elements)
+  static constexpr int PT = BN + M::PAD;   // pitch of transposed tiles
+  static constexpr int RM = BN * PR;       // elements of a row-major tile
+  static constexpr int TR = DP * PT;       // elements of a transposed tile
+  static constexpr size_t bytes(int na, int nt, int tail_floats) {
+    return (size_t)2 * (na * RM + nt * TR) * sizeof(typename M::Elt) + (size_t)tail_floats * sizeof(float);
+  }
+};
+
+template <int DP, class T>
+struct Shape {
+  static constexpr bool BF = std::is_same<T, bf16_t>::value;
+  static constexpr int BN = BF ? 64 : 32;                     // streamed rows per stage
+  static constexpr int RT_FWD = DP <= 64 ? 2 : 1;             // own 32-row tiles per wave
+  static constexpr int RT_DQ = DP <= 32 ? 2 : 1;
+  static constexpr int RT_KV = 1;
+  static constexpr int OCC = DP <= 64 ? 2 : 1;                // resident blocks per CU the kernels are built for
+};
+
+// ---------------------------------------------------------------------------------------
+// Forward.  grid = (heads, query blocks of 128 RT positions from the one that holds position Q.lo).
+// npos: positions of the queries end here (nk under the mask: query i sits at position i + nk - nq).
+// ---------------------------------------------------------------------------------------
+template <int DP, class T, int RT, int BN>
+__global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
+    Rows<const T> Q, Rows<const T> K, Rows<const T> V, const float* __restrict__ qscale,
+    const float* __restrict__ kscale, Rows<T> O, RowScalarsOut den, int npos, int nk, int d, int masked, float a0,
+    float a1, float a2, int ratio) {
+  using M = Mma<T>;
+  using Elt = typename M::Elt;
+  using Frag = typename M::Frag;
+  using L = Lds<DP, T, BN>;
+  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int PR = L::PR, PT = L::PT;
+  extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
+  Elt* Kl = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
+  Elt* Vt = Kl + 2 * L::RM;                       // [2][DP][PT]
+  float* denl = reinterpret_cast<float*>(Vt + 2 * L::TR);   // [BM]
+
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
+  // grid = (heads, row blocks): blocks are dispatched head-fastest, so under the mask the row blocks with
+  // the most keys to walk start first for every head, and (workgroups go round-robin to the 8 XCDs) the
+  // blocks of a head meet in one XCD's L2 whenever the head count is a multiple of 8
+  const int nb = gridDim.y, bx = blockIdx.y;
+  const int head = blockIdx.x, hkv = head / ratio;
+  const int tok0 = (Q.lo / BM + (masked ? nb - 1 - bx : bx)) * BM;
+  const HeadRows<const T> Qh = Q.head(head), Kh = K.head(hkv), Vh = V.head(hkv);
+  const float kq = qscale[head] * kscale[hkv];
+
+  Frag qf[RT][NF];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) load_own_frags<DP, T>(Qh, tok0 + (w * RT + rt) * 32 + i, npos, d, hh, kq, qf[rt]);
+
+  const int kend = masked ? (tok0 + BM < nk ? tok0 + BM : nk) : nk;
+  const int nst = (kend + BN - 1) / BN;
+  TileRegs<DP, T, BN> kt, vt;
+  auto stage_load = [&](int st) {
+    kt.load(Kh, st * BN, nk, d, tid);
+    vt.load(Vh, st * BN, nk, d, tid);
+  };
+  auto stage_store = [&](int buf) {
+    kt.store(Kl + buf * L::RM, PR, nullptr, 0, tid);
+    vt.store(nullptr, 0, Vt + buf * L::TR, PT, tid);
+  };
+
+  f16v acc[RT][CB];
+  float dn[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    dn[rt] = 0.f;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rt][cb][r] = 0.f;
+  }
+
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+  for (int st = 0; st < nst; ++st) {
+    const int buf = st & 1;
+    if (st + 1 < nst) stage_load(st + 1);
+    const Elt* kl = Kl + buf * L::RM;
+    const Elt* vl = Vt + buf * L::TR;
+#pragma unroll
+    for (int t32 = 0; t32 < BN / 32; ++t32) {
+      const int kb = st * BN + t32 * 32;
+      if (kb >= kend) continue;
+      bool act[RT];
+      bool any = false;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        act[rt] = !masked || kb <= tok0 + (w * RT + rt) * 32;
+        any = any || act[rt];
+      }
+      if (!any) continue;
+      // scores, transposed: rows = keys trow(r, hh), lanes = own queries
+      f16v sc[RT];
+#pragma unroll
+      for (int m = 0; m < NF; ++m) {
+        const Frag a = lds_frag<T>(kl + (t32 * 32 + i) * PR + KF * m + EPL * hh);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          if (act[rt]) sc[rt] = M::mma(a, qf[rt][m], m == 0 ? kZero16 : sc[rt]);
+      }
+      const bool tail = !masked && kb + 32 > nk;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if (!act[rt]) continue;
+        const int q0 = tok0 + (w * RT + rt) * 32;
+        const bool diag = masked && kb == q0;
+        if (diag || tail) {   // (wave-uniform: only these tiles pay for the per-element tests)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float s = sc[rt][r];
+            float f = a0 + s * (a1 + a2 * s);
+            if (diag && trow(r, hh) > i) f = 0.f;              // a key may not lie after the query
+            if (tail && kb + trow(r, hh) >= nk) f = 0.f;       // keys past the end
+            sc[rt][r] = f;
+          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float s = sc[rt][r];
+            sc[rt][r] = a0 + s * (a1 + a2 * s);
+          }
+        }
+      }
+      // own rows x channels += f(scores) (own x keys) . V (keys x channels)
+      static_for<NFA>([&](auto ftag) {
+        constexpr int F = decltype(ftag)::value;
+        Frag wa[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          wa[rt] = M::template from_acc<F>(sc[rt]);
+          if (act[rt]) dn[rt] = M::fsum(wa[rt], dn[rt]);
+        }
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+          const Frag b = lds_frag<T>(vl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            if (act[rt]) acc[rt][cb] = M::mma(wa[rt], b, acc[rt][cb]);
+        }
+      });
+    }
+    if (st + 1 < nst) stage_store(buf ^ 1);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const float tot = dn[rt] + __shfl_xor(dn[rt], 32, 64);
+    if (hh == 0) denl[(w * RT + rt) * 32 + i] = tot;
+  }
+  __syncthreads();
+  const HeadRows<T> Oh = O.head(head);
+  float* denh = den.head(head);
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = (w * RT + rt) * 32 + trow(r, hh), pos = tok0 + row;
+      if (pos < npos && pos >= Qh.lo) {
+        const float dsum = denl[row], inv = 1.0f / dsum;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+          if (cb * 32 + i < d) Oh.base[(unsigned)pos * Oh.pitch + (unsigned)(cb * 32 + i)] = from_f32<T>(acc[rt][cb][r] * inv);
+        if (i == 0) denh[(int64_t)pos * den.stride] = dsum;
+      }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// dq.  Same walk as the forward pass; the own rows carry q (times 2 a2, so that the score accumulator,
+// started at a1, is f'(s)) and g = grad_out / den.  rpart[head * gridDim.y + block] receives the block's
+// sum of dqh . qh for the normalisation chain rule (when rpart is given).
+// ---------------------------------------------------------------------------------------
+template <int DP, class T, int RT, int BN>
+__global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
+    Rows<const T> Q, Rows<const T> GO, RowScalars den, RowScalars cvec, Rows<const T> K, Rows<const T> V,
+    const float* __restrict__ qscale, const float* __restrict__ kscale, Rows<T> DQ, float* __restrict__ rpart,
+    int npos, int nk, int d, int masked, int p2, float a1, float a2, int ratio) {
+  using M = Mma<T>;
+  using Elt = typename M::Elt;
+  using Frag = typename M::Frag;
+  using L = Lds<DP, T, BN>;
+  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int PR = L::PR, PT = L::PT;
+  extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
+  Elt* Kl = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
+  Elt* Vl = Kl + 2 * L::RM;                       // [2][BN][PR]
+  Elt* Kt = Vl + 2 * L::RM;                       // [2][DP][PT]
+  float* red = reinterpret_cast<float*>(Kt + 2 * L::TR);   // [4]
+
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
+  const int nb = gridDim.y, bx = blockIdx.y;   // (heads, row blocks), as in the forward kernel
+  const int head = blockIdx.x, hkv = head / ratio;
+  const int tok0 = (Q.lo / BM + (masked ? nb - 1 - bx : bx)) * BM;
+  const HeadRows<const T> Qh = Q.head(head), Gh = GO.head(head), Kh = K.head(hkv), Vh = V.head(hkv);
+  const float* denh = den.head(head);
+  const float* ch = cvec.head(head);
+  const float kq = qscale[head] * kscale[hkv];
+
+  Frag qf[RT][NF], gf[RT][NF];
+  float cown[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int pos = tok0 + (w * RT + rt) * 32 + i;
+    const bool live = pos >= Qh.lo && pos < npos;
+    const int ps = max(pos < npos ? pos : npos - 1, Qh.lo);
+    const float rden = live ? 1.0f / denh[(int64_t)ps * den.stride] : 0.f;
+    cown[rt] = live ? ch[(int64_t)ps * cvec.stride] : 0.f;
+    if (p2) load_own_frags<DP, T>(Qh, pos, npos, d, hh, kq * 2.0f * a2, qf[rt]);
+    load_own_frags<DP, T>(Gh, pos, npos, d, hh, rden, gf[rt]);
+  }
+
+  const int kend = masked ? (tok0 + BM < nk ? tok0 + BM : nk) : nk;
+  const int nst = (kend + BN - 1) / BN;
+  TileRegs<DP, T, BN> kt, vt;
+  auto stage_load = [&](int st) {
+    kt.load(Kh, st * BN, nk, d, tid);
+    vt.load(Vh, st * BN, nk, d, tid);
+  };
+  auto stage_store = [&](int buf) {
+    kt.store(Kl + buf * L::RM, PR, Kt + buf * L::TR, PT, tid);
+    vt.store(Vl + buf * L::RM, PR, nullptr, 0, tid);
+  };
+
+  f16v acc[RT][CB];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[rt][cb][r] = 0.f;
+
+  stage_load(0);
+  stage_store(0);
+  __syncthreads();
+  for (int st = 0; st < nst; ++st) {
+    const int buf = st & 1;
+    if (st + 1 < nst) stage_load(st + 1);
+    const Elt* kl = Kl + buf * L::RM;
+    const Elt* vl = Vl + buf * L::RM;
+    const Elt* ktl = Kt + buf * L::TR;
+#pragma unroll
+    for (int t32 = 0; t32 < BN / 32; ++t32) {
+      const int kb = st * BN + t32 * 32;
+      if (kb >= kend) continue;
+      bool act[RT];
+      bool any = false;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        act[rt] = !masked || kb <= tok0 + (w * RT + rt) * 32;
+        any = any || act[rt];
+      }
+      if (!any) continue;
+      // transposed tiles (rows = keys, lanes = own queries): f'(s) and g . v - c
+      f16v sc[RT], pt[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          sc[rt][r] = a1;
+          pt[rt][r] = -cown[rt];
+        }
+#pragma unroll
+      for (int m = 0; m < NF; ++m) {
+        const Frag av = lds_frag<T>(vl + (t32 * 32 + i) * PR + KF * m + EPL * hh);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          if (act[rt]) pt[rt] = M::mma(av, gf[rt][m], pt[rt]);
+        if (p2) {
+          const Frag ak = lds_frag<T>(kl + (t32 * 32 + i) * PR + KF * m + EPL * hh);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            if (act[rt]) sc[rt] = M::mma(ak, qf[rt][m], sc[rt]);
+        }
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if (!act[rt]) continue;
+        const bool diag = masked && kb == tok0 + (w * RT + rt) * 32;
+        if (diag) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) pt[rt][r] = trow(r, hh) > i ? 0.f : sc[rt][r] * pt[rt][r];
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) pt[rt][r] = sc[rt][r] * pt[rt][r];
+        }
+      }
+      // own rows x channels += W (own x keys) . K (keys x channels)
+      static_for<NFA>([&](auto ftag) {
+        constexpr int F = decltype(ftag)::value;
+        Frag wa[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) wa[rt] = M::template from_acc<F>(pt[rt]);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+          const Frag b = lds_frag<T>(ktl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            if (act[rt]) acc[rt][cb] = M::mma(wa[rt], b, acc[rt][cb]);
+        }
+      });
+    }
+    if (st + 1 < nst) stage_store(buf ^ 1);
+    __syncthreads();
+  }
+
+  // dq = qs ks acc (the keys went in unscaled); sum of dqh . qh = qs ks sum acc . q
+  const HeadRows<T> Dh = DQ.head(head);
+  float rs = 0.f;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int pos = tok0 + (w * RT + rt) * 32 + trow(r, hh);
+      if (pos < npos && pos >= Qh.lo) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+          const int c = cb * 32 + i;
+          if (c < d) {
+            const float v = acc[rt][cb][r] * kq;
+            Dh.base[(unsigned)pos * Dh.pitch + (unsigned)c] = from_f32<T>(v);
+            if (rpart) rs += v * to_f32(Qh.base[(unsigned)pos * Qh.pitch + (unsigned)c]);
+          }
+        }
+      }
+    }
+  if (rpart) {
+    rs = block_sum_256(rs, red, tid);
+    if (tid == 0) rpart[(int64_t)head * nb + bx] = rs;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// dk and dv.  grid = (key/value heads, key blocks of 128 RT positions); the own rows are keys, the
+// streamed rows the queries at or after them (all of them when unmasked) of every query head of the
+// group in turn.  Score tiles have rows = queries, lanes = own keys.  The streamed g rows go to LDS
+// twice: times qs / den row-major (so that W comes out times qs, the factor of qh in dkh = sum W qh) and
+// times 1 / den transposed (the B operand of dv).  rpart[kvhead * gridDim.y + block] = sum dkh . kh.
+// ---------------------------------------------------------------------------------------
+template <int DP, class T, int RT, int BN>
+__global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
+    Rows<const T> K, Rows<const T> V, Rows<const T> Q, Rows<const T> GO, RowScalars den, RowScalars cvec,
+    const float* __restrict__ qscale, const float* __restrict__ kscale, Rows<T> DK, Rows<T> DV,
+    float* __restrict__ rpart, int npos, int nk, int d, int masked, float a0, float a1, float a2, int ratio) {
+  using M = Mma<T>;
+  using Elt = typename M::Elt;
+  using Frag = typename M::Frag;
+  using L = Lds<DP, T, BN>;
+  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int PR = L::PR, PT = L::PT;
+  extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
+  Elt* Ql = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
+  Elt* Gl = Ql + 2 * L::RM;                       // [2][BN][PR]
+  Elt* Qt = Gl + 2 * L::RM;                       // [2][DP][PT]
+  Elt* Gt = Qt + 2 * L::TR;                       // [2][DP][PT]
+  float* Cl = reinterpret_cast<float*>(Gt + 2 * L::TR);   // [2][BN]
+  float* red = Cl + 2 * BN;                       // [4]
+
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
+  const int nb = gridDim.y, bx = blockIdx.y;   // (key/value heads, key blocks)
+  const int hkv = blockIdx.x;
+  const int tok0 = bx * BM;   // (under the mask the first key blocks see the most queries: already first)
+  const HeadRows<const T> Kh = K.head(hkv), Vh = V.head(hkv);
+  const float ks = kscale[hkv];
+
+  Frag kf[RT][NF], vf[RT][NF];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int pos = tok0 + (w * RT + rt) * 32 + i;
+    load_own_frags<DP, T>(Kh, pos, nk, d, hh, ks, kf[rt]);
+    load_own_frags<DP, T>(Vh, pos, nk, d, hh, 1.0f, vf[rt]);
+  }
+  f16v dk[RT][CB], dv[RT][CB];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dk[rt][cb][r] = dv[rt][cb][r] = 0.f;
+
+  TileRegs<DP, T, BN> qt, gt;
+  float creg = 0.f;
+  for (int hq = 0; hq < ratio; ++hq) {
+    const int head = hkv * ratio + hq;
+    const HeadRows<const T> Qh = Q.head(head), Gh = GO.head(head);
+    const float* denh = den.head(head);
+    const float* ch = cvec.head(head);
+    const float qs = qscale[head];
+    // f and f' of s = qs sr, where sr = q . kh is what the score tile holds
+    const float c2 = a2 * qs * qs, c1 = a1 * qs, b2 = 2.0f * a2 * qs;
+    const int lo = Qh.lo;
+    const int st0 = masked ? (tok0 > lo ? tok0 : lo) / BN : 0;
+    const int nst = (npos + BN - 1) / BN;
+    auto stage_load = [&](int st) {
+      qt.load(Qh, st * BN, npos, d, tid);
+      gt.load(Gh, st * BN, npos, d, tid, denh, den.stride);
+      if (tid < BN) {
+        const int pos = st * BN + tid;
+        creg = (pos >= lo && pos < npos) ? ch[(int64_t)pos * cvec.stride] * qs : 0.f;
+      }
+    };
+    auto stage_store = [&](int buf) {
+      qt.store(Ql + buf * L::RM, PR, Qt + buf * L::TR, PT, tid);
+      gt.store_scaled(Gl + buf * L::RM, PR, qs, Gt + buf * L::TR, PT, 1.0f, tid);
+      if (tid < BN) Cl[buf * BN + tid] = creg;
+    };
+    if (st0 < nst) {
+      stage_load(st0);
+      stage_store(0);
+    }
+    __syncthreads();
+    for (int st = st0; st < nst; ++st) {
+      const int buf = (st - st0) & 1;
+      if (st + 1 < nst) stage_load(st + 1);
+      const Elt* ql = Ql + buf * L::RM;
+      const Elt* gl = Gl + buf * L::RM;
+      const Elt* qtl = Qt + buf * L::TR;
+      const Elt* gtl = Gt + buf * L::TR;
+      const float* cl = Cl + buf * BN;
+#pragma unroll
+      for (int t32 = 0; t32 < BN / 32; ++t32) {
+        const int qb = st * BN + t32 * 32;
+        if (qb >= npos) continue;
+        bool act[RT];
+        bool any = false;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          act[rt] = !masked || qb >= tok0 + (w * RT + rt) * 32;
+          any = any || act[rt];
+        }
+        if (!any) continue;
+        // tiles with rows = queries trow(r, hh), lanes = own keys: sr and qs (g . v - c)
+        float cneg[16];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float4 c4 = *reinterpret_cast<const float4*>(cl + t32 * 32 + 8 * j + 4 * hh);
+          cneg[4 * j] = -c4.x; cneg[4 * j + 1] = -c4.y; cneg[4 * j + 2] = -c4.z; cneg[4 * j + 3] = -c4.w;
+        }
+        f16v sc[RT], pt[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) pt[rt][r] = cneg[r];
+#pragma unroll
+        for (int m = 0; m < NF; ++m) {
+          const Frag aq = lds_frag<T>(ql + (t32 * 32 + i) * PR + KF * m + EPL * hh);
+          const Frag ag = lds_frag<T>(gl + (t32 * 32 + i) * PR + KF * m + EPL * hh);
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            if (act[rt]) {
+              sc[rt] = M::mma(aq, kf[rt][m], m == 0 ? kZero16 : sc[rt]);
+              pt[rt] = M::mma(ag, vf[rt][m], pt[rt]);
+            }
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          if (!act[rt]) continue;
+          const bool diag = masked && qb == tok0 + (w * RT + rt) * 32;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float s = sc[rt][r];
+            sc[rt][r] = a0 + s * (c1 + c2 * s);
+            pt[rt][r] = (a1 + b2 * s) * pt[rt][r];
+          }
+          if (diag) {   // a query may not lie before the key
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              if (trow(r, hh) < i) sc[rt][r] = pt[rt][r] = 0.f;
+          }
+        }
+        // own keys x channels: dv += f^T (keys x queries) . g,   dk += W^T . q
+        static_for<NFA>([&](auto ftag) {
+          constexpr int F = decltype(ftag)::value;
+          Frag fa[RT], wa[RT];
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) {
+            fa[rt] = M::template from_acc<F>(sc[rt]);
+            wa[rt] = M::template from_acc<F>(pt[rt]);
+          }
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) {
+            const Frag bg = lds_frag<T>(gtl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
+            const Frag bq = lds_frag<T>(qtl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+              if (act[rt]) {
+                dv[rt][cb] = M::mma(fa[rt], bg, dv[rt][cb]);
+                dk[rt][cb] = M::mma(wa[rt], bq, dk[rt][cb]);
+              }
+          }
+        });
+      }
+      if (st + 1 < nst) stage_store(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // dk = ks dkh (dkh = the accumulated sum); sum of dkh . kh = ks sum acc . k
+  const HeadRows<T> DKh = DK.head(hkv), DVh = DV.head(hkv);
+  float rs = 0.f;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int pos = tok0 + (w * RT + rt) * 32 + trow(r, hh);
+      if (pos < nk) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+          const int c = cb * 32 + i;
+          if (c < d) {
+            const float v = dk[rt][cb][r] * ks;
+            DKh.base[(unsigned)pos * DKh.pitch + (unsigned)c] = from_f32<T>(v);
+            DVh.base[(unsigned)pos * DVh.pitch + (unsigned)c] = from_f32<T>(dv[rt][cb][r]);
+            if (rpart) rs += v * to_f32(Kh.base[(unsigned)pos * Kh.pitch + (unsigned)c]);
+          }
+        }
+      }
+    }
+  if (rpart) {
+    rs = block_sum_256(rs, red, tid);
+    if (tid == 0) rpart[(int64_t)hkv * nb + bx] = rs;
+  }
+}
+
+}  // namespace dense

@@ -9,7 +9,8 @@
 // Per-head normaliser: scale[h] = lim / max_i ||x_i||_2 and the row that attains the max
 // (first one on ties).  Replaces calc_norms / find_max of the reference
 // (fastmax_cuda_forward.cu:223-253) with the PyTorch path's definition (example.py:105-108).
-// One block of NT threads per head; a row is shared by d/4 (fp32) or d/8 (bf16) threads, 16 bytes each.  (NT = 1024 when there are too few
+// One block of NT threads per head; a row is shared by d/4 (fp32) or d/8 (bf16) threads, 16 bytes each (any d that is
+// a whole number of such pieces).  (NT = 1024 when there are too few
 // heads to fill the chip with 256-thread blocks: four times the loads in flight per head.)
 // ---------------------------------------------------------------------------------------
 // a thread's piece of a row: 16 bytes = 4 fp32 or 8 bf16 elements
@@ -44,7 +45,12 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(Rows<const T> x1, int n1, i
   __shared__ int sarg[NT];
   constexpr int EPT = RowPiece<T>::N;
   const int tid = threadIdx.x;
-  const int tpr = d / EPT, rpp = NT / tpr;
+  // threads per row: the pieces of a row rounded up to a power of two (the lanes past the row's
+  // end add zero), so that a row's threads reduce with shuffles
+  const int npc = d / EPT;
+  int tpr = 1;
+  while (tpr < npc) tpr *= 2;
+  const int rpp = NT / tpr;
   const int sub = tid % tpr, rowi = tid / tpr;
   const bool second = (int)blockIdx.x >= nh1;
   const int n = second ? n2 : n1;
@@ -71,7 +77,7 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(Rows<const T> x1, int n1, i
     for (int u = 0; u < 4; ++u) {
       const int i = i0 + u * rpp + rowi;
       idx[u] = i < n ? i : n - 1;
-      ssq[u] = RowPiece<T>::sumsq(base + ((unsigned)idx[u] * pitch + (unsigned)(sub * EPT)));
+      ssq[u] = sub < npc ? RowPiece<T>::sumsq(base + ((unsigned)idx[u] * pitch + (unsigned)(sub * EPT))) : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {

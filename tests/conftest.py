@@ -33,3 +33,16 @@ def built():
 
         build.build_all()
     return _cabi.load()
+
+
+@pytest.fixture(autouse=True)
+def kernel_path(request, monkeypatch):
+    """Where the library has two kernel families for a shape (head dimensions 32 and 64: moment states, or
+    dense score tiles for short sequences) FASTMAX_PATH picks one.  The test modules written against the
+    moment kernels keep exercising them at every length; a module sets KERNEL_PATH = "dense" or "auto" to
+    test the other family or the library's own choice."""
+    path = getattr(request.module, "KERNEL_PATH", "moments")
+    if path == "auto":
+        monkeypatch.delenv("FASTMAX_PATH", raising=False)
+    else:
+        monkeypatch.setenv("FASTMAX_PATH", path)

@@ -44,10 +44,10 @@ def run_case(ops, shape, dtype=torch.float32, seed=0, check_bwd=True, **kw):
 def test_golden_vectors(ops, name):
     c = GOLD[name]
     q, k, v, go = (c[t].cuda() for t in ("q", "k", "v", "go"))
-    if q.shape[-1] not in (32, 64):
+    if q.shape[-1] % 4:   # rows are read in 16-byte pieces (the module pads such head dimensions)
         from fastmax_amd import _cabi
 
-        with pytest.raises(_cabi.FastmaxError, match="supported head dims"):
+        with pytest.raises(_cabi.FastmaxError, match="head dimension must be a multiple of 4"):
             ops.forward(q, k, v, **c["kw"])
         return
     o, den, sc, arg = ops.forward(q, k, v, **c["kw"])
