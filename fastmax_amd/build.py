@@ -32,9 +32,25 @@ def _run(cmd):
     return proc.stdout
 
 
+def _check_no_spills(remarks: str) -> None:
+    """Every kernel must fit its registers: a build in which one of the matrix kernels spilled to
+    scratch memory produced wrong accumulator values on the GPU, so a spill fails the build."""
+    import re
+
+    bad = []
+    for block in re.split(r"remark: [^\n]*Function Name: ", remarks)[1:]:
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", block)
+        if m and int(m.group(1)) > 0:
+            bad.append(f"{block.splitlines()[0].strip()}: {m.group(1)} bytes/lane")
+    if bad:
+        raise RuntimeError("kernels spill registers to scratch memory:\n  " + "\n  ".join(bad))
+
+
 def build_kernels() -> str:
     out = os.path.join(HERE, "libfastmax_hip.so")
-    _run([HIPCC, *HIP_FLAGS, "-shared", f"-I{INCLUDE}", f"-I{CSRC}", os.path.join(CSRC, "fm_api.hip"), "-o", out])
+    remarks = _run([HIPCC, *HIP_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-shared", f"-I{INCLUDE}", f"-I{CSRC}",
+                    os.path.join(CSRC, "fm_api.hip"), "-o", out])
+    _check_no_spills(remarks)
     return out
 
 

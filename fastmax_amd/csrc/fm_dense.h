@@ -231,9 +231,10 @@ struct Shape {
   static constexpr bool BF = std::is_same<T, bf16_t>::value;
   static constexpr int BN = BF ? 64 : 32;                     // streamed rows per stage
   static constexpr int RT_FWD = DP <= 64 ? 2 : 1;             // own 32-row tiles per wave
-  static constexpr int RT_DQ = DP <= 32 ? 2 : 1;
+  static constexpr int RT_DQ = DP <= 32 && BF ? 2 : 1;
   static constexpr int RT_KV = 1;
-  static constexpr int OCC = DP <= 64 ? 2 : 1;                // resident blocks per CU the kernels are built for
+  static constexpr int OCC = (BF ? DP <= 64 : DP <= 32) ? 2 : 1;   // resident blocks per CU the kernels are built for
+                                                              // (fp32 operand fragments take twice the registers)
 };
 
 // ---------------------------------------------------------------------------------------
@@ -250,6 +251,8 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
   using Frag = typename M::Frag;
   using L = Lds<DP, T, BN>;
   constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
+  static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
   extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
   Elt* Kl = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
@@ -293,74 +296,80 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
       for (int r = 0; r < 16; ++r) acc[rt][cb][r] = 0.f;
   }
 
+  // One 32-key tile against the wave's own tiles RT0 .. RT-1 (under the mask the tiles before RT0 lie
+  // wholly before the keys), as straight-line code.  diag: it is the diagonal tile of own tile RT0;
+  // tail: (unmasked) it holds keys past the end -- only those tiles pay for per-element tests.
+  auto tile = [&](auto rt0tag, int t32, int kb, bool diag, bool tail, const Elt* kl, const Elt* vl)
+                  __attribute__((always_inline)) {
+    constexpr int RT0 = decltype(rt0tag)::value;
+    // scores, transposed: rows = keys trow(r, hh), lanes = own queries
+    f16v sc[RT];
+#pragma unroll
+    for (int m0 = 0; m0 < NF; m0 += HC) {   // (HC operand fragments are read ahead of the instructions that use them)
+      Frag ka[HC];
+#pragma unroll
+      for (int m = 0; m < HC; ++m) ka[m] = lds_frag<T>(kl + (t32 * 32 + i) * PR + KF * (m0 + m) + EPL * hh);
+#pragma unroll
+      for (int m = 0; m < HC; ++m)
+#pragma unroll
+        for (int rt = RT0; rt < RT; ++rt) sc[rt] = M::mma(ka[m], qf[rt][m0 + m], m0 + m == 0 ? kZero16 : sc[rt]);
+    }
+#pragma unroll
+    for (int rt = RT0; rt < RT; ++rt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float s = sc[rt][r];
+        sc[rt][r] = a0 + s * (a1 + a2 * s);
+      }
+    if (diag) {   // (wave-uniform) a key may not lie after the query
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (trow(r, hh) > i) sc[RT0][r] = 0.f;
+    }
+    if (tail) {   // (wave-uniform) keys past the end
+#pragma unroll
+      for (int rt = RT0; rt < RT; ++rt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (kb + trow(r, hh) >= nk) sc[rt][r] = 0.f;
+    }
+    // own rows x channels += f(scores) (own x keys) . V (keys x channels)
+    static_for<NFA>([&](auto ftag) {
+      constexpr int F = decltype(ftag)::value;
+      Frag vb[CB], wa[RT];
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) vb[cb] = lds_frag<T>(vl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
+#pragma unroll
+      for (int rt = RT0; rt < RT; ++rt) {
+        wa[rt] = M::template from_acc<F>(sc[rt]);
+        dn[rt] = M::fsum(wa[rt], dn[rt]);
+      }
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int rt = RT0; rt < RT; ++rt) acc[rt][cb] = M::mma(wa[rt], vb[cb], acc[rt][cb]);
+    });
+  };
+
   stage_load(0);
   stage_store(0);
   __syncthreads();
+  const int q00 = tok0 + w * RT * 32;   // first position of the wave's own tile 0
   for (int st = 0; st < nst; ++st) {
     const int buf = st & 1;
     if (st + 1 < nst) stage_load(st + 1);
     const Elt* kl = Kl + buf * L::RM;
     const Elt* vl = Vt + buf * L::TR;
-#pragma unroll
+#pragma unroll 1
     for (int t32 = 0; t32 < BN / 32; ++t32) {
+      __builtin_amdgcn_sched_barrier(0);   // (tiles are not interleaved: register pressure)
       const int kb = st * BN + t32 * 32;
       if (kb >= kend) continue;
-      bool act[RT];
-      bool any = false;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        act[rt] = !masked || kb <= tok0 + (w * RT + rt) * 32;
-        any = any || act[rt];
-      }
-      if (!any) continue;
-      // scores, transposed: rows = keys trow(r, hh), lanes = own queries
-      f16v sc[RT];
-#pragma unroll
-      for (int m = 0; m < NF; ++m) {
-        const Frag a = lds_frag<T>(kl + (t32 * 32 + i) * PR + KF * m + EPL * hh);
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-          if (act[rt]) sc[rt] = M::mma(a, qf[rt][m], m == 0 ? kZero16 : sc[rt]);
-      }
-      const bool tail = !masked && kb + 32 > nk;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        if (!act[rt]) continue;
-        const int q0 = tok0 + (w * RT + rt) * 32;
-        const bool diag = masked && kb == q0;
-        if (diag || tail) {   // (wave-uniform: only these tiles pay for the per-element tests)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float s = sc[rt][r];
-            float f = a0 + s * (a1 + a2 * s);
-            if (diag && trow(r, hh) > i) f = 0.f;              // a key may not lie after the query
-            if (tail && kb + trow(r, hh) >= nk) f = 0.f;       // keys past the end
-            sc[rt][r] = f;
-          }
-        } else {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float s = sc[rt][r];
-            sc[rt][r] = a0 + s * (a1 + a2 * s);
-          }
-        }
-      }
-      // own rows x channels += f(scores) (own x keys) . V (keys x channels)
-      static_for<NFA>([&](auto ftag) {
-        constexpr int F = decltype(ftag)::value;
-        Frag wa[RT];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          wa[rt] = M::template from_acc<F>(sc[rt]);
-          if (act[rt]) dn[rt] = M::fsum(wa[rt], dn[rt]);
-        }
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-          const Frag b = lds_frag<T>(vl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            if (act[rt]) acc[rt][cb] = M::mma(wa[rt], b, acc[rt][cb]);
-        }
+      const int rt0 = (masked && kb > q00) ? (kb - q00) >> 5 : 0;   // own tiles that start before the keys see none of them
+      if (rt0 >= RT) continue;
+      const bool diag = masked && kb == q00 + rt0 * 32, tail = !masked && kb + 32 > nk;
+      static_for<RT>([&](auto tag) {
+        if (rt0 == decltype(tag)::value) tile(tag, t32, kb, diag, tail, kl, vl);
       });
     }
     if (st + 1 < nst) stage_store(buf ^ 1);
@@ -405,6 +414,8 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
   using Frag = typename M::Frag;
   using L = Lds<DP, T, BN>;
   constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
+  static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
   extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
   Elt* Kl = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
@@ -454,74 +465,78 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rt][cb][r] = 0.f;
 
+  auto tile = [&](auto rt0tag, int t32, bool diag, const Elt* kl, const Elt* vl, const Elt* ktl)
+                  __attribute__((always_inline)) {
+    constexpr int RT0 = decltype(rt0tag)::value;   // (diag: the diagonal tile of own tile RT0)
+    // transposed tiles (rows = keys, lanes = own queries): f'(s) and g . v - c
+    f16v sc[RT], pt[RT];
+#pragma unroll
+    for (int rt = RT0; rt < RT; ++rt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sc[rt][r] = a1;
+        pt[rt][r] = -cown[rt];
+      }
+#pragma unroll
+    for (int m0 = 0; m0 < NF; m0 += HC) {
+      Frag va[HC], ka[HC];
+#pragma unroll
+      for (int m = 0; m < HC; ++m) {
+        va[m] = lds_frag<T>(vl + (t32 * 32 + i) * PR + KF * (m0 + m) + EPL * hh);
+        if (p2) ka[m] = lds_frag<T>(kl + (t32 * 32 + i) * PR + KF * (m0 + m) + EPL * hh);
+      }
+#pragma unroll
+      for (int m = 0; m < HC; ++m)
+#pragma unroll
+        for (int rt = RT0; rt < RT; ++rt) {
+          pt[rt] = M::mma(va[m], gf[rt][m0 + m], pt[rt]);
+          if (p2) sc[rt] = M::mma(ka[m], qf[rt][m0 + m], sc[rt]);
+        }
+    }
+#pragma unroll
+    for (int rt = RT0; rt < RT; ++rt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) pt[rt][r] = sc[rt][r] * pt[rt][r];
+    if (diag) {   // (wave-uniform) a key may not lie after the query
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (trow(r, hh) > i) pt[RT0][r] = 0.f;
+    }
+    // own rows x channels += W (own x keys) . K (keys x channels)
+    static_for<NFA>([&](auto ftag) {
+      constexpr int F = decltype(ftag)::value;
+      Frag kb_[CB], wa[RT];
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) kb_[cb] = lds_frag<T>(ktl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
+#pragma unroll
+      for (int rt = RT0; rt < RT; ++rt) wa[rt] = M::template from_acc<F>(pt[rt]);
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int rt = RT0; rt < RT; ++rt) acc[rt][cb] = M::mma(wa[rt], kb_[cb], acc[rt][cb]);
+    });
+  };
+
   stage_load(0);
   stage_store(0);
   __syncthreads();
+  const int q00 = tok0 + w * RT * 32;
   for (int st = 0; st < nst; ++st) {
     const int buf = st & 1;
     if (st + 1 < nst) stage_load(st + 1);
     const Elt* kl = Kl + buf * L::RM;
     const Elt* vl = Vl + buf * L::RM;
     const Elt* ktl = Kt + buf * L::TR;
-#pragma unroll
+#pragma unroll 1
     for (int t32 = 0; t32 < BN / 32; ++t32) {
+      __builtin_amdgcn_sched_barrier(0);   // (tiles are not interleaved: register pressure)
       const int kb = st * BN + t32 * 32;
       if (kb >= kend) continue;
-      bool act[RT];
-      bool any = false;
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        act[rt] = !masked || kb <= tok0 + (w * RT + rt) * 32;
-        any = any || act[rt];
-      }
-      if (!any) continue;
-      // transposed tiles (rows = keys, lanes = own queries): f'(s) and g . v - c
-      f16v sc[RT], pt[RT];
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          sc[rt][r] = a1;
-          pt[rt][r] = -cown[rt];
-        }
-#pragma unroll
-      for (int m = 0; m < NF; ++m) {
-        const Frag av = lds_frag<T>(vl + (t32 * 32 + i) * PR + KF * m + EPL * hh);
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-          if (act[rt]) pt[rt] = M::mma(av, gf[rt][m], pt[rt]);
-        if (p2) {
-          const Frag ak = lds_frag<T>(kl + (t32 * 32 + i) * PR + KF * m + EPL * hh);
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            if (act[rt]) sc[rt] = M::mma(ak, qf[rt][m], sc[rt]);
-        }
-      }
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        if (!act[rt]) continue;
-        const bool diag = masked && kb == tok0 + (w * RT + rt) * 32;
-        if (diag) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) pt[rt][r] = trow(r, hh) > i ? 0.f : sc[rt][r] * pt[rt][r];
-        } else {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) pt[rt][r] = sc[rt][r] * pt[rt][r];
-        }
-      }
-      // own rows x channels += W (own x keys) . K (keys x channels)
-      static_for<NFA>([&](auto ftag) {
-        constexpr int F = decltype(ftag)::value;
-        Frag wa[RT];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) wa[rt] = M::template from_acc<F>(pt[rt]);
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-          const Frag b = lds_frag<T>(ktl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            if (act[rt]) acc[rt][cb] = M::mma(wa[rt], b, acc[rt][cb]);
-        }
+      const int rt0 = (masked && kb > q00) ? (kb - q00) >> 5 : 0;
+      if (rt0 >= RT) continue;
+      const bool diag = masked && kb == q00 + rt0 * 32;
+      static_for<RT>([&](auto tag) {
+        if (rt0 == decltype(tag)::value) tile(tag, t32, diag, kl, vl, ktl);
       });
     }
     if (st + 1 < nst) stage_store(buf ^ 1);
@@ -571,6 +586,8 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
   using Frag = typename M::Frag;
   using L = Lds<DP, T, BN>;
   constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
+  static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
   extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
   Elt* Ql = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
@@ -633,6 +650,74 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
       stage_store(0);
     }
     __syncthreads();
+    // One 32-query tile against the wave's own key tiles 0 .. NA-1 (under the mask the tiles after them lie
+    // wholly after the queries), as straight-line code; diag: it is the diagonal tile of own tile NA-1.
+    auto tile = [&](auto natag, int t32, bool diag, const Elt* ql, const Elt* gl, const Elt* qtl, const Elt* gtl,
+                    const float* cl) __attribute__((always_inline)) {
+      constexpr int NA = decltype(natag)::value + 1;
+      // tiles with rows = queries trow(r, hh), lanes = own keys: sr and qs (g . v - c)
+      f16v sc[RT], pt[RT];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float4 c4 = *reinterpret_cast<const float4*>(cl + t32 * 32 + 8 * j + 4 * hh);
+#pragma unroll
+        for (int rt = 0; rt < NA; ++rt) {
+          pt[rt][4 * j] = -c4.x; pt[rt][4 * j + 1] = -c4.y; pt[rt][4 * j + 2] = -c4.z; pt[rt][4 * j + 3] = -c4.w;
+        }
+      }
+#pragma unroll
+      for (int m0 = 0; m0 < NF; m0 += HC) {
+        Frag qa[HC], ga[HC];
+#pragma unroll
+        for (int m = 0; m < HC; ++m) {
+          qa[m] = lds_frag<T>(ql + (t32 * 32 + i) * PR + KF * (m0 + m) + EPL * hh);
+          ga[m] = lds_frag<T>(gl + (t32 * 32 + i) * PR + KF * (m0 + m) + EPL * hh);
+        }
+#pragma unroll
+        for (int m = 0; m < HC; ++m)
+#pragma unroll
+          for (int rt = 0; rt < NA; ++rt) {
+            sc[rt] = M::mma(qa[m], kf[rt][m0 + m], m0 + m == 0 ? kZero16 : sc[rt]);
+            pt[rt] = M::mma(ga[m], vf[rt][m0 + m], pt[rt]);
+          }
+      }
+#pragma unroll
+      for (int rt = 0; rt < NA; ++rt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float s = sc[rt][r];
+          sc[rt][r] = a0 + s * (c1 + c2 * s);
+          pt[rt][r] = (a1 + b2 * s) * pt[rt][r];
+        }
+      if (diag) {   // (wave-uniform) a query may not lie before the key
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (trow(r, hh) < i) sc[NA - 1][r] = pt[NA - 1][r] = 0.f;
+      }
+      // own keys x channels: dv += f^T (keys x queries) . g,   dk += W^T . q
+      static_for<NFA>([&](auto ftag) {
+        constexpr int F = decltype(ftag)::value;
+        Frag bg[CB], bq[CB], fa[RT], wa[RT];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+          bg[cb] = lds_frag<T>(gtl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
+          bq[cb] = lds_frag<T>(qtl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
+        }
+#pragma unroll
+        for (int rt = 0; rt < NA; ++rt) {
+          fa[rt] = M::template from_acc<F>(sc[rt]);
+          wa[rt] = M::template from_acc<F>(pt[rt]);
+        }
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+          for (int rt = 0; rt < NA; ++rt) {
+            dv[rt][cb] = M::mma(fa[rt], bg[cb], dv[rt][cb]);
+            dk[rt][cb] = M::mma(wa[rt], bq[cb], dk[rt][cb]);
+          }
+      });
+    };
+    const int k00 = tok0 + w * RT * 32;   // first position of the wave's own tile 0
     for (int st = st0; st < nst; ++st) {
       const int buf = (st - st0) & 1;
       if (st + 1 < nst) stage_load(st + 1);
@@ -641,77 +726,17 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
       const Elt* qtl = Qt + buf * L::TR;
       const Elt* gtl = Gt + buf * L::TR;
       const float* cl = Cl + buf * BN;
-#pragma unroll
+#pragma unroll 1
       for (int t32 = 0; t32 < BN / 32; ++t32) {
+        __builtin_amdgcn_sched_barrier(0);   // (tiles are not interleaved: register pressure)
         const int qb = st * BN + t32 * 32;
-        if (qb >= npos) continue;
-        bool act[RT];
-        bool any = false;
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          act[rt] = !masked || qb >= tok0 + (w * RT + rt) * 32;
-          any = any || act[rt];
-        }
-        if (!any) continue;
-        // tiles with rows = queries trow(r, hh), lanes = own keys: sr and qs (g . v - c)
-        float cneg[16];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float4 c4 = *reinterpret_cast<const float4*>(cl + t32 * 32 + 8 * j + 4 * hh);
-          cneg[4 * j] = -c4.x; cneg[4 * j + 1] = -c4.y; cneg[4 * j + 2] = -c4.z; cneg[4 * j + 3] = -c4.w;
-        }
-        f16v sc[RT], pt[RT];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) pt[rt][r] = cneg[r];
-#pragma unroll
-        for (int m = 0; m < NF; ++m) {
-          const Frag aq = lds_frag<T>(ql + (t32 * 32 + i) * PR + KF * m + EPL * hh);
-          const Frag ag = lds_frag<T>(gl + (t32 * 32 + i) * PR + KF * m + EPL * hh);
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            if (act[rt]) {
-              sc[rt] = M::mma(aq, kf[rt][m], m == 0 ? kZero16 : sc[rt]);
-              pt[rt] = M::mma(ag, vf[rt][m], pt[rt]);
-            }
-        }
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          if (!act[rt]) continue;
-          const bool diag = masked && qb == tok0 + (w * RT + rt) * 32;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float s = sc[rt][r];
-            sc[rt][r] = a0 + s * (c1 + c2 * s);
-            pt[rt][r] = (a1 + b2 * s) * pt[rt][r];
-          }
-          if (diag) {   // a query may not lie before the key
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-              if (trow(r, hh) < i) sc[rt][r] = pt[rt][r] = 0.f;
-          }
-        }
-        // own keys x channels: dv += f^T (keys x queries) . g,   dk += W^T . q
-        static_for<NFA>([&](auto ftag) {
-          constexpr int F = decltype(ftag)::value;
-          Frag fa[RT], wa[RT];
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt) {
-            fa[rt] = M::template from_acc<F>(sc[rt]);
-            wa[rt] = M::template from_acc<F>(pt[rt]);
-          }
-#pragma unroll
-          for (int cb = 0; cb < CB; ++cb) {
-            const Frag bg = lds_frag<T>(gtl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
-            const Frag bq = lds_frag<T>(qtl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-              if (act[rt]) {
-                dv[rt][cb] = M::mma(fa[rt], bg, dv[rt][cb]);
-                dk[rt][cb] = M::mma(wa[rt], bq, dk[rt][cb]);
-              }
-          }
+        if (qb >= npos || (masked && qb < k00)) continue;
+        // own tiles that start at or before the queries see them
+        int na = RT;
+        if (masked && ((qb - k00) >> 5) + 1 < RT) na = ((qb - k00) >> 5) + 1;
+        const bool diag = masked && qb == k00 + (na - 1) * 32;
+        static_for<RT>([&](auto tag) {
+          if (na == decltype(tag)::value + 1) tile(tag, t32, diag, ql, gl, qtl, gtl, cl);
         });
       }
       if (st + 1 < nst) stage_store(buf ^ 1);
