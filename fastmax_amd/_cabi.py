@@ -29,7 +29,7 @@ EXPORTS = (
     "fastmax_saved_state_bytes", "fastmax_forward_saving", "fastmax_backward_saved", "fastmax_qkv_rope",
     "fastmax_noalloc_scratch_bytes", "fastmax_forward_noalloc",
     "fastmax_workspace_bytes_strided", "fastmax_workspace_min_bytes_strided", "fastmax_saved_state_bytes_strided",
-    "fastmax_forward_strided", "fastmax_backward_strided",
+    "fastmax_forward_strided", "fastmax_backward_strided", "fastmax_uses_dense_tiles",
 )
 
 KERNEL_NAMES = ("rowstat", "build", "fwd_apply", "bwd_prep", "bwd_dq", "bwd_dk", "bwd_dv", "norm_fix")
@@ -88,6 +88,8 @@ def load() -> C.CDLL:
     lib.fastmax_last_error.argtypes = []
     lib.fastmax_check_desc.restype = C.c_int
     lib.fastmax_check_desc.argtypes = [dp]
+    lib.fastmax_uses_dense_tiles.restype = C.c_int
+    lib.fastmax_uses_dense_tiles.argtypes = [dp]
     lib.fastmax_workspace_bytes.restype = sz
     lib.fastmax_workspace_bytes.argtypes = [dp, C.c_int]
     lib.fastmax_workspace_min_bytes.restype = sz

@@ -12,10 +12,12 @@ Differences from the reference, all deliberate:
   * CPU tensors with use_custom_gradient=True raise (the reference returns q unchanged,
     example.py:10-12);
   * bfloat16 inputs are accepted (bf16 matrix instructions, fp32 accumulation);
-  * head dimensions other than 32 and 64 (up to 64) run zero-padded to the next kernel size;
+  * every head dimension up to 128 is served: d = 32 and 64 by both kernel families, every other
+    whole number of 16-byte row pieces natively by the dense score-tile kernels, and whatever is left
+    (an odd d, or a d below 64 on a sequence long enough that the moment kernels at the next of their
+    sizes are cheaper) zero-padded -- exact: zero channels change neither q.k nor the row norms;
   * a key prefix (k, v longer than q: the first nk - nq keys are visible to every query, as in
-    fastmax_cuda_forward.cu:109-150) runs with zero query rows put in front of q -- exact, at the
-    price of nk/nq times the query-side work.
+    fastmax_cuda_forward.cu:109-150) is served by the kernels as it is.
 """
 from __future__ import annotations
 
@@ -24,7 +26,7 @@ import math
 
 import torch
 
-from . import _ext
+from . import _cabi, _ext
 
 
 # fraction of the free device memory the saved prefix states of one call may take
@@ -46,6 +48,27 @@ def _states_fit_bytes(ext, q5: torch.Tensor, k4: torch.Tensor, mask: bool, p: in
     return need <= SAVE_STATES_MEMORY_FRACTION * free
 
 
+def kernel_head_dim(d: int, dtype: torch.dtype, bh: int, bhkv: int, nq: int, nk: int, mask: bool, p: int) -> int:
+    """The head dimension a call is handed to the library with (>= d; the difference is zero padding).
+    32 and 64 go as they are.  Any other d is first rounded up to whole 16-byte row pieces, which the
+    dense score-tile kernels take natively; but their cost grows with nq * nk, so when d is below 64 and
+    the library itself would take the moment kernels at the next moment-kernel size (32 or 64) for this
+    sequence length, the call is padded up to that size instead."""
+    if d in (32, 64):
+        return d
+    if d > 128:
+        raise ValueError(f"head dimension {d} is not supported (the kernels hold up to 128 channels per row)")
+    step = 8 if dtype == torch.bfloat16 else 4
+    native = -(-d // step) * step
+    if native < 64:
+        moment = 32 if native <= 32 else 64
+        code = _cabi.FASTMAX_BF16 if dtype == torch.bfloat16 else _cabi.FASTMAX_F32
+        ds = _cabi.make_desc(bh, nq, moment, code, mask, True, p, bhkv=bhkv, nk=nk)
+        if _cabi.load().fastmax_uses_dense_tiles(_cabi.C.byref(ds)) == 0:
+            return moment
+    return native
+
+
 class FASTMultiHeadAttention_Function(torch.autograd.Function):
     """Same call signature as example.py:8 / model.py:22."""
 
@@ -61,14 +84,12 @@ class FASTMultiHeadAttention_Function(torch.autograd.Function):
                              "If 3D: (b*h,n,d), if 4D: (b,h,n,d).")
         shape = q.shape
         d = q.shape[-1]
-        if d > 64:
-            raise ValueError(f"head dimension {d} is not supported (kernels exist for d <= 64)")
-        pad = (32 if d <= 32 else 64) - d
         if k.shape[-1] != d or v.shape[-1] != d:
             raise ValueError(f"q, k and v must share the head dimension (got {d}, {k.shape[-1]}, {v.shape[-1]})")
         q3 = q.reshape(-1, q.shape[-2], d)
         k3 = k.reshape(-1, k.shape[-2], d)
         v3 = v.reshape(-1, v.shape[-2], d)
+        pad = kernel_head_dim(d, q.dtype, q3.shape[0], k3.shape[0], q3.shape[1], k3.shape[1], bool(mask), int(p)) - d
         if pad:
             # zero channels change neither q.k nor the row norms, and give zero output columns
             q3, k3, v3 = (torch.nn.functional.pad(t, (0, pad)) for t in (q3, k3, v3))

@@ -365,8 +365,11 @@ int64_t saved_state_bytes_strided(torch::Tensor q, torch::Tensor k, bool mask, i
   const fastmax_desc ds = make_desc5(q, k, mask, false, 1.0, 1.0, 1.0, 0.5, 1.0, p);
   fastmax_layout lay{};
   lay.groups = (int32_t)q.size(1);
-  lay.q = lay.o = strides5(q, "q");
+  lay.q = strides5(q, "q");
   lay.k = lay.v = strides4(k, "k");
+  // the output forward_strided writes: token-major (B, T, G, R, D) memory seen as (B, G, R, T, D)
+  const int64_t G = q.size(1), R = q.size(2), T = q.size(3), D = q.size(4);
+  lay.o = fastmax_strides{T * G * R * D, R * D, D, G * R * D};
   const size_t sb = fastmax_saved_state_bytes_strided(&ds, &lay);
   TORCH_CHECK(sb > 0, "fastmax: ", fastmax_last_error());
   return (int64_t)sb;

@@ -136,7 +136,10 @@ bool use_linear_scan(const fastmax_desc* ds, const Plan& pl);
 
 // Dense score tiles cost 2 n d flop per token under the mask (4 n d without it), the moment form about
 // 2.1 d^3 (p = 2) whatever n is: below these key counts the dense kernels are the faster ones (measured,
-// forward + backward).  Head dimensions without moment kernels always take them.
+// forward + backward, 96 and 768 heads; with few heads the sequential state build of the moment form
+// fills the chip badly and the dense kernels stay ahead for longer).  A causal sequence of a single chunk
+// has no states to build either way and stays with the moment kernels' own intra-chunk tiles.  Head
+// dimensions without moment kernels always take the dense ones.
 bool use_dense(const fastmax_desc* ds) {
   if (ds->d != 32 && ds->d != 64) return true;
   // FASTMAX_PATH = moments | dense overrides the choice where both kernel families exist
@@ -147,9 +150,14 @@ bool use_dense(const fastmax_desc* ds) {
   if (ds->p != 2) return false;
   const bool bf = ds->dtype == FASTMAX_BF16;
   int limit;
-  if (ds->d == 64) limit = bf ? 4096 : 2048;
-  else limit = bf ? 1024 : 512;
-  if (!ds->mask) limit /= 2;
+  if (ds->d == 64) {
+    if (ds->mask) limit = bf ? (ds->bh <= 128 ? 4096 : 3072) : 2560;
+    else limit = bf ? 1536 : 1024;
+  } else {
+    if (ds->mask) limit = bf ? 1536 : 1024;
+    else limit = bf ? 768 : 512;
+  }
+  if (ds->mask && ds->nk <= chunk_for(ds->d, 1, ds->dtype)) return false;
   return ds->nk <= limit;
 }
 
@@ -484,6 +492,19 @@ inline int finish_state_fp32(const Plan& pl, int heads, float* state, hipStream_
   return pl.nparts;
 }
 
+// Unmasked p = 1 with bf16 tensors has two consumers of a kept state: the chunked kernels read the packed
+// form in the head's last slot, the row passes the fp32 sum.  A forward pass that keeps its states leaves
+// both (the sum in slot 0, over the first partial state), so that a backward pass may take either family
+// whatever the forward pass took.  `state` holds the fp32 partial states of `heads` heads.
+template <int D>
+inline void finish_state_both(const Plan& pl, int heads, float* state, hipStream_t stream) {
+  const int64_t ss = pl.state_floats;
+  state_pack_kernel<D><<<dim3(PackedGeo<D>::nslab(pl.p2), heads), 256, 0, stream>>>(state, pl.nslots, pl.nparts, pl.p2);
+  if (pl.nparts > 1)
+    state_accumulate_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads), 256, 0, stream>>>(
+        state, (int64_t)pl.nslots * ss, state, pl.nslots, pl.nparts, ss, 0);
+}
+
 template <int D, class T>
 int forward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v, T* o,
                  float* den, int64_t den_stride, float* scale_out, int32_t* arg_out,
@@ -529,7 +550,9 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const 
         FM_TRY((launch_build<D, T>(pl, heads, n, mk_rows(k, L.k, kv0), mk_rows(v, L.v, kv0), scale + bh + kv0, kNoScalars,
                                    kNoScalars, state, 0, stream, false)));
         (void)koff;
-        const int slot = finish_state_fp32(pl, heads, state, stream);
+        int slot = 0;
+        if (saved && kBf16Mfma<T>) finish_state_both<D>(pl, heads, state, stream);
+        else slot = finish_state_fp32(pl, heads, state, stream);
         ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
         const dim3 rgrid((n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE, heads);
 #define FM_ROWFWD(AL)                                                                                          \
@@ -550,6 +573,14 @@ int forward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const 
                            : reinterpret_cast<float*>(ws + pl.fixed_bytes + (size_t)hb * (pl.per_head_bytes - pl.scratch_bytes));
     FM_TRY((launch_build<D, T>(pl, heads / ratio, nk, kr, vr, scale + bh + kv0, kNoScalars, kNoScalars, state, 0,
                                stream, true, scratch)));
+    if constexpr (D == 64 && kBf16Mfma<T>) {
+      // (kept states of unmasked p = 1: also the fp32 sum a row-pass backward would read)
+      if (saved && !pl.masked && !pl.p2 && pl.nparts > 1) {
+        const int64_t ss = pl.state_floats;
+        state_accumulate_kernel<<<dim3((unsigned)((ss / 4 + 255) / 256), heads / ratio), 256, 0, stream>>>(
+            state, (int64_t)pl.nslots * ss, state, pl.nslots, pl.nparts, ss, 0);
+      }
+    }
     {
       ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
       const dim3 agrid(pl.nblk_q, heads);
@@ -683,7 +714,8 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
         // states of the whole sequence in fp32 (S as the forward pass left it when it was kept), then one
         // pass over the rows per gradient
         const int64_t ss = pl.state_floats, hf = (int64_t)pl.nslots * ss;
-        int slot = pl.nparts > 1 ? pl.nparts : 0;
+        // (kept bf16 states carry their fp32 sum in slot 0, the packed form in the last slot)
+        int slot = (pl.nparts > 1 && !(saved && kBf16Mfma<T>)) ? pl.nparts : 0;
         if (!saved) {
           FM_TRY((launch_build<D, T>(pl, heads, n, mk_rows(k, L.k, kv0), mk_rows(v, L.v, kv0), scale + bh + kv0,
                                      kNoScalars, kNoScalars, state, 0, stream, false)));
@@ -692,7 +724,7 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
         FM_TRY((launch_build<D, T>(pl, heads, n, mk_rows(q, L.q, h0), mk_rows(go, L.go, h0), scale + h0,
                                    mk_scalars(den, n, den_stride, h0), mk_scalars<const float>(cvec, n, 1, h0), stR, 1,
                                    stream, false)));
-        finish_state_fp32(pl, heads, stR, stream);
+        const int slot_r = finish_state_fp32(pl, heads, stR, stream);
         const int nrb = (n + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE;
         const dim3 rgrid(nrb, heads);
         {
@@ -710,14 +742,14 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
         {
           ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
           lin::linear_rowpass_kernel<T, lin::ROWPASS_DK, false, true><<<rgrid, 64, 0, stream>>>(
-              v + koff, stR + slot * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dk + toff, D, nullptr,
+              v + koff, stR + slot_r * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dk + toff, D, nullptr,
               nullptr, n, ds->a0, ds->a1);
         }
         FM_TRY(launch_status("linear_rowpass_kernel (dk)"));
         {
           ScopedKernel sk(FASTMAX_K_BWD_DV, stream);
           lin::linear_rowpass_kernel<T, lin::ROWPASS_DV, false, true><<<rgrid, 64, 0, stream>>>(
-              k + koff, stR + slot * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dv + toff, D, nullptr,
+              k + koff, stR + slot_r * ss, hf, scale + bh + kv0, nullptr, 0, nullptr, nullptr, dv + toff, D, nullptr,
               nullptr, n, ds->a0, ds->a1);
         }
         FM_TRY(launch_status("linear_rowpass_kernel (dv)"));
@@ -1087,6 +1119,12 @@ int fastmax_check_desc(const fastmax_desc* desc) {
   return check_desc(desc);
 }
 
+int fastmax_uses_dense_tiles(const fastmax_desc* desc) {
+  g_err[0] = 0;
+  FM_TRY(check_desc(desc));
+  return use_dense(desc) ? 1 : 0;
+}
+
 // (a layout only matters through "plain or not": plain tensors may take the register-resident
 // p = 1 paths, which need no state memory)
 static bool layout_is_plain(const fastmax_desc* desc, const fastmax_layout* layout, bool backward) {
@@ -1235,6 +1273,17 @@ static int backward_entry(const fastmax_desc* desc, const fastmax_layout* layout
   FM_TRY(resolve_layout(desc, layout, ldo, true, &L));
   FM_TRY(check_spans(desc, L, den_stride, true));
   const Plan pl = make_plan(desc, FASTMAX_PASS_BACKWARD, is_plain(L, desc, true));
+  if (saved_states) {
+    // The kept states are only usable when the forward pass that wrote them (planned on q, k, v, o alone) wrote
+    // kept states at all: the register-resident scan and the dense kernels keep nothing (a 256-byte token),
+    // and this pass, which also looks at grad_output and the gradients, may plan differently.  Then it
+    // rebuilds its states.  (The row passes and the chunked kernels of unmasked p = 1 read the same buffer.)
+    const Plan plf = make_plan(desc, FASTMAX_PASS_FORWARD, is_plain(L, desc, false));
+    if (plf.scan != pl.scan || plf.dense != pl.dense) {
+      saved_states = nullptr;
+      saved_bytes = 0;
+    }
+  }
   FM_TRY(check_ws(pl, workspace, workspace_bytes, saved_states != nullptr));
   FM_TRY(check_saved(pl, saved_states, saved_bytes));
   char* ws = static_cast<char*>(workspace);

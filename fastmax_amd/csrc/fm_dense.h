@@ -296,12 +296,18 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
       for (int r = 0; r < 16; ++r) acc[rt][cb][r] = 0.f;
   }
 
-  // One 32-key tile against the wave's own tiles RT0 .. RT-1 (under the mask the tiles before RT0 lie
-  // wholly before the keys), as straight-line code.  diag: it is the diagonal tile of own tile RT0;
-  // tail: (unmasked) it holds keys past the end -- only those tiles pay for per-element tests.
-  auto tile = [&](auto rt0tag, int t32, int kb, bool diag, bool tail, const Elt* kl, const Elt* vl)
-                  __attribute__((always_inline)) {
-    constexpr int RT0 = decltype(rt0tag)::value;
+  // One 32-key tile against the wave's own tiles, as straight-line code.  rel = key tile base - first
+  // position of own tile 0 (a multiple of 32; masked only): own tile rt has the key tile on its diagonal
+  // when rel == 32 rt and wholly after its queries when rel > 32 rt (its weights are then zeroed; this
+  // happens once per wave, and one code path keeps the accumulators in place).  tail: (unmasked) the tile
+  // holds keys past the end.  Only those tiles pay for per-element tests.
+  auto tile = [&](int t32, int kb, int rel, bool tail, const Elt* kl, const Elt* vl) __attribute__((always_inline)) {
+    // (the value fragments are requested first: they arrive under the score tile's work)
+    Frag vb[NFA][CB];
+#pragma unroll
+    for (int f = 0; f < NFA; ++f)
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) vb[f][cb] = lds_frag<T>(vl + (cb * 32 + i) * PT + t32 * 32 + KF * f + EPL * hh);
     // scores, transposed: rows = keys trow(r, hh), lanes = own queries
     f16v sc[RT];
 #pragma unroll
@@ -312,42 +318,40 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
 #pragma unroll
       for (int m = 0; m < HC; ++m)
 #pragma unroll
-        for (int rt = RT0; rt < RT; ++rt) sc[rt] = M::mma(ka[m], qf[rt][m0 + m], m0 + m == 0 ? kZero16 : sc[rt]);
+        for (int rt = 0; rt < RT; ++rt) sc[rt] = M::mma(ka[m], qf[rt][m0 + m], m0 + m == 0 ? kZero16 : sc[rt]);
     }
 #pragma unroll
-    for (int rt = RT0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float s = sc[rt][r];
         sc[rt][r] = a0 + s * (a1 + a2 * s);
       }
-    if (diag) {   // (wave-uniform) a key may not lie after the query
+      if (masked && rel >= 32 * rt) {   // (wave-uniform) a key may not lie after the query
+        const int lim = rel > 32 * rt ? -1 : i;
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        if (trow(r, hh) > i) sc[RT0][r] = 0.f;
-    }
-    if (tail) {   // (wave-uniform) keys past the end
-#pragma unroll
-      for (int rt = RT0; rt < RT; ++rt)
+        for (int r = 0; r < 16; ++r)
+          if (trow(r, hh) > lim) sc[rt][r] = 0.f;
+      }
+      if (tail) {   // (wave-uniform) keys past the end
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           if (kb + trow(r, hh) >= nk) sc[rt][r] = 0.f;
+      }
     }
     // own rows x channels += f(scores) (own x keys) . V (keys x channels)
     static_for<NFA>([&](auto ftag) {
       constexpr int F = decltype(ftag)::value;
-      Frag vb[CB], wa[RT];
+      Frag wa[RT];
 #pragma unroll
-      for (int cb = 0; cb < CB; ++cb) vb[cb] = lds_frag<T>(vl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
-#pragma unroll
-      for (int rt = RT0; rt < RT; ++rt) {
+      for (int rt = 0; rt < RT; ++rt) {
         wa[rt] = M::template from_acc<F>(sc[rt]);
         dn[rt] = M::fsum(wa[rt], dn[rt]);
       }
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-        for (int rt = RT0; rt < RT; ++rt) acc[rt][cb] = M::mma(wa[rt], vb[cb], acc[rt][cb]);
+        for (int rt = 0; rt < RT; ++rt) acc[rt][cb] = M::mma(wa[rt], vb[F][cb], acc[rt][cb]);
     });
   };
 
@@ -365,12 +369,8 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
       __builtin_amdgcn_sched_barrier(0);   // (tiles are not interleaved: register pressure)
       const int kb = st * BN + t32 * 32;
       if (kb >= kend) continue;
-      const int rt0 = (masked && kb > q00) ? (kb - q00) >> 5 : 0;   // own tiles that start before the keys see none of them
-      if (rt0 >= RT) continue;
-      const bool diag = masked && kb == q00 + rt0 * 32, tail = !masked && kb + 32 > nk;
-      static_for<RT>([&](auto tag) {
-        if (rt0 == decltype(tag)::value) tile(tag, t32, kb, diag, tail, kl, vl);
-      });
+      if (masked && kb > q00 + 32 * (RT - 1)) continue;   // after every own query
+      tile(t32, kb, kb - q00, !masked && kb + 32 > nk, kl, vl);
     }
     if (st + 1 < nst) stage_store(buf ^ 1);
     __syncthreads();
@@ -465,13 +465,13 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rt][cb][r] = 0.f;
 
-  auto tile = [&](auto rt0tag, int t32, bool diag, const Elt* kl, const Elt* vl, const Elt* ktl)
-                  __attribute__((always_inline)) {
-    constexpr int RT0 = decltype(rt0tag)::value;   // (diag: the diagonal tile of own tile RT0)
+  // (rel as in the forward kernel: own tile rt has the key tile on its diagonal when rel == 32 rt and
+  // wholly after its queries when rel > 32 rt)
+  auto tile = [&](int t32, int rel, const Elt* kl, const Elt* vl, const Elt* ktl) __attribute__((always_inline)) {
     // transposed tiles (rows = keys, lanes = own queries): f'(s) and g . v - c
     f16v sc[RT], pt[RT];
 #pragma unroll
-    for (int rt = RT0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         sc[rt][r] = a1;
@@ -488,19 +488,21 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
 #pragma unroll
       for (int m = 0; m < HC; ++m)
 #pragma unroll
-        for (int rt = RT0; rt < RT; ++rt) {
+        for (int rt = 0; rt < RT; ++rt) {
           pt[rt] = M::mma(va[m], gf[rt][m0 + m], pt[rt]);
           if (p2) sc[rt] = M::mma(ka[m], qf[rt][m0 + m], sc[rt]);
         }
     }
 #pragma unroll
-    for (int rt = RT0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) pt[rt][r] = sc[rt][r] * pt[rt][r];
-    if (diag) {   // (wave-uniform) a key may not lie after the query
+      if (masked && rel >= 32 * rt) {   // (wave-uniform) a key may not lie after the query
+        const int lim = rel > 32 * rt ? -1 : i;
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        if (trow(r, hh) > i) pt[RT0][r] = 0.f;
+        for (int r = 0; r < 16; ++r)
+          if (trow(r, hh) > lim) pt[rt][r] = 0.f;
+      }
     }
     // own rows x channels += W (own x keys) . K (keys x channels)
     static_for<NFA>([&](auto ftag) {
@@ -509,11 +511,11 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) kb_[cb] = lds_frag<T>(ktl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
 #pragma unroll
-      for (int rt = RT0; rt < RT; ++rt) wa[rt] = M::template from_acc<F>(pt[rt]);
+      for (int rt = 0; rt < RT; ++rt) wa[rt] = M::template from_acc<F>(pt[rt]);
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-        for (int rt = RT0; rt < RT; ++rt) acc[rt][cb] = M::mma(wa[rt], kb_[cb], acc[rt][cb]);
+        for (int rt = 0; rt < RT; ++rt) acc[rt][cb] = M::mma(wa[rt], kb_[cb], acc[rt][cb]);
     });
   };
 
@@ -532,12 +534,8 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
       __builtin_amdgcn_sched_barrier(0);   // (tiles are not interleaved: register pressure)
       const int kb = st * BN + t32 * 32;
       if (kb >= kend) continue;
-      const int rt0 = (masked && kb > q00) ? (kb - q00) >> 5 : 0;
-      if (rt0 >= RT) continue;
-      const bool diag = masked && kb == q00 + rt0 * 32;
-      static_for<RT>([&](auto tag) {
-        if (rt0 == decltype(tag)::value) tile(tag, t32, diag, kl, vl, ktl);
-      });
+      if (masked && kb > q00 + 32 * (RT - 1)) continue;   // after every own query
+      tile(t32, kb - q00, kl, vl, ktl);
     }
     if (st + 1 < nst) stage_store(buf ^ 1);
     __syncthreads();
@@ -650,18 +648,18 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
       stage_store(0);
     }
     __syncthreads();
-    // One 32-query tile against the wave's own key tiles 0 .. NA-1 (under the mask the tiles after them lie
-    // wholly after the queries), as straight-line code; diag: it is the diagonal tile of own tile NA-1.
-    auto tile = [&](auto natag, int t32, bool diag, const Elt* ql, const Elt* gl, const Elt* qtl, const Elt* gtl,
-                    const float* cl) __attribute__((always_inline)) {
-      constexpr int NA = decltype(natag)::value + 1;
+    // One 32-query tile against the wave's own key tiles, as straight-line code.  rel = query tile base -
+    // first position of own tile 0 (masked only): own tile rt has the query tile on its diagonal when
+    // rel == 32 rt and wholly before its keys when rel < 32 rt (its weights are then zeroed).
+    auto tile = [&](int t32, int rel, const Elt* ql, const Elt* gl, const Elt* qtl, const Elt* gtl, const float* cl)
+                    __attribute__((always_inline)) {
       // tiles with rows = queries trow(r, hh), lanes = own keys: sr and qs (g . v - c)
       f16v sc[RT], pt[RT];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const float4 c4 = *reinterpret_cast<const float4*>(cl + t32 * 32 + 8 * j + 4 * hh);
 #pragma unroll
-        for (int rt = 0; rt < NA; ++rt) {
+        for (int rt = 0; rt < RT; ++rt) {
           pt[rt][4 * j] = -c4.x; pt[rt][4 * j + 1] = -c4.y; pt[rt][4 * j + 2] = -c4.z; pt[rt][4 * j + 3] = -c4.w;
         }
       }
@@ -676,23 +674,25 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
 #pragma unroll
         for (int m = 0; m < HC; ++m)
 #pragma unroll
-          for (int rt = 0; rt < NA; ++rt) {
+          for (int rt = 0; rt < RT; ++rt) {
             sc[rt] = M::mma(qa[m], kf[rt][m0 + m], m0 + m == 0 ? kZero16 : sc[rt]);
             pt[rt] = M::mma(ga[m], vf[rt][m0 + m], pt[rt]);
           }
       }
 #pragma unroll
-      for (int rt = 0; rt < NA; ++rt)
+      for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float s = sc[rt][r];
           sc[rt][r] = a0 + s * (c1 + c2 * s);
           pt[rt][r] = (a1 + b2 * s) * pt[rt][r];
         }
-      if (diag) {   // (wave-uniform) a query may not lie before the key
+        if (masked && rel <= 32 * rt) {   // (wave-uniform) a query may not lie before the key
+          const int lim = rel < 32 * rt ? 32 : i;
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if (trow(r, hh) < i) sc[NA - 1][r] = pt[NA - 1][r] = 0.f;
+          for (int r = 0; r < 16; ++r)
+            if (trow(r, hh) < lim) sc[rt][r] = pt[rt][r] = 0.f;
+        }
       }
       // own keys x channels: dv += f^T (keys x queries) . g,   dk += W^T . q
       static_for<NFA>([&](auto ftag) {
@@ -704,14 +704,14 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
           bq[cb] = lds_frag<T>(qtl + (cb * 32 + i) * PT + t32 * 32 + KF * F + EPL * hh);
         }
 #pragma unroll
-        for (int rt = 0; rt < NA; ++rt) {
+        for (int rt = 0; rt < RT; ++rt) {
           fa[rt] = M::template from_acc<F>(sc[rt]);
           wa[rt] = M::template from_acc<F>(pt[rt]);
         }
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-          for (int rt = 0; rt < NA; ++rt) {
+          for (int rt = 0; rt < RT; ++rt) {
             dv[rt][cb] = M::mma(fa[rt], bg[cb], dv[rt][cb]);
             dk[rt][cb] = M::mma(wa[rt], bq[cb], dk[rt][cb]);
           }
@@ -731,13 +731,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
         __builtin_amdgcn_sched_barrier(0);   // (tiles are not interleaved: register pressure)
         const int qb = st * BN + t32 * 32;
         if (qb >= npos || (masked && qb < k00)) continue;
-        // own tiles that start at or before the queries see them
-        int na = RT;
-        if (masked && ((qb - k00) >> 5) + 1 < RT) na = ((qb - k00) >> 5) + 1;
-        const bool diag = masked && qb == k00 + (na - 1) * 32;
-        static_for<RT>([&](auto tag) {
-          if (na == decltype(tag)::value + 1) tile(tag, t32, diag, ql, gl, qtl, gtl, cl);
-        });
+        tile(t32, qb - k00, ql, gl, qtl, gtl, cl);
       }
       if (st + 1 < nst) stage_store(buf ^ 1);
       __syncthreads();

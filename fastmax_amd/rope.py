@@ -131,8 +131,10 @@ class _QKVAttention(torch.autograd.Function):
         q5, k4, v4, o5, den, scale, arg, saved, cos, sin = ctx.saved_tensors
         groups, q_per_kv, hs, rope_n = ctx.geo
         b, t, _ = ctx.shape
-        go5 = gy.contiguous().view(b, t, groups, q_per_kv, hs).permute(0, 2, 3, 1, 4)
-        dqkv = torch.empty(ctx.shape, dtype=gy.dtype, device=gy.device)
+        # the kernels work in the projection's dtype: an upstream gradient of another dtype (an output
+        # cast outside autocast, say) is brought to it, and the result goes back in the caller's
+        go5 = gy.to(q5.dtype).contiguous().view(b, t, groups, q_per_kv, hs).permute(0, 2, 3, 1, 4)
+        dqkv = torch.empty(ctx.shape, dtype=q5.dtype, device=gy.device)
         dq5, dk4, dv4 = _views(dqkv, groups, q_per_kv, hs)
         ext.backward_strided(q5, k4, v4, o5, den, go5, scale, arg, dq5, dk4, dv4, *ctx.cfg, saved)
         rope_inplace(dqkv, cos, sin, groups, q_per_kv, hs, rope_n, grad=True)
@@ -151,6 +153,10 @@ def qkv_attention(qkv: torch.Tensor, cos, sin, groups: int, q_per_kv: int, hs: i
     if not qkv.is_contiguous():
         raise RuntimeError("qkv_attention: the packed projection must be contiguous")
     _desc(qkv, groups, q_per_kv, hs, rope_n)   # shape and dtype checks
+    step = 8 if qkv.dtype == torch.bfloat16 else 4
+    if hs % step or not 0 < hs <= 128:
+        raise ValueError(f"qkv_attention: head size {hs} must be a multiple of {step} (16 bytes of a row) up to 128; "
+                         "the strided views of the packed projection cannot be padded")
     if rope_n:
         t = qkv.shape[1]
         if cos.shape != (t, rope_n) or sin.shape != (t, rope_n):

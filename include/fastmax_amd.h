@@ -62,11 +62,12 @@ typedef struct fastmax_desc {
   int32_t nq;          /* query tokens                                                   */
   int32_t nk;          /* key tokens; mask != 0: nk >= nq, the first nk - nq keys are a
                           prefix every query sees (fastmax_cuda_forward.cu:109-150)      */
-  int32_t d;           /* head dimension: 32 or 64 (the reference's kernels take d at run
-                          time, fastmax_cuda_forward.cu:331-338; this library's kernels keep
-                          a head's state tiles in registers and exist for these two sizes
-                          only -- d = 128 is deliberately not built, other d <= 64 are
-                          zero-padded by the Python module)                              */
+  int32_t d;           /* head dimension, read at run time like the reference's launcher does
+                          (fastmax_cuda_forward.cu:331-338): any whole number of 16-byte
+                          pieces of a row (a multiple of 4 for fp32, of 8 for bf16) up to
+                          128.  d = 32 and 64 have both kernel families (moment states,
+                          linear in n; dense score tiles for short sequences); every other
+                          d runs on the dense score tiles, whose cost grows with nq * nk   */
   int32_t dtype;       /* FASTMAX_F32 or FASTMAX_BF16 (bf16 in/out, fp32 accumulation)    */
   int32_t mask;        /* 0: every key visible, 1: causal (j <= i)                       */
   int32_t normalize;   /* 1: x <- lim * x / max_n ||x_n||_2 per head for q and k,
@@ -88,6 +89,13 @@ const char* fastmax_last_error(void);
 /* Checks a descriptor without touching the device.  Replaces the shape reads and the
  * implicit assumptions of fastmax_cuda_forward.cu:331-345 (d == 64). */
 int fastmax_check_desc(const fastmax_desc* desc);
+
+/* Which kernel family a descriptor runs on: 1 = dense score tiles (no states, no state memory, work
+ * ~ nq * nk * d), 0 = moment states (work ~ n * d^3 for p = 2), negative = bad descriptor.  d = 32 and
+ * 64 have both and the library picks the faster one by sequence length; the environment variable
+ * FASTMAX_PATH = moments | dense overrides that choice (read at every call).  No counterpart in the
+ * reference, whose kernels are the moment form only (fastmax_cuda_forward.cu:25-197). */
+int fastmax_uses_dense_tiles(const fastmax_desc* desc);
 
 /* Bytes of device workspace that let a pass run all heads in as few batches as a 16 GiB
  * budget allows (the passes accept anything >= fastmax_workspace_min_bytes and then loop

@@ -33,7 +33,7 @@ def test_version_and_clean_error(built):
 
 
 @pytest.mark.parametrize("over,code", [
-    (dict(d=48), -2), (dict(d=128), -2), (dict(bh=0), -2), (dict(bhkv=3), -2), (dict(bhkv=0), -2), (dict(nk=50), -2), (dict(n=0), -2),
+    (dict(d=50), -2), (dict(d=132), -2), (dict(d=0), -2), (dict(d=12, dtype=1), -2), (dict(bh=0), -2), (dict(bhkv=3), -2), (dict(bhkv=0), -2), (dict(nk=50), -2), (dict(n=0), -2),
     (dict(dtype=7), -3), (dict(p=3), -4), (dict(p=0), -4), (dict(lim=0.0), -4),
     (dict(normalize=False, temperature=0.0), -4),
 ])
@@ -41,6 +41,31 @@ def test_bad_descriptors(built, over, code):
     assert built.fastmax_check_desc(C.byref(desc(**over))) == code
     assert _cabi.last_error() != ""
     assert built.fastmax_workspace_bytes(C.byref(desc(**over)), _cabi.PASS_FORWARD) == 0
+
+
+def test_head_dimensions_and_the_dense_plan(built, monkeypatch):
+    """Any head dimension that is a whole number of 16-byte pieces up to 128 is served (the reference's
+    launcher reads d at run time, fastmax_cuda_forward.cu:331-338): dimensions other than 32 and 64 by
+    the dense score-tile kernels, which keep no states -- the workspace holds the per-head scalars (and,
+    backward, c_i and the normalisation partials) only.  Left to itself the library also takes those
+    kernels for short sequences at d = 32 / 64; the recurrent entry points keep moment states and so
+    stay with d = 32 / 64."""
+    for d, dtype in ((4, 0), (16, 0), (48, 0), (96, 0), (128, 0), (8, 1), (48, 1), (128, 1)):
+        ds = desc(d=d, dtype=dtype, bh=6, n=5000, mask=True)
+        assert built.fastmax_check_desc(C.byref(ds)) == 0, _cabi.last_error()
+        assert built.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD) == 512
+        assert built.fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_BACKWARD) == \
+            512 + (6 * 5000 * 4 + 255) // 256 * 256 + (6 * 2 * 40 * 4 + 255) // 256 * 256
+        assert built.fastmax_saved_state_bytes(C.byref(ds)) == 256
+        assert built.fastmax_state_bytes(C.byref(ds)) == 0 and "recurrent" in _cabi.last_error()
+    short, long_ = desc(bh=96, n=2048, dtype=1, mask=True), desc(bh=96, n=16384, dtype=1, mask=True)
+    assert built.fastmax_workspace_bytes(C.byref(short), _cabi.PASS_FORWARD) > 1 << 20   # (FASTMAX_PATH=moments here)
+    monkeypatch.delenv("FASTMAX_PATH")
+    assert built.fastmax_workspace_bytes(C.byref(short), _cabi.PASS_FORWARD) == 1536
+    assert built.fastmax_workspace_bytes(C.byref(long_), _cabi.PASS_FORWARD) > 1 << 20
+    assert built.fastmax_workspace_bytes(C.byref(desc(bh=96, n=2048, dtype=1, mask=True, p=1)), _cabi.PASS_FORWARD) > 1 << 20
+    monkeypatch.setenv("FASTMAX_PATH", "dense")
+    assert built.fastmax_workspace_bytes(C.byref(long_), _cabi.PASS_FORWARD) == 1536
 
 
 def test_grouped_heads_descriptor(built):

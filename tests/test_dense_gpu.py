@@ -193,3 +193,60 @@ def test_config5_attention_shape_picks_the_dense_kernels(ops, monkeypatch, built
         ro, rdq, rdk, rdv = O.dense_truth(*(t[sl].float().cpu() for t in (q, k, v, go)), **kw)
         for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
             assert_close(f"head{h}/{name}", got[sl].float(), ref, 2e-2)
+
+
+@pytest.mark.parametrize("shape,mask,dtype", [
+    ((2, 2, 3, 2), True, torch.float32), ((1, 3, 200, 16), True, torch.float32), ((2, 2, 150, 48), True, torch.float32),
+    ((1, 2, 90, 20), False, torch.float32), ((1, 2, 300, 128), True, torch.float32), ((2, 2, 260, 96), False, torch.float32),
+    ((1, 2, 300, 128), True, torch.bfloat16), ((1, 2, 200, 100), True, torch.bfloat16), ((1, 2, 3000, 48), True, torch.float32),
+    ((2, 2, 600, 48), True, torch.float32),
+])
+def test_module_head_dims(built, monkeypatch, shape, mask, dtype):
+    """Through FASTMultiHeadAttention with the library's own choice of kernels: head dimensions that are
+    whole 16-byte row pieces go to the dense kernels as they are, others are zero-padded to the next such
+    size, and a d below 64 is padded up to the moment kernels' size instead where the library would take
+    those at that size (a long sequence, or a causal one of a single chunk)."""
+    from fastmax_amd import FASTMultiHeadAttention
+    from fastmax_amd.attention import kernel_head_dim
+
+    monkeypatch.delenv("FASTMAX_PATH", raising=False)
+    b, h, n, d = shape
+    expect = {2: 32, 16: 16, 48: 48 if 256 < n <= 2560 else 64, 20: 20, 128: 128, 96: 96, 100: 104}[d]
+    assert kernel_head_dim(d, dtype, b * h, b * h, n, n, mask, 2) == expect
+    q, k, v, go = O.seeded_inputs(shape, seed=24, dtype=dtype)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = FASTMultiHeadAttention()(qd, kd, vd, None, mask, 0.0, True)
+    assert o.shape == shape and o.dtype == dtype
+    o.backward(go.cuda())
+    ro, rdq, rdk, rdv = O.dense_truth(q.float(), k.float(), v.float(), go.float(), mask=mask, normalize=True)
+    for name, got, ref in (("o", o, ro), ("dq", qd.grad, rdq), ("dk", kd.grad, rdk), ("dv", vd.grad, rdv)):
+        assert got.shape == ref.shape
+        assert_close(name, got.float(), ref, TOL[dtype], atol=1e-6)
+
+
+def test_strided_views_of_a_fused_projection_d128(built):
+    """The strided entry points on the dense kernels: q, k, v as views into a fused (B, T, G (R + 2) hs)
+    projection with hs = 128, token-major output, gradients written into the projection's gradient --
+    the reference block's layout (model.py:474-499, 572-574, 603) at a head size its kernels never had."""
+    from fastmax_amd import rope as R
+
+    b, t, g, r, hs = 2, 300, 2, 2, 128
+    gen = torch.Generator().manual_seed(3)
+    qkv = torch.randn((b, t, g * (r + 2) * hs), generator=gen)
+    gy = torch.randn((b, t, g * r * hs), generator=gen)
+    x = qkv.cuda().requires_grad_(True)
+    y = R.qkv_attention(x, None, None, g, r, hs, rope_n=0, mask=True, normalize=True, p=2)
+    y.backward(gy.cuda())
+    v5 = qkv.view(b, t, g, r + 2, hs)
+    q = v5[:, :, :, :r].permute(0, 2, 3, 1, 4).reshape(b * g * r, t, hs)
+    k = v5[:, :, :, r].permute(0, 2, 1, 3).reshape(b * g, t, hs)
+    v = v5[:, :, :, r + 1].permute(0, 2, 1, 3).reshape(b * g, t, hs)
+    go = gy.view(b, t, g * r, hs).permute(0, 2, 1, 3).reshape(b * g * r, t, hs)
+    ke, ve = k.repeat_interleave(r, dim=0), v.repeat_interleave(r, dim=0)
+    ro, rdq, rdk, rdv = O.dense_truth(q, ke, ve, go, mask=True, normalize=True)
+    fold = lambda z: z.reshape(b * g, r, t, hs).sum(1)
+    assert_close("y", y.view(b, t, g * r, hs).permute(0, 2, 1, 3).reshape(b * g * r, t, hs), ro, 1e-4)
+    gx = x.grad.view(b, t, g, r + 2, hs)
+    assert_close("dq", gx[:, :, :, :r].permute(0, 2, 3, 1, 4).reshape(b * g * r, t, hs), rdq, 1e-4, atol=1e-6)
+    assert_close("dk", gx[:, :, :, r].permute(0, 2, 1, 3).reshape(b * g, t, hs), fold(rdk), 1e-4, atol=1e-6)
+    assert_close("dv", gx[:, :, :, r + 1].permute(0, 2, 1, 3).reshape(b * g, t, hs), fold(rdv), 1e-4, atol=1e-6)

@@ -398,8 +398,9 @@ def test_module_autograd_4d(built):
 @pytest.mark.parametrize("shape,mask", [((2, 2, 3, 2), True), ((2, 2, 3, 2), False), ((1, 3, 200, 16), True),
                                          ((2, 2, 150, 48), True), ((1, 2, 90, 20), False)])
 def test_module_other_head_dims(built, shape, mask):
-    """Head dims below 64 other than 32 run zero-padded; (2,2,3,2) is the reference's demo shape
-    (example.py:227-230)."""
+    """Head dims below 64 other than 32 run zero-padded on the moment kernels (this module pins
+    FASTMAX_PATH=moments; tests/test_dense_gpu.py covers the library's own choice); (2,2,3,2) is the
+    reference's demo shape (example.py:227-230)."""
     from fastmax_amd import FASTMultiHeadAttention
 
     q, k, v, go = O.seeded_inputs(shape, seed=24)
@@ -412,8 +413,8 @@ def test_module_other_head_dims(built, shape, mask):
         assert got.shape == ref.shape
         assert_close(name, got, ref, 1e-4, atol=1e-6)
     with pytest.raises(ValueError, match="head dimension"):
-        FASTMultiHeadAttention()(torch.zeros(1, 1, 4, 128, device="cuda"), torch.zeros(1, 1, 4, 128, device="cuda"),
-                                 torch.zeros(1, 1, 4, 128, device="cuda"))
+        FASTMultiHeadAttention()(torch.zeros(1, 1, 4, 132, device="cuda"), torch.zeros(1, 1, 4, 132, device="cuda"),
+                                 torch.zeros(1, 1, 4, 132, device="cuda"))
 
 
 def test_module_output_noise_dropout(built):

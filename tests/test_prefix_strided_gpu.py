@@ -177,3 +177,33 @@ def test_strided_layout_is_checked(built):
     short = _cabi.FastmaxStrides(64 * 64 * 4, 64 * 64, 0, 32)        # token stride below d
     lay = _cabi.FastmaxLayout(1, 0, st, short, st, st, st, st, st, st)
     assert lib.fastmax_forward_strided(C.byref(ds), C.byref(lay), *args) == -4
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float32, 1e-4)])
+def test_kept_states_of_a_plain_forward_with_a_strided_backward(built, dtype, tol):
+    """Unmasked p = 1 at d = 64: a forward pass on plain tensors takes the row-pass kernels and leaves
+    an fp32 state sum in the kept-state buffer; a backward pass that writes token-major gradients takes
+    the chunked kernels, which read packed slots.  The backward pass must notice and rebuild its states
+    rather than read the other family's format."""
+    from fastmax_amd import ops
+
+    b, h, t, d = 2, 3, 300, 64
+    gen = torch.Generator().manual_seed(65)
+    q, k, v = (torch.randn((b * h, t, d), generator=gen).to(dtype).cuda() for _ in range(3))
+    go_tm = torch.randn((b, t, h, d), generator=gen).to(dtype).cuda()
+    kw = dict(mask=False, normalize=True, p=1)
+    o, den, sc, arg, saved = ops.forward(q, k, v, save_states=True, **kw)
+    q4, k4, v4, o4 = (x.view(b, h, t, d) for x in (q, k, v, o))
+    go4 = go_tm.permute(0, 2, 1, 3)
+    dq, dk, dv = ops.backward_strided(q4, k4, v4, o4, den, go4, qk_scale=sc, qk_argmax=arg, saved_states=saved, **kw)
+    ro, rdq, rdk, rdv = O.dense_truth(q.float().cpu(), k.float().cpu(), v.float().cpu(),
+                                      go4.reshape(b * h, t, d).float().cpu(), **kw)
+    for name, got, ref in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert_close(name, got.reshape(ref.shape).float(), ref, tol)
+    # and the other way round: strided forward (chunked kernels, packed slots), plain backward (row passes)
+    o5, den2, sc2, arg2, saved2 = ops.forward_strided(q4, k4, v4, save_states=True, **kw)
+    oc = o5.reshape(b * h, t, d).contiguous()
+    dq2, dk2, dv2 = ops.backward(q, k, v, oc, den2, go4.reshape(b * h, t, d).contiguous(), qk_scale=sc2, qk_argmax=arg2,
+                                 saved_states=saved2, **kw)
+    for name, got, ref in (("dq", dq2, rdq), ("dk", dk2, rdk), ("dv", dv2, rdv)):
+        assert_close(name, got.float(), ref, tol)
