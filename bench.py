@@ -167,6 +167,32 @@ def executed_mfma_flops(cfg: dict, bh: int, chunk: int = 0) -> dict:
     return out
 
 
+def executed_dense_flops(cfg: dict, bh: int) -> dict:
+    """Flops of the matrix instructions the dense score-tile kernels issue (fm_dense.h): per pair of a
+    32-row own tile and a 32-row streamed tile one score contraction over the padded head dimension and one
+    product back onto it in the forward kernel, three contractions in dq (scores, g . v, W . k), four in the
+    fused dk / dv kernel.  Under the mask a wave skips the streamed tiles that lie wholly on the far side of
+    all its own tiles; the forward kernel's waves own two tiles and also run the one pair in which only the
+    second sees the keys."""
+    d, n, masked, bf = cfg["D"], cfg["N"], cfg["mask"], cfg["dtype"] == "bf16"
+    dp = -(-d // 32) * 32
+    per = 2 * 32 * 32 * dp
+    nt = -(-n // 32)
+
+    def pairs(rt):   # own tiles are dealt to waves rt at a time
+        if not masked:
+            return -(-nt // rt) * rt * nt
+        tot = 0
+        for w0 in range(0, nt, rt):
+            tot += rt * (min(w0 + rt, nt))   # streamed tiles 0 .. last own tile of the wave, for each of its tiles
+        return tot
+    rt_fwd = 2 if dp <= 64 else 1
+    rt_dq = 2 if (dp <= 32 and bf) else 1
+    p2 = cfg["p"] == 2
+    return {"fwd_apply": bh * pairs(rt_fwd) * 2 * per, "bwd_dq": bh * pairs(rt_dq) * (3 if p2 else 2) * per,
+            "bwd_dk": bh * pairs(1) * 4 * per, "build_fwd": 0, "build_bwd": 0, "bwd_dv": 0}
+
+
 def cpu_baseline(cfg: dict, seconds_hint: float) -> dict:
     """Reference-form fwd+bwd (oracle/fastmax_oracle.py::fastmax_reference_form, the op sequence of
     the reference's fastmax_function) on one head and a token prefix that fits in memory."""
@@ -230,6 +256,278 @@ def cpu_baseline(cfg: dict, seconds_hint: float) -> dict:
     }
 
 
+def measure(name: str, args, full: bool) -> dict:
+    """Times one workload (forward + backward steps through the C ABI, inputs resident in HBM) and returns its
+    record.  full: the headline run -- every field of the output line; otherwise the short record of the
+    `configs` block (times, rates, roofline position of the slowest kernel class, parity of one sampled head)."""
+    import torch
+    from fastmax_amd import _cabi, ops
+
+    cfg = dict(WORKLOADS[name])
+    if full and args.batch:
+        cfg["B"] = args.batch
+    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
+    bh = B * H
+    dtype = torch.float32 if cfg["dtype"] == "f32" else torch.bfloat16
+    dev = torch.device("cuda:0")
+    lib = _cabi.load()
+    steps, warmup = (args.steps, args.warmup) if full else (args.config_steps, 1)
+
+    gen = torch.Generator(device=dev).manual_seed(0)
+    q, k, v, go = (torch.randn((bh, N, D), generator=gen, device=dev, dtype=torch.float32).to(dtype)
+                   for _ in range(4))
+    kw = dict(mask=cfg["mask"], normalize=COEF["normalize"], lim=COEF["lim"], temperature=COEF["temperature"],
+              a0=COEF["a0"], a1=COEF["a1"], a2=COEF["a2"], p=cfg["p"])
+    ds = ops._desc(q, k, kw["mask"], kw["normalize"], kw["p"], kw["lim"], kw["temperature"], kw["a0"], kw["a1"], kw["a2"])
+    dense = lib.fastmax_uses_dense_tiles(C.byref(ds)) == 1
+    recompute = full and args.recompute_states
+
+    def fwd():
+        return ops.forward(q, k, v, **kw)
+
+    def step():
+        if recompute:
+            o, den, sc, arg = fwd()
+            return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+        # the forward pass leaves its prefix states behind for the backward pass
+        o, den, sc, arg, saved = ops.forward(q, k, v, save_states=True, **kw)
+        return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, saved_states=saved, **kw)
+
+    def step_outputs():
+        o, den, sc, arg = fwd()
+        return (o,) + tuple(ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw))
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    _cabi.check(lib.fastmax_profile_begin())
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kt = _cabi.KernelTimes()
+    _cabi.check(lib.fastmax_profile_end(C.byref(kt)))
+    ms_step = (t1 - t0) * 1e3 / steps
+
+    # forward alone, same inputs
+    fwd()
+    torch.cuda.synchronize()
+    _cabi.check(lib.fastmax_profile_begin())
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fwd()
+    torch.cuda.synchronize()
+    ms_fwd = (time.perf_counter() - t0) * 1e3 / steps
+    ktf = _cabi.KernelTimes()
+    _cabi.check(lib.fastmax_profile_end(C.byref(ktf)))
+
+    ms_graph = None
+    if full and args.hip_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        ms_graph = (time.perf_counter() - t0) * 1e3 / steps
+        del graph
+
+    ms_module = None
+    if full and args.through_module:
+        from fastmax_amd import FASTMultiHeadAttention
+        ops.release_workspaces()
+        mod = FASTMultiHeadAttention()
+        qm, km, vm = (t.view(B, H, N, D).requires_grad_(True) for t in (q, k, v))
+        gom = go.view(B, H, N, D)
+
+        def mstep():
+            o = mod(qm, km, vm, None, cfg["mask"], 0.0, COEF["normalize"], COEF["temperature"], COEF["a0"],
+                    COEF["a1"], COEF["a2"], COEF["lim"], cfg["p"])
+            o.backward(gom)
+            qm.grad = km.grad = vm.grad = None
+
+        for _ in range(warmup):
+            mstep()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            mstep()
+        torch.cuda.synchronize()
+        ms_module = (time.perf_counter() - t0) * 1e3 / steps
+
+    if full and args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
+    fl = algorithmic_flops(D, cfg["p"])
+    token_heads = bh * N
+    peak = PEAK_TFLOPS[cfg["dtype"]]
+    kernels = {}
+    for i, kname in enumerate(_cabi.KERNEL_NAMES):
+        if kt.launches[i]:
+            kernels[kname] = {"ms_per_step": kt.ms[i] / steps, "launches_per_step": kt.launches[i] / steps}
+    # Flops per step and kernel class, two ways.  "algorithmic": the reference-form count per token-head (every
+    # ordered channel pair).  "executed": what the matrix instructions of this build really issue (moment
+    # kernels: each unordered pair once, plus intra-chunk tiles, dummy tile slots and ragged tiles; dense
+    # kernels: every score tile they walk).  Both count the state builds the timed step runs: the forward
+    # prefix build and the backward suffix build, plus the backward prefix build when the states are rebuilt.
+    n_builds = 3 if recompute else 2
+    if dense:
+        # (the fused dk / dv kernel is timed as one class: both gradients' reference-form work is its)
+        algo = {"fwd_apply": fl["fwd"] * token_heads, "bwd_dq": (fl["bwd_dq"] + fl["build"]) * token_heads,
+                "bwd_dk": (fl["bwd_dk"] + fl["bwd_dv"] + fl["build"]) * token_heads}
+    else:
+        algo = {"build": n_builds * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
+                "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dk": fl["bwd_dk"] * token_heads,
+                "bwd_dv": fl["bwd_dv"] * token_heads}
+    executed = None
+    if dense:
+        ex = executed_dense_flops(cfg, bh)
+        executed = {kk: ex[kk] for kk in ("fwd_apply", "bwd_dq", "bwd_dk")}
+        ex_fwd = ex["fwd_apply"]
+    elif cfg["p"] == 2:
+        ex = executed_mfma_flops(cfg, bh)
+        executed = {"build": ex["build_fwd"] * (n_builds - 1) + ex["build_bwd"],
+                    **{kk: ex[kk] for kk in ("fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv")}}
+        ex_fwd = ex["build_fwd"] + ex["fwd_apply"]
+    for kname, f in algo.items():
+        if kname in kernels:
+            sec = kernels[kname]["ms_per_step"] * 1e-3
+            kernels[kname]["algorithmic_tflops"] = f / sec / 1e12
+            kernels[kname]["algorithmic_frac"] = f / sec / 1e12 / peak
+            if executed:
+                kernels[kname]["executed_tflops"] = executed[kname] / sec / 1e12
+                kernels[kname]["executed_frac"] = executed[kname] / sec / 1e12 / peak
+    step_summary = {"algorithmic_tflops": sum(algo.values()) / (ms_step * 1e-3) / 1e12}
+    step_summary["algorithmic_frac"] = step_summary["algorithmic_tflops"] / peak
+    fwd_summary = {"algorithmic_tflops": fl["fwd"] * token_heads / (ms_fwd * 1e-3) / 1e12}
+    fwd_summary["algorithmic_frac"] = fwd_summary["algorithmic_tflops"] / peak
+    if executed:
+        step_summary["executed_tflops"] = sum(executed.values()) / (ms_step * 1e-3) / 1e12
+        step_summary["executed_frac"] = step_summary["executed_tflops"] / peak
+        fwd_summary["executed_tflops"] = ex_fwd / (ms_fwd * 1e-3) / 1e12
+        fwd_summary["executed_frac"] = fwd_summary["executed_tflops"] / peak
+    dom = max(algo, key=lambda kn: kernels.get(kn, {}).get("ms_per_step", 0.0))
+    dom_ms = kernels[dom]["ms_per_step"]
+    launches = kernels[dom]["launches_per_step"]
+    # fp32 inputs run every contraction on v_mfma_f32_32x32x2f32, bf16 inputs on v_mfma_f32_32x32x16_bf16.
+    # frac is the executed rate over the peak (at most 1, and what SQ_VALU_MFMA_BUSY_CYCLES over the kernel's
+    # duration shows); algorithmic_frac prices the same time with the reference-form count and can exceed 1.
+    roofline = None
+    if executed:
+        roofline = {
+            "bound": "mfma", "kernel": dom, "achieved": kernels[dom]["executed_tflops"], "peak": peak,
+            "unit": "TFLOP/s", "frac": kernels[dom]["executed_frac"],
+            "algorithmic_achieved": kernels[dom]["algorithmic_tflops"],
+            "algorithmic_frac": kernels[dom]["algorithmic_frac"], "traffic": None,
+            "flops_per_launch": executed[dom] / launches, "algorithmic_flops_per_launch": algo[dom] / launches,
+            "avg_launch_ms": dom_ms / launches,
+        }
+    if cfg["p"] == 1 and not dense:
+        # p = 1 is HBM-bound (about 19 flop per byte): price the slowest kernel against the (bh, n, d)
+        # tensors it must move; the per-token scalars and the (d+1) x (d+1) states are negligible.
+        #   causal (one scan per head and kernel): three read, one written -- forward: q, k, v -> o;
+        #     dq: grad, k, v (and o, when it forms c_i itself: no bwd_prep launch) -> dq; dk: grad, q, v -> dk;
+        #     dv: grad, q, k -> dv
+        #   unmasked (state of the whole sequence, then one pass over the rows): build k, v (or q, grad);
+        #     forward q -> o; dq grad -> dq; dk v -> dk; dv k -> dv: two tensors each
+        es = 4 if cfg["dtype"] == "f32" else 2
+        tensors = 4 if "build" not in kernels else 2
+        dom = max(algo, key=lambda kn: kernels.get(kn, {}).get("ms_per_step", 0.0)
+                  / kernels.get(kn, {}).get("launches_per_step", 1.0))
+        dom_ms = kernels[dom]["ms_per_step"]
+        launches = kernels[dom]["launches_per_step"]
+        if tensors == 4 and dom == "bwd_dq" and "bwd_prep" not in kernels:
+            tensors = 5
+        bytes_per_launch = float(tensors) * D * es * token_heads
+        gbs = bytes_per_launch / (dom_ms / launches * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": gbs / PEAK_HBM_GBS, "traffic": None, "bytes_per_launch": bytes_per_launch,
+                    "avg_launch_ms": dom_ms / launches}
+    per_th = measured_traffic_bytes_per_token_head(name if not (full and args.batch) else "").get(dom)
+    if per_th is not None and not dense:
+        n_states = n_builds if dom == "build" else 1
+        roofline["traffic"] = per_th * token_heads * n_states / launches  # bytes per launch (profiled, not live)
+        roofline["traffic_source"] = TRAFFIC_SOURCE[name]
+        # whole step: measured HBM bytes over the algorithmic 12 d es per token-head
+        all_th = measured_traffic_bytes_per_token_head(name)
+        if set(all_th) >= {"build", "fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv"}:
+            step_bytes = (all_th["build"] * n_builds + sum(all_th[c] for c in ("fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv"))) * token_heads
+            es = 4 if cfg["dtype"] == "f32" else 2
+            roofline["traffic_ratio"] = step_bytes / (12.0 * D * es * token_heads)
+
+    # parity of this very run: one sampled head of the timed tensors against the fp64 dense form (CPU oracle)
+    parity = None
+    if not args.no_parity:
+        from oracle import fastmax_oracle as O
+        h = bh // 2
+        outs = step_outputs()
+        torch.cuda.synchronize()
+        sl = slice(h, h + 1)
+        ref = O.dense_truth(*(t[sl].float().cpu().double() for t in (q, k, v, go)), mask=cfg["mask"], normalize=True,
+                            a0=COEF["a0"], a1=COEF["a1"], a2=COEF["a2"], lim=COEF["lim"], p=cfg["p"])
+        parity = {"head": h, "reference": "fp64 dense closed form on the same inputs (oracle.dense_truth)",
+                  "tolerance": 1e-4 if cfg["dtype"] == "f32" else 2e-2}
+        for pname, got, want in zip(("o", "dq", "dk", "dv"), outs, ref):
+            parity[pname] = O.error_metrics(got[sl].float().cpu(), want)
+        del outs, ref
+
+    path = ("dense score tiles (no states)" if dense else
+            "keeps every state in registers (one scan per head)" if "build" not in kernels
+            else "rebuilds the prefix states" if recompute else "reads the prefix states the forward pass kept")
+    workload = (f"{name}: Fastmax {'causal' if cfg['mask'] else 'unmasked'} fwd+bwd, "
+                f"B={B} H={H} N={N} D={D} p={cfg['p']} {cfg['dtype']}, normalize lim=1, "
+                "a=(1,1,0.5), q/k/v/grad iid N(0,1) seed 0; backward " + path)
+    del q, k, v, go
+    ops.release_workspaces()
+    torch.cuda.empty_cache()
+    if not full:
+        short = {"workload": workload, "ms_per_step": ms_step, "fwd_ms": ms_fwd,
+                 "tokens_per_s": B * N / (ms_step * 1e-3), "fwd_tokens_per_s": B * N / (ms_fwd * 1e-3),
+                 "step": step_summary, "fwd": fwd_summary,
+                 "kernels_ms": {kn: round(kv["ms_per_step"], 4) for kn, kv in kernels.items()},
+                 "roofline": {kk: roofline[kk] for kk in ("bound", "kernel", "achieved", "peak", "unit", "frac")} if roofline else None}
+        if parity:
+            short["parity"] = {"head": parity["head"], "tolerance": parity["tolerance"],
+                               **{t: {"l2": parity[t]["l2"], "maxabs": parity[t]["maxabs"]} for t in ("o", "dq", "dk", "dv")}}
+        return short
+    return {
+        "metric": "fwd+bwd tokens/sec and MFMA % of peak at B64 H16 N10000 D64 p2, 1 GPU",
+        "value": B * N / (ms_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": cfg["dtype"] if cfg["dtype"] == "f32" else "bf16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": workload},
+        "fwd_ms": ms_fwd, "fwd_tokens_per_s": B * N / (ms_fwd * 1e-3),
+        "module_autograd_ms_per_step": ms_module,
+        "hip_graph_replay_ms_per_step": ms_graph,
+        "fwd_tflops": fwd_summary["algorithmic_tflops"],
+        "fwd": fwd_summary,
+        "step": step_summary,
+        "kernels": kernels,
+        "roofline": roofline,
+        "parity": parity,
+    }
+
+
+# the other configurations of the benchmark set, timed after the headline in the same process
+CONFIG_BLOCK = ("c1", "c2", "headline-unmasked", "headline-p1", "headline-unmasked-p1", "c4", "c5-layer", "c5-layer-p1")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -244,6 +542,10 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true",
                     help="skip the error metrics of one sampled head against the CPU oracle")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="time the chosen workload only (the default headline run also times every other "
+                         "configuration of the benchmark set and the GPT step, reported under \"configs\")")
+    ap.add_argument("--config-steps", type=int, default=3, help="timed steps per entry of the configs block")
     ap.add_argument("--recompute-states", action="store_true",
                     help="backward rebuilds the prefix states instead of reading the ones the forward pass "
                          "kept (saves bhkv * chunks * 592 KB of HBM, costs one more state build)")
@@ -260,229 +562,24 @@ def main() -> int:
         return 2
 
     import torch
-    from fastmax_amd import _cabi, ops
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3
-    cfg = dict(WORKLOADS[args.workload])
-    if args.batch:
-        cfg["B"] = args.batch
-    B, H, N, D = cfg["B"], cfg["H"], cfg["N"], cfg["D"]
-    bh = B * H
-    dtype = torch.float32 if cfg["dtype"] == "f32" else torch.bfloat16
-    dev = torch.device("cuda:0")
-    lib = _cabi.load()
-
-    gen = torch.Generator(device=dev).manual_seed(0)
-    q, k, v, go = (torch.randn((bh, N, D), generator=gen, device=dev, dtype=torch.float32).to(dtype)
-                   for _ in range(4))
-    kw = dict(mask=cfg["mask"], normalize=COEF["normalize"], lim=COEF["lim"], temperature=COEF["temperature"],
-              a0=COEF["a0"], a1=COEF["a1"], a2=COEF["a2"], p=cfg["p"])
-
-    def fwd():
-        return ops.forward(q, k, v, **kw)
-
-    def step():
-        if args.recompute_states:
-            o, den, sc, arg = fwd()
-            return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
-        # the forward pass leaves its prefix states behind for the backward pass
-        o, den, sc, arg, saved = ops.forward(q, k, v, save_states=True, **kw)
-        return ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, saved_states=saved, **kw)
-
-    def step_outputs():
-        o, den, sc, arg = fwd()
-        return (o,) + tuple(ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw))
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    _cabi.check(lib.fastmax_profile_begin())
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    kt = _cabi.KernelTimes()
-    _cabi.check(lib.fastmax_profile_end(C.byref(kt)))
-    ms_step = (t1 - t0) * 1e3 / args.steps
-
-    # forward alone, same inputs
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        fwd()
-    torch.cuda.synchronize()
-    ms_fwd = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    ms_graph = None
-    if args.hip_graph:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step()
-        torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step()
-        graph.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            graph.replay()
-        torch.cuda.synchronize()
-        ms_graph = (time.perf_counter() - t0) * 1e3 / args.steps
-        del graph
-
-    ms_module = None
-    if args.through_module:
-        from fastmax_amd import FASTMultiHeadAttention
-        ops.release_workspaces()
-        mod = FASTMultiHeadAttention()
-        qm, km, vm = (t.view(B, H, N, D).requires_grad_(True) for t in (q, k, v))
-        gom = go.view(B, H, N, D)
-
-        def mstep():
-            o = mod(qm, km, vm, None, cfg["mask"], 0.0, COEF["normalize"], COEF["temperature"], COEF["a0"],
-                    COEF["a1"], COEF["a2"], COEF["lim"], cfg["p"])
-            o.backward(gom)
-            qm.grad = km.grad = vm.grad = None
-
-        for _ in range(args.warmup):
-            mstep()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            mstep()
-        torch.cuda.synchronize()
-        ms_module = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    if args.copy_calibration:
-        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
-
-    fl = algorithmic_flops(D, cfg["p"])
-    token_heads = bh * N
-    peak = PEAK_TFLOPS[cfg["dtype"]]
-    kernels = {}
-    for i, name in enumerate(_cabi.KERNEL_NAMES):
-        if kt.launches[i]:
-            kernels[name] = {"ms_per_step": kt.ms[i] / args.steps, "launches_per_step": kt.launches[i] / args.steps}
-    # Flops per step and kernel class, two ways.  "algorithmic": the reference-form count per token-head (every
-    # ordered channel pair).  "executed": what the matrix instructions of this build really issue (each unordered
-    # pair once, plus intra-chunk tiles, dummy tile slots and ragged tiles).  Both count the state builds the timed
-    # step runs: the forward prefix build and the backward suffix build, plus the backward prefix build when the
-    # states are rebuilt instead of kept.
-    n_builds = 3 if args.recompute_states else 2
-    algo = {"build": n_builds * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
-            "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dk": fl["bwd_dk"] * token_heads,
-            "bwd_dv": fl["bwd_dv"] * token_heads}
-    executed = None
-    if cfg["p"] == 2:
-        ex = executed_mfma_flops(cfg, bh)
-        executed = {"build": ex["build_fwd"] * (n_builds - 1) + ex["build_bwd"],
-                    **{k: ex[k] for k in ("fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv")}}
-    for name, f in algo.items():
-        if name in kernels:
-            sec = kernels[name]["ms_per_step"] * 1e-3
-            kernels[name]["algorithmic_tflops"] = f / sec / 1e12
-            kernels[name]["algorithmic_frac"] = f / sec / 1e12 / peak
-            if executed:
-                kernels[name]["executed_tflops"] = executed[name] / sec / 1e12
-                kernels[name]["executed_frac"] = executed[name] / sec / 1e12 / peak
-    step_summary = {"algorithmic_tflops": sum(algo.values()) / (ms_step * 1e-3) / 1e12}
-    step_summary["algorithmic_frac"] = step_summary["algorithmic_tflops"] / peak
-    if executed:
-        step_summary["executed_tflops"] = sum(executed.values()) / (ms_step * 1e-3) / 1e12
-        step_summary["executed_frac"] = step_summary["executed_tflops"] / peak
-    dom = max(algo, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0))
-    dom_ms = kernels[dom]["ms_per_step"]
-    launches = kernels[dom]["launches_per_step"]
-    # fp32 inputs run every contraction on v_mfma_f32_32x32x2f32, bf16 inputs on v_mfma_f32_32x32x16_bf16.
-    # frac is the executed rate over the peak (at most 1, and what SQ_VALU_MFMA_BUSY_CYCLES over the kernel's
-    # duration shows); algorithmic_frac prices the same time with the reference-form count and can exceed 1.
-    if executed:
-        roofline = {
-            "bound": "mfma", "kernel": dom, "achieved": kernels[dom]["executed_tflops"], "peak": peak,
-            "unit": "TFLOP/s", "frac": kernels[dom]["executed_frac"],
-            "algorithmic_achieved": kernels[dom]["algorithmic_tflops"],
-            "algorithmic_frac": kernels[dom]["algorithmic_frac"], "traffic": None,
-            "flops_per_launch": executed[dom] / launches, "algorithmic_flops_per_launch": algo[dom] / launches,
-            "avg_launch_ms": dom_ms / launches,
-        }
-    if cfg["p"] == 1:
-        # p = 1 is HBM-bound (about 19 flop per byte): price the slowest kernel against the (bh, n, d)
-        # tensors it must move; the per-token scalars and the (d+1) x (d+1) states are negligible.
-        #   causal (one scan per head and kernel): three read, one written -- forward: q, k, v -> o;
-        #     dq: grad, k, v (and o, when it forms c_i itself: no bwd_prep launch) -> dq; dk: grad, q, v -> dk;
-        #     dv: grad, q, k -> dv
-        #   unmasked (state of the whole sequence, then one pass over the rows): build k, v (or q, grad);
-        #     forward q -> o; dq grad -> dq; dk v -> dk; dv k -> dv: two tensors each
-        es = 4 if cfg["dtype"] == "f32" else 2
-        tensors = 4 if "build" not in kernels else 2
-        dom = max(algo, key=lambda n: kernels.get(n, {}).get("ms_per_step", 0.0)
-                  / kernels.get(n, {}).get("launches_per_step", 1.0))
-        dom_ms = kernels[dom]["ms_per_step"]
-        launches = kernels[dom]["launches_per_step"]
-        if tensors == 4 and dom == "bwd_dq" and "bwd_prep" not in kernels:
-            tensors = 5
-        bytes_per_launch = float(tensors) * D * es * token_heads
-        gbs = bytes_per_launch / (dom_ms / launches * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": gbs / PEAK_HBM_GBS, "traffic": None, "bytes_per_launch": bytes_per_launch,
-                    "avg_launch_ms": dom_ms / launches}
-    per_th = measured_traffic_bytes_per_token_head(args.workload if not args.batch else "").get(dom)
-    if per_th is not None:
-        n_states = n_builds if dom == "build" else 1
-        roofline["traffic"] = per_th * token_heads * n_states / launches  # bytes per launch (profiled, not live)
-        roofline["traffic_source"] = TRAFFIC_SOURCE[args.workload]
-
-    # parity of this very run: one sampled head of the timed tensors against the fp64 dense form (CPU oracle)
-    parity = None
-    if not args.no_parity:
-        from oracle import fastmax_oracle as O
-        h = bh // 2
-        outs = step_outputs()
-        torch.cuda.synchronize()
-        sl = slice(h, h + 1)
-        ref = O.dense_truth(*(t[sl].float().cpu().double() for t in (q, k, v, go)), mask=cfg["mask"], normalize=True,
-                            a0=COEF["a0"], a1=COEF["a1"], a2=COEF["a2"], lim=COEF["lim"], p=cfg["p"])
-        parity = {"head": h, "reference": "fp64 dense closed form on the same inputs (oracle.dense_truth)",
-                  "tolerance": 1e-4 if cfg["dtype"] == "f32" else 2e-2}
-        for name, got, want in zip(("o", "dq", "dk", "dv"), outs, ref):
-            parity[name] = O.error_metrics(got[sl].float().cpu(), want)
-        del outs, ref
-
-    result = {
-        "metric": "fwd+bwd tokens/sec and MFMA % of peak at B64 H16 N10000 D64 p2, 1 GPU",
-        "value": B * N / (ms_step * 1e-3),
-        "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": cfg["dtype"] if cfg["dtype"] == "f32" else "bf16 (fp32 accumulate)", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: Fastmax {'causal' if cfg['mask'] else 'unmasked'} fwd+bwd, "
-                               f"B={B} H={H} N={N} D={D} p={cfg['p']} {cfg['dtype']}, normalize lim=1, "
-                               "a=(1,1,0.5), q/k/v/grad iid N(0,1) seed 0; backward "
-                               + ("keeps every state in registers (one scan per head)" if "build" not in kernels
-                                  else "rebuilds the prefix states" if args.recompute_states
-                                  else "reads the prefix states the forward pass kept")},
-        "fwd_ms": ms_fwd, "fwd_tokens_per_s": B * N / (ms_fwd * 1e-3),
-        "module_autograd_ms_per_step": ms_module,
-        "hip_graph_replay_ms_per_step": ms_graph,
-        "fwd_tflops": fl["fwd"] * token_heads / (ms_fwd * 1e-3) / 1e12,
-        "step": step_summary,
-        "kernels": kernels,
-        "roofline": roofline,
-        "parity": parity,
-    }
+    result = measure(args.workload, args, True)
+    if args.workload == "headline" and not args.no_configs and not args.batch:
+        configs = {}
+        for name in CONFIG_BLOCK:
+            configs[name] = measure(name, args, False)
+        import bench_gpt
+        g = bench_gpt.run(steps=args.config_steps, warmup=2)
+        configs["gpt-step"] = {"workload": g["config"]["workload"], "ms_per_step": g["ms_per_step"],
+                               "tokens_per_s": g["value"], "attention_fwd_bwd_ms_per_step": g["attention_fwd_bwd_ms_per_step"],
+                               "attention_share_of_step": g["attention_share_of_step"],
+                               "loss_first_last": g["loss_first_last"], "finite": g["finite"]}
+        result["configs"] = configs
     if not args.no_cpu_baseline:
-        del q, k, v, go
-        result["cpu_baseline"] = cpu_baseline(cfg, args.cpu_seconds)
+        result["cpu_baseline"] = cpu_baseline(dict(WORKLOADS[args.workload]), args.cpu_seconds)
     print(json.dumps(result))
     return 0
 

@@ -147,6 +147,60 @@ class TimedAttention(nn.Module):
         return t
 
 
+def run(steps: int = 5, warmup: int = 2, p: int = 2, layers: int = 12, batch: int = 8, seq: int = 2048,
+        pytorch_attention: bool = False, split_rope: bool = False, unfused_rope: bool = False) -> dict:
+    """Times the training step and returns the result record (main() prints it as one JSON line)."""
+    from fastmax_amd import FASTMultiHeadAttention
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    layout = "pytorch" if unfused_rope else ("split" if (split_rope or pytorch_attention) else "packed")
+    if layout == "packed":
+        attn = TimedAttention(PackedAttention())
+    else:
+        attn = TimedAttention(FASTMultiHeadAttention(use_custom_gradient=not pytorch_attention))
+    model = MiniGPT(50304, 768, layers, 12, 3072, seq, attn, p, layout).to(dev)
+    opt = torch.optim.AdamW(model.parameters(), lr=3e-4, weight_decay=0.1)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    idx = torch.randint(0, 50304, (batch, seq + 1), device=dev, generator=gen)
+    x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
+
+    def step():
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            logits = model(x)
+        loss = F.cross_entropy(logits.float().view(-1, logits.size(-1)), y.view(-1))
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        opt.step()
+        return loss.detach()
+
+    losses = []
+    for _ in range(warmup):
+        losses.append(float(step()))
+    attn.total_ms()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        losses.append(float(step()))
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    attn_ms = attn.total_ms() / steps
+    return {
+        "metric": "GPT training step with Fastmax causal attention in every layer",
+        "value": batch * seq / (ms * 1e-3), "unit": "tokens/s", "ms_per_step": ms,
+        "attention_fwd_bwd_ms_per_step": attn_ms, "attention_share_of_step": attn_ms / ms,
+        "dtype": "bf16 autocast (attention: bf16 in/out, bf16 matrix instructions, fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"{layers} layers, d_model 768, 12 heads x 64, MLP 3072 GELU, RoPE, vocab 50304, "
+                               f"seq {seq}, batch {batch}, p={p}, AdamW",
+                   "attention": "pytorch function" if pytorch_attention else "hip kernels",
+                   "qkv split + rope": {"pytorch": "pytorch ops", "split": "fused hip kernel, contiguous q/k/v",
+                                        "packed": "rotated q, k to a packed tensor, attention on strided views of it and of the projection, "
+                                                  "token-major output (includes the rope pass in the attention time)"}[layout]},
+        "loss_first_last": [losses[0], losses[-1]], "steps": steps, "warmup": warmup,
+        "finite": all(math.isfinite(v) for v in losses),
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--steps", type=int, default=5)
@@ -167,55 +221,10 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench_gpt.py: no GPU visible", file=sys.stderr)
         return 3
-    from fastmax_amd import FASTMultiHeadAttention
-
-    dev = torch.device("cuda:0")
-    torch.manual_seed(0)
-    layout = "pytorch" if args.unfused_rope else ("split" if (args.split_rope or args.pytorch_attention) else "packed")
-    if layout == "packed":
-        attn = TimedAttention(PackedAttention())
-    else:
-        attn = TimedAttention(FASTMultiHeadAttention(use_custom_gradient=not args.pytorch_attention))
-    model = MiniGPT(50304, 768, args.layers, 12, 3072, args.seq, attn, args.p, layout).to(dev)
-    opt = torch.optim.AdamW(model.parameters(), lr=3e-4, weight_decay=0.1)
-    gen = torch.Generator(device=dev).manual_seed(0)
-    idx = torch.randint(0, 50304, (args.batch, args.seq + 1), device=dev, generator=gen)
-    x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
-
-    def step():
-        with torch.autocast("cuda", dtype=torch.bfloat16):
-            logits = model(x)
-        loss = F.cross_entropy(logits.float().view(-1, logits.size(-1)), y.view(-1))
-        opt.zero_grad(set_to_none=True)
-        loss.backward()
-        opt.step()
-        return loss.detach()
-
-    losses = []
-    for _ in range(args.warmup):
-        losses.append(float(step()))
-    attn.total_ms()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        losses.append(float(step()))
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    attn_ms = attn.total_ms() / args.steps
-    print(json.dumps({
-        "metric": "GPT training step with Fastmax causal attention in every layer",
-        "value": args.batch * args.seq / (ms * 1e-3), "unit": "tokens/s", "ms_per_step": ms,
-        "attention_fwd_bwd_ms_per_step": attn_ms, "attention_share_of_step": attn_ms / ms,
-        "dtype": "bf16 autocast (attention: bf16 in/out, bf16 matrix instructions, fp32 accumulate)", "data": "synthetic",
-        "config": {"workload": f"{args.layers} layers, d_model 768, 12 heads x 64, MLP 3072 GELU, RoPE, vocab 50304, "
-                               f"seq {args.seq}, batch {args.batch}, p={args.p}, AdamW",
-                   "attention": "pytorch function" if args.pytorch_attention else "hip kernels",
-                   "qkv split + rope": {"pytorch": "pytorch ops", "split": "fused hip kernel, contiguous q/k/v",
-                                        "packed": "rotated q, k to a packed tensor, attention on strided views of it and of the projection, "
-                                                  "token-major output (includes the rope pass in the attention time)"}[layout]},
-        "loss_first_last": [losses[0], losses[-1]], "steps": args.steps, "warmup": args.warmup,
-    }))
-    return 0 if all(math.isfinite(v) for v in losses) else 1
+    res = run(args.steps, args.warmup, args.p, args.layers, args.batch, args.seq, args.pytorch_attention,
+              args.split_rope, args.unfused_rope)
+    print(json.dumps(res))
+    return 0 if res["finite"] else 1
 
 
 if __name__ == "__main__":

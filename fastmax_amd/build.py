@@ -18,7 +18,10 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(ROOT, "include")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-# -packed-fp32-ops off: scalar fp32 code must not be fused into v_pk_*_f32 on this hardware pool
+# -packed-fp32-ops off: scalar fp32 code must not be fused into v_pk_*_f32 on this hardware pool.  The
+# feature switch acts on the device pass (a float2 multiply-add compiles to v_pk_fma_f32 without it and to
+# two v_fma_f32 with it: tests/test_build_flags_cpu.py); the "not a recognized feature" warning hipcc
+# prints for it comes from the host pass, which has no such feature, and is harmless.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

@@ -154,7 +154,7 @@ bool use_dense(const fastmax_desc* ds) {
     if (ds->mask) limit = bf ? (ds->bh <= 128 ? 4096 : 3072) : 2560;
     else limit = bf ? 1536 : 1024;
   } else {
-    if (ds->mask) limit = bf ? 1536 : 1024;
+    if (ds->mask) limit = bf ? 1536 : 768;
     else limit = bf ? 768 : 512;
   }
   if (ds->mask && ds->nk <= chunk_for(ds->d, 1, ds->dtype)) return false;
@@ -1235,7 +1235,13 @@ int fastmax_forward(const fastmax_desc* desc, const void* q, const void* k, cons
                                 workspace_bytes, nullptr, 0, stream);
 }
 
-size_t fastmax_noalloc_scratch_bytes(void) { return FASTMAX_NOALLOC_SCRATCH_BYTES; }
+size_t fastmax_noalloc_scratch_bytes(void) {
+  // (also the warm-up a graph-capturing caller needs: the per-device address is resolved here)
+  void* p = nullptr;
+  (void)scratch_on_current_device(&p);
+  g_err[0] = 0;
+  return FASTMAX_NOALLOC_SCRATCH_BYTES;
+}
 
 int fastmax_forward_noalloc(const fastmax_desc* desc, const void* q, const void* k, const void* v, void* o,
                             int64_t ldo, float* den, int64_t den_stride, float* qk_scale,

@@ -209,7 +209,11 @@ int fastmax_backward_saved(const fastmax_desc* desc, const void* q, const void* 
  * The call allocates and frees nothing.  Problems whose smallest workspace
  * (fastmax_workspace_min_bytes(desc, FASTMAX_PASS_FORWARD)) exceeds the array are refused with
  * FASTMAX_E_WORKSPACE.  All calls on one GPU share the array: calls that overlap in time on
- * one GPU (different streams, or threads) race and must be serialised by the caller. */
+ * one GPU (different streams, or threads) race and must be serialised by the caller.
+ * The address lookup of the first call on a device is a host-side runtime query behind a mutex: a
+ * caller that captures a HIP graph makes it happen before the capture begins, either with one
+ * uncaptured call or with fastmax_noalloc_scratch_bytes(), which also resolves the address on the
+ * current device (and still returns the size when no device is current). */
 #define FASTMAX_NOALLOC_SCRATCH_BYTES (64u << 20)
 size_t fastmax_noalloc_scratch_bytes(void);
 int fastmax_forward_noalloc(const fastmax_desc* desc, const void* q, const void* k, const void* v,

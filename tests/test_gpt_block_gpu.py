@@ -6,6 +6,7 @@ import torch
 import torch.nn.functional as F
 
 pytestmark = pytest.mark.gpu
+KERNEL_PATH = "auto"   # (conftest) the library's own choice of kernels; the config-5 tests also pin each family
 
 
 def _hip_attention(layout):
@@ -55,14 +56,19 @@ class _Fp32PyTorchAttention(torch.nn.Module):
         return o.to(q.dtype)
 
 
+@pytest.mark.parametrize("path", ["auto", "moments"])
 @pytest.mark.parametrize("p,layout", [(2, "split"), (1, "split"), (2, "packed"), (1, "packed")])
-def test_gpt_at_config5_widths_bf16_gradients(built, p, layout):
+def test_gpt_at_config5_widths_bf16_gradients(built, monkeypatch, p, layout, path):
     """d_model 768, 12 heads x 64, MLP 3072, T = 2048, bf16 autocast, fused projection split + RoPE
     (two layers, batch 2, a small vocabulary): loss and every parameter gradient of the model on the
     HIP kernels against the same model with the PyTorch attention function, at the bf16 tolerance."""
     import bench_gpt
     from fastmax_amd import FASTMultiHeadAttention
 
+    if path == "moments":   # (auto takes the dense score tiles for p = 2 at this length)
+        if p == 1:
+            pytest.skip("p = 1 runs on the moment kernels either way")
+        monkeypatch.setenv("FASTMAX_PATH", "moments")
     dev = torch.device("cuda:0")
     vocab, T = 1024, 2048
     torch.manual_seed(0)
@@ -109,3 +115,35 @@ def test_bf16_autocast_step_runs_and_learns(built):
         opt.step()
         losses.append(float(loss.detach()))
     assert all(v == v for v in losses) and losses[-1] < losses[0]
+
+
+@pytest.mark.parametrize("path", ["auto", "moments"])
+def test_config5_full_depth_step(built, monkeypatch, path):
+    """One forward + backward of the whole configuration-5 model -- 12 layers, d_model 768, 12 heads x 64,
+    MLP 3072, RoPE, vocabulary 50304, batch 8, T = 2048, bf16 autocast -- on the HIP kernels (the library's
+    own choice, which is the dense score tiles at this length, and the moment kernels): finite loss near
+    ln(vocabulary) for random weights, finite gradients in every parameter, none of them all zero."""
+    import math
+
+    import bench_gpt
+
+    if path == "moments":
+        monkeypatch.setenv("FASTMAX_PATH", "moments")
+    dev = torch.device("cuda:0")
+    vocab, T, B = 50304, 2048, 8
+    torch.manual_seed(0)
+    model = bench_gpt.MiniGPT(vocab, 768, 12, 12, 3072, T, bench_gpt.PackedAttention(), 2, "packed").to(dev)
+    idx = torch.randint(0, vocab, (B, T + 1), device=dev, generator=torch.Generator(device=dev).manual_seed(4))
+    x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        logits = model(x)
+    loss = F.cross_entropy(logits.float().view(-1, vocab), y.view(-1))
+    loss.backward()
+    lv = float(loss.detach())
+    print("loss", lv, flush=True)
+    assert math.isfinite(lv) and abs(lv - math.log(vocab)) < 0.5
+    for name, prm in model.named_parameters():
+        assert prm.grad is not None and bool(torch.isfinite(prm.grad).all()), name
+        assert float(prm.grad.abs().max()) > 0.0, name
+    del model, logits, loss
+    torch.cuda.empty_cache()

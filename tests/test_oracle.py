@@ -182,6 +182,30 @@ def test_key_prefix_is_the_tail_of_a_longer_causal_pass():
     assert torch.allclose(full[:, :, 4:], tail, rtol=1e-12, atol=1e-13)
 
 
+def test_rope_cache_known_values():
+    """The frequency table of the rotary embedding against numbers written out by hand (reference:
+    model.py:694-760: theta_c = base^(-2c / n_elem) for channel pair c, angle = position * theta_c, the
+    table repeated over both halves).  n_elem = 4, base 10000: theta = (1, 0.01); n_elem = 8: theta =
+    (1, 0.1, 0.01, 0.001).  A wrong exponent, base, pairing or repeat fails here."""
+    cos, sin = O.rope_cache(4, 4)
+    assert cos.shape == sin.shape == (4, 4)
+    # position 1: angles (1, 0.01, 1, 0.01); position 3: angles (3, 0.03, 3, 0.03)
+    want_cos = {1: (0.5403023058681398, 0.9999500004166653), 3: (-0.9899924966004454, 0.9995500337489875)}
+    want_sin = {1: (0.8414709848078965, 0.009999833334166664), 3: (0.1411200080598672, 0.02999550020249566)}
+    for pos in (1, 3):
+        for c in (0, 1):
+            for half in (0, 2):
+                assert abs(float(cos[pos, half + c]) - want_cos[pos][c]) < 1e-12
+                assert abs(float(sin[pos, half + c]) - want_sin[pos][c]) < 1e-12
+    cos8, sin8 = O.rope_cache(6, 8)
+    # position 5, pairs 1 and 3: angles 0.5 and 0.005
+    assert abs(float(cos8[5, 1]) - 0.8775825618903728) < 1e-12 and abs(float(sin8[5, 5]) - 0.479425538604203) < 1e-12
+    assert abs(float(cos8[5, 7]) - 0.9999875000260416) < 1e-12 and abs(float(sin8[5, 3]) - 0.004999979166692708) < 1e-12
+    # another base: theta_1 = 100^(-1/2) = 0.1 at n_elem = 4
+    cb, sb = O.rope_cache(3, 4, base=100.0)
+    assert abs(float(cb[2, 1]) - 0.9800665778412416) < 1e-12 and abs(float(sb[2, 3]) - 0.19866933079506122) < 1e-12
+
+
 def test_rope_is_a_rotation_and_identity_at_position_zero():
     """apply_rope rotates channel pairs (c, c + hs/2): norms are kept, position 0 is the identity,
     and relative positions are what q.k sees (the defining property of the rotary embedding)."""

@@ -26,10 +26,15 @@ def _forward_both(lib, cabi, q, k, v, **kw):
         scale = torch.zeros(2 * bh, dtype=torch.float32, device=q.device)
         arg = torch.zeros(2 * bh, dtype=torch.int32, device=q.device)
         if noalloc:
-            before = torch.cuda.memory_allocated()
+            lib.fastmax_noalloc_scratch_bytes()   # (resolves the scratch address: not part of what is measured)
+            torch.cuda.synchronize()
+            before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
             cabi.check(lib.fastmax_forward_noalloc(C.byref(ds), q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                                    d, den.data_ptr(), 1, scale.data_ptr(), arg.data_ptr(), stream))
+            torch.cuda.synchronize()
+            # neither torch's allocator nor the device itself (hipMemGetInfo: a raw hipMalloc would show) moved
             assert torch.cuda.memory_allocated() == before
+            assert torch.cuda.mem_get_info()[0] == free_before
         else:
             nbytes = lib.fastmax_workspace_bytes(C.byref(ds), cabi.PASS_FORWARD)
             ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
@@ -74,3 +79,44 @@ def test_noalloc_forward_refuses_what_does_not_fit(built):
     rc = lib.fastmax_forward_noalloc(C.byref(ds), x.data_ptr(), x.data_ptr(), x.data_ptr(), x.data_ptr(), d,
                                      den.data_ptr(), 1, None, None, torch.cuda.current_stream().cuda_stream)
     assert rc == -5 and "allocation-free" in _cabi.last_error()
+
+
+def test_noalloc_forward_under_graph_capture(built):
+    """After the warm-up the header asks for (fastmax_noalloc_scratch_bytes resolves the scratch address),
+    the entry point captures into a HIP graph; every replay is checked against the eager result, with eager
+    work and synchronisations between the replays."""
+    from fastmax_amd import _cabi
+
+    lib = built
+    bh, n, d = 6, 700, 64
+    ds = _cabi.make_desc(bh, n, d, _cabi.FASTMAX_F32, True, True, 2)
+    data = [tuple(t.cuda() for t in O.seeded_inputs((bh, n, d), seed=s)[:3]) for s in (91, 92, 93)]
+    static = [t.clone() for t in data[0]]
+    o = torch.empty((bh, n, d), device="cuda")
+    den = torch.empty((bh, n), device="cuda")
+    scale = torch.empty(2 * bh, device="cuda")
+    arg = torch.empty(2 * bh, dtype=torch.int32, device="cuda")
+
+    def call(q, k, v, o_, den_):
+        _cabi.check(lib.fastmax_forward_noalloc(C.byref(ds), q.data_ptr(), k.data_ptr(), v.data_ptr(), o_.data_ptr(), d,
+                                                den_.data_ptr(), 1, scale.data_ptr(), arg.data_ptr(),
+                                                torch.cuda.current_stream().cuda_stream))
+
+    assert lib.fastmax_noalloc_scratch_bytes() == 64 << 20   # the warm-up
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(*static, o, den)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(*static, o, den)
+    eo, eden = torch.empty_like(o), torch.empty_like(den)
+    for rep, inputs in enumerate(data + data[:1]):
+        call(*inputs, eo, eden)                    # eager work between the replays
+        torch.cuda.synchronize()
+        for dst, src in zip(static, inputs):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(o, eo) and torch.equal(den, eden), f"replay {rep} differs from the eager result"
