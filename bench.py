@@ -172,8 +172,8 @@ def executed_dense_flops(cfg: dict, bh: int) -> dict:
     32-row own tile and a 32-row streamed tile one score contraction over the padded head dimension and one
     product back onto it in the forward kernel, three contractions in dq (scores, g . v, W . k), four in the
     fused dk / dv kernel.  Under the mask a wave skips the streamed tiles that lie wholly on the far side of
-    all its own tiles; the forward kernel's waves own two tiles and also run the one pair in which only the
-    second sees the keys."""
+    all its own tiles (pairs(rt) also prices kernels whose waves own rt tiles, which run every pair that any
+    of the wave's tiles sees)."""
     d, n, masked, bf = cfg["D"], cfg["N"], cfg["mask"], cfg["dtype"] == "bf16"
     dp = -(-d // 32) * 32
     per = 2 * 32 * 32 * dp
@@ -186,8 +186,7 @@ def executed_dense_flops(cfg: dict, bh: int) -> dict:
         for w0 in range(0, nt, rt):
             tot += rt * (min(w0 + rt, nt))   # streamed tiles 0 .. last own tile of the wave, for each of its tiles
         return tot
-    rt_fwd = 2 if dp <= 64 else 1
-    rt_dq = 2 if (dp <= 32 and bf) else 1
+    rt_fwd = rt_dq = 1   # own tiles per wave in the forward and dq kernels (the dk / dv kernel: 1)
     p2 = cfg["p"] == 2
     return {"fwd_apply": bh * pairs(rt_fwd) * 2 * per, "bwd_dq": bh * pairs(rt_dq) * (3 if p2 else 2) * per,
             "bwd_dk": bh * pairs(1) * 4 * per, "build_fwd": 0, "build_bwd": 0, "bwd_dv": 0}

@@ -859,14 +859,14 @@ template <int DP, class T>
 int dense_forward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v, T* o,
                      float* den, int64_t den_stride, const float* scale, hipStream_t stream) {
   using S = dense::Shape<DP, T>;
-  constexpr int RT = S::RT_FWD, BN = S::BN, BM = 128 * RT;
+  constexpr int RT = S::RT_FWD, BN = S::BN, NW = S::NW_FWD, BM = 32 * RT * NW;
   const size_t smem = dense::Lds<DP, T, BN>::bytes(1, 1, BM);
-  auto kern = dense::dense_fwd_kernel<DP, T, RT, BN>;
+  auto kern = dense::dense_fwd_kernel<DP, T, RT, BN, NW>;
   FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
   const int npos = pl.masked ? pl.nk : pl.nq;
   const int nb = (npos + BM - 1) / BM - pl.off / BM;
   ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
-  kern<<<dim3(pl.bh, nb), 256, smem, stream>>>(mk_rows(q, L.q, 0, pl.off), mk_rows(k, L.k), mk_rows(v, L.v), scale,
+  kern<<<dim3(pl.bh, nb), 64 * NW, smem, stream>>>(mk_rows(q, L.q, 0, pl.off), mk_rows(k, L.k), mk_rows(v, L.v), scale,
                                                scale + pl.bh, mk_rows(o, L.o, 0, pl.off),
                                                mk_scalars(den, pl.nq, den_stride, 0, pl.off), npos, pl.nk, ds->d,
                                                pl.masked, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f, pl.ratio);
@@ -901,27 +901,27 @@ int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, c
   const Rows<const T> qr = mk_rows(q, L.q, 0, pl.off), gr = mk_rows(go, L.go, 0, pl.off);
   const Rows<const T> kr = mk_rows(k, L.k), vr = mk_rows(v, L.v);
   {
-    constexpr int RT = S::RT_DQ, BM = 128 * RT;
-    const size_t smem = dense::Lds<DP, T, BN>::bytes(2, 1, 4);
-    auto kern = dense::dense_dq_kernel<DP, T, RT, BN>;
+    constexpr int RT = S::RT_DQ, NW = S::NW_DQ, BM = 32 * RT * NW;
+    const size_t smem = dense::Lds<DP, T, BN>::bytes(2, 1, NW);
+    auto kern = dense::dense_dq_kernel<DP, T, RT, BN, NW>;
     FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
     const int nb = (npos + BM - 1) / BM - pl.off / BM;
     *nbq_out = nb;
     ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
-    kern<<<dim3(pl.bh, nb), 256, smem, stream>>>(qr, gr, dn, cv, kr, vr, scale, scale + pl.bh, mk_rows(dq, L.dq, 0, pl.off), rq,
+    kern<<<dim3(pl.bh, nb), 64 * NW, smem, stream>>>(qr, gr, dn, cv, kr, vr, scale, scale + pl.bh, mk_rows(dq, L.dq, 0, pl.off), rq,
                                                  npos, pl.nk, ds->d, pl.masked, pl.p2 && a2 != 0.f, ds->a1, a2, pl.ratio);
     FM_TRY(launch_status("dense_dq_kernel"));
   }
   {
-    constexpr int RT = S::RT_KV, BM = 128 * RT;
-    const size_t smem = dense::Lds<DP, T, BN>::bytes(2, 2, 2 * BN + 4);
-    auto kern = dense::dense_dkdv_kernel<DP, T, RT, BN>;
+    constexpr int RT = S::RT_KV, NW = S::NW_KV, BM = 32 * RT * NW;
+    const size_t smem = dense::Lds<DP, T, BN>::bytes(2, 2, 2 * BN + NW);
+    auto kern = dense::dense_dkdv_kernel<DP, T, RT, BN, NW>;
     FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
     const int nb = (pl.nk + BM - 1) / BM;
     *nbk_out = nb;
     float* rk = ds->normalize ? rpart + (int64_t)pl.bh * (*nbq_out) : nullptr;
     ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
-    kern<<<dim3(pl.bhkv, nb), 256, smem, stream>>>(kr, vr, qr, gr, dn, cv, scale, scale + pl.bh, mk_rows(dk, L.dk),
+    kern<<<dim3(pl.bhkv, nb), 64 * NW, smem, stream>>>(kr, vr, qr, gr, dn, cv, scale, scale + pl.bh, mk_rows(dk, L.dk),
                                                    mk_rows(dv, L.dv), rk, npos, pl.nk, ds->d, pl.masked, ds->a0, ds->a1,
                                                    a2, pl.ratio);
     FM_TRY(launch_status("dense_dkdv_kernel"));

@@ -13,9 +13,9 @@
 // (reference: example.py:199-212 is this dense form; fastmax_cuda_forward.cu:102-197 and
 // fastmax_cuda_backward.cu:26-882 are the token loops it replaces).
 //
-// One block = 4 waves; a wave owns RT tiles of 32 "own" rows (queries in forward / dq, keys in dk/dv)
+// One block = 4 or 8 waves; a wave owns RT tiles of 32 "own" rows (queries in forward / dq, keys in dk/dv)
 // whose operands stay in registers, and walks the "streamed" rows (keys, resp. queries) in stages of
-// BN rows that all four waves share through LDS (double buffered, one barrier per stage).  Score tiles
+// BN rows that all the block's waves share through LDS (double buffered, one barrier per stage).  Score tiles
 // are formed with the streamed rows as the A operand (rows of the tile) and the own rows as the B
 // operand (columns = lanes), so that f(score), still in the accumulator registers, is directly the A
 // operand of the second contraction (rows = own... of the transposed tile), whose B operand is the
@@ -111,25 +111,45 @@ struct Mma<float> {
   }
 };
 
+// The per-element mask tests of a score tile sit in blocks that only the diagonal and the ragged last tiles
+// enter (a wave-uniform condition).  Left alone the compiler turns such a block into selects that every tile
+// executes -- 16 compares and 32 selects per tile, half as many instructions again as the tile's arithmetic;
+// a statement it may not speculate keeps the block a branch.
+#define FM_KEEP_BRANCH() asm volatile("" ::: "memory")
+
 // an all-zero accumulator tile (the C operand of a contraction's first step)
 constexpr f16v kZero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+// sum over the NW waves of a block; red is NW floats of LDS; the result is valid in every thread
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red, int tid) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  __syncthreads();
+  if ((tid & 63) == 0) red[tid >> 6] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) t += red[w];
+  return t;
+}
 
 template <class T>
 __device__ __forceinline__ typename Mma<T>::Frag lds_frag(const typename Mma<T>::Elt* p) {
   return *reinterpret_cast<const typename Mma<T>::Frag*>(p);
 }
 
-// R rows x DP channels of one head on their way global -> registers -> LDS, by 256 threads.
+// R rows x DP channels of one head on their way global -> registers -> LDS, by the NT threads of a block.
 // Consecutive threads take consecutive rows (16 bytes of a row each), which makes both the row-major
 // and the transposed LDS writes conflict-free.  Rows outside [lo, pend) and channels past d are zero.
-template <int DP, class T, int R>
+template <int DP, class T, int R, int NT>
 struct TileRegs {
   using M = Mma<T>;
   using Elt = typename M::Elt;
   static constexpr int EPP = 16 / (int)sizeof(T);   // elements per 16-byte piece
   static constexpr int PPR = DP / EPP;
   static constexpr int TOTAL = R * PPR;
-  static constexpr int NV = (TOTAL + 255) / 256;
+  static constexpr int NV = (TOTAL + NT - 1) / NT;
   uint4 raw[NV];
   float rf[NV];   // row factor of scaled tiles: 1 / rowdiv[row], 0 for a row that does not exist
 
@@ -137,7 +157,7 @@ struct TileRegs {
                                        const float* rowdiv = nullptr, int64_t rdstride = 0) {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int idx = tid + u * 256;
+      const int idx = tid + u * NT;
       const bool in = idx < TOTAL;
       const int row = in ? idx % R : 0, pc = in ? idx / R : 0;
       const int pos = pos0 + row;
@@ -153,7 +173,7 @@ struct TileRegs {
   __device__ __forceinline__ void store(Elt* rm, int pr, Elt* tr, int pt, int tid) const {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int idx = tid + u * 256;
+      const int idx = tid + u * NT;
       if (idx < TOTAL) {
         const int row = idx % R, pc = idx / R;
         if (rm) *reinterpret_cast<uint4*>(rm + row * pr + pc * EPP) = raw[u];
@@ -169,7 +189,7 @@ struct TileRegs {
   __device__ __forceinline__ void store_scaled(Elt* rm, int pr, float srm, Elt* tr, int pt, float str, int tid) const {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
-      const int idx = tid + u * 256;
+      const int idx = tid + u * NT;
       if (idx < TOTAL) {
         const int row = idx % R, pc = idx / R;
         float x[EPP], y[EPP];
@@ -230,19 +250,32 @@ template <int DP, class T>
 struct Shape {
   static constexpr bool BF = std::is_same<T, bf16_t>::value;
   static constexpr int BN = BF ? 64 : 32;                     // streamed rows per stage
-  static constexpr int RT_FWD = DP <= 64 ? 2 : 1;             // own 32-row tiles per wave
-  static constexpr int RT_DQ = DP <= 32 && BF ? 2 : 1;
+  // Own 32-row tiles per wave.  Matrix instructions and everything else a SIMD issues (VALU, LDS reads)
+  // take turns rather than overlap on this chip, and with one own tile every matrix instruction needs a
+  // 16-byte LDS operand read of its own -- the CU's whole LDS bandwidth; two own tiles share each
+  // streamed operand and halve that, at the price of the registers of a second set of accumulators,
+  // which for the backward kernels means one resident block per CU.
+  // Waves per block.  Staging a stage of streamed rows costs a block the same whatever its size, so the
+  // backward kernels, whose stages are the costliest (four staged tiles, one of them rescaled), run eight
+  // waves on it where the registers allow two waves per SIMD.
+  static constexpr int NW_FWD = 4;
+  static constexpr int NW_DQ = (BF && DP == 64) ? 8 : 4;
+  static constexpr int NW_KV = (BF && DP == 64) ? 8 : 4;
+  static constexpr int RT_FWD = 1;
+  static constexpr int RT_DQ = 1;
   static constexpr int RT_KV = 1;
-  static constexpr int OCC = (BF ? DP <= 64 : DP <= 32) ? 2 : 1;   // resident blocks per CU the kernels are built for
-                                                              // (fp32 operand fragments take twice the registers)
+  // resident blocks per CU each kernel is built for (fp32 operand fragments take twice the registers)
+  static constexpr int OCC_FWD = (BF && DP <= 64) ? 3 : (DP <= 32) ? 2 : 1;
+  static constexpr int OCC_DQ = (BF && DP == 64) ? 1 : (DP <= 32) ? 2 : 1;   // (8-wave blocks: one is two waves per SIMD)
+  static constexpr int OCC_KV = (BF && DP == 64) ? 1 : (DP <= 32) ? 2 : 1;
 };
 
 // ---------------------------------------------------------------------------------------
 // Forward.  grid = (heads, query blocks of 128 RT positions from the one that holds position Q.lo).
 // npos: positions of the queries end here (nk under the mask: query i sits at position i + nk - nq).
 // ---------------------------------------------------------------------------------------
-template <int DP, class T, int RT, int BN>
-__global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
+template <int DP, class T, int RT, int BN, int NW>
+__global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_FWD)) void dense_fwd_kernel(
     Rows<const T> Q, Rows<const T> K, Rows<const T> V, const float* __restrict__ qscale,
     const float* __restrict__ kscale, Rows<T> O, RowScalarsOut den, int npos, int nk, int d, int masked, float a0,
     float a1, float a2, int ratio) {
@@ -250,7 +283,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
   using Elt = typename M::Elt;
   using Frag = typename M::Frag;
   using L = Lds<DP, T, BN>;
-  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, NT = 64 * NW, BM = 32 * RT * NW;
   constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
   static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
@@ -275,7 +308,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
 
   const int kend = masked ? (tok0 + BM < nk ? tok0 + BM : nk) : nk;
   const int nst = (kend + BN - 1) / BN;
-  TileRegs<DP, T, BN> kt, vt;
+  TileRegs<DP, T, BN, NT> kt, vt;
   auto stage_load = [&](int st) {
     kt.load(Kh, st * BN, nk, d, tid);
     vt.load(Vh, st * BN, nk, d, tid);
@@ -328,12 +361,14 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
         sc[rt][r] = a0 + s * (a1 + a2 * s);
       }
       if (masked && rel >= 32 * rt) {   // (wave-uniform) a key may not lie after the query
+        FM_KEEP_BRANCH();
         const int lim = rel > 32 * rt ? -1 : i;
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           if (trow(r, hh) > lim) sc[rt][r] = 0.f;
       }
       if (tail) {   // (wave-uniform) keys past the end
+        FM_KEEP_BRANCH();
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           if (kb + trow(r, hh) >= nk) sc[rt][r] = 0.f;
@@ -404,8 +439,8 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_fwd_kernel(
 // started at a1, is f'(s)) and g = grad_out / den.  rpart[head * gridDim.y + block] receives the block's
 // sum of dqh . qh for the normalisation chain rule (when rpart is given).
 // ---------------------------------------------------------------------------------------
-template <int DP, class T, int RT, int BN>
-__global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
+template <int DP, class T, int RT, int BN, int NW>
+__global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kernel(
     Rows<const T> Q, Rows<const T> GO, RowScalars den, RowScalars cvec, Rows<const T> K, Rows<const T> V,
     const float* __restrict__ qscale, const float* __restrict__ kscale, Rows<T> DQ, float* __restrict__ rpart,
     int npos, int nk, int d, int masked, int p2, float a1, float a2, int ratio) {
@@ -413,7 +448,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
   using Elt = typename M::Elt;
   using Frag = typename M::Frag;
   using L = Lds<DP, T, BN>;
-  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, NT = 64 * NW, BM = 32 * RT * NW;
   constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
   static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
@@ -421,7 +456,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
   Elt* Kl = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
   Elt* Vl = Kl + 2 * L::RM;                       // [2][BN][PR]
   Elt* Kt = Vl + 2 * L::RM;                       // [2][DP][PT]
-  float* red = reinterpret_cast<float*>(Kt + 2 * L::TR);   // [4]
+  float* red = reinterpret_cast<float*>(Kt + 2 * L::TR);   // [NW]
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int nb = gridDim.y, bx = blockIdx.y;   // (heads, row blocks), as in the forward kernel
@@ -447,7 +482,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
 
   const int kend = masked ? (tok0 + BM < nk ? tok0 + BM : nk) : nk;
   const int nst = (kend + BN - 1) / BN;
-  TileRegs<DP, T, BN> kt, vt;
+  TileRegs<DP, T, BN, NT> kt, vt;
   auto stage_load = [&](int st) {
     kt.load(Kh, st * BN, nk, d, tid);
     vt.load(Vh, st * BN, nk, d, tid);
@@ -498,6 +533,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) pt[rt][r] = sc[rt][r] * pt[rt][r];
       if (masked && rel >= 32 * rt) {   // (wave-uniform) a key may not lie after the query
+        FM_KEEP_BRANCH();
         const int lim = rel > 32 * rt ? -1 : i;
 #pragma unroll
         for (int r = 0; r < 16; ++r)
@@ -562,7 +598,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
       }
     }
   if (rpart) {
-    rs = block_sum_256(rs, red, tid);
+    rs = block_sum<NW>(rs, red, tid);
     if (tid == 0) rpart[(int64_t)head * nb + bx] = rs;
   }
 }
@@ -574,8 +610,8 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dq_kernel(
 // twice: times qs / den row-major (so that W comes out times qs, the factor of qh in dkh = sum W qh) and
 // times 1 / den transposed (the B operand of dv).  rpart[kvhead * gridDim.y + block] = sum dkh . kh.
 // ---------------------------------------------------------------------------------------
-template <int DP, class T, int RT, int BN>
-__global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
+template <int DP, class T, int RT, int BN, int NW>
+__global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_KV)) void dense_dkdv_kernel(
     Rows<const T> K, Rows<const T> V, Rows<const T> Q, Rows<const T> GO, RowScalars den, RowScalars cvec,
     const float* __restrict__ qscale, const float* __restrict__ kscale, Rows<T> DK, Rows<T> DV,
     float* __restrict__ rpart, int npos, int nk, int d, int masked, float a0, float a1, float a2, int ratio) {
@@ -583,7 +619,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
   using Elt = typename M::Elt;
   using Frag = typename M::Frag;
   using L = Lds<DP, T, BN>;
-  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, BM = 128 * RT;
+  constexpr int KF = M::KF, EPL = M::EPL, NF = DP / KF, CB = DP / 32, NFA = 32 / KF, NT = 64 * NW, BM = 32 * RT * NW;
   constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
   static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
@@ -592,8 +628,8 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
   Elt* Gl = Ql + 2 * L::RM;                       // [2][BN][PR]
   Elt* Qt = Gl + 2 * L::RM;                       // [2][DP][PT]
   Elt* Gt = Qt + 2 * L::TR;                       // [2][DP][PT]
-  float* Cl = reinterpret_cast<float*>(Gt + 2 * L::TR);   // [2][BN]
-  float* red = Cl + 2 * BN;                       // [4]
+  float* Cl = reinterpret_cast<float*>(Gt + 2 * L::TR);   // [2][BN]: -qs c of the streamed queries
+  float* red = Cl + 2 * BN;                       // [NW]
 
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
   const int nb = gridDim.y, bx = blockIdx.y;   // (key/value heads, key blocks)
@@ -617,7 +653,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) dk[rt][cb][r] = dv[rt][cb][r] = 0.f;
 
-  TileRegs<DP, T, BN> qt, gt;
+  TileRegs<DP, T, BN, NT> qt, gt;
   float creg = 0.f;
   for (int hq = 0; hq < ratio; ++hq) {
     const int head = hkv * ratio + hq;
@@ -635,7 +671,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
       gt.load(Gh, st * BN, npos, d, tid, denh, den.stride);
       if (tid < BN) {
         const int pos = st * BN + tid;
-        creg = (pos >= lo && pos < npos) ? ch[(int64_t)pos * cvec.stride] * qs : 0.f;
+        creg = (pos >= lo && pos < npos) ? -ch[(int64_t)pos * cvec.stride] * qs : 0.f;   // (-qs c: the tile's start value)
       }
     };
     auto stage_store = [&](int buf) {
@@ -660,7 +696,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
         const float4 c4 = *reinterpret_cast<const float4*>(cl + t32 * 32 + 8 * j + 4 * hh);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-          pt[rt][4 * j] = -c4.x; pt[rt][4 * j + 1] = -c4.y; pt[rt][4 * j + 2] = -c4.z; pt[rt][4 * j + 3] = -c4.w;
+          pt[rt][4 * j] = c4.x; pt[rt][4 * j + 1] = c4.y; pt[rt][4 * j + 2] = c4.z; pt[rt][4 * j + 3] = c4.w;
         }
       }
 #pragma unroll
@@ -688,6 +724,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
           pt[rt][r] = (a1 + b2 * s) * pt[rt][r];
         }
         if (masked && rel <= 32 * rt) {   // (wave-uniform) a query may not lie before the key
+          FM_KEEP_BRANCH();
           const int lim = rel < 32 * rt ? 32 : i;
 #pragma unroll
           for (int r = 0; r < 16; ++r)
@@ -760,7 +797,7 @@ __global__ __launch_bounds__(256, (Shape<DP, T>::OCC)) void dense_dkdv_kernel(
       }
     }
   if (rpart) {
-    rs = block_sum_256(rs, red, tid);
+    rs = block_sum<NW>(rs, red, tid);
     if (tid == 0) rpart[(int64_t)hkv * nb + bx] = rs;
   }
 }
