@@ -250,3 +250,38 @@ def test_strided_views_of_a_fused_projection_d128(built):
     assert_close("dq", gx[:, :, :, :r].permute(0, 2, 3, 1, 4).reshape(b * g * r, t, hs), rdq, 1e-4, atol=1e-6)
     assert_close("dk", gx[:, :, :, r].permute(0, 2, 1, 3).reshape(b * g, t, hs), fold(rdk), 1e-4, atol=1e-6)
     assert_close("dv", gx[:, :, :, r + 1].permute(0, 2, 1, 3).reshape(b * g, t, hs), fold(rdv), 1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape,mask,dtype", [((12, 640, 64), True, torch.bfloat16),     # (dk/dv kernel: 74 KB of LDS)
+                                              ((6, 500, 128), True, torch.float32), ((8, 300, 48), False, torch.float32)])
+def test_graph_replays_match_eager(ops, shape, mask, dtype):
+    """The dense kernels allocate nothing, clear nothing and never synchronise either: a forward + backward
+    step captures into a HIP graph, and every replay equals the eager result."""
+    kw = dict(mask=mask, normalize=True, p=2)
+
+    def step(q, k, v, go):
+        o, den, sc, arg = ops.forward(q, k, v, **kw)
+        dq, dk, dv = ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+        return o, dq, dk, dv
+
+    data = [tuple(t.to(dtype).cuda() for t in O.seeded_inputs(shape, seed=s)) for s in (1, 2, 3)]
+    static = [t.clone() for t in data[0]]
+    step(*static)            # workspaces exist before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(*static)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step(*static)
+    for rep, inputs in enumerate(data + data[:1]):
+        eager = step(*inputs)                      # eager work between the replays
+        torch.cuda.synchronize()
+        for dst, src in zip(static, inputs):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("o", "dq", "dk", "dv"), outs, eager):
+            assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager result"
