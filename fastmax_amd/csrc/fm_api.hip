@@ -913,9 +913,9 @@ int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, c
     FM_TRY(launch_status("dense_dq_kernel"));
   }
   {
-    constexpr int RT = S::RT_KV, NW = S::NW_KV, BM = 32 * RT * NW;
-    const size_t smem = dense::Lds<DP, T, BN>::bytes(2, 2, 2 * BN + NW);
-    auto kern = dense::dense_dkdv_kernel<DP, T, RT, BN, NW>;
+    constexpr int RT = S::RT_KV, NW = S::NW_KV, BM = 32 * RT * NW, BNK = S::BN_KV;
+    const size_t smem = dense::Lds<DP, T, BNK>::bytes(2, 2, 2 * BNK + NW);
+    auto kern = dense::dense_dkdv_kernel<DP, T, RT, BNK, NW>;
     FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
     const int nb = (pl.nk + BM - 1) / BM;
     *nbk_out = nb;
