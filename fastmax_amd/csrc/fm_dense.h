@@ -259,15 +259,15 @@ struct Shape {
   // Waves per block.  Staging a stage of streamed rows costs a block the same whatever its size, so the
   // backward kernels, whose stages are the costliest (four staged tiles, one of them rescaled), run eight
   // waves on it where the registers allow two waves per SIMD.
-  static constexpr int NW_FWD = 4;
+  static constexpr int NW_FWD = (BF && DP == 64) ? 8 : 4;
   static constexpr int NW_DQ = (BF && DP == 64) ? 8 : 4;
   static constexpr int NW_KV = (BF && DP == 64) ? 8 : 4;
   static constexpr int RT_FWD = 1;
   static constexpr int RT_DQ = 1;
   static constexpr int RT_KV = 1;
   // resident blocks per CU each kernel is built for (fp32 operand fragments take twice the registers)
-  static constexpr int OCC_FWD = (BF && DP <= 64) ? 3 : (DP <= 32) ? 2 : 1;
-  static constexpr int OCC_DQ = (BF && DP == 64) ? 1 : (DP <= 32) ? 2 : 1;   // (8-wave blocks: one is two waves per SIMD)
+  static constexpr int OCC_FWD = (BF && DP == 64) ? 2 : (BF && DP <= 32) ? 3 : (DP <= 32) ? 2 : 1;
+  static constexpr int OCC_DQ = (BF && DP == 64) ? 2 : (DP <= 32) ? 2 : 1;   // (8-wave blocks: one is two waves per SIMD)
   static constexpr int OCC_KV = (BF && DP == 64) ? 1 : (DP <= 32) ? 2 : 1;
 };
 
