@@ -299,6 +299,12 @@ def measure(name: str, args, full: bool) -> dict:
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
+    if not full:
+        # short workloads are timed over enough steps to fill about 60 ms (at most 100 steps)
+        t0 = time.perf_counter()
+        step()
+        torch.cuda.synchronize()
+        steps = max(steps, min(100, int(0.06 / max(time.perf_counter() - t0, 1e-5))))
     _cabi.check(lib.fastmax_profile_begin())
     t0 = time.perf_counter()
     for _ in range(steps):

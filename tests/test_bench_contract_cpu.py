@@ -57,6 +57,26 @@ def test_executed_flops_model():
     assert bench.executed_mfma_flops(cb, 4)["fwd_apply"] == 2 * 34 * 64 * 96 * th
 
 
+def test_executed_flops_of_the_dense_kernels():
+    """Dense score tiles: 2 x 32 x 32 x d flop per contraction and (own tile, streamed tile) pair; unmasked
+    every pair, causal the pairs at or below the diagonal; forward two contractions, dq three, dk/dv four."""
+    sys.path.insert(0, ROOT)
+    import bench
+
+    cfg = dict(B=1, H=3, N=2048, D=64, mask=False, p=2, dtype="bf16")
+    ex = bench.executed_dense_flops(cfg, 3)
+    per = 2 * 32 * 32 * 64
+    assert ex["fwd_apply"] == 3 * 64 * 64 * 2 * per
+    assert ex["bwd_dq"] == 3 * 64 * 64 * 3 * per and ex["bwd_dk"] == 3 * 64 * 64 * 4 * per
+    exm = bench.executed_dense_flops(dict(cfg, mask=True), 3)
+    assert exm["fwd_apply"] == 3 * (64 * 65 // 2) * 2 * per
+    # a head dimension of 48 runs as 64 padded channels, 100 tokens as 4 tiles of 32
+    e48 = bench.executed_dense_flops(dict(cfg, D=48, N=100, mask=True), 1)
+    assert e48["bwd_dk"] == 10 * 4 * per
+    # p = 1 needs no score tile in dq
+    assert bench.executed_dense_flops(dict(cfg, p=1), 3)["bwd_dq"] == 3 * 64 * 64 * 2 * per
+
+
 def test_traffic_figures_are_read_from_the_committed_profiles():
     """roofline.traffic is priced with the HBM bytes per token-head that the rocprofv3 summaries under
     profiles/ list for each kernel class; the summaries of both chunked workloads parse."""
