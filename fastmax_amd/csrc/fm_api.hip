@@ -104,6 +104,9 @@ struct Plan {
   bool rowpass;        // unmasked p = 1: states from the build kernel, one pass over the rows per output
   bool dense;          // dense score tiles, no moment states (fm_dense.h): short sequences, and every head
                        // dimension other than 32 and 64
+  bool lin;            // dense kernels in linear mode (p = 1, long sequences): chunk states of (dp + 1) rows in
+                       // the workspace, lslots of them per head, one per lchunk positions
+  int lchunk, lslots, ldp;
   bool split;          // causal p = 1 with few heads: the chunks of a head are built side by side as partial
                        // states and a prefix pass over the chunks makes the causal states of them
   size_t scratch_bytes;   // per head: where the fp32 partial states of a split build go when the
@@ -125,6 +128,11 @@ int64_t slot_floats_for(int d, int p2, bool packed) {
 }
 
 size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+
+int64_t lin_state_floats(int dp, int nblk) {
+  return dp == 32 ? dense::LinState<32>::floats(nblk) : dp == 64 ? dense::LinState<64>::floats(nblk)
+       : dp == 96 ? dense::LinState<96>::floats(nblk) : dense::LinState<128>::floats(nblk);
+}
 
 // Causal p = 1 at d = 64 runs as one sequential scan per head (fm_linear.h: one wave per head, the
 // state never leaves its registers) once there are enough heads to fill the chip's 1024 SIMDs
@@ -189,6 +197,17 @@ Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true, bool allow_d
     if (pass == FASTMAX_PASS_BACKWARD) {
       fx += align256((size_t)pl.bh * pl.nq * sizeof(float));
       fx += align256((size_t)pl.bh * (pl.nblk_q + pl.nblk_k) * sizeof(float));
+    }
+    // p = 1 is linear in the keys: past these lengths the tiles of a 256-position chunk plus one state of
+    // everything outside it cost less than the tiles of the whole sequence
+    pl.lchunk = 256;
+    pl.lslots = (pl.n + pl.lchunk - 1) / pl.lchunk;
+    pl.ldp = (pl.d + 31) / 32 * 32;
+    pl.lin = !pl.p2 && pl.n > (pl.masked ? 1024 : 512);
+    if (pl.lin) {
+      // key-side states (one layout of the d x d block per pass), query-side states (both layouts)
+      fx += align256((size_t)pl.bhkv * pl.lslots * lin_state_floats(pl.ldp, 1) * sizeof(float));
+      if (pass == FASTMAX_PASS_BACKWARD) fx += align256((size_t)pl.bh * pl.lslots * lin_state_floats(pl.ldp, 2) * sizeof(float));
     }
     pl.fixed_bytes = fx;
     return pl;
@@ -856,20 +875,38 @@ int allow_lds(const void* kernel, size_t bytes) {
 }
 
 template <int DP, class T>
+int dense_key_states(const Plan& pl, const Layout& L, const T* k, const T* v, int d, float a1, bool transposed,
+                     float* kstate, hipStream_t stream) {
+  // a1 sum k (x) v and the sums of k, of v of every chunk of keys alone, then (masked) of the chunks before each /
+  // (unmasked) of all, in slot 0; the forward kernel reads rows of the transposed block, dq of the natural one
+  const int64_t sf = dense::LinState<DP>::floats(1);
+  ScopedKernel sk(FASTMAX_K_BUILD, stream);
+  dense::dense_state_kernel<DP, T, false><<<dim3(pl.bhkv, pl.lslots), 256, 0, stream>>>(
+      mk_rows(k, L.k), mk_rows(v, L.v), RowScalars{nullptr, 0, 0}, RowScalars{nullptr, 0, 0}, nullptr, a1, kstate, 1,
+      transposed ? -1 : 0, transposed ? 0 : -1, pl.nk, d, pl.lchunk);
+  dense::lin_scan_kernel<<<dim3((unsigned)((sf / 4 + 255) / 256), pl.bhkv), 256, 0, stream>>>(kstate, pl.lslots, sf,
+                                                                                           pl.masked ? 0 : 2);
+  return launch_status("dense_state_kernel");
+}
+
+template <int DP, class T>
 int dense_forward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v, T* o,
-                     float* den, int64_t den_stride, const float* scale, hipStream_t stream) {
+                     float* den, int64_t den_stride, const float* scale, float* kstate, hipStream_t stream) {
   using S = dense::Shape<DP, T>;
   constexpr int RT = S::RT_FWD, BN = S::BN, NW = S::NW_FWD, BM = 32 * RT * NW;
+  static_assert(256 % BM == 0 && 256 % BN == 0, "blocks and stages do not straddle the chunks of the linear mode");
   const size_t smem = dense::Lds<DP, T, BN>::bytes(1, 1, BM);
   auto kern = dense::dense_fwd_kernel<DP, T, RT, BN, NW>;
   FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
   const int npos = pl.masked ? pl.nk : pl.nq;
   const int nb = (npos + BM - 1) / BM - pl.off / BM;
+  if (pl.lin) FM_TRY((dense_key_states<DP, T>(pl, L, k, v, ds->d, ds->a1, true, kstate, stream)));
   ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
   kern<<<dim3(pl.bh, nb), 64 * NW, smem, stream>>>(mk_rows(q, L.q, 0, pl.off), mk_rows(k, L.k), mk_rows(v, L.v), scale,
                                                scale + pl.bh, mk_rows(o, L.o, 0, pl.off),
                                                mk_scalars(den, pl.nq, den_stride, 0, pl.off), npos, pl.nk, ds->d,
-                                               pl.masked, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f, pl.ratio);
+                                               pl.masked, ds->a0, ds->a1, pl.p2 ? ds->a2 : 0.f, pl.ratio,
+                                               pl.lin ? kstate : nullptr, pl.lchunk, pl.lslots);
   return launch_status("dense_fwd_kernel");
 }
 
@@ -879,7 +916,8 @@ int dense_forward(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
   float* scale = scale_out ? scale_out : reinterpret_cast<float*>(ws);
   int* arg = arg_out ? arg_out : reinterpret_cast<int*>(ws + align256((size_t)2 * pl.bh * sizeof(float)));
   FM_TRY(compute_scales<T>(ds, L, q, k, scale, arg, stream));
-#define FM_DENSE_FWD(DP) return dense_forward_dp<DP, T>(ds, pl, L, q, k, v, o, den, den_stride, scale, stream)
+  float* kstate = reinterpret_cast<float*>(ws + align256((size_t)2 * pl.bh * sizeof(float)) + align256((size_t)2 * pl.bh * sizeof(int)));
+#define FM_DENSE_FWD(DP) return dense_forward_dp<DP, T>(ds, pl, L, q, k, v, o, den, den_stride, scale, kstate, stream)
   if (ds->d <= 32) FM_DENSE_FWD(32);
   if (ds->d <= 64) FM_DENSE_FWD(64);
   if (ds->d <= 96) FM_DENSE_FWD(96);
@@ -890,7 +928,8 @@ int dense_forward(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
 template <int DP, class T>
 int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v,
                       const float* den, int64_t den_stride, const T* go, T* dq, T* dk, T* dv, const float* scale,
-                      const float* cvec, float* rpart, int* nbq_out, int* nbk_out, hipStream_t stream) {
+                      const float* cvec, float* rpart, float* kstate, float* qstate, int* nbq_out, int* nbk_out,
+                      hipStream_t stream) {
   using S = dense::Shape<DP, T>;
   constexpr int BN = S::BN;
   const int npos = pl.masked ? pl.nk : pl.nq;
@@ -900,8 +939,23 @@ int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, c
   const RowScalars cv = mk_scalars<const float>(cvec, pl.nq, 1, 0, pl.off);
   const Rows<const T> qr = mk_rows(q, L.q, 0, pl.off), gr = mk_rows(go, L.go, 0, pl.off);
   const Rows<const T> kr = mk_rows(k, L.k), vr = mk_rows(v, L.v);
+  if (pl.lin) {
+    // key-side states as in the forward pass; query-side states sum [q; 1] (x) [g, c] of every chunk alone, then
+    // (masked) of the chunks after each / (unmasked) of all, in slot 0
+    FM_TRY((dense_key_states<DP, T>(pl, L, k, v, ds->d, ds->a1, false, kstate, stream)));
+    const int64_t sf = dense::LinState<DP>::floats(2);
+    ScopedKernel sk(FASTMAX_K_BUILD, stream);
+    dense::dense_state_kernel<DP, T, true><<<dim3(pl.bh, pl.lslots), 256, 0, stream>>>(qr, gr, dn, cv, scale, ds->a1, qstate, 2, 0, 1,
+                                                                            npos, ds->d, pl.lchunk);
+    dense::lin_scan_kernel<<<dim3((unsigned)((sf / 4 + 255) / 256), pl.bh), 256, 0, stream>>>(qstate, pl.lslots, sf,
+                                                                                          pl.masked ? 1 : 2);
+    FM_TRY(launch_status("dense_state_kernel"));
+  }
+  const float* ksl = pl.lin ? kstate : nullptr;
+  const float* qsl = pl.lin ? qstate : nullptr;
   {
     constexpr int RT = S::RT_DQ, NW = S::NW_DQ, BM = 32 * RT * NW;
+    static_assert(256 % BM == 0, "blocks do not straddle the chunks of the linear mode");
     const size_t smem = dense::Lds<DP, T, BN>::bytes(2, 1, NW);
     auto kern = dense::dense_dq_kernel<DP, T, RT, BN, NW>;
     FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
@@ -909,11 +963,13 @@ int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, c
     *nbq_out = nb;
     ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
     kern<<<dim3(pl.bh, nb), 64 * NW, smem, stream>>>(qr, gr, dn, cv, kr, vr, scale, scale + pl.bh, mk_rows(dq, L.dq, 0, pl.off), rq,
-                                                 npos, pl.nk, ds->d, pl.masked, pl.p2 && a2 != 0.f, ds->a1, a2, pl.ratio);
+                                                 npos, pl.nk, ds->d, pl.masked, pl.p2 && a2 != 0.f, ds->a1, a2, pl.ratio,
+                                                 ksl, pl.lchunk, pl.lslots);
     FM_TRY(launch_status("dense_dq_kernel"));
   }
   {
     constexpr int RT = S::RT_KV, NW = S::NW_KV, BM = 32 * RT * NW, BNK = S::BN_KV;
+    static_assert(256 % BM == 0 && 256 % BNK == 0, "blocks and stages do not straddle the chunks of the linear mode");
     const size_t smem = dense::Lds<DP, T, BNK>::bytes(2, 2, 2 * BNK + NW);
     auto kern = dense::dense_dkdv_kernel<DP, T, RT, BNK, NW>;
     FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
@@ -923,7 +979,7 @@ int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, c
     ScopedKernel sk(FASTMAX_K_BWD_DK, stream);
     kern<<<dim3(pl.bhkv, nb), 64 * NW, smem, stream>>>(kr, vr, qr, gr, dn, cv, scale, scale + pl.bh, mk_rows(dk, L.dk),
                                                    mk_rows(dv, L.dv), rk, npos, pl.nk, ds->d, pl.masked, ds->a0, ds->a1,
-                                                   a2, pl.ratio);
+                                                   a2, pl.ratio, qsl, pl.lchunk, pl.lslots);
     FM_TRY(launch_status("dense_dkdv_kernel"));
   }
   return FASTMAX_OK;
@@ -945,12 +1001,16 @@ int dense_backward(const fastmax_desc* ds, const Plan& pl, const Layout& L, cons
   float* cvec = reinterpret_cast<float*>(p);
   p += align256((size_t)bh * pl.nq * sizeof(float));
   float* rpart = reinterpret_cast<float*>(p);
+  p += align256((size_t)bh * (pl.nblk_q + pl.nblk_k) * sizeof(float));
+  float* kstate = reinterpret_cast<float*>(p);
+  float* qstate = kstate;
+  if (pl.lin) qstate = reinterpret_cast<float*>(p + align256((size_t)pl.bhkv * pl.lslots * lin_state_floats(pl.ldp, 1) * sizeof(float)));
   if (!given) FM_TRY(compute_scales<T>(ds, L, q, k, scale_ws, arg_ws, stream));
   FM_TRY((launch_bwd_prep<T>(pl, L, go, o, den, den_stride, cvec, stream)));
   int nbq = 0, nbk = 0;
 #define FM_DENSE_BWD(DP)                                                                                          \
-  FM_TRY((dense_backward_dp<DP, T>(ds, pl, L, q, k, v, den, den_stride, go, dq, dk, dv, scale, cvec, rpart, &nbq, \
-                                   &nbk, stream)))
+  FM_TRY((dense_backward_dp<DP, T>(ds, pl, L, q, k, v, den, den_stride, go, dq, dk, dv, scale, cvec, rpart, kstate, \
+                                   qstate, &nbq, &nbk, stream)))
   if (ds->d <= 32) FM_DENSE_BWD(32);
   else if (ds->d <= 64) FM_DENSE_BWD(64);
   else if (ds->d <= 96) FM_DENSE_BWD(96);

@@ -77,6 +77,7 @@ struct Mma<bf16_t> {
     const uint32_t w = e < 2 ? r.x : e < 4 ? r.y : e < 6 ? r.z : r.w;
     return (Elt)((e & 1) ? (w >> 16) : w);
   }
+  static __device__ __forceinline__ Elt to_elt(float v) { return (Elt)pack_bf2(v, 0.f); }
 };
 
 template <>
@@ -109,6 +110,7 @@ struct Mma<float> {
   static __device__ __forceinline__ Elt elt(const uint4& r, int e) {
     return __uint_as_float(e == 0 ? r.x : e == 1 ? r.y : e == 2 ? r.z : r.w);
   }
+  static __device__ __forceinline__ Elt to_elt(float v) { return v; }
 };
 
 // The per-element mask tests of a score tile sit in blocks that only the diagonal and the ragged last tiles
@@ -134,6 +136,9 @@ __device__ __forceinline__ float block_sum(float v, float* red, int tid) {
   return t;
 }
 
+__device__ __forceinline__ float to_f32_elt(float v) { return v; }
+__device__ __forceinline__ float to_f32_elt(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
 template <class T>
 __device__ __forceinline__ typename Mma<T>::Frag lds_frag(const typename Mma<T>::Elt* p) {
   return *reinterpret_cast<const typename Mma<T>::Frag*>(p);
@@ -151,7 +156,7 @@ struct TileRegs {
   static constexpr int TOTAL = R * PPR;
   static constexpr int NV = (TOTAL + NT - 1) / NT;
   uint4 raw[NV];
-  float rf[NV];   // row factor of scaled tiles: 1 / rowdiv[row], 0 for a row that does not exist
+  float rf[NV];   // row divisor of scaled tiles: rowdiv[row] (of the nearest row that exists: the others' elements are zero)
 
   __device__ __forceinline__ void load(const HeadRows<const T>& hr, int pos0, int pend, int d, int tid,
                                        const float* rowdiv = nullptr, int64_t rdstride = 0) {
@@ -165,8 +170,9 @@ struct TileRegs {
       const int ps = max(pos < pend ? pos : pend - 1, hr.lo);
       const uint4 t = *reinterpret_cast<const uint4*>(hr.base + ((unsigned)ps * hr.pitch + (unsigned)(live ? pc * EPP : 0)));
       raw[u] = live ? t : make_uint4(0u, 0u, 0u, 0u);
-      rf[u] = 0.f;
-      if (rowdiv) rf[u] = live ? 1.0f / rowdiv[(unsigned)ps * (unsigned)rdstride] : 0.f;
+      // (the divisor as loaded: anything computed from it here would make this a wait for every load above it)
+      rf[u] = 1.0f;
+      if (rowdiv) rf[u] = rowdiv[(unsigned)ps * (unsigned)rdstride];
     }
   }
   // as loaded: row-major [R][pr] and / or transposed [DP][pt] (row x at column tpos(x))
@@ -185,7 +191,7 @@ struct TileRegs {
       }
     }
   }
-  // times the row factor and a constant each: srm for the row-major copy, str for the transposed one
+  // over the row divisor and times a constant each: srm for the row-major copy, str for the transposed one
   __device__ __forceinline__ void store_scaled(Elt* rm, int pr, float srm, Elt* tr, int pt, float str, int tid) const {
 #pragma unroll
     for (int u = 0; u < NV; ++u) {
@@ -194,17 +200,19 @@ struct TileRegs {
         const int row = idx % R, pc = idx / R;
         float x[EPP], y[EPP];
         M::unpack(raw[u], x);
-        const float f1 = rf[u] * srm, f2 = rf[u] * str;
+        const float inv = 1.0f / rf[u], f1 = inv * srm, f2 = inv * str;
 #pragma unroll
         for (int e = 0; e < EPP; ++e) {
           y[e] = x[e] * f2;
           x[e] *= f1;
         }
-        *reinterpret_cast<uint4*>(rm + row * pr + pc * EPP) = M::pack(x);
-        const uint4 yt = M::pack(y);
-        Elt* t0 = tr + pc * EPP * pt + M::tpos(row);
+        if (rm) *reinterpret_cast<uint4*>(rm + row * pr + pc * EPP) = M::pack(x);
+        if (tr) {
+          const uint4 yt = M::pack(y);
+          Elt* t0 = tr + pc * EPP * pt + M::tpos(row);
 #pragma unroll
-        for (int e = 0; e < EPP; ++e) t0[e * pt] = M::elt(yt, e);
+          for (int e = 0; e < EPP; ++e) t0[e * pt] = M::elt(yt, e);
+        }
       }
     }
   }
@@ -272,6 +280,218 @@ struct Shape {
 };
 
 // ---------------------------------------------------------------------------------------
+// p = 1 in linear time on top of the dense tiles ("linear mode").  With f(s) = a0 + a1 s everything a query
+// needs from the keys before its chunk is one small state
+//     S = sum_j [k_j; 1] (x) [v_j, 1]        (DP + 1) x (DP + 1) floats
+// (sum k (x) v, sum k, sum v, the count; reference: example.py:167-193), and the backward pass needs the
+// mirror image R = sum_i [q_i; 1] (x) [g_i, c_i] over the queries after a key's chunk.  The sequence is cut
+// into chunks of `lchunk` positions; dense_state_kernel forms the state of every chunk alone, a scan over
+// the chunks (lin_scan_kernel; unmasked: their plain sum) turns them into what each chunk needs, and
+// the three dense kernels start from that state and walk only their own chunk's score tiles.  Cost per
+// token: ~lchunk d (tiles) + ~4 d^2 (state), whatever the sequence length, for every head dimension.
+// The states are built from the rows as stored (no normaliser scale): the kernels' register-side operands
+// and epilogues carry the scales, as in the tile part.
+//
+// A state slot in memory: nblk blocks of DP rows x LD floats -- the DP x DP part sum X (x) Y, times a
+// constant the consumer wants folded in, as [x][y] ("natural") and / or [y][x] ("transposed"), whichever
+// layouts the consumers read rows of -- then the vectors: sum_t e_t X_t, sum_t Y_t, and sum_t e_t.
+// ---------------------------------------------------------------------------------------
+template <int DP>
+struct LinState {
+  static constexpr int LD = DP + 4;            // row pitch of a block: rows stay 16-byte aligned
+  static constexpr int BLOCK = DP * LD;
+  __host__ __device__ static constexpr int64_t floats(int nblk) {
+    return ((int64_t)nblk * BLOCK + 2 * DP + 4 + 63) / 64 * 64;
+  }
+};
+
+// slots of fp32 states, in place: mode 0: slot c = sum of the slots before c; 1: of the slots after c;
+// 2: slot 0 = the sum of all.  grid = (ceil(ss / 1024), heads), one float4 per thread.
+__global__ __launch_bounds__(256) void lin_scan_kernel(float* __restrict__ state, int nslots, int64_t ss, int mode) {
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= ss) return;
+  float* base = state + (int64_t)blockIdx.y * nslots * ss + idx;
+  float4 run = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int step = 0; step < nslots; ++step) {
+    const int c = mode == 1 ? nslots - 1 - step : step;
+    float4* p = reinterpret_cast<float4*>(base + c * ss);
+    const float4 t = *p;
+    if (mode != 2) *p = run;
+    run.x += t.x; run.y += t.y; run.z += t.z; run.w += t.w;
+  }
+  if (mode == 2) *reinterpret_cast<float4*>(base) = run;
+}
+
+__device__ __forceinline__ void lin_store4(float* p, const float4& v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void lin_store4(uint16_t* p, const float4& v) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf2(v.x, v.y), pack_bf2(v.z, v.w));
+}
+
+// One block of a state on its way into LDS as a matrix operand: DP rows of DP elements, pitch DP + PAD.
+// Up to eight 16-byte loads per thread are in flight before the first is used.
+template <int DP, class T, int NT>
+__device__ __forceinline__ void lin_stage_block(const float* __restrict__ g, typename Mma<T>::Elt* l, int tid) {
+  using M = Mma<T>;
+  constexpr int PS = DP + M::PAD, LD = LinState<DP>::LD, V4 = DP / 4, TOTAL = DP * V4, NV = (TOTAL + NT - 1) / NT;
+  constexpr int B = NV < 8 ? NV : 8;
+  static_assert(TOTAL % NT == 0, "every thread moves the same number of pieces");
+  static_for<(NV + B - 1) / B>([&](auto btag) {
+    constexpr int U0 = decltype(btag)::value * B, N = NV - U0 < B ? NV - U0 : B;
+    float4 t[N];
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+      const int idx = tid + (U0 + u) * NT;
+      t[u] = *reinterpret_cast<const float4*>(g + (idx / V4) * LD + (idx % V4) * 4);
+    }
+#pragma unroll
+    for (int u = 0; u < N; ++u) {
+      const int idx = tid + (U0 + u) * NT;
+      lin_store4(l + (idx / V4) * PS + (idx % V4) * 4, t[u]);
+    }
+  });
+}
+
+// t + (own rows x DP, fragments af) . B, where brow is the LDS row that holds output column i's DP
+// contraction elements, already offset by the lane half's EPL hh
+template <int DP, class T>
+__device__ __forceinline__ f16v lin_own_times(const typename Mma<T>::Frag (&af)[DP / Mma<T>::KF],
+                                              const typename Mma<T>::Elt* brow, f16v t) {
+  using M = Mma<T>;
+#pragma unroll
+  for (int m0 = 0; m0 < DP / M::KF; m0 += 2) {   // (two operand reads in flight, not all of them: register pressure)
+    const typename M::Frag b0 = lds_frag<T>(brow + M::KF * m0), b1 = lds_frag<T>(brow + M::KF * (m0 + 1));
+    t = M::mma(af[m0], b0, t);
+    t = M::mma(af[m0 + 1], b1, t);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  return t;
+}
+
+// The state of every chunk alone.  With X_t, Y_t the rows at position t of chunk c (Y_t divided by ydiv_t when
+// given), e_t = ew_t (1 when not given) and bs = cscale hscale[head] (hscale: 1 when not given):
+//   block nat_blk [x][y] = block trn_blk [y][x] = bs sum_t X_t[x] Y_t[y]          (a block index < 0: not written)
+//   vectors: [x] = sum_t e_t X_t[x],   [DP + y] = sum_t Y_t[y],   [2 DP] = sum_t e_t
+// grid = (heads, chunks), 256 threads; the (DP / 32)^2 tiles of the x-by-y block are dealt to the four waves,
+// and the wave that has column block 0 (row block 0) of a block row (column) also sums that row block's X e
+// (column block's Y) from the operand fragments it reads anyway.
+template <int DP, class T, bool HAS_E>
+__global__ __launch_bounds__(256) void dense_state_kernel(Rows<const T> X, Rows<const T> Y, RowScalars ydiv,
+                                                          RowScalars ew, const float* __restrict__ hscale, float cscale,
+                                                          float* __restrict__ state, int nblk, int nat_blk, int trn_blk,
+                                                          int npos, int d, int lchunk) {
+  using M = Mma<T>;
+  using Elt = typename M::Elt;
+  using Frag = typename M::Frag;
+  using LS = LinState<DP>;
+  constexpr int KF = M::KF, EPL = M::EPL, CB = DP / 32, NTL = CB * CB, TPW = (NTL + 3) / 4;
+  constexpr int BN = Shape<DP, T>::BN, PT = BN + M::PAD;
+  static_assert(256 % BN == 0, "a thread stages the same row of every stage");
+  __shared__ __attribute__((aligned(16))) Elt Xt[DP * PT];
+  __shared__ __attribute__((aligned(16))) Elt Yt[DP * PT];
+  __shared__ __attribute__((aligned(16))) float El[BN];
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
+  const int head = blockIdx.x, c = blockIdx.y, nch = gridDim.y;
+  const HeadRows<const T> Xh = X.head(head), Yh = Y.head(head);
+  const float* ydh = ydiv.head(head);
+  const float* ewh = ew.head(head);
+  const int lo = Xh.lo;
+  const int t0 = c * lchunk, t1 = (t0 + lchunk < npos ? t0 + lchunk : npos);
+
+  f16v acc[TPW];
+  float xs[TPW], ys[TPW];   // this lane's part of sum e X[rb 32 + i] / sum Y[cb 32 + i] where tile t is the one that sums
+#pragma unroll
+  for (int t = 0; t < TPW; ++t) {
+    xs[t] = ys[t] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  }
+  float esum = 0.f;   // threads < BN: sum of e over the positions tb + tid of every stage
+
+  TileRegs<DP, T, BN, 256> xt, yt;
+  float ev = 1.0f, em = 0.f;   // e of the position this thread stages, as loaded, and whether the position exists
+  auto stage_load = [&](int tb) {
+    xt.load(Xh, tb, t1, d, tid);
+    yt.load(Yh, tb, t1, d, tid, ydh, ydiv.stride);
+    // (every thread, clamped, not predicated, nothing computed from it yet: a wait here would wait for the rows too)
+    const int pos = tb + tid % BN;
+    if (HAS_E) ev = ewh[(int64_t)max(pos < t1 ? pos : t1 - 1, lo) * ew.stride];
+    em = (pos >= lo && pos < t1) ? 1.0f : 0.f;
+  };
+  if (t0 < t1) stage_load(t0);
+  for (int tb = t0; tb < t1; tb += BN) {
+    __syncthreads();   // the previous stage has been read
+    xt.store(nullptr, 0, Xt, PT, tid);
+    if (ydh) yt.store_scaled(nullptr, 0, 1.0f, Yt, PT, 1.0f, tid);
+    else yt.store(nullptr, 0, Yt, PT, tid);
+    if (tid < BN) {
+      const float e = ev * em;
+      esum += e;
+      El[M::tpos(tid)] = e;   // (same column order as the transposed tiles)
+    }
+    __syncthreads();
+    if (tb + BN < t1) stage_load(tb + BN);   // (the next stage's rows arrive under this stage's tiles)
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+      const int tile = w + 4 * t;
+      if (tile < NTL) {
+        const int rb = tile / CB, cb = (tile % CB + rb) % CB;   // (skewed: every wave gets its share of the summing tiles)
+#pragma unroll
+        for (int f = 0; f < BN / KF; ++f) {
+          const Frag a = lds_frag<T>(Xt + (rb * 32 + i) * PT + KF * f + EPL * hh);
+          const Frag b = lds_frag<T>(Yt + (cb * 32 + i) * PT + KF * f + EPL * hh);
+          acc[t] = M::mma(a, b, acc[t]);
+          if (cb == 0) {
+            float x[EPL];
+            M::unpack(__builtin_bit_cast(uint4, a), x);
+#pragma unroll
+            for (int e4 = 0; e4 < EPL; e4 += 4) {
+              const float4 ev = *reinterpret_cast<const float4*>(El + KF * f + EPL * hh + e4);
+              xs[t] += x[e4] * ev.x + x[e4 + 1] * ev.y + x[e4 + 2] * ev.z + x[e4 + 3] * ev.w;
+            }
+          }
+          if (rb == 0) {
+            float y[EPL];
+            M::unpack(__builtin_bit_cast(uint4, b), y);
+#pragma unroll
+            for (int e4 = 0; e4 < EPL; ++e4) ys[t] += y[e4];
+          }
+        }
+      }
+    }
+  }
+  float* st = state + ((int64_t)head * nch + c) * LS::floats(nblk);
+  float* vec = st + (int64_t)nblk * LS::BLOCK;
+  const float bs = cscale * (hscale ? hscale[head] : 1.0f);
+#pragma unroll
+  for (int t = 0; t < TPW; ++t) {
+    const int tile = w + 4 * t;
+    if (tile < NTL) {
+      const int rb = tile / CB, cb = (tile % CB + rb) % CB;
+      if (nat_blk >= 0) {
+        float* nb = st + (int64_t)nat_blk * LS::BLOCK;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) nb[(rb * 32 + trow(r, hh)) * LS::LD + cb * 32 + i] = bs * acc[t][r];
+      }
+      if (trn_blk >= 0) {   // registers 4 j .. 4 j + 3 are four consecutive x
+        float* tb = st + (int64_t)trn_blk * LS::BLOCK + (cb * 32 + i) * LS::LD + rb * 32 + 4 * hh;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          *reinterpret_cast<float4*>(tb + 8 * j) =
+              make_float4(bs * acc[t][4 * j], bs * acc[t][4 * j + 1], bs * acc[t][4 * j + 2], bs * acc[t][4 * j + 3]);
+      }
+      const float xsum = xs[t] + __shfl_xor(xs[t], 32, 64), ysum = ys[t] + __shfl_xor(ys[t], 32, 64);
+      if (cb == 0 && hh == 0) vec[rb * 32 + i] = xsum;
+      if (rb == 0 && hh == 0) vec[DP + cb * 32 + i] = ysum;
+    }
+  }
+  if (w == 0) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) esum += __shfl_xor(esum, off, 64);
+    if (tid == 0) vec[2 * DP] = esum;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Forward.  grid = (heads, query blocks of 128 RT positions from the one that holds position Q.lo).
 // npos: positions of the queries end here (nk under the mask: query i sits at position i + nk - nq).
 // ---------------------------------------------------------------------------------------
@@ -279,7 +499,7 @@ template <int DP, class T, int RT, int BN, int NW>
 __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_FWD)) void dense_fwd_kernel(
     Rows<const T> Q, Rows<const T> K, Rows<const T> V, const float* __restrict__ qscale,
     const float* __restrict__ kscale, Rows<T> O, RowScalarsOut den, int npos, int nk, int d, int masked, float a0,
-    float a1, float a2, int ratio) {
+    float a1, float a2, int ratio, const float* __restrict__ lstate, int lchunk, int lslots) {
   using M = Mma<T>;
   using Elt = typename M::Elt;
   using Frag = typename M::Frag;
@@ -288,6 +508,7 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_FWD)) void dense_fwd_ke
   constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
   static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
+  static_assert(L::bytes(1, 1, 0) >= (size_t)DP * (DP + M::PAD) * sizeof(Elt) + 2 * DP * sizeof(float), "a state fits the stage buffers");
   extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
   Elt* Kl = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
   Elt* Vt = Kl + 2 * L::RM;                       // [2][DP][PT]
@@ -309,6 +530,9 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_FWD)) void dense_fwd_ke
 
   const int kend = masked ? (tok0 + BM < nk ? tok0 + BM : nk) : nk;
   const int nst = (kend + BN - 1) / BN;
+  // linear mode: the keys before the block's chunk (unmasked: all keys) come as a state
+  const int lc = (lstate && masked) ? tok0 / lchunk : 0;
+  const int st0 = lstate ? (masked ? lc * (lchunk / BN) : nst) : 0;
   TileRegs<DP, T, BN, NT> kt, vt;
   auto stage_load = [&](int st) {
     kt.load(Kh, st * BN, nk, d, tid);
@@ -328,6 +552,41 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_FWD)) void dense_fwd_ke
     for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rt][cb][r] = 0.f;
+  }
+
+  if (st0 < nst) stage_load(st0);   // (requested before the state is: one memory latency, not two)
+  if (lstate && (!masked || lc > 0)) {
+    // o += a1 qh . S1 + a0 sum v,  den += a1 qh . sum k + a0 count   (S1 = sum k (x) v of the keys in the state)
+    constexpr int PS = DP + M::PAD;
+    Elt* St = reinterpret_cast<Elt*>(dense_smem);             // a1 S1 as [value channel][key channel]
+    float* sk = reinterpret_cast<float*>(St + DP * PS);       // sum k
+    float* sv = sk + DP;                                      // sum v
+    const float* sp = lstate + ((int64_t)hkv * lslots + lc) * LinState<DP>::floats(1);   // (one block: transposed)
+    lin_stage_block<DP, T, NT>(sp, St, tid);
+    for (int idx = tid; idx < 2 * DP; idx += NT) sk[idx] = sp[LinState<DP>::BLOCK + idx];
+    __syncthreads();
+    const int before = masked ? lc * lchunk : nk;
+    const float cnt = (float)(before < nk ? before : nk);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const float z = a0 * sv[cb * 32 + i];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[rt][cb][r] = z;
+        acc[rt][cb] = lin_own_times<DP, T>(qf[rt], St + (cb * 32 + i) * PS + EPL * hh, acc[rt][cb]);
+      }
+      float dd = 0.f;
+#pragma unroll
+      for (int m = 0; m < NF; ++m) {
+        float x[EPL];
+        M::unpack(__builtin_bit_cast(uint4, qf[rt][m]), x);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) dd += x[e] * sk[KF * m + EPL * hh + e];
+      }
+      dn[rt] = a1 * dd + (hh == 0 ? a0 * cnt : 0.f);
+    }
+    __syncthreads();
   }
 
   // One 32-key tile against the wave's own tiles, as straight-line code.  rel = key tile base - first
@@ -391,12 +650,11 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_FWD)) void dense_fwd_ke
     });
   };
 
-  stage_load(0);
-  stage_store(0);
+  if (st0 < nst) stage_store(0);
   __syncthreads();
   const int q00 = tok0 + w * RT * 32;   // first position of the wave's own tile 0
-  for (int st = 0; st < nst; ++st) {
-    const int buf = st & 1;
+  for (int st = st0; st < nst; ++st) {
+    const int buf = (st - st0) & 1;
     if (st + 1 < nst) stage_load(st + 1);
     const Elt* kl = Kl + buf * L::RM;
     const Elt* vl = Vt + buf * L::TR;
@@ -444,7 +702,8 @@ template <int DP, class T, int RT, int BN, int NW>
 __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kernel(
     Rows<const T> Q, Rows<const T> GO, RowScalars den, RowScalars cvec, Rows<const T> K, Rows<const T> V,
     const float* __restrict__ qscale, const float* __restrict__ kscale, Rows<T> DQ, float* __restrict__ rpart,
-    int npos, int nk, int d, int masked, int p2, float a1, float a2, int ratio) {
+    int npos, int nk, int d, int masked, int p2, float a1, float a2, int ratio, const float* __restrict__ lstate,
+    int lchunk, int lslots) {
   using M = Mma<T>;
   using Elt = typename M::Elt;
   using Frag = typename M::Frag;
@@ -453,6 +712,7 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kern
   constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
   static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
+  static_assert(L::bytes(2, 1, 0) >= (size_t)DP * (DP + M::PAD) * sizeof(Elt) + DP * sizeof(float), "a state fits the stage buffers");
   extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
   Elt* Kl = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
   Elt* Vl = Kl + 2 * L::RM;                       // [2][BN][PR]
@@ -475,14 +735,19 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kern
     const int pos = tok0 + (w * RT + rt) * 32 + i;
     const bool live = pos >= Qh.lo && pos < npos;
     const int ps = max(pos < npos ? pos : npos - 1, Qh.lo);
-    const float rden = live ? 1.0f / denh[(int64_t)ps * den.stride] : 0.f;
-    cown[rt] = live ? ch[(int64_t)ps * cvec.stride] : 0.f;
+    // (clamped loads whose values are used whatever `live` says: the compiler moves a load that only one side of a
+    // select uses under that condition, where it gets a wait of its own -- for every load issued before it)
+    const float dnv = denh[(int64_t)ps * den.stride], cvv = ch[(int64_t)ps * cvec.stride], lm = live ? 1.0f : 0.f;
+    const float rden = lm / dnv;
+    cown[rt] = lm * cvv;
     if (p2) load_own_frags<DP, T>(Qh, pos, npos, d, hh, kq * 2.0f * a2, qf[rt]);
     load_own_frags<DP, T>(Gh, pos, npos, d, hh, rden, gf[rt]);
   }
 
   const int kend = masked ? (tok0 + BM < nk ? tok0 + BM : nk) : nk;
   const int nst = (kend + BN - 1) / BN;
+  const int lc = (lstate && masked) ? tok0 / lchunk : 0;   // (linear mode, as in the forward kernel)
+  const int st0 = lstate ? (masked ? lc * (lchunk / BN) : nst) : 0;
   TileRegs<DP, T, BN, NT> kt, vt;
   auto stage_load = [&](int st) {
     kt.load(Kh, st * BN, nk, d, tid);
@@ -500,6 +765,36 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kern
     for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[rt][cb][r] = 0.f;
+
+  if (st0 < nst) stage_load(st0);   // (requested before the state is: one memory latency, not two)
+  if (lstate && (!masked || lc > 0)) {
+    // sum_j a1 (g . v_j - c) k_j over the keys in the state = a1 (g . S1^T - c sum k)
+    constexpr int PS = DP + M::PAD;
+    Elt* Sn = reinterpret_cast<Elt*>(dense_smem);             // a1 S1 as [key channel][value channel]
+    float* sk = reinterpret_cast<float*>(Sn + DP * PS);       // sum k
+    const float* sp = lstate + ((int64_t)hkv * lslots + lc) * LinState<DP>::floats(1);   // (one block: natural)
+    lin_stage_block<DP, T, NT>(sp, Sn, tid);
+    for (int idx = tid; idx < DP; idx += NT) sk[idx] = sp[LinState<DP>::BLOCK + idx];
+    __syncthreads();
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float crow[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int pos = tok0 + (w * RT + rt) * 32 + trow(r, hh);
+        const float cvv = ch[(int64_t)max(pos < npos ? pos : npos - 1, Qh.lo) * cvec.stride];   // (clamped, not predicated)
+        crow[r] = -a1 * cvv * ((pos >= Qh.lo && pos < npos) ? 1.0f : 0.f);
+      }
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const float z = sk[cb * 32 + i];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[rt][cb][r] = crow[r] * z;
+        acc[rt][cb] = lin_own_times<DP, T>(gf[rt], Sn + (cb * 32 + i) * PS + EPL * hh, acc[rt][cb]);
+      }
+    }
+    __syncthreads();
+  }
 
   // (rel as in the forward kernel: own tile rt has the key tile on its diagonal when rel == 32 rt and
   // wholly after its queries when rel > 32 rt)
@@ -556,12 +851,11 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kern
     });
   };
 
-  stage_load(0);
-  stage_store(0);
+  if (st0 < nst) stage_store(0);
   __syncthreads();
   const int q00 = tok0 + w * RT * 32;
-  for (int st = 0; st < nst; ++st) {
-    const int buf = st & 1;
+  for (int st = st0; st < nst; ++st) {
+    const int buf = (st - st0) & 1;
     if (st + 1 < nst) stage_load(st + 1);
     const Elt* kl = Kl + buf * L::RM;
     const Elt* vl = Vl + buf * L::RM;
@@ -582,7 +876,20 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kern
   const HeadRows<T> Dh = DQ.head(head);
   float rs = 0.f;
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+  for (int rt = 0; rt < RT; ++rt) {
+    // (the q elements are all requested before the first store: a load that had to stay behind a store that
+    // may alias it would cost one memory round trip per element)
+    float qv[CB][16];
+    if (rpart) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int pos = tok0 + (w * RT + rt) * 32 + trow(r, hh);
+        const int ps = max(pos < npos ? pos : npos - 1, Qh.lo);   // (clamped, not predicated: predicated loads get a wait each)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+          qv[cb][r] = to_f32(Qh.base[(unsigned)ps * Qh.pitch + (unsigned)(cb * 32 + i < d ? cb * 32 + i : 0)]);
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int pos = tok0 + (w * RT + rt) * 32 + trow(r, hh);
@@ -593,11 +900,12 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kern
           if (c < d) {
             const float v = acc[rt][cb][r] * kq;
             Dh.base[(unsigned)pos * Dh.pitch + (unsigned)c] = from_f32<T>(v);
-            if (rpart) rs += v * to_f32(Qh.base[(unsigned)pos * Qh.pitch + (unsigned)c]);
+            if (rpart) rs += v * qv[cb][r];
           }
         }
       }
     }
+  }
   if (rpart) {
     rs = block_sum<NW>(rs, red, tid);
     if (tid == 0) rpart[(int64_t)head * nb + bx] = rs;
@@ -615,7 +923,8 @@ template <int DP, class T, int RT, int BN, int NW>
 __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_KV)) void dense_dkdv_kernel(
     Rows<const T> K, Rows<const T> V, Rows<const T> Q, Rows<const T> GO, RowScalars den, RowScalars cvec,
     const float* __restrict__ qscale, const float* __restrict__ kscale, Rows<T> DK, Rows<T> DV,
-    float* __restrict__ rpart, int npos, int nk, int d, int masked, float a0, float a1, float a2, int ratio) {
+    float* __restrict__ rpart, int npos, int nk, int d, int masked, float a0, float a1, float a2, int ratio,
+    const float* __restrict__ lstate, int lchunk, int lslots) {
   using M = Mma<T>;
   using Elt = typename M::Elt;
   using Frag = typename M::Frag;
@@ -624,6 +933,7 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_KV)) void dense_dkdv_ke
   constexpr int HC = (Shape<DP, T>::BF && NF % 4 == 0) ? 4 : 2;   // operand fragments read ahead at a time
   static_assert(NF % HC == 0, "whole groups of fragments");
   constexpr int PR = L::PR, PT = L::PT;
+  static_assert(L::bytes(2, 2, 0) >= (size_t)2 * DP * (DP + M::PAD) * sizeof(Elt) + 2 * DP * sizeof(float), "a state fits the stage buffers");
   extern __shared__ __attribute__((aligned(16))) unsigned char dense_smem[];
   Elt* Ql = reinterpret_cast<Elt*>(dense_smem);   // [2][BN][PR]
   Elt* Gl = Ql + 2 * L::RM;                       // [2][BN][PR]
@@ -654,8 +964,11 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_KV)) void dense_dkdv_ke
 #pragma unroll
       for (int r = 0; r < 16; ++r) dk[rt][cb][r] = dv[rt][cb][r] = 0.f;
 
+  float dvc[CB], dkc[CB];   // (linear mode) what every own row's dv / dk gets on top, per channel cb * 32 + i
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb) dvc[cb] = dkc[cb] = 0.f;
   TileRegs<DP, T, BN, NT> qt, gt;
-  float creg = 0.f;
+  float creg = 0.f, cmask = 0.f;
   for (int hq = 0; hq < ratio; ++hq) {
     const int head = hkv * ratio + hq;
     const HeadRows<const T> Qh = Q.head(head), Gh = GO.head(head);
@@ -665,25 +978,59 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_KV)) void dense_dkdv_ke
     // f and f' of s = qs sr, where sr = q . kh is what the score tile holds
     const float c2 = a2 * qs * qs, c1 = a1 * qs, b2 = 2.0f * a2 * qs;
     const int lo = Qh.lo;
-    const int st0 = masked ? (tok0 > lo ? tok0 : lo) / BN : 0;
-    const int nst = (npos + BN - 1) / BN;
+    // linear mode: the queries after the block's chunk (unmasked: all queries) come as a state
+    const int lc = (lstate && masked) ? tok0 / lchunk : 0;
+    const int qend = (lstate && masked && (lc + 1) * lchunk < npos) ? (lc + 1) * lchunk : npos;
+    const int nst = (qend + BN - 1) / BN;
+    const int st0 = lstate && !masked ? nst : masked ? (tok0 > lo ? tok0 : lo) / BN : 0;
     auto stage_load = [&](int st) {
       qt.load(Qh, st * BN, npos, d, tid);
       gt.load(Gh, st * BN, npos, d, tid, denh, den.stride);
-      if (tid < BN) {
-        const int pos = st * BN + tid;
-        creg = (pos >= lo && pos < npos) ? -ch[(int64_t)pos * cvec.stride] * qs : 0.f;   // (-qs c: the tile's start value)
+      {   // (every thread, clamped, not predicated: a predicated load gets a wait that would also wait for the tiles' loads)
+        const int pos = st * BN + tid % BN;
+        creg = ch[(int64_t)max(pos < npos ? pos : npos - 1, lo) * cvec.stride];   // (as loaded: nothing here may wait for it)
+        cmask = (pos >= lo && pos < npos) ? 1.0f : 0.f;
       }
     };
     auto stage_store = [&](int buf) {
       qt.store(Ql + buf * L::RM, PR, Qt + buf * L::TR, PT, tid);
       gt.store_scaled(Gl + buf * L::RM, PR, qs, Gt + buf * L::TR, PT, 1.0f, tid);
-      if (tid < BN) Cl[buf * BN + tid] = creg;
+      if (tid < BN) Cl[buf * BN + tid] = -creg * qs * cmask;   // (-qs c: the tile's start value)
     };
-    if (st0 < nst) {
-      stage_load(st0);
-      stage_store(0);
+    // (requested before the state is -- one memory latency, not two -- where the registers are there: with fp32
+    // fragments of 96 or 128 channels the state's own loads would be left with one register set and a wait each)
+    constexpr bool EARLY = Shape<DP, T>::BF || DP <= 64;
+    if (EARLY && st0 < nst) stage_load(st0);
+    if (lstate && (!masked || lc + 1 < lslots)) {
+      // dv += a0 sum g + a1 qs kh . R1,  dk += a1 qs (v . R1^T - sum c q)   (R1 = sum q (x) g of the queries in the state);
+      // the two sums, the same for every own row, wait in dvc / dkc for the epilogue
+      constexpr int PS = DP + M::PAD;
+      Elt* Rn = reinterpret_cast<Elt*>(dense_smem);             // a1 qs R1 as [query channel][value channel]
+      Elt* Rt = Rn + DP * PS;                                   // and as [value channel][query channel]
+      float* rq = reinterpret_cast<float*>(Rt + DP * PS);       // sum c q
+      float* rg = rq + DP;                                      // sum g
+      const float aq = a1 * qs;
+      const float* sp = lstate + ((int64_t)head * lslots + lc) * LinState<DP>::floats(2);   // (two blocks: natural, transposed)
+      lin_stage_block<DP, T, NT>(sp, Rn, tid);
+      lin_stage_block<DP, T, NT>(sp + LinState<DP>::BLOCK, Rt, tid);
+      for (int idx = tid; idx < 2 * DP; idx += NT) rq[idx] = sp[2 * LinState<DP>::BLOCK + idx];
+      __syncthreads();
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        dvc[cb] += a0 * rg[cb * 32 + i];
+        dkc[cb] -= aq * rq[cb * 32 + i];
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+          dv[rt][cb] = lin_own_times<DP, T>(kf[rt], Rt + (cb * 32 + i) * PS + EPL * hh, dv[rt][cb]);
+          dk[rt][cb] = lin_own_times<DP, T>(vf[rt], Rn + (cb * 32 + i) * PS + EPL * hh, dk[rt][cb]);
+        }
+      __syncthreads();
     }
+    if (!EARLY && st0 < nst) stage_load(st0);
+    if (st0 < nst) stage_store(0);
     __syncthreads();
     // One 32-query tile against the wave's own key tiles, as straight-line code.  rel = query tile base -
     // first position of own tile 0 (masked only): own tile rt has the query tile on its diagonal when
@@ -780,7 +1127,18 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_KV)) void dense_dkdv_ke
   const HeadRows<T> DKh = DK.head(hkv), DVh = DV.head(hkv);
   float rs = 0.f;
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+  for (int rt = 0; rt < RT; ++rt) {
+    float kv[CB][16];   // (requested before the first store, as in the dq kernel)
+    if (rpart) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int pos = tok0 + (w * RT + rt) * 32 + trow(r, hh);
+        const int ps = pos < nk ? pos : nk - 1;   // (clamped, not predicated: predicated loads get a wait each)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+          kv[cb][r] = to_f32(Kh.base[(unsigned)ps * Kh.pitch + (unsigned)(cb * 32 + i < d ? cb * 32 + i : 0)]);
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int pos = tok0 + (w * RT + rt) * 32 + trow(r, hh);
@@ -789,14 +1147,15 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_KV)) void dense_dkdv_ke
         for (int cb = 0; cb < CB; ++cb) {
           const int c = cb * 32 + i;
           if (c < d) {
-            const float v = dk[rt][cb][r] * ks;
+            const float v = (dk[rt][cb][r] + dkc[cb]) * ks;
             DKh.base[(unsigned)pos * DKh.pitch + (unsigned)c] = from_f32<T>(v);
-            DVh.base[(unsigned)pos * DVh.pitch + (unsigned)c] = from_f32<T>(dv[rt][cb][r]);
-            if (rpart) rs += v * to_f32(Kh.base[(unsigned)pos * Kh.pitch + (unsigned)c]);
+            DVh.base[(unsigned)pos * DVh.pitch + (unsigned)c] = from_f32<T>(dv[rt][cb][r] + dvc[cb]);
+            if (rpart) rs += v * kv[cb][r];
           }
         }
       }
     }
+  }
   if (rpart) {
     rs = block_sum<NW>(rs, red, tid);
     if (tid == 0) rpart[(int64_t)hkv * nb + bx] = rs;

@@ -58,6 +58,21 @@ def test_head_dimensions_and_the_dense_plan(built, monkeypatch):
             512 + (6 * 5000 * 4 + 255) // 256 * 256 + (6 * 2 * 40 * 4 + 255) // 256 * 256
         assert built.fastmax_saved_state_bytes(C.byref(ds)) == 256
         assert built.fastmax_state_bytes(C.byref(ds)) == 0 and "recurrent" in _cabi.last_error()
+    # p = 1 past 1024 causal / 512 unmasked positions: the dense kernels take one small state per 256 positions
+    # with them (linear time): per key/value head and slot the d x d block in one layout plus the sums,
+    # backward also per query head the block in both layouts
+    a256 = lambda x: (x + 255) // 256 * 256
+    r64 = lambda x: (x + 63) // 64 * 64
+    for d, dp in ((128, 128), (48, 64), (80, 96)):
+        one, two = r64(dp * (dp + 4) + 2 * dp + 4), r64(2 * dp * (dp + 4) + 2 * dp + 4)
+        ds = desc(d=d, dtype=0, bh=6, bhkv=3, n=5000, mask=True, p=1)
+        assert built.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD) == 512 + a256(3 * 20 * one * 4)
+        assert built.fastmax_workspace_min_bytes(C.byref(ds), _cabi.PASS_BACKWARD) == \
+            512 + a256(6 * 5000 * 4) + a256(6 * 2 * 40 * 4) + a256(3 * 20 * one * 4) + a256(6 * 20 * two * 4)
+        assert built.fastmax_saved_state_bytes(C.byref(ds)) == 256
+        assert built.fastmax_workspace_bytes(C.byref(desc(d=d, bh=6, n=1000, mask=True, p=1)), _cabi.PASS_FORWARD) == 512
+        assert built.fastmax_workspace_bytes(C.byref(desc(d=d, bh=6, n=600, mask=False, p=1)), _cabi.PASS_FORWARD) == \
+            512 + a256(6 * 3 * one * 4)
     short, long_ = desc(bh=96, n=2048, dtype=1, mask=True), desc(bh=96, n=16384, dtype=1, mask=True)
     assert built.fastmax_workspace_bytes(C.byref(short), _cabi.PASS_FORWARD) > 1 << 20   # (FASTMAX_PATH=moments here)
     monkeypatch.delenv("FASTMAX_PATH")

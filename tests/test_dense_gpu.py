@@ -252,12 +252,14 @@ def test_strided_views_of_a_fused_projection_d128(built):
     assert_close("dv", gx[:, :, :, r + 1].permute(0, 2, 1, 3).reshape(b * g, t, hs), fold(rdv), 1e-4, atol=1e-6)
 
 
-@pytest.mark.parametrize("shape,mask,dtype", [((12, 640, 64), True, torch.bfloat16),     # (dk/dv kernel: 74 KB of LDS)
-                                              ((6, 500, 128), True, torch.float32), ((8, 300, 48), False, torch.float32)])
-def test_graph_replays_match_eager(ops, shape, mask, dtype):
+@pytest.mark.parametrize("shape,mask,dtype,p", [((12, 640, 64), True, torch.bfloat16, 2),     # (dk/dv kernel: 74 KB of LDS)
+                                                ((6, 500, 128), True, torch.float32, 2), ((8, 300, 48), False, torch.float32, 2),
+                                                ((3, 1400, 128), True, torch.bfloat16, 1),   # (linear mode: chunk states)
+                                                ((3, 1100, 96), False, torch.float32, 1)])
+def test_graph_replays_match_eager(ops, shape, mask, dtype, p):
     """The dense kernels allocate nothing, clear nothing and never synchronise either: a forward + backward
     step captures into a HIP graph, and every replay equals the eager result."""
-    kw = dict(mask=mask, normalize=True, p=2)
+    kw = dict(mask=mask, normalize=True, p=p)
 
     def step(q, k, v, go):
         o, den, sc, arg = ops.forward(q, k, v, **kw)
@@ -285,3 +287,76 @@ def test_graph_replays_match_eager(ops, shape, mask, dtype):
         torch.cuda.synchronize()
         for name, a, b in zip(("o", "dq", "dk", "dv"), outs, eager):
             assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager result"
+
+
+# ---- p = 1 past the lengths where the dense kernels switch to chunk states plus the own chunk's tiles ----
+
+@pytest.mark.parametrize("d", [16, 48, 64, 96, 128])
+@pytest.mark.parametrize("mask", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_mode_head_dims(ops, d, mask, dtype):
+    # whole chunks, a ragged last chunk, a last chunk of one position
+    for n in (1280, 1337, 1025):
+        run_case(ops, (2, n, d), dtype=dtype, seed=n + d, mask=mask, normalize=True, p=1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mask", [False, True])
+def test_linear_mode_coefficients_and_grouped_heads(ops, dtype, mask):
+    run_case(ops, (2, 1500, 128), dtype=dtype, seed=71, mask=mask, normalize=True, p=1, a0=1.5, a1=0.5)
+    run_case(ops, (2, 1100, 96), dtype=dtype, seed=72, mask=mask, normalize=True, p=1, a0=0.7, a1=1.3, lim=1.5)
+    run_case(ops, (2, 1100, 48), dtype=dtype, seed=73, mask=mask, normalize=False, p=1, scale=0.1)
+    run_case(ops, (6, 1300, 128), dtype=dtype, seed=74, kv_shape=(2, 1300, 128), ratio=3, mask=mask, normalize=True, p=1)
+    run_case(ops, (4, 1111, 64), dtype=dtype, seed=75, kv_shape=(1, 1111, 64), ratio=4, mask=mask, normalize=True, p=1)
+
+
+@pytest.mark.parametrize("nq,nk,d,dtype", [(1100, 1400, 128, torch.float32), (700, 1300, 96, torch.float32),
+                                           (1200, 1200 + 255, 48, torch.float32), (1100, 1500, 128, torch.bfloat16),
+                                           (3, 1290, 64, torch.bfloat16), (1300, 600, 128, torch.float32)])
+def test_linear_mode_key_prefix_and_unequal_lengths(ops, nq, nk, d, dtype):
+    q, _, _, go = O.seeded_inputs((3, nq, d), seed=81, dtype=dtype)
+    _, k, v, _ = O.seeded_inputs((3, nk, d), seed=82, dtype=dtype)
+    for mask in (True, False):
+        if mask and nq > nk:
+            continue
+        kw = dict(mask=mask, normalize=True, p=1)
+        qd, kd, vd, god = (t.cuda() for t in (q, k, v, go))
+        print("linear-mode prefix case", nq, nk, d, dtype, mask, flush=True)
+        o, den, sc, arg = ops.forward(qd, kd, vd, **kw)
+        dq, dk, dv = ops.backward(qd, kd, vd, o, den, god, qk_scale=sc, qk_argmax=arg, **kw)
+        ro, rdq, rdk, rdv = O.dense_truth(q.float(), k.float(), v.float(), go.float(), **kw)
+        tol = TOL[dtype]
+        for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+            assert_close(f"mask={mask}/{name}", got.float(), ref, tol, atol=1e-6)
+
+
+def test_linear_mode_long_sequence_matches_the_moment_kernels(ops, monkeypatch):
+    # a length the oracle's dense closed form would take long on: the other kernel family is the reference
+    for mask in (True, False):
+        for dtype in (torch.float32, torch.bfloat16):
+            q, k, v, go = (t.cuda() for t in O.seeded_inputs((4, 9000, 64), seed=91, dtype=dtype))
+            kw = dict(mask=mask, normalize=True, p=1)
+            monkeypatch.setenv("FASTMAX_PATH", "dense")
+            o, den, sc, arg = ops.forward(q, k, v, **kw)
+            g = ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+            monkeypatch.setenv("FASTMAX_PATH", "moments")
+            o2, den2, sc2, arg2 = ops.forward(q, k, v, **kw)
+            g2 = ops.backward(q, k, v, o2, den2, go, qk_scale=sc2, qk_argmax=arg2, **kw)
+            tol = 2e-4 if dtype == torch.float32 else 3e-2
+            assert_close("o", o.float(), o2.float(), tol)
+            assert_close("den", den, den2, tol)
+            for name, a, b in zip(("dq", "dk", "dv"), g, g2):
+                assert_close(name, a.float(), b.float(), tol, atol=1e-6)
+
+
+def test_linear_mode_is_deterministic(ops):
+    q, k, v, go = (t.cuda() for t in O.seeded_inputs((3, 1400, 128), seed=95, dtype=torch.bfloat16))
+    kw = dict(mask=True, normalize=True, p=1)
+    o, den, sc, arg = ops.forward(q, k, v, **kw)
+    g = ops.backward(q, k, v, o, den, go, qk_scale=sc, qk_argmax=arg, **kw)
+    for _ in range(2):
+        o2, den2, sc2, arg2 = ops.forward(q, k, v, **kw)
+        g2 = ops.backward(q, k, v, o2, den2, go, qk_scale=sc2, qk_argmax=arg2, **kw)
+        assert torch.equal(o, o2) and torch.equal(den, den2)
+        for a, b in zip(g, g2):
+            assert torch.equal(a, b)
