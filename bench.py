@@ -167,6 +167,11 @@ def executed_mfma_flops(cfg: dict, bh: int, chunk: int = 0) -> dict:
     return out
 
 
+def dense_linear_mode(cfg: dict) -> bool:
+    """Whether the dense kernels run a p = 1 workload in their linear mode (fm_api.hip::make_plan)."""
+    return cfg["p"] == 1 and cfg["N"] > (1024 if cfg["mask"] else 512)
+
+
 def executed_dense_flops(cfg: dict, bh: int) -> dict:
     """Flops of the matrix instructions the dense score-tile kernels issue (fm_dense.h): per pair of a
     32-row own tile and a 32-row streamed tile one score contraction over the padded head dimension and one
@@ -188,6 +193,17 @@ def executed_dense_flops(cfg: dict, bh: int) -> dict:
         return tot
     rt_fwd = rt_dq = 1   # own tiles per wave in the forward and dq kernels (the dk / dv kernel: 1)
     p2 = cfg["p"] == 2
+    if dense_linear_mode(cfg):
+        # p = 1 past 1024 causal / 512 unmasked positions: every own tile starts from a state (one contraction of
+        # 32 x dp x dp; the dk / dv kernel two) and walks the streamed tiles of its own 256-position chunk up to
+        # itself only (unmasked: none); one state kernel builds the key-side states of the forward pass, two the
+        # key- and query-side states of the backward pass (dp x dp per position each)
+        tiles_per_chunk = 256 // 32
+        walked = sum(min(j % tiles_per_chunk + 1, nt) for j in range(nt)) if masked else 0
+        state = 2 * 32 * dp * dp
+        build = 2 * n * dp * dp
+        return {"fwd_apply": bh * (walked * 2 * per + nt * state), "bwd_dq": bh * (walked * 2 * per + nt * state),
+                "bwd_dk": bh * (walked * 4 * per + nt * 2 * state), "build": 3 * bh * build, "bwd_dv": 0}
     return {"fwd_apply": bh * pairs(rt_fwd) * 2 * per, "bwd_dq": bh * pairs(rt_dq) * (3 if p2 else 2) * per,
             "bwd_dk": bh * pairs(1) * 4 * per, "build_fwd": 0, "build_bwd": 0, "bwd_dv": 0}
 
@@ -390,7 +406,11 @@ def measure(name: str, args, full: bool) -> dict:
     # kernels: every score tile they walk).  Both count the state builds the timed step runs: the forward
     # prefix build and the backward suffix build, plus the backward prefix build when the states are rebuilt.
     n_builds = 3 if recompute else 2
-    if dense:
+    if dense and dense_linear_mode(cfg):
+        # (three state builds: key-side forward, key- and query-side backward; dk and dv are one kernel class)
+        algo = {"build": 3 * fl["build"] * token_heads, "fwd_apply": fl["fwd_apply"] * token_heads,
+                "bwd_dq": fl["bwd_dq"] * token_heads, "bwd_dk": (fl["bwd_dk"] + fl["bwd_dv"]) * token_heads}
+    elif dense:
         # (the fused dk / dv kernel is timed as one class: both gradients' reference-form work is its)
         algo = {"fwd_apply": fl["fwd"] * token_heads, "bwd_dq": (fl["bwd_dq"] + fl["build"]) * token_heads,
                 "bwd_dk": (fl["bwd_dk"] + fl["bwd_dv"] + fl["build"]) * token_heads}
@@ -401,8 +421,8 @@ def measure(name: str, args, full: bool) -> dict:
     executed = None
     if dense:
         ex = executed_dense_flops(cfg, bh)
-        executed = {kk: ex[kk] for kk in ("fwd_apply", "bwd_dq", "bwd_dk")}
-        ex_fwd = ex["fwd_apply"]
+        executed = {kk: ex[kk] for kk in ("build", "fwd_apply", "bwd_dq", "bwd_dk") if kk in ex}
+        ex_fwd = ex["fwd_apply"] + ex.get("build", 0) / 3
     elif cfg["p"] == 2:
         ex = executed_mfma_flops(cfg, bh)
         executed = {"build": ex["build_fwd"] * (n_builds - 1) + ex["build_bwd"],
@@ -462,6 +482,20 @@ def measure(name: str, args, full: bool) -> dict:
         roofline = {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": gbs / PEAK_HBM_GBS, "traffic": None, "bytes_per_launch": bytes_per_launch,
                     "avg_launch_ms": dom_ms / launches}
+    if dense and dense_linear_mode(cfg):
+        # p = 1 on the dense kernels' linear mode is HBM-bound as well: the slowest kernel against the tensors it
+        # must move -- forward q, k, v -> o; dq grad, k, v, q -> dq (q for the normalisation sum); the fused
+        # dk / dv kernel k, v, q, grad -> dk, dv; a state kernel two tensors (three launches a step).  The
+        # chunk states (d x d floats per 256 positions and head) come on top and are not counted.
+        es = 4 if cfg["dtype"] == "f32" else 2
+        dom = max(algo, key=lambda kn: kernels.get(kn, {}).get("ms_per_step", 0.0))
+        dom_ms = kernels[dom]["ms_per_step"]
+        tensors = {"fwd_apply": 4, "bwd_dq": 5, "bwd_dk": 6, "build": 6}[dom]
+        bytes_per_step = float(tensors) * D * es * token_heads
+        gbs = bytes_per_step / (dom_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": gbs / PEAK_HBM_GBS, "traffic": None, "bytes_per_step_of_this_kernel_class": bytes_per_step,
+                    "ms_per_step_of_this_kernel_class": dom_ms}
     per_th = measured_traffic_bytes_per_token_head(name if not (full and args.batch) else "").get(dom)
     if per_th is not None and not dense:
         n_states = n_builds if dom == "build" else 1
@@ -490,7 +524,8 @@ def measure(name: str, args, full: bool) -> dict:
             parity[pname] = O.error_metrics(got[sl].float().cpu(), want)
         del outs, ref
 
-    path = ("dense score tiles (no states)" if dense else
+    path = ("dense score tiles from chunk states (p = 1 linear mode; states rebuilt)" if dense and dense_linear_mode(cfg) else
+            "dense score tiles (no states)" if dense else
             "keeps every state in registers (one scan per head)" if "build" not in kernels
             else "rebuilds the prefix states" if recompute else "reads the prefix states the forward pass kept")
     workload = (f"{name}: Fastmax {'causal' if cfg['mask'] else 'unmasked'} fwd+bwd, "

@@ -90,7 +90,9 @@ std::vector<torch::Tensor> forward_ex(torch::Tensor q, torch::Tensor k, torch::T
     const size_t sb = fastmax_saved_state_bytes(&ds);
     TORCH_CHECK(sb > 0, "fastmax: ", fastmax_last_error());
     saved = torch::empty({(int64_t)sb}, q.options().dtype(torch::kUInt8));
-    wsb = (size_t)16 * ds.bh + 512;  // the per-head scalars only: the states go to `saved`
+    // the per-head scalars only: the states go to `saved` -- unless the kernels keep nothing (the 256-byte token)
+    // and work as in a plain forward pass
+    wsb = sb > 256 ? (size_t)16 * ds.bh + 512 : fastmax_workspace_bytes(&ds, FASTMAX_PASS_FORWARD);
     ws = torch::empty({(int64_t)wsb}, q.options().dtype(torch::kUInt8));
   } else {
     saved = torch::empty({0}, q.options().dtype(torch::kUInt8));
@@ -212,7 +214,7 @@ std::vector<torch::Tensor> forward_strided(torch::Tensor q, torch::Tensor k, tor
     const size_t sb = fastmax_saved_state_bytes_strided(&ds, &lay);
     TORCH_CHECK(sb > 0, "fastmax: ", fastmax_last_error());
     saved = torch::empty({(int64_t)sb}, q.options().dtype(torch::kUInt8));
-    wsb = (size_t)16 * ds.bh + 512;
+    wsb = sb > 256 ? (size_t)16 * ds.bh + 512 : fastmax_workspace_bytes_strided(&ds, &lay, FASTMAX_PASS_FORWARD);   // (as in forward_ex)
   } else {
     saved = torch::empty({0}, q.options().dtype(torch::kUInt8));
     wsb = fastmax_workspace_bytes_strided(&ds, &lay, FASTMAX_PASS_FORWARD);

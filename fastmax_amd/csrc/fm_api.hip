@@ -147,7 +147,7 @@ bool use_linear_scan(const fastmax_desc* ds, const Plan& pl);
 // forward + backward, 96 and 768 heads; with few heads the sequential state build of the moment form
 // fills the chip badly and the dense kernels stay ahead for longer).  A causal sequence of a single chunk
 // has no states to build either way and stays with the moment kernels' own intra-chunk tiles.  Head
-// dimensions without moment kernels always take the dense ones.
+// dimensions without moment kernels always take the dense ones (p = 1 at d = 32 / 64: see below).
 bool use_dense(const fastmax_desc* ds) {
   if (ds->d != 32 && ds->d != 64) return true;
   // FASTMAX_PATH = moments | dense overrides the choice where both kernel families exist
@@ -155,8 +155,18 @@ bool use_dense(const fastmax_desc* ds) {
     if (!strcmp(e, "moments")) return false;
     if (!strcmp(e, "dense")) return true;
   }
-  if (ds->p != 2) return false;
   const bool bf = ds->dtype == FASTMAX_BF16;
+  if (ds->p != 2) {
+    // p = 1: the moment states are tiny and the moment kernels win -- except for bf16 inputs under the mask
+    // past 1024 keys, where the dense kernels' linear mode (chunk states plus the own chunk's tiles, all of it
+    // parallel over heads and chunks) beats the chunked moment kernels at every head count measured (16 .. 768
+    // heads: 1.0 - 1.4x), and the one-scan-per-head kernels too unless their waves fill the chip's 1024 SIMDs
+    // to about three quarters (a scan costs 0.92 us per position and round of 1024 heads, the linear mode
+    // 1.23 us per 1000 positions and head)
+    if (!(bf && ds->mask && ds->nk > 1024)) return false;
+    const bool scan = ds->d == 64 && ds->bh == ds->bhkv && ds->nq == ds->nk && ds->a1 != 0.f && ds->bh >= FM_LINEAR_MIN_HEADS;
+    return !scan || ds->bh < 750 * ((ds->bh + 1023) / 1024);
+  }
   int limit;
   if (ds->d == 64) {
     if (ds->mask) limit = bf ? (ds->bh <= 128 ? 4096 : 3072) : 2560;

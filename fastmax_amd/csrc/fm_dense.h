@@ -258,7 +258,7 @@ template <int DP, class T>
 struct Shape {
   static constexpr bool BF = std::is_same<T, bf16_t>::value;
   static constexpr int BN = BF ? 64 : 32;           // streamed rows per stage
-  static constexpr int BN_KV = (BF && DP == 64) ? 128 : BN;   // (the dk / dv kernel's eight-wave blocks: fewer barriers)
+  static constexpr int BN_KV = BN;                  // (the dk / dv kernel's; 128 at bf16 d = 64 measured 5 % slower)
   // Own 32-row tiles per wave.  Matrix instructions and everything else a SIMD issues (VALU, LDS reads)
   // take turns rather than overlap on this chip, and with one own tile every matrix instruction needs a
   // 16-byte LDS operand read of its own -- the CU's whole LDS bandwidth; two own tiles share each

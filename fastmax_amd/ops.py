@@ -75,7 +75,10 @@ def forward(q, k, v, *, mask=False, normalize=False, lim=1.0, temperature=1.0, a
         saved = None
         if save_states:
             saved = torch.empty(lib.fastmax_saved_state_bytes(C.byref(ds)), dtype=torch.uint8, device=q.device)
-            nbytes = workspace_bytes or (64 * bh + 4096)  # only the per-head scalars live in the workspace
+            # states that are kept go to `saved` and only the per-head scalars live in the workspace; kernels that
+            # keep nothing (the 256-byte token) work as in a plain forward pass
+            nbytes = workspace_bytes or (64 * bh + 4096 if saved.numel() > 256 else
+                                         lib.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD))
         else:
             nbytes = workspace_bytes or lib.fastmax_workspace_bytes(C.byref(ds), _cabi.PASS_FORWARD)
         ws = _workspace(q.device, nbytes, 0)
@@ -259,7 +262,8 @@ def forward_strided(q, k, v, *, mask=False, normalize=False, lim=1.0, temperatur
         if save_states:
             saved = torch.empty(lib.fastmax_saved_state_bytes_strided(C.byref(ds), C.byref(lay)), dtype=torch.uint8,
                                 device=q.device)
-            nbytes = 64 * bh + 4096
+            nbytes = (64 * bh + 4096 if saved.numel() > 256 else   # (as in forward)
+                      lib.fastmax_workspace_bytes_strided(C.byref(ds), C.byref(lay), _cabi.PASS_FORWARD))
         else:
             nbytes = lib.fastmax_workspace_bytes_strided(C.byref(ds), C.byref(lay), _cabi.PASS_FORWARD)
         ws = _workspace(q.device, nbytes, 0)

@@ -182,10 +182,13 @@ int fastmax_backward_strided(const fastmax_desc* desc, const fastmax_layout* lay
  * need not hold the prefix states: 16*bh + 512 bytes suffice for fastmax_forward_saving, and
  * fastmax_backward_saved needs one state per head less.  (The size query is the contract: for
  * causal p = 1 with few heads and bf16 tensors the buffer also holds, behind the states, the
- * fp32 per-chunk partial states the forward pass adds up.)  (Causal p = 1 at d = 64 with at
- * least 512 heads runs as one register-resident scan per head that keeps no state in memory:
- * there the size is a token 256 bytes, the buffer is left untouched and the workspace only
- * holds per-head and per-token scalars.) */
+ * fp32 per-chunk partial states the forward pass adds up.)  Kernels that keep nothing answer the
+ * size query with a token 256 bytes: the buffer is then left untouched and the two calls need the
+ * workspace of fastmax_forward / fastmax_backward.  Those are the one register-resident scan per
+ * head of causal p = 1 at d = 64 with at least 512 heads (workspace: per-head and per-token scalars
+ * only) and the dense score tiles (fastmax_uses_dense_tiles; their workspace holds scalars -- and for
+ * p = 1 past 1024 causal / 512 unmasked positions the chunk states of their linear mode, which both
+ * passes rebuild). */
 size_t fastmax_saved_state_bytes(const fastmax_desc* desc);
 int fastmax_forward_saving(const fastmax_desc* desc, const void* q, const void* k, const void* v,
                            void* o, int64_t ldo, float* den, int64_t den_stride,

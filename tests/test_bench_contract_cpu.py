@@ -74,7 +74,16 @@ def test_executed_flops_of_the_dense_kernels():
     e48 = bench.executed_dense_flops(dict(cfg, D=48, N=100, mask=True), 1)
     assert e48["bwd_dk"] == 10 * 4 * per
     # p = 1 needs no score tile in dq
-    assert bench.executed_dense_flops(dict(cfg, p=1), 3)["bwd_dq"] == 3 * 64 * 64 * 2 * per
+    assert bench.executed_dense_flops(dict(cfg, p=1, N=512), 3)["bwd_dq"] == 3 * 16 * 16 * 2 * per
+    # p = 1 past 1024 causal / 512 unmasked positions: chunk states.  Every own tile starts from a state (one
+    # 32 x d x d contraction; dk / dv two) and walks the tiles of its own 256-position chunk up to itself (1 .. 8
+    # of them; unmasked none); three state builds of d x d per position
+    lin = bench.executed_dense_flops(dict(cfg, p=1, mask=True), 3)
+    state, walked = 2 * 32 * 64 * 64, 8 * (1 + 2 + 3 + 4 + 5 + 6 + 7 + 8)
+    assert lin["fwd_apply"] == lin["bwd_dq"] == 3 * (walked * 2 * per + 64 * state)
+    assert lin["bwd_dk"] == 3 * (walked * 4 * per + 64 * 2 * state)
+    assert lin["build"] == 3 * 3 * 2 * 2048 * 64 * 64
+    assert bench.executed_dense_flops(dict(cfg, p=1), 3)["fwd_apply"] == 3 * 64 * state
 
 
 def test_traffic_figures_are_read_from_the_committed_profiles():

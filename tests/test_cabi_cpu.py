@@ -83,6 +83,26 @@ def test_head_dimensions_and_the_dense_plan(built, monkeypatch):
     assert built.fastmax_workspace_bytes(C.byref(long_), _cabi.PASS_FORWARD) == 1536
 
 
+def test_kernel_choice_for_p1(built, monkeypatch):
+    """p = 1 at d = 32 / 64 stays with the moment kernels except for bf16 inputs under the mask past 1024 keys:
+    there the dense kernels' linear mode runs, unless the one-scan-per-head kernels (d = 64, ungrouped heads,
+    >= 512 of them) have heads enough to fill about three quarters of a round of 1024 waves."""
+    monkeypatch.delenv("FASTMAX_PATH")
+    uses = lambda **kw: built.fastmax_uses_dense_tiles(C.byref(desc(p=1, **kw)))
+    assert uses(bh=96, n=2048, dtype=1, mask=True) == 1
+    assert uses(bh=512, n=16384, dtype=1, mask=True) == 1
+    assert uses(bh=749, n=4096, dtype=1, mask=True) == 1
+    assert uses(bh=750, n=4096, dtype=1, mask=True) == 0
+    assert uses(bh=1024, n=10000, dtype=1, mask=True) == 0
+    assert uses(bh=1100, n=4096, dtype=1, mask=True) == 1      # (a second round of scans for 76 heads)
+    assert uses(bh=1024, bhkv=256, n=4096, dtype=1, mask=True) == 1   # (grouped heads: no scan kernels)
+    assert uses(bh=1024, n=4096, d=32, dtype=1, mask=True) == 1       # (d = 32: no scan kernels)
+    assert uses(bh=96, n=1024, dtype=1, mask=True) == 0
+    assert uses(bh=96, n=2048, dtype=1, mask=False) == 0
+    assert uses(bh=96, n=2048, dtype=0, mask=True) == 0
+    assert uses(bh=96, n=2048, d=48, dtype=0, mask=True) == 1
+
+
 def test_grouped_heads_descriptor(built):
     """bhkv must divide bh (fastmax_cuda_forward.cu:38 maps head i to key/value head i / (bh/bhkv)); the
     smallest workspace then holds one whole group."""
