@@ -360,3 +360,28 @@ def test_linear_mode_is_deterministic(ops):
         assert torch.equal(o, o2) and torch.equal(den, den2)
         for a, b in zip(g, g2):
             assert torch.equal(a, b)
+
+
+def test_linear_mode_is_what_bf16_causal_p1_runs_on_by_default(ops, monkeypatch):
+    """Left to itself the library takes the dense kernels' linear mode for bf16 causal p = 1 past 1024 keys at
+    d = 32 / 64 (few heads: no scan kernels); the saving forward then keeps nothing and backward rebuilds."""
+    import ctypes as C
+    from fastmax_amd import _cabi
+
+    monkeypatch.delenv("FASTMAX_PATH")
+    for d, bh, bhkv in ((64, 6, 6), (32, 6, 2)):
+        q, _, _, go = O.seeded_inputs((bh, 1500, d), seed=97, dtype=torch.bfloat16)
+        _, k, v, _ = O.seeded_inputs((bhkv, 1500, d), seed=98, dtype=torch.bfloat16)
+        kw = dict(mask=True, normalize=True, p=1)
+        qd, kd, vd, god = (t.cuda() for t in (q, k, v, go))
+        ds = ops._desc(qd, kd, True, True, 1, 1.0, 1.0, 1.0, 1.0, 0.5)
+        assert _cabi.load().fastmax_uses_dense_tiles(C.byref(ds)) == 1
+        o, den, sc, arg, saved = ops.forward(qd, kd, vd, save_states=True, **kw)
+        assert saved.numel() == 256
+        dq, dk, dv = ops.backward(qd, kd, vd, o, den, god, qk_scale=sc, qk_argmax=arg, saved_states=saved, **kw)
+        r = bh // bhkv
+        ke, ve = k.repeat_interleave(r, dim=0), v.repeat_interleave(r, dim=0)
+        ro, rdq, rdk, rdv = O.dense_truth(q.float(), ke.float(), ve.float(), go.float(), **kw)
+        fold = lambda t: t.reshape(bhkv, r, *t.shape[1:]).sum(1)
+        for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, fold(rdk)), ("dv", dv, fold(rdv))):
+            assert_close(name, got.float(), ref, TOL[torch.bfloat16], atol=1e-6)
