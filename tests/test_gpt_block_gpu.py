@@ -65,9 +65,7 @@ def test_gpt_at_config5_widths_bf16_gradients(built, monkeypatch, p, layout, pat
     import bench_gpt
     from fastmax_amd import FASTMultiHeadAttention
 
-    if path == "moments":   # (auto takes the dense score tiles for p = 2 at this length)
-        if p == 1:
-            pytest.skip("p = 1 runs on the moment kernels either way")
+    if path == "moments":   # (auto takes the dense kernels at this length: score tiles for p = 2, their linear mode for p = 1)
         monkeypatch.setenv("FASTMAX_PATH", "moments")
     dev = torch.device("cuda:0")
     vocab, T = 1024, 2048
@@ -117,12 +115,13 @@ def test_bf16_autocast_step_runs_and_learns(built):
     assert all(v == v for v in losses) and losses[-1] < losses[0]
 
 
-@pytest.mark.parametrize("path", ["auto", "moments"])
-def test_config5_full_depth_step(built, monkeypatch, path):
+@pytest.mark.parametrize("path,p", [("auto", 2), ("moments", 2), ("auto", 1)])
+def test_config5_full_depth_step(built, monkeypatch, path, p):
     """One forward + backward of the whole configuration-5 model -- 12 layers, d_model 768, 12 heads x 64,
     MLP 3072, RoPE, vocabulary 50304, batch 8, T = 2048, bf16 autocast -- on the HIP kernels (the library's
-    own choice, which is the dense score tiles at this length, and the moment kernels): finite loss near
-    ln(vocabulary) for random weights, finite gradients in every parameter, none of them all zero."""
+    own choice, which is the dense score tiles at this length -- at p = 1, the order the reference model sets
+    (model.py:212), their linear mode -- and the moment kernels): finite loss near ln(vocabulary) for random
+    weights, finite gradients in every parameter, none of them all zero."""
     import math
 
     import bench_gpt
@@ -132,7 +131,7 @@ def test_config5_full_depth_step(built, monkeypatch, path):
     dev = torch.device("cuda:0")
     vocab, T, B = 50304, 2048, 8
     torch.manual_seed(0)
-    model = bench_gpt.MiniGPT(vocab, 768, 12, 12, 3072, T, bench_gpt.PackedAttention(), 2, "packed").to(dev)
+    model = bench_gpt.MiniGPT(vocab, 768, 12, 12, 3072, T, bench_gpt.PackedAttention(), p, "packed").to(dev)
     idx = torch.randint(0, vocab, (B, T + 1), device=dev, generator=torch.Generator(device=dev).manual_seed(4))
     x, y = idx[:, :-1].contiguous(), idx[:, 1:].contiguous()
     with torch.autocast("cuda", dtype=torch.bfloat16):
