@@ -712,8 +712,9 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
       FM_TRY(launch_status("linear_dv_kernel"));
       if (ds->normalize) {
         ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
-        norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), qs, arg, rq, 1, n, D, ds->lim);
-        norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), ks, arg + bh, rq, 1, n, D, ds->lim);
+        norm_fix_kernel<T><<<2 * bh, D, 0, stream>>>(NormFixSide<T>{mk_rows(dq, L.dq), mk_rows(q, L.q), qs, arg, rq, bh, 1, n},
+                                                     NormFixSide<T>{mk_rows(dk, L.dk), mk_rows(k, L.k), ks, arg + bh, rq, bh, 1, n},
+                                                     D, ds->lim);
         FM_TRY(launch_status("norm_fix_kernel"));
       }
       return FASTMAX_OK;
@@ -862,14 +863,16 @@ int backward_impl(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
     // one partial per row block of the dq pass; sum_j dk_hat_j . k_hat_j is the same number
     const int nrb = (nq + lin::ROWS_PER_WAVE - 1) / lin::ROWS_PER_WAVE;
     ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
-    norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, nrb, nq, D, ds->lim);
-    norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh, rpart, nrb, nk, D, ds->lim);
+    norm_fix_kernel<T><<<2 * bh, D, 0, stream>>>(
+        NormFixSide<T>{mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, bh, nrb, nq},
+        NormFixSide<T>{mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh, rpart, bh, nrb, nk}, D, ds->lim);
     FM_TRY(launch_status("norm_fix_kernel"));
   } else if (ds->normalize) {
     ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
-    norm_fix_kernel<T><<<bh, D, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, pl.nblk_q, nq, D, ds->lim);
-    norm_fix_kernel<T><<<bhkv, D, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh, rpart_k,
-                                               pl.nblk_k * ratio, nk, D, ds->lim);
+    norm_fix_kernel<T><<<bh + bhkv, D, 0, stream>>>(
+        NormFixSide<T>{mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, bh, pl.nblk_q, nq},
+        NormFixSide<T>{mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh, rpart_k, bhkv, pl.nblk_k * ratio, nk}, D,
+        ds->lim);
     FM_TRY(launch_status("norm_fix_kernel"));
   }
   return FASTMAX_OK;
@@ -884,18 +887,30 @@ int allow_lds(const void* kernel, size_t bytes) {
   return FASTMAX_OK;
 }
 
+// The states of the dense kernels' linear mode.  Key side: cscale sum k (x) v and the sums of k, of v of every chunk
+// of keys alone, then (masked) of the chunks before each / (unmasked) of all, in slot 0; the forward kernel reads rows
+// of the transposed block, dq of the natural one.  Query side (backward; qstate == nullptr: none): qs a1 sum q (x) g,
+// sum c q, sum g (g = grad_out / den) of every chunk of queries alone, then of the chunks after each / of all, in both
+// layouts.  One state launch and one scan launch serve both sides.
 template <int DP, class T>
-int dense_key_states(const Plan& pl, const Layout& L, const T* k, const T* v, int d, float a1, bool transposed,
-                     float* kstate, hipStream_t stream) {
-  // a1 sum k (x) v and the sums of k, of v of every chunk of keys alone, then (masked) of the chunks before each /
-  // (unmasked) of all, in slot 0; the forward kernel reads rows of the transposed block, dq of the natural one
-  const int64_t sf = dense::LinState<DP>::floats(1);
+int dense_lin_states(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v,
+                     const T* go, const float* den, int64_t den_stride, const float* cvec, const float* scale,
+                     bool transposed, float* kstate, float* qstate, hipStream_t stream) {
+  const int npos = pl.masked ? pl.nk : pl.nq;
+  const RowScalars none{nullptr, 0, 0};
+  dense::StateSide<T> ks{mk_rows(k, L.k), mk_rows(v, L.v), none, none, nullptr, ds->a1, kstate, 1,
+                         transposed ? -1 : 0, transposed ? 0 : -1, pl.nk, pl.bhkv};
+  dense::StateSide<T> qs = ks;
+  qs.heads = 0;
+  const int64_t sfk = dense::LinState<DP>::floats(1), sfq = dense::LinState<DP>::floats(2);
+  if (qstate)
+    qs = dense::StateSide<T>{mk_rows(q, L.q, 0, pl.off), mk_rows(go, L.go, 0, pl.off), mk_scalars(den, pl.nq, den_stride, 0, pl.off),
+                             mk_scalars<const float>(cvec, pl.nq, 1, 0, pl.off), scale, ds->a1, qstate, 2, 0, 1, npos, pl.bh};
   ScopedKernel sk(FASTMAX_K_BUILD, stream);
-  dense::dense_state_kernel<DP, T, false><<<dim3(pl.bhkv, pl.lslots), 256, 0, stream>>>(
-      mk_rows(k, L.k), mk_rows(v, L.v), RowScalars{nullptr, 0, 0}, RowScalars{nullptr, 0, 0}, nullptr, a1, kstate, 1,
-      transposed ? -1 : 0, transposed ? 0 : -1, pl.nk, d, pl.lchunk);
-  dense::lin_scan_kernel<<<dim3((unsigned)((sf / 4 + 255) / 256), pl.bhkv), 256, 0, stream>>>(kstate, pl.lslots, sf,
-                                                                                           pl.masked ? 0 : 2);
+  dense::dense_state_kernel<DP, T><<<dim3(ks.heads + qs.heads, pl.lslots), 256, 0, stream>>>(ks, qs, ds->d, pl.lchunk);
+  const int64_t sfmax = qstate ? sfq : sfk;
+  dense::lin_scan_kernel<<<dim3((unsigned)((sfmax / 4 + 255) / 256), ks.heads + qs.heads), 256, 0, stream>>>(
+      kstate, sfk, ks.heads, pl.masked ? 0 : 2, qstate, sfq, pl.masked ? 1 : 2, pl.lslots);
   return launch_status("dense_state_kernel");
 }
 
@@ -910,7 +925,8 @@ int dense_forward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, co
   FM_TRY(allow_lds(reinterpret_cast<const void*>(kern), smem));
   const int npos = pl.masked ? pl.nk : pl.nq;
   const int nb = (npos + BM - 1) / BM - pl.off / BM;
-  if (pl.lin) FM_TRY((dense_key_states<DP, T>(pl, L, k, v, ds->d, ds->a1, true, kstate, stream)));
+  if (pl.lin)
+    FM_TRY((dense_lin_states<DP, T>(ds, pl, L, q, k, v, nullptr, nullptr, 0, nullptr, scale, true, kstate, nullptr, stream)));
   ScopedKernel sk(FASTMAX_K_FWD_APPLY, stream);
   kern<<<dim3(pl.bh, nb), 64 * NW, smem, stream>>>(mk_rows(q, L.q, 0, pl.off), mk_rows(k, L.k), mk_rows(v, L.v), scale,
                                                scale + pl.bh, mk_rows(o, L.o, 0, pl.off),
@@ -949,18 +965,8 @@ int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, c
   const RowScalars cv = mk_scalars<const float>(cvec, pl.nq, 1, 0, pl.off);
   const Rows<const T> qr = mk_rows(q, L.q, 0, pl.off), gr = mk_rows(go, L.go, 0, pl.off);
   const Rows<const T> kr = mk_rows(k, L.k), vr = mk_rows(v, L.v);
-  if (pl.lin) {
-    // key-side states as in the forward pass; query-side states sum [q; 1] (x) [g, c] of every chunk alone, then
-    // (masked) of the chunks after each / (unmasked) of all, in slot 0
-    FM_TRY((dense_key_states<DP, T>(pl, L, k, v, ds->d, ds->a1, false, kstate, stream)));
-    const int64_t sf = dense::LinState<DP>::floats(2);
-    ScopedKernel sk(FASTMAX_K_BUILD, stream);
-    dense::dense_state_kernel<DP, T, true><<<dim3(pl.bh, pl.lslots), 256, 0, stream>>>(qr, gr, dn, cv, scale, ds->a1, qstate, 2, 0, 1,
-                                                                            npos, ds->d, pl.lchunk);
-    dense::lin_scan_kernel<<<dim3((unsigned)((sf / 4 + 255) / 256), pl.bh), 256, 0, stream>>>(qstate, pl.lslots, sf,
-                                                                                          pl.masked ? 1 : 2);
-    FM_TRY(launch_status("dense_state_kernel"));
-  }
+  if (pl.lin)
+    FM_TRY((dense_lin_states<DP, T>(ds, pl, L, q, k, v, go, den, den_stride, cvec, scale, false, kstate, qstate, stream)));
   const float* ksl = pl.lin ? kstate : nullptr;
   const float* qsl = pl.lin ? qstate : nullptr;
   {
@@ -1028,9 +1034,10 @@ int dense_backward(const fastmax_desc* ds, const Plan& pl, const Layout& L, cons
 #undef FM_DENSE_BWD
   if (ds->normalize) {
     ScopedKernel sk(FASTMAX_K_NORM_FIX, stream);
-    norm_fix_kernel<T><<<bh, ds->d, 0, stream>>>(mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, nbq, pl.nq, ds->d, ds->lim);
-    norm_fix_kernel<T><<<pl.bhkv, ds->d, 0, stream>>>(mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh,
-                                                      rpart + (int64_t)bh * nbq, nbk, pl.nk, ds->d, ds->lim);
+    norm_fix_kernel<T><<<bh + pl.bhkv, ds->d, 0, stream>>>(
+        NormFixSide<T>{mk_rows(dq, L.dq), mk_rows(q, L.q), scale, arg, rpart, bh, nbq, pl.nq},
+        NormFixSide<T>{mk_rows(dk, L.dk), mk_rows(k, L.k), scale + bh, arg + bh, rpart + (int64_t)bh * nbq, pl.bhkv, nbk, pl.nk},
+        ds->d, ds->lim);
     FM_TRY(launch_status("norm_fix_kernel"));
   }
   return FASTMAX_OK;

@@ -51,22 +51,33 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(Rows<const T> go, Rows<co
 // ---------------------------------------------------------------------------------------
 // Chain rule through x_hat = lim * x / max_n ||x_n||: the scaling by lim/M is already in dx;
 // the max-norm row i* additionally gets  dx[i*] -= (sum dx_hat.x_hat) * x[i*] / M^2.
-// One block per head; blockDim.x = d.  A row index outside [0, n) (only a caller-supplied
-// qk_argmax can hold one) leaves the head untouched.
+// One launch serves both sides: blocks [0, heads of side a) fix dq, the rest dk; one block per head,
+// blockDim.x = d.  A row index outside [0, n) (only a caller-supplied qk_argmax can hold one) leaves
+// the head untouched.
 // ---------------------------------------------------------------------------------------
 template <class T>
-__global__ void norm_fix_kernel(Rows<T> dx, Rows<const T> x,
-                                const float* __restrict__ scale, const int* __restrict__ arg,
-                                const float* __restrict__ rpart, int nblk, int n, int d, float lim) {
-  const int head = blockIdx.x, c = threadIdx.x;
-  const int row = arg[head];
-  if (row < 0 || row >= n) return;
+struct NormFixSide {
+  Rows<T> dx;
+  Rows<const T> x;
+  const float* scale;
+  const int* arg;
+  const float* rpart;
+  int heads, nblk, n;
+};
+
+template <class T>
+__global__ void norm_fix_kernel(NormFixSide<T> a, NormFixSide<T> b, int d, float lim) {
+  const bool first = (int)blockIdx.x < a.heads;
+  const NormFixSide<T>& sd = first ? a : b;
+  const int head = first ? blockIdx.x : blockIdx.x - a.heads, c = threadIdx.x;
+  const int row = sd.arg[head];
+  if (row < 0 || row >= sd.n) return;
   float r = 0.f;
-  for (int b = 0; b < nblk; ++b) r += rpart[(int64_t)head * nblk + b];
-  const float s = scale[head];
+  for (int bl = 0; bl < sd.nblk; ++bl) r += sd.rpart[(int64_t)head * sd.nblk + bl];
+  const float s = sd.scale[head];
   const float fac = r * s * s / (lim * lim);
-  const HeadRows<T> dh = dx.head(head);
-  const HeadRows<const T> xh = x.head(head);
+  const HeadRows<T> dh = sd.dx.head(head);
+  const HeadRows<const T> xh = sd.x.head(head);
   T* dst = dh.row(row) + c;
   *dst = from_f32<T>(to_f32(*dst) - fac * to_f32(xh.row(row)[c]));
 }

@@ -306,11 +306,16 @@ struct LinState {
 };
 
 // slots of fp32 states, in place: mode 0: slot c = sum of the slots before c; 1: of the slots after c;
-// 2: slot 0 = the sum of all.  grid = (ceil(ss / 1024), heads), one float4 per thread.
-__global__ __launch_bounds__(256) void lin_scan_kernel(float* __restrict__ state, int nslots, int64_t ss, int mode) {
+// 2: slot 0 = the sum of all.  One launch serves two arrays of states (the key side's and the query side's of a
+// backward pass; heads_b = 0: one): grid = (ceil(max slot floats / 1024), heads_a + heads_b), one float4 per thread.
+__global__ __launch_bounds__(256) void lin_scan_kernel(float* __restrict__ sa, int64_t ssa, int heads_a, int mode_a,
+                                                       float* __restrict__ sb, int64_t ssb, int mode_b, int nslots) {
+  const bool first = (int)blockIdx.y < heads_a;
+  const int64_t ss = first ? ssa : ssb;
+  const int mode = first ? mode_a : mode_b, head = first ? blockIdx.y : blockIdx.y - heads_a;
   const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (idx >= ss) return;
-  float* base = state + (int64_t)blockIdx.y * nslots * ss + idx;
+  float* base = (first ? sa : sb) + (int64_t)head * nslots * ss + idx;
   float4 run = make_float4(0.f, 0.f, 0.f, 0.f);
   for (int step = 0; step < nslots; ++step) {
     const int c = mode == 1 ? nslots - 1 - step : step;
@@ -371,14 +376,22 @@ __device__ __forceinline__ f16v lin_own_times(const typename Mma<T>::Frag (&af)[
 // given), e_t = ew_t (1 when not given) and bs = cscale hscale[head] (hscale: 1 when not given):
 //   block nat_blk [x][y] = block trn_blk [y][x] = bs sum_t X_t[x] Y_t[y]          (a block index < 0: not written)
 //   vectors: [x] = sum_t e_t X_t[x],   [DP + y] = sum_t Y_t[y],   [2 DP] = sum_t e_t
-// grid = (heads, chunks), 256 threads; the (DP / 32)^2 tiles of the x-by-y block are dealt to the four waves,
-// and the wave that has column block 0 (row block 0) of a block row (column) also sums that row block's X e
+// One launch serves two sets of tensors (the key side and the query side of a backward pass; b.heads = 0: one):
+// grid = (a.heads + b.heads, chunks), 256 threads; the (DP / 32)^2 tiles of the x-by-y block are dealt to the four
+// waves, and the wave that has column block 0 (row block 0) of a block row (column) also sums that row block's X e
 // (column block's Y) from the operand fragments it reads anyway.
-template <int DP, class T, bool HAS_E>
-__global__ __launch_bounds__(256) void dense_state_kernel(Rows<const T> X, Rows<const T> Y, RowScalars ydiv,
-                                                          RowScalars ew, const float* __restrict__ hscale, float cscale,
-                                                          float* __restrict__ state, int nblk, int nat_blk, int trn_blk,
-                                                          int npos, int d, int lchunk) {
+template <class T>
+struct StateSide {
+  Rows<const T> X, Y;
+  RowScalars ydiv, ew;
+  const float* hscale;
+  float cscale;
+  float* state;
+  int nblk, nat_blk, trn_blk, npos, heads;
+};
+
+template <int DP, class T>
+__global__ __launch_bounds__(256) void dense_state_kernel(StateSide<T> sa, StateSide<T> sb, int d, int lchunk) {
   using M = Mma<T>;
   using Elt = typename M::Elt;
   using Frag = typename M::Frag;
@@ -390,10 +403,17 @@ __global__ __launch_bounds__(256) void dense_state_kernel(Rows<const T> X, Rows<
   __shared__ __attribute__((aligned(16))) Elt Yt[DP * PT];
   __shared__ __attribute__((aligned(16))) float El[BN];
   const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, i = l & 31, hh = l >> 5;
-  const int head = blockIdx.x, c = blockIdx.y, nch = gridDim.y;
-  const HeadRows<const T> Xh = X.head(head), Yh = Y.head(head);
+  const bool first = (int)blockIdx.x < sa.heads;
+  const StateSide<T>& sd = first ? sa : sb;
+  const int head = first ? blockIdx.x : blockIdx.x - sa.heads, c = blockIdx.y, nch = gridDim.y;
+  const HeadRows<const T> Xh = sd.X.head(head), Yh = sd.Y.head(head);
+  const RowScalars ydiv = sd.ydiv, ew = sd.ew;
   const float* ydh = ydiv.head(head);
   const float* ewh = ew.head(head);
+  const int nblk = sd.nblk, nat_blk = sd.nat_blk, trn_blk = sd.trn_blk, npos = sd.npos;
+  const float* hscale = sd.hscale;
+  const float cscale = sd.cscale;
+  float* state = sd.state;
   const int lo = Xh.lo;
   const int t0 = c * lchunk, t1 = (t0 + lchunk < npos ? t0 + lchunk : npos);
 
@@ -414,7 +434,7 @@ __global__ __launch_bounds__(256) void dense_state_kernel(Rows<const T> X, Rows<
     yt.load(Yh, tb, t1, d, tid, ydh, ydiv.stride);
     // (every thread, clamped, not predicated, nothing computed from it yet: a wait here would wait for the rows too)
     const int pos = tb + tid % BN;
-    if (HAS_E) ev = ewh[(int64_t)max(pos < t1 ? pos : t1 - 1, lo) * ew.stride];
+    if (ewh) ev = ewh[(int64_t)max(pos < t1 ? pos : t1 - 1, lo) * ew.stride];
     em = (pos >= lo && pos < t1) ? 1.0f : 0.f;
   };
   if (t0 < t1) stage_load(t0);
