@@ -72,8 +72,14 @@ __global__ void norm_fix_kernel(NormFixSide<T> a, NormFixSide<T> b, int d, float
   const int head = first ? blockIdx.x : blockIdx.x - a.heads, c = threadIdx.x;
   const int row = sd.arg[head];
   if (row < 0 || row >= sd.n) return;
+  // the block's threads share the partials (fixed order per thread and in the tree: the same sum every run)
+  __shared__ float red[128];
   float r = 0.f;
-  for (int bl = 0; bl < sd.nblk; ++bl) r += sd.rpart[(int64_t)head * sd.nblk + bl];
+  for (int bl = c; bl < sd.nblk; bl += blockDim.x) r += sd.rpart[(int64_t)head * sd.nblk + bl];
+  red[c] = r;
+  __syncthreads();
+  r = 0.f;
+  for (int t = 0; t < (int)blockDim.x; ++t) r += red[t];
   const float s = sd.scale[head];
   const float fac = r * s * s / (lim * lim);
   const HeadRows<T> dh = sd.dx.head(head);

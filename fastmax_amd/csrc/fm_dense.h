@@ -317,12 +317,24 @@ __global__ __launch_bounds__(256) void lin_scan_kernel(float* __restrict__ sa, i
   if (idx >= ss) return;
   float* base = (first ? sa : sb) + (int64_t)head * nslots * ss + idx;
   float4 run = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int step = 0; step < nslots; ++step) {
-    const int c = mode == 1 ? nslots - 1 - step : step;
-    float4* p = reinterpret_cast<float4*>(base + c * ss);
-    const float4 t = *p;
-    if (mode != 2) *p = run;
-    run.x += t.x; run.y += t.y; run.z += t.z; run.w += t.w;
+  // eight slots at a time: their loads are all requested before the first store (a load that had to stay behind
+  // a store that may alias it would make the walk one memory round trip per slot)
+  for (int s0 = 0; s0 < nslots; s0 += 8) {
+    float4 t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int step = s0 + u < nslots ? s0 + u : nslots - 1;
+      const int c = mode == 1 ? nslots - 1 - step : step;
+      t[u] = *reinterpret_cast<const float4*>(base + c * ss);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (s0 + u < nslots) {
+        const int c = mode == 1 ? nslots - 1 - (s0 + u) : s0 + u;
+        if (mode != 2) *reinterpret_cast<float4*>(base + c * ss) = run;
+        run.x += t[u].x; run.y += t[u].y; run.z += t[u].z; run.w += t[u].w;
+      }
+    }
   }
   if (mode == 2) *reinterpret_cast<float4*>(base) = run;
 }

@@ -19,16 +19,15 @@ struct RowPiece;
 template <>
 struct RowPiece<float> {
   static constexpr int N = 4;
-  __device__ __forceinline__ static float sumsq(const float* p) {
-    const float4 t = *reinterpret_cast<const float4*>(p);
-    return t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w;
+  __device__ __forceinline__ static float sumsq(const uint4& r) {
+    const float x = __uint_as_float(r.x), y = __uint_as_float(r.y), z = __uint_as_float(r.z), w = __uint_as_float(r.w);
+    return x * x + y * y + z * z + w * w;
   }
 };
 template <>
 struct RowPiece<bf16_t> {
   static constexpr int N = 8;
-  __device__ __forceinline__ static float sumsq(const bf16_t* p) {
-    const uint4 t = *reinterpret_cast<const uint4*>(p);
+  __device__ __forceinline__ static float sumsq(const uint4& t) {
     const float a0 = bf_lo(t.x), a1 = bf_hi(t.x), a2 = bf_lo(t.y), a3 = bf_hi(t.y);
     const float a4 = bf_lo(t.z), a5 = bf_hi(t.z), a6 = bf_lo(t.w), a7 = bf_hi(t.w);
     return (a0 * a0 + a1 * a1 + a2 * a2 + a3 * a3) + (a4 * a4 + a5 * a5 + a6 * a6 + a7 * a7);
@@ -68,20 +67,29 @@ __global__ __launch_bounds__(NT) void rowstat_kernel(Rows<const T> x1, int n1, i
   };
   float best = -1.f;
   int bi = 0;
-  // four row groups per trip, loaded before any of them is reduced (rows past the end are
-  // clamped to the last row: a duplicate cannot change the maximum or its first index)
-  for (int i0 = 0; i0 < n; i0 += 4 * rpp) {
-    float ssq[4];
-    int idx[4];
+  // U row groups per trip, loaded before any of them is reduced (rows past the end are clamped to the
+  // last row: a duplicate cannot change the maximum or its first index).  With few heads a block walks
+  // its head alone and only what it has in flight hides the memory latency: 16 loads per thread there.
+  constexpr int U = NT >= 1024 ? 16 : 8;
+  for (int i0 = 0; i0 < n; i0 += U * rpp) {
+    uint4 raw[U];
+    int idx[U];
+    // (unconditional loads of clamped addresses, nothing computed from them yet: a load under a condition, or
+    // one whose value is used at once, gets a wait of its own and the trip becomes one memory round trip per group)
+    const unsigned piece = (unsigned)((sub < npc ? sub : npc - 1) * EPT);
+    const unsigned keep = sub < npc ? 0xffffffffu : 0u;   // (the lanes past the row's end: their piece, a duplicate, becomes zeros)
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int i = i0 + u * rpp + rowi;
       idx[u] = i < n ? i : n - 1;
-      ssq[u] = sub < npc ? RowPiece<T>::sumsq(base + ((unsigned)idx[u] * pitch + (unsigned)(sub * EPT))) : 0.f;
+      raw[u] = *reinterpret_cast<const uint4*>(base + ((unsigned)idx[u] * pitch + piece));
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      float ss = ssq[u];
+    for (int u = 0; u < U; ++u) {
+      if (tpr != npc) {   // (block-uniform: only head dimensions whose pieces are not a power of two have such lanes)
+        raw[u].x &= keep; raw[u].y &= keep; raw[u].z &= keep; raw[u].w &= keep;
+      }
+      float ss = RowPiece<T>::sumsq(raw[u]);
       for (int off = tpr >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
       if (better(ss, idx[u], best, bi)) {
         best = ss;
