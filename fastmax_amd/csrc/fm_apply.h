@@ -133,10 +133,20 @@ __global__ __launch_bounds__(256, 2) void apply_kernel(
   if (n_tile > 0) tiles_load(0);
   if (n_state > 0) slab_dma(0, Sl0);
   // the order-0 row of the state: value columns i and 32 + i, and the extra column
+  // (requested together and whatever n_state says -- a slot that is not used is still memory of the state
+  // array -- and masked afterwards: a load under a condition gets a wait of its own, for it and for every
+  // transfer requested before it, one memory round trip per value)
   float z0[CB], zd = 0.f;
+  {
+    float zraw[CB + 1];
 #pragma unroll
-  for (int cb = 0; cb < CB; ++cb) z0[cb] = n_state > 0 ? a0 * sbase[(rows2 + D) * LD + cb * 32 + i] : 0.f;
-  if (FWD && n_state > 0 && hh == 0) zd = a0 * sbase[(rows2 + D) * LD + D];
+    for (int cb = 0; cb < CB; ++cb) zraw[cb] = sbase[(rows2 + D) * LD + cb * 32 + i];
+    zraw[CB] = sbase[(rows2 + D) * LD + D];
+    const unsigned keep = n_state > 0 ? 0xffffffffu : 0u;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) z0[cb] = a0 * __uint_as_float(__float_as_uint(zraw[cb]) & keep);
+    if (FWD) zd = a0 * __uint_as_float(__float_as_uint(zraw[CB]) & (hh == 0 ? keep : 0u));
+  }
   xt.store(Xl, LD, xs, tid);
   if (n_state == 0 && n_tile > 0) tiles_store(0);
   FM_WAIT_VM(0);
@@ -529,9 +539,17 @@ __global__ __launch_bounds__(256, 2) void apply_kernel_bf(
   // the order-2 slabs carry their pair weights; a2 is applied to their sum, a1 to the order-1
   // features and a0 to the order-0 row
   float zc[CB], zd = 0.f;
+  {   // (requested together and whatever n_state says, masked afterwards: a load under a condition gets a wait
+      // of its own -- for it and for every transfer requested before it)
+    float zraw[CB + 1];
 #pragma unroll
-  for (int cb = 0; cb < CB; ++cb) zc[cb] = n_state > 0 ? a0 * zsec[cb * 32 + i] : 0.f;
-  if (FWD && n_state > 0) zd = a0 * zsec[D];
+    for (int cb = 0; cb < CB; ++cb) zraw[cb] = zsec[cb * 32 + i];
+    zraw[CB] = zsec[D];
+    const unsigned keep = n_state > 0 ? 0xffffffffu : 0u;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) zc[cb] = a0 * __uint_as_float(__float_as_uint(zraw[cb]) & keep);
+    if (FWD) zd = a0 * __uint_as_float(__float_as_uint(zraw[CB]) & keep);
+  }
 
   // One pipeline step = two slabs and one barrier: start the transfers of slabs st+2, st+3 into the
   // buffers the previous step read from (every wave is past them: it has passed the barrier),
