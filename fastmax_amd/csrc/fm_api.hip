@@ -135,11 +135,20 @@ int64_t lin_state_floats(int dp, int nblk) {
 }
 
 // Causal p = 1 at d = 64 runs as one sequential scan per head (fm_linear.h: one wave per head, the
-// state never leaves its registers) once there are enough heads to fill the chip's 1024 SIMDs
-// about half way; below that the chunked kernels, which split a head over many blocks, win.
+// state never leaves its registers) once there are enough heads: with fp32 tensors (fp32 matrix
+// instruction, matrix-bound) from about half of the chip's 1024 SIMDs filled, below which the chunked
+// kernels, which split a head over many blocks, win; with bf16 tensors (bf16 matrix instruction: a
+// scan then costs 0.24 us per position up to 256 heads and is memory-bound beyond) from 208 heads, below
+// which the dense kernels' linear mode wins (1.2 ns per position and head).
 #ifndef FM_LINEAR_MIN_HEADS
 #define FM_LINEAR_MIN_HEADS 512
 #endif
+#ifndef FM_LINEAR_MIN_HEADS_BF16
+#define FM_LINEAR_MIN_HEADS_BF16 208
+#endif
+int linear_min_heads(const fastmax_desc* ds) {
+  return ds->dtype == FASTMAX_BF16 ? FM_LINEAR_MIN_HEADS_BF16 : FM_LINEAR_MIN_HEADS;
+}
 bool use_linear_scan(const fastmax_desc* ds, const Plan& pl);
 
 // Dense score tiles cost 2 n d flop per token under the mask (4 n d without it), the moment form about
@@ -158,14 +167,13 @@ bool use_dense(const fastmax_desc* ds) {
   const bool bf = ds->dtype == FASTMAX_BF16;
   if (ds->p != 2) {
     // p = 1: the moment states are tiny and the moment kernels win -- except for bf16 inputs under the mask
-    // past 1024 keys, where the dense kernels' linear mode (chunk states plus the own chunk's tiles, all of it
-    // parallel over heads and chunks) beats the chunked moment kernels at every head count measured (16 .. 768
-    // heads: 1.0 - 1.4x), and the one-scan-per-head kernels too unless their waves fill the chip's 1024 SIMDs
-    // to about three quarters (a scan costs 0.92 us per position and round of 1024 heads, the linear mode
-    // 1.23 us per 1000 positions and head)
+    // past 1024 keys with too few heads for the one-scan-per-head kernels (linear_min_heads; or no such kernels:
+    // d = 32, grouped heads, a key prefix, a1 = 0): there the dense kernels' linear mode (chunk states plus the
+    // own chunk's tiles, all of it parallel over heads and chunks) beats the chunked moment kernels at every
+    // head count measured (16 .. 768 heads: 1.0 - 1.4x)
     if (!(bf && ds->mask && ds->nk > 1024)) return false;
-    const bool scan = ds->d == 64 && ds->bh == ds->bhkv && ds->nq == ds->nk && ds->a1 != 0.f && ds->bh >= FM_LINEAR_MIN_HEADS;
-    return !scan || ds->bh < 750 * ((ds->bh + 1023) / 1024);
+    const bool scan = ds->d == 64 && ds->bh == ds->bhkv && ds->nq == ds->nk && ds->a1 != 0.f && ds->bh >= linear_min_heads(ds);
+    return !scan;
   }
   int limit;
   if (ds->d == 64) {
@@ -282,7 +290,7 @@ Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true, bool allow_d
 bool use_linear_scan(const fastmax_desc* ds, const Plan& pl) {
   // (its kernels keep the weights divided by a1, and every tile is a full 32 rows)
   return !pl.p2 && pl.masked && pl.d == 64 && pl.ratio == 1 && pl.n >= 32 && ds->a1 != 0.f &&
-         pl.bh >= FM_LINEAR_MIN_HEADS && pl.plain && pl.nq == pl.nk;
+         pl.bh >= linear_min_heads(ds) && pl.plain && pl.nq == pl.nk;
 }
 
 // Heads per launch that fit the workspace.  When several batches are needed the batch is

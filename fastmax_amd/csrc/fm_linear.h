@@ -10,7 +10,8 @@
 //   weights, which sit in accumulator registers and are fed back as the A operand)
 //   + 64 (own rows x running state, the state's accumulator registers being the B operand)
 //   + 64 (state update).
-// bf16 inputs take the same path (fp32 matrix instruction, half the memory traffic).
+// bf16 inputs take the same path with eight of those instructions at a time as one
+// v_mfma_f32_32x32x16_bf16 (24 per tile; kPackedMma below) and half the memory traffic.
 //
 // Operand layouts (lane l: i = l % 32, hh = l / 32; trow(t, hh) = row of accumulator register t):
 //   channel-major X^ch[c][t] = X[tile row trow(t, hh)][chan(c, i)], c = 0, 1: the lane's two channels
@@ -225,40 +226,122 @@ __device__ __forceinline__ float vec_dot(const float* lds64, const Lane<T>& L, c
 // own rows x running state, O[own row][chan(cc, n)] = sum_ch own[ch] State[ch][chan(cc, n)] (the
 // state's accumulator registers are the B operand).  The three accumulation chains are
 // independent and issued interleaved.
+// With bf16 tensors the contractions run on v_mfma_f32_32x32x16_bf16: eight of the per-lane operand values
+// that the fp32 path feeds to eight v_mfma_f32_32x32x2f32 make one instruction (the k index of a contraction
+// may be permuted freely as long as both operands agree, so any eight pairs will do).  Operands that come
+// from the tensors are bf16 values already (the conversion back is exact); weights and the running state,
+// which live in fp32 accumulator registers, are rounded to bf16 on their way into an operand, as everywhere
+// on the bf16 paths.
+template <class T>
+constexpr bool kPackedMma = false;
+template <>
+constexpr bool kPackedMma<bf16_t> = true;
+
+__device__ __forceinline__ bf8v pk8(float a, float b, float c, float d, float e, float f, float g, float h) {
+  return __builtin_bit_cast(bf8v, fm_u4{pack_bf2(a, b), pack_bf2(c, d), pack_bf2(e, f), pack_bf2(g, h)});
+}
+__device__ __forceinline__ bf8v pk8(const float* x) { return pk8(x[0], x[1], x[2], x[3], x[4], x[5], x[6], x[7]); }
+// registers 8 F .. 8 F + 7 of an accumulator tile
+template <int F>
+__device__ __forceinline__ bf8v pk8(const f16v& a) {
+  return pk8(a[8 * F], a[8 * F + 1], a[8 * F + 2], a[8 * F + 3], a[8 * F + 4], a[8 * F + 5], a[8 * F + 6], a[8 * F + 7]);
+}
+// the own-row elements that meet registers 8 F .. 8 F + 7 of a state tile of row class rc
+template <class T, int F, int RC>
+__device__ __forceinline__ bf8v pk8_own(const float (&own)[32]) {
+  return pk8(own[Map<T>::tok_of(8 * F, RC)], own[Map<T>::tok_of(8 * F + 1, RC)], own[Map<T>::tok_of(8 * F + 2, RC)],
+             own[Map<T>::tok_of(8 * F + 3, RC)], own[Map<T>::tok_of(8 * F + 4, RC)], own[Map<T>::tok_of(8 * F + 5, RC)],
+             own[Map<T>::tok_of(8 * F + 6, RC)], own[Map<T>::tok_of(8 * F + 7, RC)]);
+}
+
+// own rows x state, O[own row][chan(cc, n)] (+)= sum_ch own[ch] State[ch][chan(cc, n)]: the state's accumulator
+// registers are the B operand
+template <class T>
+__device__ __forceinline__ void own_times_state(const float (&own)[32], const f16v (&S)[2][2], f16v (&O)[2]) {
+  if constexpr (kPackedMma<T>) {
+    const bf8v a00 = pk8_own<T, 0, 0>(own), a10 = pk8_own<T, 1, 0>(own), a01 = pk8_own<T, 0, 1>(own), a11 = pk8_own<T, 1, 1>(own);
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      O[cc] = FM_MFMA_BF16(a00, pk8<0>(S[0][cc]), O[cc]);
+      O[cc] = FM_MFMA_BF16(a10, pk8<1>(S[0][cc]), O[cc]);
+      O[cc] = FM_MFMA_BF16(a01, pk8<0>(S[1][cc]), O[cc]);
+      O[cc] = FM_MFMA_BF16(a11, pk8<1>(S[1][cc]), O[cc]);
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+#pragma unroll
+      for (int rc = 0; rc < 2; ++rc) {
+        O[0] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][0][t], O[0]);
+        O[1] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][1][t], O[1]);
+      }
+  }
+}
+
+// Score tile P (rows = rows of `a`, columns = rows of `b`, contraction over the 64 channels) and
+// own rows x running state.  The three accumulation chains are independent and issued interleaved.
 template <class T>
 __device__ __forceinline__ void score_and_state(const float (&a)[32], const float (&b)[32],
                                                 const float (&own)[32], const f16v (&S)[2][2], f16v& P,
                                                 f16v (&O)[2]) {
 #pragma unroll
   for (int t = 0; t < 16; ++t) P[t] = 0.f, O[0][t] = 0.f, O[1][t] = 0.f;
+  if constexpr (kPackedMma<T>) {
 #pragma unroll
-  for (int t = 0; t < 16; ++t)
+    for (int m = 0; m < 4; ++m) P = FM_MFMA_BF16(pk8(a + 8 * m), pk8(b + 8 * m), P);
+    own_times_state<T>(own, S, O);
+  } else {
 #pragma unroll
-    for (int rc = 0; rc < 2; ++rc) {
-      P = FM_MFMA(a[2 * t + rc], b[2 * t + rc], P);
-      O[0] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][0][t], O[0]);
-      O[1] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][1][t], O[1]);
-    }
+    for (int t = 0; t < 16; ++t)
+#pragma unroll
+      for (int rc = 0; rc < 2; ++rc) {
+        P = FM_MFMA(a[2 * t + rc], b[2 * t + rc], P);
+        O[0] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][0][t], O[0]);
+        O[1] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][1][t], O[1]);
+      }
+  }
 }
 
 // State[chan(rc, m)][chan(cc, n)] += sum over the tile's rows of ua[row][chan(rc, m)] * ub[row][chan(cc, n)]
+template <class T>
 __device__ __forceinline__ void state_update(f16v (&S)[2][2], const float (&ua)[2][16], const float (&ub)[2][16]) {
+  if constexpr (kPackedMma<T>) {
 #pragma unroll
-  for (int t = 0; t < 16; ++t) {
-    S[0][0] = FM_MFMA(ua[0][t], ub[0][t], S[0][0]);
-    S[0][1] = FM_MFMA(ua[0][t], ub[1][t], S[0][1]);
-    S[1][0] = FM_MFMA(ua[1][t], ub[0][t], S[1][0]);
-    S[1][1] = FM_MFMA(ua[1][t], ub[1][t], S[1][1]);
+    for (int f = 0; f < 2; ++f) {
+      const bf8v a0 = pk8(ua[0] + 8 * f), a1 = pk8(ua[1] + 8 * f), b0 = pk8(ub[0] + 8 * f), b1 = pk8(ub[1] + 8 * f);
+      S[0][0] = FM_MFMA_BF16(a0, b0, S[0][0]);
+      S[0][1] = FM_MFMA_BF16(a0, b1, S[0][1]);
+      S[1][0] = FM_MFMA_BF16(a1, b0, S[1][0]);
+      S[1][1] = FM_MFMA_BF16(a1, b1, S[1][1]);
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      S[0][0] = FM_MFMA(ua[0][t], ub[0][t], S[0][0]);
+      S[0][1] = FM_MFMA(ua[0][t], ub[1][t], S[0][1]);
+      S[1][0] = FM_MFMA(ua[1][t], ub[0][t], S[1][0]);
+      S[1][1] = FM_MFMA(ua[1][t], ub[1][t], S[1][1]);
+    }
   }
 }
 
 // O[own row][chan(cc, n)] += sum over streamed rows of W[streamed][own] * ub[streamed][chan(cc, n)];
 // the weights are fed from their accumulator registers as the A operand
+template <class T>
 __device__ __forceinline__ void weight_product(const f16v& W, const float (&ub)[2][16], f16v (&O)[2]) {
+  if constexpr (kPackedMma<T>) {
+    const bf8v w0 = pk8<0>(W), w1 = pk8<1>(W);
 #pragma unroll
-  for (int t = 0; t < 16; ++t) {
-    O[0] = FM_MFMA(W[t], ub[0][t], O[0]);
-    O[1] = FM_MFMA(W[t], ub[1][t], O[1]);
+    for (int cc = 0; cc < 2; ++cc) {
+      O[cc] = FM_MFMA_BF16(w0, pk8(ub[cc]), O[cc]);
+      O[cc] = FM_MFMA_BF16(w1, pk8(ub[cc] + 8), O[cc]);
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      O[0] = FM_MFMA(W[t], ub[0][t], O[0]);
+      O[1] = FM_MFMA(W[t], ub[1][t], O[1]);
+    }
   }
 }
 
@@ -346,7 +429,7 @@ __global__ __launch_bounds__(64) void linear_fwd_kernel(const T* __restrict__ q,
 
     // the previous tile joins the state
     kc.ready();
-    state_update(S1, kc.x, vc.x);
+    state_update<T>(S1, kc.x, vc.x);
     {
       float ks[2], vs[2];
       column_sums(kc.x, ks);
@@ -384,7 +467,7 @@ __global__ __launch_bounds__(64) void linear_fwd_kernel(const T* __restrict__ q,
 
     // intra-tile part: weights x values
     vc.ready();
-    weight_product(P, vc.x, O);
+    weight_product<T>(P, vc.x, O);
 
     // denominators move from "lane = token" to the row order of the output registers
     if (L.l < 32 && L.l >= skip) dh[(int64_t)(base + L.l) * den_stride] = den_i;
@@ -465,7 +548,7 @@ __global__ __launch_bounds__(64) void linear_dq_kernel(const T* __restrict__ go,
     }
 
     // the previous tile joins the state
-    state_update(S, vc, kc);
+    state_update<T>(S, vc, kc);
     {
       float ks[2];
       column_sums(kc, ks);
@@ -514,7 +597,7 @@ __global__ __launch_bounds__(64) void linear_dq_kernel(const T* __restrict__ go,
     rows_from_lanes(c_cur, cl, L, cT);
     rows_from_lanes(inv_l, dl, L, inv);
 
-    weight_product(W, kc, O);
+    weight_product<T>(W, kc, O);
 
     float x[2][16];
 #pragma unroll
@@ -573,7 +656,7 @@ __global__ __launch_bounds__(64) void linear_dv_kernel(const T* __restrict__ go,
     const float inv_l = L.i < hi ? rcp(den_l) : 0.f;
 
     // the previous tile (its g rows already divided by den) joins the state
-    state_update(S, qc, gc);
+    state_update<T>(S, qc, gc);
     {
       float gs[2];
       column_sums(gc, gs);
@@ -604,7 +687,7 @@ __global__ __launch_bounds__(64) void linear_dv_kernel(const T* __restrict__ go,
 #pragma unroll
       for (int t = 0; t < 16; ++t) gc[c][t] *= inv[t];
 
-    weight_product(P, gc, O);
+    weight_product<T>(P, gc, O);
 
     float x[2][16];
 #pragma unroll
@@ -659,7 +742,7 @@ __global__ __launch_bounds__(64) void linear_dk_kernel(const T* __restrict__ go,
     rows_from_lanes(c_cur, cl, L, cT);
 
     // the previous tile (its g rows already divided by den) joins the state
-    state_update(S, gc, qc);
+    state_update<T>(S, gc, qc);
     r1[0] += r1next[0];
     r1[1] += r1next[1];
     FM_PIN();
@@ -694,7 +777,7 @@ __global__ __launch_bounds__(64) void linear_dk_kernel(const T* __restrict__ go,
       r1next[1] = half_swap_add(cb);
     }
 
-    weight_product(W, qc, O);
+    weight_product<T>(W, qc, O);
 
     float x[2][16];
 #pragma unroll
@@ -732,13 +815,7 @@ template <class T>
 __device__ __forceinline__ void state_only(const float (&own)[32], const f16v (&S)[2][2], f16v (&O)[2]) {
 #pragma unroll
   for (int t = 0; t < 16; ++t) O[0][t] = 0.f, O[1][t] = 0.f;
-#pragma unroll
-  for (int t = 0; t < 16; ++t)
-#pragma unroll
-    for (int rc = 0; rc < 2; ++rc) {
-      O[0] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][0][t], O[0]);
-      O[1] = FM_MFMA(own[Map<T>::tok_of(t, rc)], S[rc][1][t], O[1]);
-    }
+  own_times_state<T>(own, S, O);
 }
 
 template <class T, int MODE, bool NORM, bool ALIGNED>

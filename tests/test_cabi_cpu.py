@@ -84,23 +84,27 @@ def test_head_dimensions_and_the_dense_plan(built, monkeypatch):
 
 
 def test_kernel_choice_for_p1(built, monkeypatch):
-    """p = 1 at d = 32 / 64 stays with the moment kernels except for bf16 inputs under the mask past 1024 keys:
-    there the dense kernels' linear mode runs, unless the one-scan-per-head kernels (d = 64, ungrouped heads,
-    >= 512 of them) have heads enough to fill about three quarters of a round of 1024 waves."""
+    """p = 1 at d = 32 / 64 stays with the moment kernels except for bf16 inputs under the mask past 1024 keys
+    when the one-scan-per-head kernels are not there to take them (d = 64, ungrouped heads, no key prefix,
+    at least 208 heads with bf16 tensors): then the dense kernels' linear mode runs."""
     monkeypatch.delenv("FASTMAX_PATH")
     uses = lambda **kw: built.fastmax_uses_dense_tiles(C.byref(desc(p=1, **kw)))
     assert uses(bh=96, n=2048, dtype=1, mask=True) == 1
-    assert uses(bh=512, n=16384, dtype=1, mask=True) == 1
-    assert uses(bh=749, n=4096, dtype=1, mask=True) == 1
-    assert uses(bh=750, n=4096, dtype=1, mask=True) == 0
+    assert uses(bh=207, n=4096, dtype=1, mask=True) == 1
+    assert uses(bh=208, n=4096, dtype=1, mask=True) == 0
+    assert uses(bh=512, n=16384, dtype=1, mask=True) == 0
     assert uses(bh=1024, n=10000, dtype=1, mask=True) == 0
-    assert uses(bh=1100, n=4096, dtype=1, mask=True) == 1      # (a second round of scans for 76 heads)
     assert uses(bh=1024, bhkv=256, n=4096, dtype=1, mask=True) == 1   # (grouped heads: no scan kernels)
     assert uses(bh=1024, n=4096, d=32, dtype=1, mask=True) == 1       # (d = 32: no scan kernels)
+    assert uses(bh=1024, n=4096, nk=5000, dtype=1, mask=True) == 1    # (a key prefix: no scan kernels)
     assert uses(bh=96, n=1024, dtype=1, mask=True) == 0
     assert uses(bh=96, n=2048, dtype=1, mask=False) == 0
     assert uses(bh=96, n=2048, dtype=0, mask=True) == 0
     assert uses(bh=96, n=2048, d=48, dtype=0, mask=True) == 1
+    # the scan kernels keep no states: with bf16 tensors from 208 heads on, with fp32 tensors from 512
+    tiny = lambda **kw: built.fastmax_workspace_bytes(C.byref(desc(p=1, mask=True, n=1000, **kw)), _cabi.PASS_FORWARD)
+    assert tiny(bh=208, dtype=1) == 2 * 256 * ((208 * 8 + 255) // 256) and tiny(bh=207, dtype=1) > 1 << 16
+    assert tiny(bh=511, dtype=0) > 1 << 16
 
 
 def test_grouped_heads_descriptor(built):
