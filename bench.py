@@ -565,7 +565,8 @@ def measure(name: str, args, full: bool) -> dict:
 
 
 # the other configurations of the benchmark set, timed after the headline in the same process
-CONFIG_BLOCK = ("c1", "c2", "headline-unmasked", "headline-p1", "headline-unmasked-p1", "c4", "c5-layer", "c5-layer-p1")
+CONFIG_BLOCK = ("c1", "c2", "headline-unmasked", "headline-p1", "headline-unmasked-p1", "headline-p1-bf16", "c4", "c5-layer",
+                "c5-layer-p1")
 
 
 def main() -> int:
