@@ -1,5 +1,6 @@
 """The register-resident scan kernels that serve causal p = 1 at head dim 64 once there are at
-least 512 heads (fastmax_amd/csrc/fm_linear.h), through the C ABI: parity with the fp64 closed
+least 512 heads (208 with bf16 tensors, whose contractions run on the bf16 matrix instruction;
+fastmax_amd/csrc/fm_linear.h), through the C ABI: parity with the fp64 closed
 form (reference op sequence: example.py:183-193, 101-108) on whole tensors and on sampled heads,
 agreement with the chunked kernels the same call takes for fewer heads, and the dispatch
 conditions."""
@@ -11,7 +12,8 @@ from oracle import fastmax_oracle as O
 from helpers import TOL, assert_close
 
 pytestmark = pytest.mark.gpu
-BH = 512   # smallest head count that takes the scan kernels
+BH = 512   # smallest head count that takes the scan kernels with fp32 tensors
+BH_BF16 = 208   # ... with bf16 tensors
 
 
 @pytest.fixture(scope="module")
@@ -74,6 +76,17 @@ def test_bf16(ops):
     check_whole(ops, BH, 77, dtype=torch.bfloat16, seed=11, mask=True, normalize=True, p=1)
 
 
+@pytest.mark.parametrize("n", [32, 33, 65, 100, 333, 1030])
+def test_bf16_lengths_at_the_smallest_head_count(ops, n):
+    check_whole(ops, BH_BF16, n, dtype=torch.bfloat16, seed=n, mask=True, normalize=True, p=1)
+
+
+def test_bf16_coefficients_and_unnormalised(ops):
+    check_whole(ops, BH_BF16, 150, dtype=torch.bfloat16, seed=13, mask=True, normalize=True, p=1, a0=0.7, a1=1.3, lim=1.5)
+    check_whole(ops, BH_BF16, 150, dtype=torch.bfloat16, seed=14, mask=True, normalize=False, p=1, scale=0.1)
+    check_whole(ops, 1030, 90, dtype=torch.bfloat16, seed=15, mask=True, normalize=True, p=1)   # (more heads than SIMDs)
+
+
 def test_denominator_column_layout(ops):
     """o with row pitch d+1 and the denominator in column d (fastmax_cuda_forward.cu:353)."""
     q, k, v, go = (t.cuda() for t in O.seeded_inputs((BH, 90, 64), seed=12))
@@ -93,16 +106,18 @@ def test_denominator_column_layout(ops):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_agrees_with_the_chunked_kernels(ops, dtype):
-    """The same heads in one call (scan kernels) and in two calls of 256 heads (chunked kernels)."""
+    """The same heads in one call (scan kernels) and in calls of fewer heads than the scan takes (chunked kernels)."""
     n = 1500
     g = torch.Generator(device="cuda").manual_seed(3)
     q, k, v, go = (torch.randn((BH, n, 64), device="cuda", generator=g).to(dtype) for _ in range(4))
     kw = dict(mask=True, normalize=True, p=1)
     one = fwd_bwd(ops, q, k, v, go, **kw)
-    halves = [fwd_bwd(ops, q[s], k[s], v[s], go[s], **kw) for s in (slice(0, 256), slice(256, 512))]
+    step = 256 if dtype == torch.float32 else 128
+    parts = [fwd_bwd(ops, q[s:s + step], k[s:s + step], v[s:s + step], go[s:s + step], **kw) for s in range(0, BH, step)]
     tol = 2e-5 if dtype == torch.float32 else 1e-2
-    for name, a, b0, b1 in zip(("o", "den", "dq", "dk", "dv"), one, *halves):
-        assert_close(name, a.float(), torch.cat([b0, b1]).float().reshape(a.shape), tol)
+    for idx, name in enumerate(("o", "den", "dq", "dk", "dv")):
+        a = one[idx]
+        assert_close(name, a.float(), torch.cat([pt[idx] for pt in parts]).float().reshape(a.shape), tol)
 
 
 def test_long_sequence_sampled_heads(ops):
