@@ -289,12 +289,13 @@ struct Shape {
 // the chunks (lin_scan_kernel; unmasked: their plain sum) turns them into what each chunk needs, and
 // the three dense kernels start from that state and walk only their own chunk's score tiles.  Cost per
 // token: ~lchunk d (tiles) + ~4 d^2 (state), whatever the sequence length, for every head dimension.
-// The states are built from the rows as stored (no normaliser scale): the kernels' register-side operands
-// and epilogues carry the scales, as in the tile part.
+// The states are sums over the rows as stored; the normaliser scales ride on the kernels' register-side
+// operands and epilogues, as in the tile part, except where a whole block can carry them (below).
 //
 // A state slot in memory: nblk blocks of DP rows x LD floats -- the DP x DP part sum X (x) Y, times a
-// constant the consumer wants folded in, as [x][y] ("natural") and / or [y][x] ("transposed"), whichever
-// layouts the consumers read rows of -- then the vectors: sum_t e_t X_t, sum_t Y_t, and sum_t e_t.
+// constant the consumer wants folded in (a1; on the query side a1 times the head's query scale), as [x][y]
+// ("natural") and / or [y][x] ("transposed"), whichever layouts the consumers read rows of -- then the
+// vectors as they are: sum_t e_t X_t, sum_t Y_t, and sum_t e_t.
 // ---------------------------------------------------------------------------------------
 template <int DP>
 struct LinState {
