@@ -185,7 +185,7 @@ int fastmax_backward_strided(const fastmax_desc* desc, const fastmax_layout* lay
  * fp32 per-chunk partial states the forward pass adds up.)  Kernels that keep nothing answer the
  * size query with a token 256 bytes: the buffer is then left untouched and the two calls need the
  * workspace of fastmax_forward / fastmax_backward.  Those are the one register-resident scan per
- * head of causal p = 1 at d = 64 with at least 512 heads (workspace: per-head and per-token scalars
+ * head of causal p = 1 at d = 64 with at least 512 heads (bf16: 208; workspace: per-head and per-token scalars
  * only) and the dense score tiles (fastmax_uses_dense_tiles; their workspace holds scalars -- and for
  * p = 1 past 1024 causal / 512 unmasked positions the chunk states of their linear mode, which both
  * passes rebuild). */
