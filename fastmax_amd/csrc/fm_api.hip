@@ -157,7 +157,7 @@ bool use_linear_scan(const fastmax_desc* ds, const Plan& pl);
 // fills the chip badly and the dense kernels stay ahead for longer).  A causal sequence of a single chunk
 // has no states to build either way and stays with the moment kernels' own intra-chunk tiles.  Head
 // dimensions without moment kernels always take the dense ones (p = 1 at d = 32 / 64: see below).
-bool use_dense(const fastmax_desc* ds) {
+bool use_dense(const fastmax_desc* ds, bool plain = true) {
   if (ds->d != 32 && ds->d != 64) return true;
   // FASTMAX_PATH = moments | dense overrides the choice where both kernel families exist
   if (const char* e = getenv("FASTMAX_PATH")) {
@@ -168,11 +168,11 @@ bool use_dense(const fastmax_desc* ds) {
   if (ds->p != 2) {
     // p = 1: the moment states are tiny and the moment kernels win -- except for bf16 inputs under the mask
     // past 1024 keys with too few heads for the one-scan-per-head kernels (linear_min_heads; or no such kernels:
-    // d = 32, grouped heads, a key prefix, a1 = 0): there the dense kernels' linear mode (chunk states plus the
+    // d = 32, grouped heads, a key prefix, a1 = 0, strided tensors): there the dense kernels' linear mode (chunk states plus the
     // own chunk's tiles, all of it parallel over heads and chunks) beats the chunked moment kernels at every
     // head count measured (16 .. 768 heads: 1.0 - 1.4x)
     if (!(bf && ds->mask && ds->nk > 1024)) return false;
-    const bool scan = ds->d == 64 && ds->bh == ds->bhkv && ds->nq == ds->nk && ds->a1 != 0.f && ds->bh >= linear_min_heads(ds);
+    const bool scan = plain && ds->d == 64 && ds->bh == ds->bhkv && ds->nq == ds->nk && ds->a1 != 0.f && ds->bh >= linear_min_heads(ds);
     return !scan;
   }
   int limit;
@@ -190,7 +190,7 @@ bool use_dense(const fastmax_desc* ds) {
 Plan make_plan(const fastmax_desc* ds, int pass, bool plain = true, bool allow_dense = true) {
   Plan pl;
   pl.pass = pass;
-  pl.dense = allow_dense && use_dense(ds);
+  pl.dense = allow_dense && use_dense(ds, plain);
   pl.d = ds->d;
   pl.p2 = ds->p == 2;
   pl.masked = ds->mask != 0;

@@ -385,3 +385,41 @@ def test_linear_mode_is_what_bf16_causal_p1_runs_on_by_default(ops, monkeypatch)
         fold = lambda t: t.reshape(bhkv, r, *t.shape[1:]).sum(1)
         for name, got, ref in (("o", o, ro), ("dq", dq, rdq), ("dk", dk, fold(rdk)), ("dv", dv, fold(rdv))):
             assert_close(name, got.float(), ref, TOL[torch.bfloat16], atol=1e-6)
+
+
+def test_strided_views_with_many_heads_take_the_linear_mode(built, monkeypatch):
+    """bf16 causal p = 1 past 1024 keys with enough heads for the one-scan-per-head kernels, but as strided views of
+    a fused projection, which those kernels do not read: left to itself the library takes the dense kernels' linear
+    mode then (contiguous tensors of the same shape take the scan).  Checked against the fp64 closed form on a
+    few heads and against the contiguous call on all of them."""
+    import ctypes as C
+    from fastmax_amd import _cabi, ops as _ops, rope as R
+
+    monkeypatch.delenv("FASTMAX_PATH")
+    b, t, g, r, hs = 20, 1100, 12, 1, 64      # 240 heads
+    gen = torch.Generator().manual_seed(5)
+    qkv = torch.randn((b, t, g * (r + 2) * hs), generator=gen).to(torch.bfloat16)
+    gy = torch.randn((b, t, g * r * hs), generator=gen).to(torch.bfloat16)
+    x = qkv.cuda().requires_grad_(True)
+    y = R.qkv_attention(x, None, None, g, r, hs, rope_n=0, mask=True, normalize=True, p=1)
+    y.backward(gy.cuda())
+    v5 = qkv.view(b, t, g, r + 2, hs)
+    q = v5[:, :, :, 0].permute(0, 2, 1, 3).reshape(b * g, t, hs).contiguous()
+    k = v5[:, :, :, 1].permute(0, 2, 1, 3).reshape(b * g, t, hs).contiguous()
+    v = v5[:, :, :, 2].permute(0, 2, 1, 3).reshape(b * g, t, hs).contiguous()
+    go = gy.view(b, t, g, hs).permute(0, 2, 1, 3).reshape(b * g, t, hs).contiguous()
+    got_o = y.view(b, t, g, hs).permute(0, 2, 1, 3).reshape(b * g, t, hs)
+    gx = x.grad.view(b, t, g, 3, hs)
+    got = [got_o] + [gx[:, :, :, j].permute(0, 2, 1, 3).reshape(b * g, t, hs) for j in range(3)]
+    kw = dict(mask=True, normalize=True, p=1)
+    heads = [0, 117, 239]
+    ref = O.dense_truth(q[heads].float(), k[heads].float(), v[heads].float(), go[heads].float(), **kw)
+    for name, a, want in zip(("o", "dq", "dk", "dv"), got, ref):
+        assert_close(name, a[heads].float().cpu(), want, TOL[torch.bfloat16], atol=1e-6)
+    # the contiguous call: the scan kernels (same descriptor, plain layout)
+    qd, kd, vd, god = (z.cuda() for z in (q, k, v, go))
+    assert _cabi.load().fastmax_uses_dense_tiles(C.byref(_ops._desc(qd, kd, True, True, 1, 1.0, 1.0, 1.0, 1.0, 0.5))) == 0
+    o2, den2, sc2, arg2 = _ops.forward(qd, kd, vd, **kw)
+    g2 = _ops.backward(qd, kd, vd, o2, den2, god, qk_scale=sc2, qk_argmax=arg2, **kw)
+    for name, a, b2 in zip(("o", "dq", "dk", "dv"), got, (o2,) + tuple(g2)):
+        assert_close(name, a.float(), b2.float(), 3e-2, atol=1e-6)
