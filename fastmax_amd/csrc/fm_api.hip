@@ -961,9 +961,14 @@ int dense_forward(const fastmax_desc* ds, const Plan& pl, const Layout& L, const
 
 template <int DP, class T>
 int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, const T* q, const T* k, const T* v,
-                      const float* den, int64_t den_stride, const T* go, T* dq, T* dk, T* dv, const float* scale,
-                      const float* cvec, float* rpart, float* kstate, float* qstate, int* nbq_out, int* nbk_out,
-                      hipStream_t stream) {
+                      const T* o, const float* den, int64_t den_stride, const T* go, T* dq, T* dk, T* dv,
+                      const float* scale, float* cvec_w, float* rpart, float* kstate, float* qstate, int* nbq_out,
+                      int* nbk_out, hipStream_t stream) {
+  // c_i = grad_out_i . out_i / den_i: the dq kernel forms it from rows it holds anyway and leaves it in cvec for the
+  // dk / dv kernel -- except in the linear mode, whose query-side states need it before any of them runs
+  const bool prep_in_dq = !pl.lin;
+  if (!prep_in_dq) FM_TRY((launch_bwd_prep<T>(pl, L, go, o, den, den_stride, cvec_w, stream)));
+  const float* cvec = cvec_w;
   using S = dense::Shape<DP, T>;
   constexpr int BN = S::BN;
   const int npos = pl.masked ? pl.nk : pl.nq;
@@ -988,7 +993,8 @@ int dense_backward_dp(const fastmax_desc* ds, const Plan& pl, const Layout& L, c
     ScopedKernel sk(FASTMAX_K_BWD_DQ, stream);
     kern<<<dim3(pl.bh, nb), 64 * NW, smem, stream>>>(qr, gr, dn, cv, kr, vr, scale, scale + pl.bh, mk_rows(dq, L.dq, 0, pl.off), rq,
                                                  npos, pl.nk, ds->d, pl.masked, pl.p2 && a2 != 0.f, ds->a1, a2, pl.ratio,
-                                                 ksl, pl.lchunk, pl.lslots);
+                                                 ksl, pl.lchunk, pl.lslots, mk_rows(o, L.o, 0, pl.off),
+                                                 prep_in_dq ? mk_scalars<float>(cvec_w, pl.nq, 1, 0, pl.off) : RowScalarsOut{nullptr, 0, 0});
     FM_TRY(launch_status("dense_dq_kernel"));
   }
   {
@@ -1030,10 +1036,9 @@ int dense_backward(const fastmax_desc* ds, const Plan& pl, const Layout& L, cons
   float* qstate = kstate;
   if (pl.lin) qstate = reinterpret_cast<float*>(p + align256((size_t)pl.bhkv * pl.lslots * lin_state_floats(pl.ldp, 1) * sizeof(float)));
   if (!given) FM_TRY(compute_scales<T>(ds, L, q, k, scale_ws, arg_ws, stream));
-  FM_TRY((launch_bwd_prep<T>(pl, L, go, o, den, den_stride, cvec, stream)));
   int nbq = 0, nbk = 0;
-#define FM_DENSE_BWD(DP)                                                                                          \
-  FM_TRY((dense_backward_dp<DP, T>(ds, pl, L, q, k, v, den, den_stride, go, dq, dk, dv, scale, cvec, rpart, kstate, \
+#define FM_DENSE_BWD(DP)                                                                                              \
+  FM_TRY((dense_backward_dp<DP, T>(ds, pl, L, q, k, v, o, den, den_stride, go, dq, dk, dv, scale, cvec, rpart, kstate, \
                                    qstate, &nbq, &nbk, stream)))
   if (ds->d <= 32) FM_DENSE_BWD(32);
   else if (ds->d <= 64) FM_DENSE_BWD(64);

@@ -240,6 +240,37 @@ __device__ __forceinline__ void load_own_frags(const HeadRows<const T>& hr, int 
   }
 }
 
+// The own-row fragments of g = grad_out / den for position pos, and c = grad_out . out / den of that row (the lane
+// half's channels summed with the other half's): what a separate pass over grad_out and out would leave in memory.
+template <int DP, class T>
+__device__ __forceinline__ float load_g_frags_and_c(const HeadRows<const T>& gr, const HeadRows<const T>& orow, int pos,
+                                                    int pend, int d, int hh, float rden,
+                                                    typename Mma<T>::Frag (&f)[DP / Mma<T>::KF]) {
+  using M = Mma<T>;
+  const bool live = pos >= gr.lo && pos < pend;
+  const int ps = max(pos < pend ? pos : pend - 1, gr.lo);
+  const T* grow = gr.base + (unsigned)ps * gr.pitch;
+  const T* orw = orow.base + (unsigned)ps * orow.pitch;
+  float dot = 0.f;
+#pragma unroll
+  for (int m = 0; m < DP / M::KF; ++m) {
+    const int ch = M::KF * m + M::EPL * hh;
+    const bool ok = live && ch < d;
+    const uint4 tg = *reinterpret_cast<const uint4*>(grow + (ok ? ch : 0));
+    const uint4 to = *reinterpret_cast<const uint4*>(orw + (ok ? ch : 0));
+    float x[M::EPL], y[M::EPL];
+    M::unpack(tg, x);
+    M::unpack(to, y);
+#pragma unroll
+    for (int e = 0; e < M::EPL; ++e) {
+      dot += ok ? x[e] * y[e] : 0.f;
+      x[e] = ok ? x[e] * rden : 0.f;
+    }
+    f[m] = __builtin_bit_cast(typename M::Frag, M::pack(x));
+  }
+  return (dot + __shfl_xor(dot, 32, 64)) * rden;
+}
+
 // LDS layout shared by the three kernels: NA row-major and NT transposed streamed tiles per buffer, two
 // buffers, then `tail` floats.
 template <int DP, class T, int BN>
@@ -729,14 +760,16 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_FWD)) void dense_fwd_ke
 // ---------------------------------------------------------------------------------------
 // dq.  Same walk as the forward pass; the own rows carry q (times 2 a2, so that the score accumulator,
 // started at a1, is f'(s)) and g = grad_out / den.  rpart[head * gridDim.y + block] receives the block's
-// sum of dqh . qh for the normalisation chain rule (when rpart is given).
+// sum of dqh . qh for the normalisation chain rule (when rpart is given).  cprep given: c is not read from cvec
+// but formed from OUTF, the forward output, and written to cprep (the same array) for the kernel that runs after
+// this one.
 // ---------------------------------------------------------------------------------------
 template <int DP, class T, int RT, int BN, int NW>
 __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kernel(
     Rows<const T> Q, Rows<const T> GO, RowScalars den, RowScalars cvec, Rows<const T> K, Rows<const T> V,
     const float* __restrict__ qscale, const float* __restrict__ kscale, Rows<T> DQ, float* __restrict__ rpart,
     int npos, int nk, int d, int masked, int p2, float a1, float a2, int ratio, const float* __restrict__ lstate,
-    int lchunk, int lslots) {
+    int lchunk, int lslots, Rows<const T> OUTF, RowScalarsOut cprep) {
   using M = Mma<T>;
   using Elt = typename M::Elt;
   using Frag = typename M::Frag;
@@ -759,6 +792,7 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kern
   const HeadRows<const T> Qh = Q.head(head), Gh = GO.head(head), Kh = K.head(hkv), Vh = V.head(hkv);
   const float* denh = den.head(head);
   const float* ch = cvec.head(head);
+  float* cw = cprep.head(head);
   const float kq = qscale[head] * kscale[hkv];
 
   Frag qf[RT][NF], gf[RT][NF];
@@ -770,11 +804,18 @@ __global__ __launch_bounds__(64 * NW, (Shape<DP, T>::OCC_DQ)) void dense_dq_kern
     const int ps = max(pos < npos ? pos : npos - 1, Qh.lo);
     // (clamped loads whose values are used whatever `live` says: the compiler moves a load that only one side of a
     // select uses under that condition, where it gets a wait of its own -- for every load issued before it)
-    const float dnv = denh[(int64_t)ps * den.stride], cvv = ch[(int64_t)ps * cvec.stride], lm = live ? 1.0f : 0.f;
+    const float dnv = denh[(int64_t)ps * den.stride], lm = live ? 1.0f : 0.f;
     const float rden = lm / dnv;
-    cown[rt] = lm * cvv;
     if (p2) load_own_frags<DP, T>(Qh, pos, npos, d, hh, kq * 2.0f * a2, qf[rt]);
-    load_own_frags<DP, T>(Gh, pos, npos, d, hh, rden, gf[rt]);
+    if (cw) {   // (block-uniform)
+      // c_i = grad_out_i . out_i / den_i is formed here from rows the block reads anyway (plus those of out) and left
+      // in cvec for the dk / dv kernel: no separate pass over grad_out and out
+      cown[rt] = load_g_frags_and_c<DP, T>(Gh, OUTF.head(head), pos, npos, d, hh, rden, gf[rt]);
+      if (live && hh == 0) cw[(int64_t)pos * cprep.stride] = cown[rt];
+    } else {
+      cown[rt] = lm * ch[(int64_t)ps * cvec.stride];
+      load_own_frags<DP, T>(Gh, pos, npos, d, hh, rden, gf[rt]);
+    }
   }
 
   const int kend = masked ? (tok0 + BM < nk ? tok0 + BM : nk) : nk;
