@@ -175,13 +175,14 @@ bool use_dense(const fastmax_desc* ds, bool plain = true) {
     const bool scan = plain && ds->d == 64 && ds->bh == ds->bhkv && ds->nq == ds->nk && ds->a1 != 0.f && ds->bh >= linear_min_heads(ds);
     return !scan;
   }
+  const bool few = ds->bh <= 128;   // (few heads: the moment form's sequential state build fills the chip badly)
   int limit;
   if (ds->d == 64) {
-    if (ds->mask) limit = bf ? (ds->bh <= 128 ? 4096 : 3072) : 2560;
-    else limit = bf ? 1536 : 1024;
+    if (ds->mask) limit = bf ? (few ? 5632 : 4096) : (few ? 3584 : 3072);
+    else limit = bf ? (few ? 2048 : 1536) : 1024;
   } else {
-    if (ds->mask) limit = bf ? 1536 : 768;
-    else limit = bf ? 768 : 512;
+    if (ds->mask) limit = bf ? (few ? 3072 : 2048) : (few ? 1536 : 1024);
+    else limit = bf ? (few ? 1024 : 768) : 512;
   }
   if (ds->mask && ds->nk <= chunk_for(ds->d, 1, ds->dtype)) return false;
   return ds->nk <= limit;

@@ -199,6 +199,7 @@ def test_config5_attention_shape_picks_the_dense_kernels(ops, monkeypatch, built
     ((2, 2, 3, 2), True, torch.float32), ((1, 3, 200, 16), True, torch.float32), ((2, 2, 150, 48), True, torch.float32),
     ((1, 2, 90, 20), False, torch.float32), ((1, 2, 300, 128), True, torch.float32), ((2, 2, 260, 96), False, torch.float32),
     ((1, 2, 300, 128), True, torch.bfloat16), ((1, 2, 200, 100), True, torch.bfloat16), ((1, 2, 3000, 48), True, torch.float32),
+    ((1, 2, 3700, 48), True, torch.float32),
     ((2, 2, 600, 48), True, torch.float32),
 ])
 def test_module_head_dims(built, monkeypatch, shape, mask, dtype):
@@ -211,7 +212,7 @@ def test_module_head_dims(built, monkeypatch, shape, mask, dtype):
 
     monkeypatch.delenv("FASTMAX_PATH", raising=False)
     b, h, n, d = shape
-    expect = {2: 32, 16: 16, 48: 48 if 256 < n <= 2560 else 64, 20: 20, 128: 128, 96: 96, 100: 104}[d]
+    expect = {2: 32, 16: 16, 48: 48 if 256 < n <= 3584 else 64, 20: 20, 128: 128, 96: 96, 100: 104}[d]
     assert kernel_head_dim(d, dtype, b * h, b * h, n, n, mask, 2) == expect
     q, k, v, go = O.seeded_inputs(shape, seed=24, dtype=dtype)
     qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
