@@ -272,24 +272,33 @@ struct RowTile {
   using Raw = typename std::conditional<std::is_same<T, float>::value, float4, uint2>::type;
   Raw raw[NV];
   float rdiv[NV];  // per-row divisors fetched by load(), applied by the stores
-  bool live[NV];
+  uint32_t keep[NV];   // all ones for a row inside the range, zero for one outside: the stores AND it in
   __device__ __forceinline__ static int row_of(int idx) { return ROWFAST ? idx % ROWS : idx / VPR; }
   __device__ __forceinline__ static int c4_of(int idx) { return ROWFAST ? idx / ROWS : idx % VPR; }
-  __device__ __forceinline__ static void unpack(const float4& r, float (&o)[4]) {
-    o[0] = r.x; o[1] = r.y; o[2] = r.z; o[3] = r.w;
+  // whether piece idx exists (compile-time true when the pieces fill the block's sweeps)
+  __device__ __forceinline__ static bool has(int idx) { return TOTAL % 256 == 0 || idx < TOTAL; }
+  __device__ __forceinline__ static void unpack(const float4& r, uint32_t k, float (&o)[4]) {
+    o[0] = __uint_as_float(__float_as_uint(r.x) & k);
+    o[1] = __uint_as_float(__float_as_uint(r.y) & k);
+    o[2] = __uint_as_float(__float_as_uint(r.z) & k);
+    o[3] = __uint_as_float(__float_as_uint(r.w) & k);
   }
-  __device__ __forceinline__ static void unpack(const uint2& r, float (&o)[4]) {
-    o[0] = __uint_as_float(r.x << 16);
-    o[1] = __uint_as_float(r.x & 0xffff0000u);
-    o[2] = __uint_as_float(r.y << 16);
-    o[3] = __uint_as_float(r.y & 0xffff0000u);
+  __device__ __forceinline__ static void unpack(const uint2& r, uint32_t k, float (&o)[4]) {
+    const uint32_t x = r.x & k, y = r.y & k;
+    o[0] = __uint_as_float(x << 16);
+    o[1] = __uint_as_float(x & 0xffff0000u);
+    o[2] = __uint_as_float(y << 16);
+    o[3] = __uint_as_float(y & 0xffff0000u);
   }
-  // piece u converted, times `scale` over the row's divisor; zero for a row past the end
+  // piece u converted, times `scale` over the row's divisor; zero for a row outside the range.  The mask
+  // goes on as bits, on the piece and on the factor (whose divisor is that of the nearest row inside): as
+  // a choice between the value and zero it would become a branch around the use of the fetched registers,
+  // and a loop that reuses them would then have to wait for every older memory operation first.
   __device__ __forceinline__ void piece(int u, float scale, float (&o)[4]) const {
-    const float sc = live[u] ? scale / rdiv[u] : 0.f;
-    unpack(raw[u], o);
+    const float sc = __uint_as_float(__float_as_uint(scale / rdiv[u]) & keep[u]);
+    unpack(raw[u], keep[u], o);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = live[u] ? o[e] * sc : 0.f;
+    for (int e = 0; e < 4; ++e) o[e] *= sc;
   }
 
   // rows tok0.. of one head; rows outside [lo, n) read as zero (they are fetched from the nearest
@@ -303,7 +312,7 @@ struct RowTile {
       const bool in = idx < TOTAL;
       const int row = in ? row_of(idx) : 0, c4 = in ? c4_of(idx) : 0;
       const int tok = tok0 + row;
-      live[u] = in && tok < n && tok >= hr.lo;
+      keep[u] = (in && tok < n && tok >= hr.lo) ? 0xffffffffu : 0u;
       const int tk = max(tok < n ? tok : n - 1, hr.lo);
       raw[u] = *reinterpret_cast<const Raw*>(hr.base + ((unsigned)tk * hr.pitch + (unsigned)(c4 * 4)));
       rdiv[u] = 1.0f;
@@ -316,7 +325,7 @@ struct RowTile {
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
-      if (idx < TOTAL) {
+      if (has(idx)) {
         float x[4];
         piece(u, scale, x);
         *reinterpret_cast<float4*>(dst + row * ld + c4 * 4) = make_float4(x[0], x[1], x[2], x[3]);
@@ -329,7 +338,7 @@ struct RowTile {
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
-      if (idx < TOTAL) {
+      if (has(idx)) {
         float x[4];
         piece(u, scale, x);
 #pragma unroll
@@ -343,7 +352,7 @@ struct RowTile {
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
-      if (idx < TOTAL) {
+      if (has(idx)) {
         float x[4];
         piece(u, scale, x);
         const uint32_t p01 = pack_bf2(x[0], x[1]), p23 = pack_bf2(x[2], x[3]);
@@ -360,7 +369,7 @@ struct RowTile {
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
-      if (idx < TOTAL) {
+      if (has(idx)) {
         float x[4];
         piece(u, scale, x);
         *reinterpret_cast<uint2*>(dst + row * ld + c4 * 4) = make_uint2(pack_bf2(x[0], x[1]), pack_bf2(x[2], x[3]));
@@ -373,7 +382,7 @@ struct RowTile {
     for (int u = 0; u < NV; ++u) {
       const int idx = tid + u * 256;
       const int row = row_of(idx), c4 = c4_of(idx);
-      if (idx < TOTAL) {
+      if (has(idx)) {
         float x[4];
         piece(u, scale, x);
 #pragma unroll
