@@ -47,20 +47,20 @@ COEF = dict(a0=1.0, a1=1.0, a2=0.5, lim=1.0, normalize=True, temperature=1.0)
 # summarised under profiles/ (counter KiB per dispatch, scaled by the factors a 1 GiB copy reads: fetch
 # x2.0, write x1.0).  The summaries of the chunked kernels list the figure per kernel ("... B per
 # token-head"); it is read from the committed file at run time, so it changes with the profile and not
-# with an edit here.  The scan-kernel summary lists GiB per launch only: its figures are kept here
-# (algorithmic: 1024 B per token-head and kernel, 1280 B for dq, which also reads the forward output).
+# with an edit here.  The scan-kernel summaries list scaled GiB per launch (of the headline shape, 64 x 16 heads x
+# 10000 tokens); algorithmic: four tensors per token-head and kernel, five for dq, which also reads the forward output.
 TRAFFIC_SOURCE = {"headline": "profiles/headline_causal_fp32_all_kernels.txt",
                   "c4": "profiles/config4_causal_bf16_all_kernels.txt",
-                  "headline-p1": "profiles/headline_p1_causal_fp32_scan_kernels.txt"}
-SCAN_TRAFFIC_BYTES_PER_TOKEN_HEAD = {"fwd_apply": 1164.0, "bwd_dq": 1504.0, "bwd_dk": 1186.0, "bwd_dv": 1178.0}
+                  "headline-p1": "profiles/headline_p1_causal_fp32_scan_kernels.txt",
+                  "headline-p1-bf16": "profiles/headline_p1_causal_bf16_scan_kernels.txt"}
+_SCAN_KERNEL_CLASS = {"linear_fwd_kernel": "fwd_apply", "linear_dq_kernel": "bwd_dq", "linear_dk_kernel": "bwd_dk",
+                      "linear_dv_kernel": "bwd_dv"}
 _PROFILE_KERNEL_CLASS = (("build_kernel", None, "build"), ("apply_kernel", 0, "fwd_apply"), ("apply_kernel", 1, "bwd_dv"),
                          ("grad_kernel", 0, "bwd_dq"), ("grad_kernel", 1, "bwd_dk"))
 
 
 def measured_traffic_bytes_per_token_head(workload: str) -> dict:
     """{kernel class: HBM bytes per token-head (and state, for the build)} of a workload, or {}."""
-    if workload == "headline-p1":
-        return dict(SCAN_TRAFFIC_BYTES_PER_TOKEN_HEAD)
     path = TRAFFIC_SOURCE.get(workload)
     if path is None:
         return {}
@@ -69,6 +69,11 @@ def measured_traffic_bytes_per_token_head(workload: str) -> dict:
         return {}
     out = {}
     for line in open(path):
+        # scan kernels: "lin::linear_dq_kernel<...>   dispatches   FETCH KiB   WRITE KiB   scaled GiB/launch"
+        m = re.match(r"lin::(linear_\w+_kernel)<.*>\s+\d+\s+[\d.]+e[+-]\d+\s+[\d.]+e[+-]\d+\s+([\d.]+)\s*$", line)
+        if m and m.group(1) in _SCAN_KERNEL_CLASS:
+            out[_SCAN_KERNEL_CLASS[m.group(1)]] = float(m.group(2)) * 2.0 ** 30 / (64 * 16 * 10000)
+            continue
         m = re.match(r"\s+(\w+)<(.*)>\s+\d+ launches\s+[\d.]+ GB\s+([\d.]+) B per token-head", line)
         if not m:
             continue
@@ -501,6 +506,10 @@ def measure(name: str, args, full: bool) -> dict:
         n_states = n_builds if dom == "build" else 1
         roofline["traffic"] = per_th * token_heads * n_states / launches  # bytes per launch (profiled, not live)
         roofline["traffic_source"] = TRAFFIC_SOURCE[name]
+        if roofline["bound"] == "hbm":
+            # what the kernel really moved (the bf16 dq scan also reads q, for the normalisation sum), over its time
+            roofline["traffic_gbs"] = roofline["traffic"] / (roofline["avg_launch_ms"] * 1e-3) / 1e9
+            roofline["traffic_frac"] = roofline["traffic_gbs"] / PEAK_HBM_GBS
         # whole step: measured HBM bytes over the algorithmic 12 d es per token-head
         all_th = measured_traffic_bytes_per_token_head(name)
         if set(all_th) >= {"build", "fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv"}:

@@ -95,4 +95,11 @@ def test_traffic_figures_are_read_from_the_committed_profiles():
         t = bench.measured_traffic_bytes_per_token_head(workload)
         assert set(t) == {"build", "fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv"}, (workload, t)
         assert all(500.0 < v < 20000.0 for v in t.values()), (workload, t)
+    # the scan kernels' summaries list GiB per launch of the headline shape: four tensors of d elements per
+    # token-head and kernel at least, and dq (which also reads the forward output) moves the most
+    for workload, es in (("headline-p1", 4), ("headline-p1-bf16", 2)):
+        t = bench.measured_traffic_bytes_per_token_head(workload)
+        assert set(t) == {"fwd_apply", "bwd_dq", "bwd_dk", "bwd_dv"}, (workload, t)
+        assert all(4 * 64 * es <= v < 8 * 64 * es for v in t.values()), (workload, t)
+        assert max(t, key=t.get) == "bwd_dq"
     assert bench.measured_traffic_bytes_per_token_head("c2") == {}
