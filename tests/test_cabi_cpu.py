@@ -107,6 +107,35 @@ def test_kernel_choice_for_p1(built, monkeypatch):
     assert tiny(bh=511, dtype=0) > 1 << 16
 
 
+def test_kernel_choice_for_p2(built, monkeypatch):
+    """p = 2 at d = 32 / 64: the dense score tiles up to the measured crossover (key counts; the first figure
+    of a pair is for at most 128 heads), the moment kernels beyond; a causal sequence of a single chunk stays
+    with the moment kernels; other head dimensions have dense kernels only."""
+    monkeypatch.delenv("FASTMAX_PATH")
+    uses = lambda **kw: built.fastmax_uses_dense_tiles(C.byref(desc(p=2, **kw)))
+    table = [  # d, dtype (0 fp32, 1 bf16), mask, limit with few heads, limit with many
+        (64, 1, True, 5632, 4096), (64, 1, False, 2048, 1536), (64, 0, True, 3584, 3072), (64, 0, False, 1024, 1024),
+        (32, 1, True, 3072, 2048), (32, 1, False, 1024, 768), (32, 0, True, 1536, 1024), (32, 0, False, 512, 512),
+    ]
+    for d, dtype, mask, few, many in table:
+        for bh, limit in ((96, few), (128, few), (129, many), (768, many)):
+            assert uses(d=d, dtype=dtype, mask=mask, bh=bh, n=limit) == 1, (d, dtype, mask, bh, limit)
+            assert uses(d=d, dtype=dtype, mask=mask, bh=bh, n=limit + 1) == 0, (d, dtype, mask, bh, limit)
+    # a single causal chunk (384 positions for bf16, 256 for fp32 at d = 64, 128 at d = 32)
+    assert uses(d=64, dtype=1, mask=True, bh=96, n=384) == 0 and uses(d=64, dtype=1, mask=True, bh=96, n=385) == 1
+    assert uses(d=64, dtype=0, mask=True, bh=96, n=256) == 0 and uses(d=64, dtype=0, mask=True, bh=96, n=257) == 1
+    assert uses(d=32, dtype=0, mask=True, bh=96, n=128) == 0 and uses(d=32, dtype=0, mask=True, bh=96, n=129) == 1
+    assert uses(d=64, dtype=1, mask=False, bh=96, n=32) == 1
+    # the configurations of the benchmark: 1 and 3 (headline) and 4 on the moment kernels, 2 and 5 on the dense ones
+    assert uses(d=32, dtype=0, mask=False, bh=64, n=1024) == 0
+    assert uses(d=32, dtype=0, mask=True, bh=512, n=1000) == 1
+    assert uses(d=64, dtype=0, mask=True, bh=1024, n=10000) == 0
+    assert uses(d=64, dtype=1, mask=True, bh=512, n=16384) == 0
+    assert uses(d=64, dtype=1, mask=True, bh=96, n=2048) == 1
+    for d in (16, 48, 96, 128):
+        assert uses(d=d, dtype=0, mask=True, bh=4, n=20000) == 1
+
+
 def test_grouped_heads_descriptor(built):
     """bhkv must divide bh (fastmax_cuda_forward.cu:38 maps head i to key/value head i / (bh/bhkv)); the
     smallest workspace then holds one whole group."""
